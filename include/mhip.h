@@ -1,0 +1,192 @@
+/* mhip.h — C-ABI launch shim for the gfx950 (MI355X) kernel library.
+ *
+ * This is the boundary a host (the reference's Swift executor, the C++ host in
+ * this repository, or any FFI) binds in place of the reference's Metal kernel
+ * library: one entry point per fused operator, taking a HIP stream, raw device
+ * pointers, shape scalars and a small set of flags.  It mirrors the reference's
+ * kernel ABI — buffers in operand order, then outputs, then scalars
+ * (Sources/MetalHLOCore/Compiler/KernelTypes.swift:259-313,
+ *  Sources/MetalHLOCore/Compiler/CodeGenerator.swift:5681-5879).
+ *
+ * All tensors are dense row-major with the last dimension contiguous.
+ * Every call only enqueues work on `stream` (NULL = the default stream) and
+ * returns; nothing synchronises.  Return value: MHIP_OK or an MHIP_ERR_* code;
+ * mhip_last_error() then holds a message (thread-local).
+ */
+#ifndef MHIP_H
+#define MHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Element types use the numbering of MHLOElementType
+ * (Sources/CMetalHLO/include/metalhlo.h:62-76). */
+typedef enum {
+    MHIP_F16 = 0,
+    MHIP_F32 = 1,
+    MHIP_F64 = 2,
+    MHIP_BF16 = 3,
+    MHIP_I1 = 4,
+    MHIP_I8 = 5,
+    MHIP_I16 = 6,
+    MHIP_I32 = 7,
+    MHIP_I64 = 8,
+    MHIP_UI8 = 9,
+    MHIP_UI16 = 10,
+    MHIP_UI32 = 11,
+    MHIP_UI64 = 12
+} mhip_dtype;
+
+typedef enum {
+    MHIP_OK = 0,
+    MHIP_ERR_INVALID_ARGUMENT = 1, /* NULL pointer, non-positive size, misaligned buffer */
+    MHIP_ERR_UNSUPPORTED = 2,      /* dtype / shape outside what the kernels cover */
+    MHIP_ERR_LAUNCH = 3,           /* HIP reported an error for the launch */
+    MHIP_ERR_NO_DEVICE = 4
+} mhip_status;
+
+/* Activation of fused_matmul_bias_activation
+ * (Sources/MetalHLOCore/Compiler/IntegrationTypes.swift:328-355). */
+typedef enum {
+    MHIP_ACT_NONE = 0,
+    MHIP_ACT_RELU = 1,
+    MHIP_ACT_GELU = 2, /* tanh approximation, CustomCallHandlers.swift:540-558 */
+    MHIP_ACT_SILU = 3,
+    MHIP_ACT_TANH = 4,
+    MHIP_ACT_SIGMOID = 5
+} mhip_activation;
+
+/* Library / device ------------------------------------------------------- */
+
+/* Version string, static storage (cf. mhlo_version, metalhlo.h:23). */
+const char* mhip_version(void);
+
+/* Last error message of the calling thread, "" if none
+ * (cf. mhlo_get_last_error, metalhlo.h:53). */
+const char* mhip_last_error(void);
+
+/* Number of visible HIP devices; 0 when there is none. */
+int mhip_device_count(void);
+
+/* Device facts used by launch heuristics and reports: compute units, LDS bytes
+ * per workgroup, gcn arch name (written into `arch`, NUL-terminated). Replaces
+ * MTLDevice queries in Metal/Kernels/KernelRegistry.swift:122-165. */
+int mhip_device_info(int device, int* out_cus, int* out_lds_bytes, char* arch, size_t arch_len);
+
+/* Row operators (HBM-bound) ---------------------------------------------- */
+
+/* y = softmax(x) over the last axis of x[rows, cols].
+ * Replaces SoftmaxKernel (Metal/Kernels/SoftmaxKernel.swift:16-215) and
+ * generateSoftmaxSource (Compiler/CodeGenerator.swift:4690-4794).
+ * dtype: F32, F16, BF16 (16-bit types compute in fp32, one final rounding). */
+int mhip_softmax(void* stream, const void* x, void* y, int64_t rows, int64_t cols, int dtype);
+
+/* Softmax over a middle axis: x viewed as [outer, axis_len, inner], inner > 1.
+ * (Compiler/CodeGenerator.swift:4690-4697 general-axis variant.) */
+int mhip_softmax_strided(void* stream, const void* x, void* y, int64_t outer, int64_t axis_len,
+                         int64_t inner, int dtype);
+
+/* y = (x - mean) * rsqrt(var + eps) * gamma + beta over the last axis.
+ * gamma / beta may be NULL (layer_norm_no_affine_kernel).
+ * Replaces LayerNormKernel (Metal/Kernels/LayerNormKernel.swift:34-408);
+ * operand order [x, gamma, beta] of FusedLayerNormHandler
+ * (Compiler/CustomCallHandlers.swift:285-346). Variance is two-pass. */
+int mhip_layer_norm(void* stream, const void* x, const void* gamma, const void* beta, void* y,
+                    int64_t rows, int64_t cols, float eps, int dtype);
+
+/* y = x * rsqrt(mean(x^2) + eps) * gamma; gamma may be NULL.
+ * Replaces RMSNormKernel (Metal/Kernels/LayerNormKernel.swift:420-733). */
+int mhip_rms_norm(void* stream, const void* x, const void* gamma, void* y, int64_t rows,
+                  int64_t cols, float eps, int dtype);
+
+/* y = gelu_tanh(x + bias[col]); bias may be NULL (plain fused_gelu).
+ * Replaces GELUKernel (Metal/Kernels/GELUKernel.swift:15-123) and the epilogue
+ * of generateMatMulBiasActSource (Compiler/CodeGenerator.swift:4797-4850). */
+int mhip_bias_gelu(void* stream, const void* x, const void* bias, void* y, int64_t rows,
+                   int64_t cols, int dtype);
+
+/* dot_general ------------------------------------------------------------ */
+
+/* C[b] = act(op(A[b]) . op(B[b]) + bias[col]) for b in [0, batch).
+ * op(A) is [M,K] (stored [K,M] when trans_a), op(B) is [K,N] (stored [N,K]
+ * when trans_b); strides are in elements between consecutive batch matrices
+ * (0 broadcasts an operand).  bias (length N, same dtype) may be NULL.
+ * fp32 accumulate, one rounding at the store.  dtype: BF16, F16, F32.
+ * Replaces the kernel_matmul family and kernel_matmul_bias_act
+ * (Compiler/CodeGenerator.swift:3155-4068, 4797-4850); M/K/N/batch are what
+ * dotGeneralDims (:5939-5970) derives. */
+int mhip_gemm(void* stream, const void* a, const void* b, const void* bias, void* c, int64_t M,
+              int64_t N, int64_t K, int64_t batch, int64_t stride_a, int64_t stride_b,
+              int64_t stride_c, int trans_a, int trans_b, int activation, int dtype);
+
+/* Attention -------------------------------------------------------------- */
+
+/* O = softmax(scale * Q K^T + mask, causal) V.
+ * Q,O [B,H,Sq,D]; K,V [B,H,Skv,D]; mask NULL or additive [B,H,Sq,Skv] with
+ * batch/head strides `mask_stride_b`, `mask_stride_h` in elements (0 = broadcast).
+ * Causal rule: key position > query position is masked; a row with no
+ * unmasked key yields zeros.  fp32 softmax state and accumulation.
+ * Replaces FlashAttentionTiledKernel (Metal/Kernels/FlashAttentionKernel.swift:462-671)
+ * launched from MetalExecutor.executeFlashAttentionDirect
+ * (Runtime/MetalExecutor.swift:502-564). dtype: BF16, F16, F32. D in {64, 128}
+ * for the MFMA path; other D up to 256 take a scalar path. */
+int mhip_flash_attention(void* stream, const void* q, const void* k, const void* v,
+                         const void* mask, void* o, int64_t B, int64_t H, int64_t Sq, int64_t Skv,
+                         int64_t D, float scale, int is_causal, int64_t mask_stride_b,
+                         int64_t mask_stride_h, int dtype);
+
+/* Glue operators (index / data movement; integer results are bit-exact) ---- */
+
+/* out[i, :] = table[clamp(idx[i], 0, n_rows-1), :], rows of `row_elems` elements.
+ * StableHLO gather with whole-row slices; the clamp is the specification's
+ * ([0, dim - slice_size]), not the reference's (Compiler/CodeGenerator.swift:1252-1254).
+ * Replaces the gather kernels of Compiler/CodeGenerator.swift:1133-1397.
+ * table_dtype: any 1/2/4/8-byte type; idx_dtype: I32 or I64. */
+int mhip_gather_rows(void* stream, const void* table, const void* indices, void* out,
+                     int64_t n_idx, int64_t n_rows, int64_t row_elems, int table_dtype,
+                     int idx_dtype);
+
+/* out[b, s, :] = convert(wte[ids[b, s], :] + wpe[s, :]) — token + position
+ * embedding in one pass (gather :1133-1397, add :921, convert :1012-1078 of
+ * Compiler/CodeGenerator.swift).  ids are I32 [B,S]; params F32 or the output
+ * type; the sum is formed in fp32 and rounded once (RNE). */
+int mhip_embed_tokens(void* stream, const void* ids, const void* wte, const void* wpe, void* out,
+                      int64_t B, int64_t S, int64_t d_model, int64_t vocab, int param_dtype,
+                      int out_dtype);
+
+/* y = a + b elementwise over n elements (Compiler/CodeGenerator.swift:921).
+ * F32/F16/BF16 add in fp32 and round once; I32/I64 wrap. */
+int mhip_add(void* stream, const void* a, const void* b, void* y, int64_t n, int dtype);
+
+/* y = convert(x), n elements (Compiler/CodeGenerator.swift:1012-1078).
+ * Float narrowing is round-to-nearest-even; float -> int truncates toward zero. */
+int mhip_convert(void* stream, const void* x, void* y, int64_t n, int src_dtype, int dst_dtype);
+
+/* [d0,d1,d2,d3] -> [d0,d2,d1,d3] (head split / merge;
+ * Compiler/CodeGenerator.swift:2840-3056). Any 2/4-byte type. */
+int mhip_transpose_0213(void* stream, const void* x, void* y, int64_t d0, int64_t d1, int64_t d2,
+                        int64_t d3, int dtype);
+
+/* qkv [B,S,3*H*D] -> q,k,v each [B,H,S,D] (slice + reshape + transpose fused). */
+int mhip_split_qkv_heads(void* stream, const void* qkv, void* q, void* k, void* v, int64_t B,
+                         int64_t S, int64_t H, int64_t D, int dtype);
+
+/* y[o, i, j] = i for a tensor viewed as [outer, n, inner]
+ * (stablehlo.iota, Compiler/CodeGenerator.swift:1977). Integer and float types. */
+int mhip_iota(void* stream, void* y, int64_t outer, int64_t n, int64_t inner, int dtype);
+
+/* Last-axis argmax of x[rows, cols]: lowest index among equal maxima, a NaN
+ * wins over any number (JAX's tie-break; the reference has no native
+ * arg-reduction, python/README.md:122).  out_val may be NULL.
+ * idx_dtype: I32 or I64. */
+int mhip_argmax(void* stream, const void* x, void* out_idx, void* out_val, int64_t rows,
+                int64_t cols, int dtype, int idx_dtype);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MHIP_H */

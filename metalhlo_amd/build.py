@@ -1,0 +1,101 @@
+"""Builds the gfx950 kernel library (``libmetalhlo_hip.so``) and the C++ host
+libraries in-tree with hipcc / g++.  ``python -m metalhlo_amd.build`` rebuilds
+everything; nothing here needs a GPU (hipcc cross-compiles)."""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+import tempfile
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIBDIR = os.path.join(HERE, "lib")
+ROOT = os.path.dirname(HERE)
+
+HIP_SOURCES = ["runtime.hip", "row_kernels.hip", "gemm.hip", "attention.hip", "glue_kernels.hip"]
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=fast",
+    # packed fp32 VALU forms are kept out of generated code on this hardware pool
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option",
+]
+
+
+def _run(cmd):
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        sys.stderr.write(" ".join(cmd) + "\n" + r.stdout + r.stderr)
+        raise RuntimeError("build step failed: " + os.path.basename(cmd[-1]))
+    noisy = [l for l in r.stderr.splitlines()
+             if l.strip() and "packed-fp32-ops" not in l and "is not a recognized feature" not in l]
+    if noisy:
+        sys.stderr.write("\n".join(noisy) + "\n")
+
+
+def hipcc() -> str:
+    for cand in (os.environ.get("HIPCC"), "/opt/rocm/bin/hipcc", "hipcc"):
+        if cand and (os.path.isabs(cand) and os.path.exists(cand) or not os.path.isabs(cand)):
+            return cand
+    return "hipcc"
+
+
+def build_kernels(verbose: bool = True) -> str:
+    os.makedirs(LIBDIR, exist_ok=True)
+    objdir = tempfile.mkdtemp(prefix="mhip_obj_")
+    srcs = [s for s in HIP_SOURCES if os.path.exists(os.path.join(CSRC, s))]
+    objs = [os.path.join(objdir, s.replace(".hip", ".o")) for s in srcs]
+
+    def one(pair):
+        src, obj = pair
+        _run([hipcc(), *HIPCC_FLAGS, "-I", os.path.join(ROOT, "include"), "-c",
+              os.path.join(CSRC, src), "-o", obj])
+        if verbose:
+            print("  hipcc", src, flush=True)
+
+    with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as ex:
+        list(ex.map(one, zip(srcs, objs)))
+    out = os.path.join(LIBDIR, "libmetalhlo_hip.so")
+    _run([hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out, *objs])
+    if verbose:
+        print("  link ", os.path.relpath(out, ROOT), flush=True)
+    return out
+
+
+def build_host(verbose: bool = True) -> list:
+    """C++ host libraries above the kernel C-ABI (built when their sources exist)."""
+    outs = []
+    host = os.path.join(CSRC, "host")
+    if not os.path.isdir(host):
+        return outs
+    srcs = sorted(os.path.join(host, f) for f in os.listdir(host) if f.endswith(".cpp"))
+    if not srcs:
+        return outs
+    out = os.path.join(LIBDIR, "libCMetalHLO.so")
+    _run([hipcc(), "-O2", "-std=c++17", "-fPIC", "-shared", "-D__HIP_PLATFORM_AMD__",
+          "-I", os.path.join(ROOT, "include"), "-I", "/opt/rocm/include", "-o", out, *srcs,
+          "-L", LIBDIR, "-lmetalhlo_hip", "-Wl,-rpath,$ORIGIN"])
+    if verbose:
+        print("  link ", os.path.relpath(out, ROOT), flush=True)
+    outs.append(out)
+    return outs
+
+
+def build_oracle(verbose: bool = True) -> str:
+    d = os.path.join(ROOT, "oracle")
+    _run(["make", "-C", d, "-B", "liboracle.so"])
+    if verbose:
+        print("  make  oracle/liboracle.so", flush=True)
+    return os.path.join(d, "liboracle.so")
+
+
+def build_all(verbose: bool = True):
+    build_kernels(verbose)
+    build_host(verbose)
+    build_oracle(verbose)
+
+
+if __name__ == "__main__":
+    build_all()

@@ -1,0 +1,452 @@
+// Flash-attention forward for gfx950: O = softmax(scale * Q K^T + mask, causal) V.
+//
+// MFMA path (16-bit types, D in {64, 128}).  A workgroup of four waves owns 128
+// query rows of one (batch, head); each wave owns 32 of them.  Keys/values are
+// walked in blocks of 64, staged in LDS and double-buffered.
+//
+// The scores are computed TRANSPOSED, S^T = K . Q^T, with v_mfma_f32_32x32x16:
+// in the accumulator layout every lane then holds 16 keys of ONE query column,
+// so the online-softmax row statistics are plain per-lane loops plus a single
+// exchange between the two 32-lane halves, and the probabilities can be fed
+// straight back as the B operand of O^T += V^T . P^T without any cross-lane
+// movement.  V is transposed (and its keys put in the order that B operand
+// needs) in registers on the way into LDS.  Softmax state and both
+// accumulations are fp32; the output is rounded once.
+//
+// Everything else (fp32, other head sizes) takes a wave-per-query scalar path.
+#include <math.h>
+
+#include "common.h"
+
+namespace mhip {
+
+constexpr uint32_t kOobA = 0x80000000u;
+constexpr int kBQ = 128;   // query rows per workgroup
+constexpr int kBKV = 64;   // keys per LDS stage
+constexpr float kLog2e = 1.4426950408889634f;
+
+struct FaArgs {
+    const void* q;
+    const void* k;
+    const void* v;
+    const void* mask;
+    void* o;
+    int B, H, Sq, Skv;
+    float c;          // |scale| * log2(e)
+    int negate_q;     // scale < 0: flip the sign of Q instead
+    int is_causal;    // read by the scalar path (the MFMA path is templated on it)
+    int64_t mask_sb, mask_sh;
+    int nqb;          // query blocks per (batch, head)
+    int xcd_map;      // 1: (batch*head) % 8 == 0, use the XCD-aware block order
+};
+
+template <typename T> struct Mfma32A;
+template <> struct Mfma32A<bf16_t> {
+    __device__ static f32x16 run(u32x4 a, u32x4 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                       __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+    __device__ static uint32_t pack2(float lo, float hi) {
+        typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+        bf16x2 t = {(__bf16)lo, (__bf16)hi};
+        return __builtin_bit_cast(uint32_t, t);
+    }
+};
+template <> struct Mfma32A<f16_t> {
+    __device__ static f32x16 run(u32x4 a, u32x4 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
+                                                      __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+    __device__ static uint32_t pack2(float lo, float hi) {
+        typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+        f16x2 t = {(_Float16)lo, (_Float16)hi};
+        return __builtin_bit_cast(uint32_t, t);
+    }
+};
+
+__device__ inline __amdgpu_buffer_rsrc_t fa_rsrc(const void* p, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
+}
+
+// K tile [64 keys][D] : 16-byte chunks XOR-swizzled inside each row.
+template <int D>
+__device__ inline uint32_t k_off(int row, int chunk) {
+    const int s = (D == 128) ? (row & 15) : (((row >> 1) ^ (row >> 4)) & 7);
+    return (uint32_t)(row * (D * 2) + ((chunk ^ s) << 4));
+}
+// V^T tile [D][64 keys] : 128-byte rows.
+__device__ inline uint32_t vt_off(int row, int chunk) {
+    const int s = ((row >> 1) ^ (row >> 4)) & 7;
+    return (uint32_t)(row * 128 + ((chunk ^ s) << 4));
+}
+
+template <typename T, int D, bool CAUSAL, bool HAS_MASK>
+__global__ __launch_bounds__(256) void fa_fwd_kernel(FaArgs a) {
+    constexpr int CPR = D / 8;                  // 16-byte chunks per K row
+    constexpr int kKTile = kBKV * D * 2;        // bytes
+    constexpr int kVTile = D * 128;             // bytes
+    constexpr int kKIters = kBKV * CPR / 128;   // K chunks per loading thread
+    constexpr int kVBlocks = 8 * (D / 8);       // 8x8 blocks of the V tile
+    constexpr int ND = D / 32, NS = D / 16;
+    __shared__ __attribute__((aligned(16))) char smem[2 * (kKTile + kVTile)];
+    auto k_tile = [&](int buf) { return smem + buf * kKTile; };
+    auto v_tile = [&](int buf) { return smem + 2 * kKTile + buf * kVTile; };
+
+    // ---- which (batch*head, query block) -----------------------------------
+    int bh, qb;
+    {
+        const int id = blockIdx.x;
+        if (a.xcd_map) {
+            const int xcd = id & 7, local = id >> 3;
+            bh = (local / a.nqb) * 8 + xcd;
+            qb = a.nqb - 1 - local % a.nqb;   // long (late) causal rows first
+        } else {
+            bh = id / a.nqb;
+            qb = a.nqb - 1 - id % a.nqb;
+        }
+    }
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int lrow = lane & 31, lhalf = lane >> 5;
+    const int qblk0 = qb * kBQ;
+    const int qw = qblk0 + wave * 32;          // first query row of this wave
+    const int qpos = qw + lrow;
+
+    const T* qp = static_cast<const T*>(a.q) + (int64_t)bh * a.Sq * D;
+    const T* kp = static_cast<const T*>(a.k) + (int64_t)bh * a.Skv * D;
+    const T* vp = static_cast<const T*>(a.v) + (int64_t)bh * a.Skv * D;
+    T* op = static_cast<T*>(a.o) + (int64_t)bh * a.Sq * D;
+    const __amdgpu_buffer_rsrc_t rq = fa_rsrc(qp, (uint32_t)((int64_t)a.Sq * D * 2));
+    const __amdgpu_buffer_rsrc_t rk = fa_rsrc(kp, (uint32_t)((int64_t)a.Skv * D * 2));
+    const __amdgpu_buffer_rsrc_t rv = fa_rsrc(vp, (uint32_t)((int64_t)a.Skv * D * 2));
+
+    // ---- Q^T operand: lane = query column, 8 consecutive d per k-step ------
+    u32x4 qf[NS];
+#pragma unroll
+    for (int s = 0; s < NS; s++) {
+        const uint32_t off = qpos < a.Sq ? (uint32_t)((qpos * D + 16 * s + 8 * lhalf) * 2) : kOobA;
+        qf[s] = __builtin_amdgcn_raw_buffer_load_b128(rq, off, 0, 0);
+        if (a.negate_q) {
+            const uint32_t flip = sizeof(T) == 2 ? 0x80008000u : 0u;
+            qf[s].x ^= flip; qf[s].y ^= flip; qf[s].z ^= flip; qf[s].w ^= flip;
+        }
+    }
+
+    int nkv = (a.Skv + kBKV - 1) / kBKV;
+    if (CAUSAL) {
+        const int last_q = min(qblk0 + kBQ, a.Sq) - 1;
+        nkv = min(nkv, last_q / kBKV + 1);
+    }
+
+    // ---- staging registers: waves 0,1 fetch K, waves 2,3 fetch + transpose V
+    u32x4 stage[8];
+    auto load_tile = [&](int kv0) {
+        if (wave < 2) {
+#pragma unroll
+            for (int i = 0; i < kKIters; i++) {
+                const int idx = tid + i * 128;
+                const int row = idx / CPR, c = idx % CPR;
+                const int key = kv0 + row;
+                const uint32_t off = key < a.Skv ? (uint32_t)((key * D + c * 8) * 2) : kOobA;
+                stage[i] = __builtin_amdgcn_raw_buffer_load_b128(rk, off, 0, 0);
+            }
+        } else {
+            const int blk = tid - 128;
+            if (blk < kVBlocks) {
+                const int dg = blk % (D / 8), ch = blk / (D / 8);
+                const int u = ch >> 1, h = ch & 1;
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    const int key = kv0 + 16 * u + 8 * (j >> 2) + 4 * h + (j & 3);
+                    const uint32_t off = key < a.Skv ? (uint32_t)((key * D + dg * 8) * 2) : kOobA;
+                    stage[j] = __builtin_amdgcn_raw_buffer_load_b128(rv, off, 0, 0);
+                }
+            }
+        }
+    };
+    auto store_tile = [&](int buf) {
+        if (wave < 2) {
+#pragma unroll
+            for (int i = 0; i < kKIters; i++) {
+                const int idx = tid + i * 128;
+                const int row = idx / CPR, c = idx % CPR;
+                *reinterpret_cast<u32x4*>(k_tile(buf) + k_off<D>(row, c)) = stage[i];
+            }
+        } else {
+            const int blk = tid - 128;
+            if (blk < kVBlocks) {
+                const int dg = blk % (D / 8), ch = blk / (D / 8);
+#pragma unroll
+                for (int q = 0; q < 4; q++) {   // dword q of a key row holds d = 2q, 2q+1
+                    u32x4 even, odd;
+                    even.x = __builtin_amdgcn_perm(stage[1][q], stage[0][q], 0x05040100);
+                    even.y = __builtin_amdgcn_perm(stage[3][q], stage[2][q], 0x05040100);
+                    even.z = __builtin_amdgcn_perm(stage[5][q], stage[4][q], 0x05040100);
+                    even.w = __builtin_amdgcn_perm(stage[7][q], stage[6][q], 0x05040100);
+                    odd.x = __builtin_amdgcn_perm(stage[1][q], stage[0][q], 0x07060302);
+                    odd.y = __builtin_amdgcn_perm(stage[3][q], stage[2][q], 0x07060302);
+                    odd.z = __builtin_amdgcn_perm(stage[5][q], stage[4][q], 0x07060302);
+                    odd.w = __builtin_amdgcn_perm(stage[7][q], stage[6][q], 0x07060302);
+                    const int d = dg * 8 + 2 * q;
+                    *reinterpret_cast<u32x4*>(v_tile(buf) + vt_off(d, ch)) = even;
+                    *reinterpret_cast<u32x4*>(v_tile(buf) + vt_off(d + 1, ch)) = odd;
+                }
+            }
+        }
+    };
+
+    f32x16 oacc[ND];
+#pragma unroll
+    for (int i = 0; i < ND; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) oacc[i][r] = 0.f;
+    float m_run = -INFINITY, l_run = 0.f;
+
+    load_tile(0);
+    store_tile(0);
+    __syncthreads();
+
+    for (int it = 0; it < nkv; it++) {
+        const int cur = it & 1, kv0 = it * kBKV;
+        if (it + 1 < nkv) load_tile(kv0 + kBKV);
+
+        const bool wave_active = !CAUSAL || kv0 <= qw + 31;
+        if (wave_active) {
+            // ---- S^T = K . Q^T ---------------------------------------------
+            f32x16 sacc[2];
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) sacc[t][r] = 0.f;
+#pragma unroll
+            for (int s = 0; s < NS; s++) {
+#pragma unroll
+                for (int t = 0; t < 2; t++) {
+                    const u32x4 kf = *reinterpret_cast<const u32x4*>(
+                        k_tile(cur) + k_off<D>(32 * t + lrow, 2 * s + lhalf));
+                    sacc[t] = Mfma32A<T>::run(kf, qf[s], sacc[t]);
+                }
+            }
+            // ---- to the log2 domain, additive mask, causal / tail masking ---
+            float sv[32];
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) sv[t * 16 + r] = sacc[t][r] * a.c;
+            if (HAS_MASK) {
+                const T* mp = static_cast<const T*>(a.mask) + (int64_t)(bh / a.H) * a.mask_sb +
+                              (int64_t)(bh % a.H) * a.mask_sh;
+#pragma unroll
+                for (int i = 0; i < 32; i++) {
+                    const int key = kv0 + 32 * (i >> 4) + 8 * ((i & 15) >> 2) + 4 * lhalf + (i & 3);
+                    if (qpos < a.Sq && key < a.Skv)
+                        sv[i] += Elem<T>::to_f32(mp[(int64_t)qpos * a.Skv + key]) * kLog2e;
+                }
+            }
+            const bool boundary = (CAUSAL && kv0 + kBKV - 1 > qw) || kv0 + kBKV > a.Skv;
+            if (boundary) {
+#pragma unroll
+                for (int i = 0; i < 32; i++) {
+                    const int key = kv0 + 32 * (i >> 4) + 8 * ((i & 15) >> 2) + 4 * lhalf + (i & 3);
+                    if ((CAUSAL && key > qpos) || key >= a.Skv) sv[i] = -INFINITY;
+                }
+            }
+            // ---- online softmax ---------------------------------------------
+            float mloc = sv[0];
+#pragma unroll
+            for (int i = 1; i < 32; i++) mloc = fmaxf(mloc, sv[i]);
+            mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
+            const float m_new = fmaxf(m_run, mloc);
+            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+            const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
+            m_run = m_new;
+            float lsum = 0.f;
+#pragma unroll
+            for (int i = 0; i < 32; i++) {
+                sv[i] = __builtin_amdgcn_exp2f(sv[i] - m_use);
+                lsum += sv[i];
+            }
+            l_run = l_run * alpha + lsum;
+#pragma unroll
+            for (int i = 0; i < ND; i++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) oacc[i][r] *= alpha;
+            // ---- P^T as B operand: slot j of step u is register 8u + j ------
+            u32x4 pb[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                pb[u].x = Mfma32A<T>::pack2(sv[8 * u + 0], sv[8 * u + 1]);
+                pb[u].y = Mfma32A<T>::pack2(sv[8 * u + 2], sv[8 * u + 3]);
+                pb[u].z = Mfma32A<T>::pack2(sv[8 * u + 4], sv[8 * u + 5]);
+                pb[u].w = Mfma32A<T>::pack2(sv[8 * u + 6], sv[8 * u + 7]);
+            }
+            // ---- O^T += V^T . P^T -------------------------------------------
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+#pragma unroll
+                for (int dt = 0; dt < ND; dt++) {
+                    const u32x4 vf = *reinterpret_cast<const u32x4*>(
+                        v_tile(cur) + vt_off(32 * dt + lrow, 2 * u + lhalf));
+                    oacc[dt] = Mfma32A<T>::run(vf, pb[u], oacc[dt]);
+                }
+            }
+        }
+        if (it + 1 < nkv) store_tile(cur ^ 1);
+        __syncthreads();
+    }
+
+    // ---- normalise and store: lane holds 4 consecutive d per register group -
+    const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+    const float inv = l_tot > 1e-10f ? 1.f / l_tot : 0.f;
+    if (qpos < a.Sq) {
+        T* orow = op + (int64_t)qpos * D;
+#pragma unroll
+        for (int dt = 0; dt < ND; dt++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                u32x2 w;
+                w.x = Mfma32A<T>::pack2(oacc[dt][4 * g + 0] * inv, oacc[dt][4 * g + 1] * inv);
+                w.y = Mfma32A<T>::pack2(oacc[dt][4 * g + 2] * inv, oacc[dt][4 * g + 3] * inv);
+                *reinterpret_cast<u32x2*>(orow + 32 * dt + 8 * g + 4 * lhalf) = w;
+            }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Scalar path: one wave per query row, any type, D <= 256.
+// Per block of 64 keys: lanes own keys for the scores, then own head-dim
+// columns for the weighted sum.  The recurrence is the reference's
+// (FlashAttentionKernel.swift:589-598) applied per block of keys.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void fa_scalar_kernel(FaArgs a, int D, float scale) {
+    __shared__ float qs[4][256];
+    __shared__ float ps[4][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t row = (int64_t)blockIdx.x * 4 + wave;      // over B*H*Sq
+    const int64_t nrows = (int64_t)a.B * a.H * a.Sq;
+    const bool live = row < nrows;
+    const int64_t bh = live ? row / a.Sq : 0;
+    const int qpos = live ? (int)(row % a.Sq) : 0;
+    const T* qp = static_cast<const T*>(a.q) + (bh * a.Sq + qpos) * D;
+    const T* kp = static_cast<const T*>(a.k) + bh * a.Skv * D;
+    const T* vp = static_cast<const T*>(a.v) + bh * a.Skv * D;
+    const T* mp = a.mask ? static_cast<const T*>(a.mask) + (bh / a.H) * a.mask_sb +
+                               (bh % a.H) * a.mask_sh + (int64_t)qpos * a.Skv
+                         : nullptr;
+    for (int d = lane; d < D; d += 64) qs[wave][d] = live ? Elem<T>::to_f32(qp[d]) : 0.f;
+    __syncthreads();
+    float oacc[4] = {0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.f;
+    const int kv_end = live ? (a.is_causal ? min(a.Skv, qpos + 1) : a.Skv) : 0;
+    for (int kv0 = 0; kv0 < kv_end; kv0 += 64) {
+        const int key = kv0 + lane;
+        float s = -INFINITY;
+        if (key < kv_end) {
+            float acc = 0.f;
+            const T* kr = kp + (int64_t)key * D;
+            for (int d = 0; d < D; d++) acc = fmaf(qs[wave][d], Elem<T>::to_f32(kr[d]), acc);
+            s = acc * scale;
+            if (mp) s += Elem<T>::to_f32(mp[key]);
+        }
+        const float m_new = fmaxf(m_run, wave_max(s));
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        const float alpha = expf(m_run - m_use);
+        const float p = expf(s - m_use);
+        m_run = m_new;
+        l_run = l_run * alpha + wave_sum(p);
+        ps[wave][lane] = p;
+        __builtin_amdgcn_wave_barrier();
+        const int nk = min(64, kv_end - kv0);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int d = lane + 64 * j;
+            if (d < D) {
+                float acc = oacc[j] * alpha;
+                for (int t = 0; t < nk; t++)
+                    acc = fmaf(ps[wave][t], Elem<T>::to_f32(vp[(int64_t)(kv0 + t) * D + d]), acc);
+                oacc[j] = acc;
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+    if (live) {
+        const float inv = l_run > 1e-10f ? 1.f / l_run : 0.f;
+        T* orow = static_cast<T*>(a.o) + (bh * a.Sq + qpos) * D;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int d = lane + 64 * j;
+            if (d < D) orow[d] = Elem<T>::from_f32(oacc[j] * inv);
+        }
+    }
+}
+
+template <typename T, int D>
+static int launch_fa(hipStream_t s, FaArgs a, bool causal, bool has_mask) {
+    a.nqb = (a.Sq + kBQ - 1) / kBQ;
+    const int64_t bh = (int64_t)a.B * a.H;
+    a.xcd_map = (bh % 8 == 0) ? 1 : 0;
+    const int64_t grid = bh * a.nqb;
+    if (grid > 0x7FFFFFFFLL) return fail(MHIP_ERR_UNSUPPORTED, "flash_attention: grid too large");
+#define MHIP_FA(C, M)                                                                       \
+    hipLaunchKernelGGL((fa_fwd_kernel<T, D, C, M>), dim3((unsigned)grid), dim3(256), 0, s, a)
+    if (causal && has_mask) MHIP_FA(true, true);
+    else if (causal) MHIP_FA(true, false);
+    else if (has_mask) MHIP_FA(false, true);
+    else MHIP_FA(false, false);
+#undef MHIP_FA
+    return check_launch("flash_attention");
+}
+
+template <typename T>
+static int launch_fa_scalar(hipStream_t s, FaArgs a, int D, float scale) {
+    const int64_t rows = (int64_t)a.B * a.H * a.Sq;
+    const int64_t grid = (rows + 3) / 4;
+    if (grid > 0x7FFFFFFFLL) return fail(MHIP_ERR_UNSUPPORTED, "flash_attention: grid too large");
+    hipLaunchKernelGGL((fa_scalar_kernel<T>), dim3((unsigned)grid), dim3(256), 0, s, a, D, scale);
+    return check_launch("flash_attention_scalar");
+}
+
+}  // namespace mhip
+
+using namespace mhip;
+
+extern "C" int mhip_flash_attention(void* stream, const void* q, const void* k, const void* v,
+                                    const void* mask, void* o, int64_t B, int64_t H, int64_t Sq,
+                                    int64_t Skv, int64_t D, float scale, int is_causal,
+                                    int64_t mask_stride_b, int64_t mask_stride_h, int dtype) {
+    if (!q || !k || !v || !o)
+        return fail(MHIP_ERR_INVALID_ARGUMENT, "mhip_flash_attention: NULL tensor pointer");
+    if (B < 0 || H < 0 || Sq < 0 || Skv < 0 || D <= 0)
+        return fail(MHIP_ERR_INVALID_ARGUMENT, "mhip_flash_attention: bad size");
+    if (D > 256) return fail(MHIP_ERR_UNSUPPORTED, "mhip_flash_attention: head_dim %lld > 256", (long long)D);
+    if (B == 0 || H == 0 || Sq == 0) return MHIP_OK;
+    if (Sq > 0x7FFFFFFF || Skv > 0x7FFFFFFF || B * H > 0x7FFFFFFF)
+        return fail(MHIP_ERR_UNSUPPORTED, "mhip_flash_attention: dimension exceeds 2^31-1");
+    hipStream_t s = as_stream(stream);
+    FaArgs a;
+    a.q = q; a.k = k; a.v = v; a.mask = mask; a.o = o;
+    a.B = (int)B; a.H = (int)H; a.Sq = (int)Sq; a.Skv = (int)Skv;
+    a.c = fabsf(scale) * kLog2e;
+    a.negate_q = scale < 0.f;
+    a.is_causal = is_causal ? 1 : 0;
+    a.mask_sb = mask_stride_b; a.mask_sh = mask_stride_h;
+    a.nqb = 0; a.xcd_map = 0;
+    const bool is16 = dtype == MHIP_BF16 || dtype == MHIP_F16;
+    const bool aligned = ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) |
+                           reinterpret_cast<uintptr_t>(v) | reinterpret_cast<uintptr_t>(o)) & 15) == 0;
+    const bool fits = Sq * D * 2 < 0x7FFFFFFFLL && Skv * D * 2 < 0x7FFFFFFFLL;
+    if (is16 && aligned && fits && Skv > 0 && (D == 64 || D == 128)) {
+        const bool hm = mask != nullptr;
+        if (dtype == MHIP_BF16)
+            return D == 128 ? launch_fa<bf16_t, 128>(s, a, is_causal, hm)
+                            : launch_fa<bf16_t, 64>(s, a, is_causal, hm);
+        return D == 128 ? launch_fa<f16_t, 128>(s, a, is_causal, hm)
+                        : launch_fa<f16_t, 64>(s, a, is_causal, hm);
+    }
+    switch (dtype) {
+        case MHIP_F32: return launch_fa_scalar<float>(s, a, (int)D, scale);
+        case MHIP_BF16: return launch_fa_scalar<bf16_t>(s, a, (int)D, scale);
+        case MHIP_F16: return launch_fa_scalar<f16_t>(s, a, (int)D, scale);
+        default: return fail(MHIP_ERR_UNSUPPORTED, "mhip_flash_attention: dtype %d", dtype);
+    }
+}

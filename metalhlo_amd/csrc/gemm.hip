@@ -1,0 +1,401 @@
+// dot_general GEMM for gfx950: C[b] = act(op(A[b]) . op(B[b]) + bias).
+//
+// 16-bit types run on v_mfma_f32_32x32x16_{bf16,f16}: a workgroup owns a
+// BM x BN tile of C, walks K in steps of 64 with both operand tiles staged in
+// LDS (double-buffered, XOR-swizzled 16-byte chunks so that every 128-bit LDS
+// access is conflict free), and each wave accumulates a (BM/WGM) x (BN/WGN)
+// sub-tile in fp32 registers.  Operand tiles always sit in LDS "k-major"
+// ([row][64 k]) because the MFMA wants eight consecutive k per lane; an operand
+// whose memory layout has k as the slow axis is transposed in registers on the
+// way in (16-byte global loads either way).
+// Everything else (fp32, shapes that are not 16-byte friendly) goes through a
+// plain LDS-tiled kernel.
+#include <math.h>
+
+#include <mutex>
+
+#include "common.h"
+
+namespace mhip {
+
+constexpr int kBK = 64;              // k extent of one LDS stage
+constexpr int kRowBytes = kBK * 2;   // bytes per LDS tile row (16-bit elements)
+constexpr uint32_t kOob = 0x80000000u;  // byte offset beyond any buffer: load returns 0
+
+struct GemmArgs {
+    const void* a;
+    const void* b;
+    const void* bias;
+    void* c;
+    int M, N, K;
+    int lda, ldb;           // leading dimensions in elements of the stored matrices
+    int64_t sa, sb, sc;     // batch strides in elements
+    int act;
+    int tiles_m, tiles_n;
+};
+
+template <typename T> struct Mfma32;
+template <> struct Mfma32<bf16_t> {
+    __device__ static f32x16 run(u32x4 a, u32x4 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                       __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+};
+template <> struct Mfma32<f16_t> {
+    __device__ static f32x16 run(u32x4 a, u32x4 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
+                                                      __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+};
+
+__device__ inline float apply_act(float v, int act) {
+    switch (act) {
+        case MHIP_ACT_RELU: return fmaxf(v, 0.f);
+        case MHIP_ACT_GELU: {
+            const float inner = 0.7978845608028654f * (v + 0.044715f * v * v * v);
+            return 0.5f * v * (1.f + tanhf(inner));
+        }
+        case MHIP_ACT_SILU: return v / (1.f + expf(-v));
+        case MHIP_ACT_TANH: return tanhf(v);
+        case MHIP_ACT_SIGMOID: return 1.f / (1.f + expf(-v));
+        default: return v;
+    }
+}
+
+// Swizzle of the 16-byte chunk index inside a 128-byte LDS row.  Rows r..r+15
+// (r % 16 == 0) map one chunk column onto 16 distinct bank groups.
+__device__ inline int swz(int row) { return ((row >> 1) ^ (row >> 4)) & 7; }
+
+__device__ inline uint32_t lds_off(int row, int chunk) {
+    return (uint32_t)(row * kRowBytes + ((chunk ^ swz(row)) << 4));
+}
+
+__device__ inline __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
+}
+
+// ---- operand with k contiguous in memory: [rows_total][ld] ----------------
+template <int ROWS, int NT>
+struct KMajorLoader {
+    static constexpr int kIters = ROWS * 8 / NT;
+    u32x4 regs[kIters];
+    __device__ void load(__amdgpu_buffer_rsrc_t rsrc, int row0, int k0, int rows_total, int K,
+                         int ld) {
+        const int c = threadIdx.x & 7;
+#pragma unroll
+        for (int i = 0; i < kIters; i++) {
+            const int r = (threadIdx.x >> 3) + i * (NT / 8);
+            const int grow = row0 + r, gk = k0 + c * 8;
+            const uint32_t off =
+                (grow < rows_total && gk < K) ? (uint32_t)(((int64_t)grow * ld + gk) * 2) : kOob;
+            regs[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, 0);
+        }
+    }
+    __device__ void store(char* tile) const {
+        const int c = threadIdx.x & 7;
+#pragma unroll
+        for (int i = 0; i < kIters; i++) {
+            const int r = (threadIdx.x >> 3) + i * (NT / 8);
+            *reinterpret_cast<u32x4*>(tile + lds_off(r, c)) = regs[i];
+        }
+    }
+};
+
+// ---- operand with k as the slow axis in memory: [K][ld] -------------------
+// A thread fetches a 4(k) x 8(mn) block with four 16-byte loads, transposes it
+// in registers and writes eight 8-byte k-runs into the k-major LDS tile.
+template <int ROWS, int NT>
+struct MnMajorLoader {
+    static constexpr int kBlocks = 16 * (ROWS / 8);
+    static constexpr int kIters = kBlocks / NT;
+    static_assert(kBlocks % NT == 0, "tile does not split evenly over the workgroup");
+    u32x4 regs[kIters][4];
+    __device__ void load(__amdgpu_buffer_rsrc_t rsrc, int col0, int k0, int cols_total, int K,
+                         int ld) {
+#pragma unroll
+        for (int i = 0; i < kIters; i++) {
+            const int blk = threadIdx.x + i * NT;
+            const int ng = blk % (ROWS / 8), kg = blk / (ROWS / 8);
+            const int gcol = col0 + ng * 8;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int gk = k0 + kg * 4 + j;
+                const uint32_t off = (gk < K && gcol < cols_total)
+                                         ? (uint32_t)(((int64_t)gk * ld + gcol) * 2)
+                                         : kOob;
+                regs[i][j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, 0);
+            }
+        }
+    }
+    __device__ void store(char* tile) const {
+#pragma unroll
+        for (int i = 0; i < kIters; i++) {
+            const int blk = threadIdx.x + i * NT;
+            const int ng = blk % (ROWS / 8), kg = blk / (ROWS / 8);
+#pragma unroll
+            for (int q = 0; q < 4; q++) {  // dword q of each row holds columns 2q, 2q+1
+                const uint32_t r0 = regs[i][0][q], r1 = regs[i][1][q];
+                const uint32_t r2 = regs[i][2][q], r3 = regs[i][3][q];
+                u32x2 even, odd;
+                even.x = __builtin_amdgcn_perm(r1, r0, 0x05040100);
+                even.y = __builtin_amdgcn_perm(r3, r2, 0x05040100);
+                odd.x = __builtin_amdgcn_perm(r1, r0, 0x07060302);
+                odd.y = __builtin_amdgcn_perm(r3, r2, 0x07060302);
+                const int row = ng * 8 + q * 2;
+                *reinterpret_cast<u32x2*>(tile + lds_off(row, kg >> 1) + (kg & 1) * 8) = even;
+                *reinterpret_cast<u32x2*>(tile + lds_off(row + 1, kg >> 1) + (kg & 1) * 8) = odd;
+            }
+        }
+    }
+};
+
+template <int ROWS, int NT, bool KMAJOR> struct LoaderSel { using type = KMajorLoader<ROWS, NT>; };
+template <int ROWS, int NT> struct LoaderSel<ROWS, NT, false> { using type = MnMajorLoader<ROWS, NT>; };
+
+// Maps the linear workgroup id to a C tile.  Consecutive ids go to different
+// XCDs (round-robin dispatch), so ids are first regrouped so that each XCD's
+// share is a contiguous range, then walked in bands of kGroupM tile rows:
+// the workgroups resident on one XCD then share A row panels and B column
+// panels through that XCD's L2.
+constexpr int kXcds = 8;
+constexpr int kGroupM = 4;
+__device__ inline void tile_of(int pid, int grid, int tiles_m, int tiles_n, int& tm, int& tn) {
+    const int per = (grid + kXcds - 1) / kXcds;
+    const int tall = (grid % kXcds == 0) ? kXcds : grid % kXcds;
+    const int xcd = pid % kXcds, local = pid / kXcds;
+    const int lpid = (xcd < tall) ? xcd * per + local
+                                  : tall * per + (xcd - tall) * (per - 1) + local;
+    const int band = kGroupM * tiles_n;
+    const int g = lpid / band, first = g * kGroupM;
+    const int gsz = min(tiles_m - first, kGroupM);
+    tm = first + (lpid % band) % gsz;
+    tn = (lpid % band) / gsz;
+}
+
+template <typename T, int BM, int BN, int WGM, int WGN, bool TA, bool TB>
+__global__ __launch_bounds__(WGM* WGN * 64) void gemm_mfma_kernel(GemmArgs g) {
+    constexpr int NT = WGM * WGN * 64;
+    constexpr int WTM = BM / WGM, WTN = BN / WGN;
+    constexpr int TM = WTM / 32, TN = WTN / 32;
+    constexpr int kATile = BM * kRowBytes, kBTile = BN * kRowBytes;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    auto a_tile = [&](int buf) { return smem + buf * kATile; };
+    auto b_tile = [&](int buf) { return smem + 2 * kATile + buf * kBTile; };
+
+    int tm, tn;
+    tile_of(blockIdx.x, gridDim.x, g.tiles_m, g.tiles_n, tm, tn);
+    const int m0 = tm * BM, n0 = tn * BN;
+    const int64_t batch = blockIdx.y;
+    const T* a = static_cast<const T*>(g.a) + batch * g.sa;
+    const T* b = static_cast<const T*>(g.b) + batch * g.sb;
+    T* c = static_cast<T*>(g.c) + batch * g.sc;
+
+    // A is stored [M][K] (k contiguous) unless TA ([K][M]); B is stored [K][N]
+    // (k slow) unless TB ([N][K]).
+    const uint32_t a_bytes = (uint32_t)((int64_t)(TA ? g.K : g.M) * g.lda * 2);
+    const uint32_t b_bytes = (uint32_t)((int64_t)(TB ? g.N : g.K) * g.ldb * 2);
+    const __amdgpu_buffer_rsrc_t ra = make_rsrc(a, a_bytes), rb = make_rsrc(b, b_bytes);
+
+    typename LoaderSel<BM, NT, !TA>::type la;
+    typename LoaderSel<BN, NT, TB>::type lb;
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int wm = wave / WGN, wn = wave % WGN;
+    const int lrow = lane & 31, lhalf = lane >> 5;
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+    const int KT = (g.K + kBK - 1) / kBK;
+    la.load(ra, m0, 0, g.M, g.K, g.lda);
+    lb.load(rb, n0, 0, g.N, g.K, g.ldb);
+    la.store(a_tile(0));
+    lb.store(b_tile(0));
+    __syncthreads();
+
+    for (int kt = 0; kt < KT; kt++) {
+        const int cur = kt & 1;
+        if (kt + 1 < KT) {
+            la.load(ra, m0, (kt + 1) * kBK, g.M, g.K, g.lda);
+            lb.load(rb, n0, (kt + 1) * kBK, g.N, g.K, g.ldb);
+        }
+#pragma unroll
+        for (int s = 0; s < kBK / 16; s++) {
+            u32x4 af[TM], bf[TN];
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+                af[i] = *reinterpret_cast<const u32x4*>(
+                    a_tile(cur) + lds_off(wm * WTM + i * 32 + lrow, 2 * s + lhalf));
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+                bf[j] = *reinterpret_cast<const u32x4*>(
+                    b_tile(cur) + lds_off(wn * WTN + j * 32 + lrow, 2 * s + lhalf));
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++) acc[i][j] = Mfma32<T>::run(af[i], bf[j], acc[i][j]);
+        }
+        if (kt + 1 < KT) {
+            la.store(a_tile(cur ^ 1));
+            lb.store(b_tile(cur ^ 1));
+        }
+        __syncthreads();
+    }
+
+    // Epilogue: lane holds column n = lrow and rows 8*(r/4) + 4*lhalf + r%4 of
+    // every 32x32 accumulator tile.
+    const T* bias = static_cast<const T*>(g.bias);
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+        const int n = n0 + wn * WTN + j * 32 + lrow;
+        if (n >= g.N) continue;
+        const float bv = bias ? Elem<T>::to_f32(bias[n]) : 0.f;
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+            const int mb = m0 + wm * WTM + i * 32 + 4 * lhalf;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int m = mb + 8 * (r >> 2) + (r & 3);
+                if (m < g.M) {
+                    float v = acc[i][j][r] + bv;
+                    if (g.act != MHIP_ACT_NONE) v = apply_act(v, g.act);
+                    c[(int64_t)m * g.N + n] = Elem<T>::from_f32(v);
+                }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Plain tiled kernel: any type, any shape.  16x16 threads, one output each.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void gemm_simple_kernel(GemmArgs g, int trans_a, int trans_b) {
+    __shared__ float As[16][17];
+    __shared__ float Bs[16][17];
+    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+    const int64_t batch = blockIdx.z;
+    const T* a = static_cast<const T*>(g.a) + batch * g.sa;
+    const T* b = static_cast<const T*>(g.b) + batch * g.sb;
+    T* c = static_cast<T*>(g.c) + batch * g.sc;
+    const int m = blockIdx.y * 16 + ty, n = blockIdx.x * 16 + tx;
+    float acc = 0.f;
+    for (int k0 = 0; k0 < g.K; k0 += 16) {
+        const int ka = k0 + tx, kb = k0 + ty;
+        float av = 0.f, bv = 0.f;
+        if (m < g.M && ka < g.K)
+            av = Elem<T>::to_f32(trans_a ? a[(int64_t)ka * g.lda + m] : a[(int64_t)m * g.lda + ka]);
+        if (n < g.N && kb < g.K)
+            bv = Elem<T>::to_f32(trans_b ? b[(int64_t)n * g.ldb + kb] : b[(int64_t)kb * g.ldb + n]);
+        As[ty][tx] = av;
+        Bs[ty][tx] = bv;
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < 16; k++) acc = fmaf(As[ty][k], Bs[k][tx], acc);
+        __syncthreads();
+    }
+    if (m < g.M && n < g.N) {
+        if (g.bias) acc += Elem<T>::to_f32(static_cast<const T*>(g.bias)[n]);
+        if (g.act != MHIP_ACT_NONE) acc = apply_act(acc, g.act);
+        c[(int64_t)m * g.N + n] = Elem<T>::from_f32(acc);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Host dispatch
+// ---------------------------------------------------------------------------
+template <typename T, int BM, int BN, int WGM, int WGN, bool TA, bool TB>
+static int launch_mfma(hipStream_t s, GemmArgs g, int64_t batch) {
+    constexpr int NT = WGM * WGN * 64;
+    constexpr int kSmem = 2 * (BM + BN) * kRowBytes;
+    auto kern = gemm_mfma_kernel<T, BM, BN, WGM, WGN, TA, TB>;
+    static std::once_flag once;
+    static hipError_t attr_err = hipSuccess;
+    std::call_once(once, [&] {
+        attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kSmem);
+    });
+    if (attr_err != hipSuccess)
+        return fail(MHIP_ERR_LAUNCH, "gemm: cannot reserve %d bytes of LDS: %s", kSmem,
+                    hipGetErrorString(attr_err));
+    g.tiles_m = (g.M + BM - 1) / BM;
+    g.tiles_n = (g.N + BN - 1) / BN;
+    const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
+    if (tiles > 0x7FFFFFFFLL || batch > 65535) return fail(MHIP_ERR_UNSUPPORTED, "gemm: grid too large");
+    hipLaunchKernelGGL(kern, dim3((unsigned)tiles, (unsigned)batch), dim3(NT), kSmem, s, g);
+    return check_launch("gemm_mfma");
+}
+
+template <typename T, bool TA, bool TB>
+static int pick_tile(hipStream_t s, const GemmArgs& g, int64_t batch) {
+    const int64_t big = (int64_t)((g.M + 255) / 256) * ((g.N + 255) / 256) * batch;
+    if (big >= 192) return launch_mfma<T, 256, 256, 2, 4, TA, TB>(s, g, batch);
+    return launch_mfma<T, 128, 128, 2, 2, TA, TB>(s, g, batch);
+}
+
+template <typename T>
+static int pick_layout(hipStream_t s, const GemmArgs& g, int64_t batch, int ta, int tb) {
+    if (!ta && !tb) return pick_tile<T, false, false>(s, g, batch);
+    if (!ta && tb) return pick_tile<T, false, true>(s, g, batch);
+    if (ta && !tb) return pick_tile<T, true, false>(s, g, batch);
+    return pick_tile<T, true, true>(s, g, batch);
+}
+
+template <typename T>
+static int launch_simple(hipStream_t s, const GemmArgs& g, int64_t batch, int ta, int tb) {
+    const int64_t gx = (g.N + 15) / 16, gy = (g.M + 15) / 16;
+    if (gy > 65535 || batch > 65535) return fail(MHIP_ERR_UNSUPPORTED, "gemm: grid too large");
+    hipLaunchKernelGGL((gemm_simple_kernel<T>), dim3((unsigned)gx, (unsigned)gy, (unsigned)batch),
+                       dim3(256), 0, s, g, ta, tb);
+    return check_launch("gemm_simple");
+}
+
+}  // namespace mhip
+
+using namespace mhip;
+
+extern "C" int mhip_gemm(void* stream, const void* a, const void* b, const void* bias, void* c,
+                         int64_t M, int64_t N, int64_t K, int64_t batch, int64_t stride_a,
+                         int64_t stride_b, int64_t stride_c, int trans_a, int trans_b,
+                         int activation, int dtype) {
+    if (!a || !b || !c) return fail(MHIP_ERR_INVALID_ARGUMENT, "mhip_gemm: NULL matrix pointer");
+    if (M < 0 || N < 0 || K < 0 || batch < 0)
+        return fail(MHIP_ERR_INVALID_ARGUMENT, "mhip_gemm: negative size");
+    if (activation < MHIP_ACT_NONE || activation > MHIP_ACT_SIGMOID)
+        return fail(MHIP_ERR_INVALID_ARGUMENT, "mhip_gemm: unknown activation %d", activation);
+    if (M == 0 || N == 0 || batch == 0) return MHIP_OK;
+    if (M > 0x7FFFFFFF || N > 0x7FFFFFFF || K > 0x7FFFFFFF)
+        return fail(MHIP_ERR_UNSUPPORTED, "mhip_gemm: dimension exceeds 2^31-1");
+    hipStream_t s = as_stream(stream);
+    GemmArgs g;
+    g.a = a; g.b = b; g.bias = bias; g.c = c;
+    g.M = (int)M; g.N = (int)N; g.K = (int)K;
+    g.lda = trans_a ? (int)M : (int)K;
+    g.ldb = trans_b ? (int)K : (int)N;
+    g.sa = stride_a; g.sb = stride_b; g.sc = stride_c;
+    g.act = activation;
+    g.tiles_m = g.tiles_n = 0;
+
+    const bool is16 = dtype == MHIP_BF16 || dtype == MHIP_F16;
+    // 16-byte global loads need every row start and every 8-element chunk aligned.
+    const bool vec_ok = is16 && K > 0 && g.lda % 8 == 0 && g.ldb % 8 == 0 &&
+                        (reinterpret_cast<uintptr_t>(a) & 15) == 0 &&
+                        (reinterpret_cast<uintptr_t>(b) & 15) == 0 && stride_a % 8 == 0 &&
+                        stride_b % 8 == 0 && (int64_t)M * K * 2 < 0x7FFFFFFFLL &&
+                        (int64_t)N * K * 2 < 0x7FFFFFFFLL;
+    if (vec_ok) {
+        if (dtype == MHIP_BF16) return pick_layout<bf16_t>(s, g, batch, trans_a, trans_b);
+        return pick_layout<f16_t>(s, g, batch, trans_a, trans_b);
+    }
+    switch (dtype) {
+        case MHIP_F32: return launch_simple<float>(s, g, batch, trans_a, trans_b);
+        case MHIP_BF16: return launch_simple<bf16_t>(s, g, batch, trans_a, trans_b);
+        case MHIP_F16: return launch_simple<f16_t>(s, g, batch, trans_a, trans_b);
+        default: return fail(MHIP_ERR_UNSUPPORTED, "mhip_gemm: dtype %d (need f32, f16 or bf16)", dtype);
+    }
+}

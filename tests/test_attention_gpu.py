@@ -1,0 +1,127 @@
+"""GPU parity: flash-attention forward through the C-ABI vs the float64
+materialised-scores oracle.  fp32: 1e-5 relative; bf16/fp16: 2e-2 relative
+(floor max(tol, tol*|e|))."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle
+from tests.util import NAME, TOL, as_f64, assert_close, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def _qkv(B, H, Sq, Skv, D, dtype, seed):
+    rng = np.random.default_rng(seed)
+    q = to_dev(rng.standard_normal((B, H, Sq, D)), dtype)
+    k = to_dev(rng.standard_normal((B, H, Skv, D)), dtype)
+    v = to_dev(rng.standard_normal((B, H, Skv, D)), dtype)
+    return q, k, v
+
+
+def test_c1_fp32_causal_sdpa():
+    """BASELINE config 0: fp32, B1 H4 S128 D64, causal, scale 1/8, seed 1234 —
+    causal flag and additive -inf mask variants must both match the oracle."""
+    from metalhlo_amd import kernels
+    q, k, v = _qkv(1, 4, 128, 128, 64, torch.float32, 1234)
+    exp = oracle.attention(as_f64(q), as_f64(k), as_f64(v), scale=0.125, is_causal=True)
+    o = kernels.flash_attention(q, k, v, scale=0.125, is_causal=True)
+    assert o.shape == (1, 4, 128, 64)
+    assert_close(o, exp, 1e-5, "C1 causal flag")
+    m = np.where(np.arange(128)[None, :] > np.arange(128)[:, None], -np.inf, 0.0)
+    om = kernels.flash_attention(q, k, v, scale=0.125, mask=to_dev(m, torch.float32))
+    assert_close(om, exp, 1e-5, "C1 additive mask")
+    # causal row 0 attends to key 0 only
+    assert_close(o[:, :, 0], as_f64(v)[:, :, 0], 1e-6, "row 0 == V[0]")
+
+
+CASES = [  # B, H, Sq, Skv, D, causal
+    (1, 2, 128, 128, 128, False), (1, 2, 128, 128, 128, True),
+    (2, 3, 256, 256, 64, True), (2, 3, 256, 256, 64, False),
+    (1, 8, 200, 200, 128, True),      # ragged: S not a multiple of the 128/64 tiles
+    (1, 2, 77, 333, 64, False),       # cross attention, ragged both ways
+    (1, 1, 333, 77, 128, True),       # more queries than keys (rows past Skv see every key)
+    (1, 8, 1024, 1024, 64, True),     # GPT-2-small head shape
+    (2, 2, 96, 160, 32, True),        # head size without an MFMA path
+    (1, 1, 1, 1, 128, True),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=lambda d: NAME[d])
+@pytest.mark.parametrize("case", CASES, ids=lambda c: "B%dH%dq%dk%dD%d%s" % (*c[:5], "c" if c[5] else ""))
+def test_attention_16bit(case, dtype):
+    from metalhlo_amd import kernels
+    B, H, Sq, Skv, D, causal = case
+    q, k, v = _qkv(B, H, Sq, Skv, D, dtype, 41)
+    o = kernels.flash_attention(q, k, v, is_causal=causal)
+    exp = oracle.attention(as_f64(q), as_f64(k), as_f64(v), is_causal=causal)
+    assert_close(o, exp, TOL[dtype], f"attention {case}")
+
+
+def test_attention_mask_scale_variants():
+    from metalhlo_amd import kernels
+    rng = np.random.default_rng(42)
+    q, k, v = _qkv(2, 4, 192, 192, 128, torch.bfloat16, 43)
+    # per-(b,h) mask, broadcast-over-heads mask, broadcast-over-everything mask
+    for shape in [(2, 4, 192, 192), (2, 1, 192, 192), (1, 1, 192, 192)]:
+        m = rng.standard_normal(shape)
+        m[..., :, 100:] = -np.inf          # padded keys
+        md = to_dev(m, torch.bfloat16)
+        o = kernels.flash_attention(q, k, v, mask=md, scale=0.05)
+        exp = oracle.attention(as_f64(q), as_f64(k), as_f64(v), scale=0.05, mask=as_f64(md))
+        assert_close(o, exp, 2e-2, f"mask {shape}")
+    # mask + causal together, negative scale, fully masked rows -> zeros
+    m = np.zeros((1, 1, 192, 192)); m[..., 5, :] = -np.inf
+    md = to_dev(m, torch.bfloat16)
+    o = kernels.flash_attention(q, k, v, mask=md, is_causal=True, scale=-0.1)
+    exp = oracle.attention(as_f64(q), as_f64(k), as_f64(v), scale=-0.1, is_causal=True, mask=as_f64(md))
+    assert_close(o, exp, 2e-2, "mask+causal, negative scale")
+    assert torch.count_nonzero(o[:, :, 5]) == 0
+
+
+def test_attention_invariants():
+    from metalhlo_amd import kernels
+    q, k, v = _qkv(1, 2, 256, 256, 128, torch.bfloat16, 44)
+    # uniform V rows -> every output row equals that row (softmax weights sum to 1)
+    vu = v[:, :, :1].expand_as(v).contiguous()
+    o = kernels.flash_attention(q, k, vu, is_causal=True)
+    assert_close(o, as_f64(vu), 2e-2, "uniform V")
+    # causal flag == additive upper-triangular -inf mask
+    m = np.where(np.arange(256)[None, :] > np.arange(256)[:, None], -np.inf, 0.0)[None, None]
+    a = kernels.flash_attention(q, k, v, is_causal=True)
+    b = kernels.flash_attention(q, k, v, mask=to_dev(m, torch.bfloat16))
+    assert_close(a, as_f64(b), 2e-2, "causal == mask")
+    # one dominant key: q.k huge for key 7 -> output ~ V[7]
+    kk = k.clone(); kk[:, :, 7] = q[:, :, 0] * 8
+    o = kernels.flash_attention(q, kk, v, scale=1.0)
+    assert_close(o[:, :, 0], as_f64(v[:, :, 7]), 2e-2, "dominant key")
+
+
+@pytest.mark.parametrize("causal,S", [(True, 4096), (False, 2048)], ids=["causal4096", "full2048"])
+def test_attention_baseline_shape_sampled(causal, S):
+    """BASELINE config 3: bf16 B4 H32 D128 (seed 4). Oracle on sampled (b,h) slices and rows."""
+    from metalhlo_amd import kernels
+    B, H, D = 4, 32, 128
+    g = torch.Generator(device="cuda").manual_seed(4)
+    q, k, v = (torch.randn(B, H, S, D, generator=g, device="cuda").to(torch.bfloat16) for _ in range(3))
+    o = kernels.flash_attention(q, k, v, is_causal=causal)
+    rng = np.random.default_rng(4)
+    rows = np.r_[0, 1, 31, 32, 63, 64, 127, 128, S - 129, S - 1, rng.integers(0, S, 22)]
+    for b, h in [(0, 0), (1, 7), (3, 31), (2, 16)]:
+        exp = oracle.attention_rows(as_f64(q[b, h]), as_f64(k[b, h]), as_f64(v[b, h]), rows,
+                                    is_causal=causal)
+        assert_close(o[b, h][rows], exp, 2e-2, f"slice {(b, h)}")
+    if causal:
+        assert torch.equal(o[:, :, 0], v[:, :, 0])     # first causal row copies V[0] exactly
+    assert torch.isfinite(o.float()).all()
+
+
+def test_attention_errors(lib):
+    x = torch.zeros(16, dtype=torch.float32, device="cuda")
+    p = x.data_ptr()
+    assert lib.mhip_flash_attention(None, None, p, p, None, p, 1, 1, 1, 1, 4, 1.0, 0, 0, 0, 1) == 1
+    assert lib.mhip_flash_attention(None, p, p, p, None, p, 1, 1, 1, 1, 512, 1.0, 0, 0, 0, 1) == 2
+    assert lib.mhip_flash_attention(None, p, p, p, None, p, 0, 1, 1, 1, 4, 1.0, 0, 0, 0, 1) == 0
+    assert lib.mhip_flash_attention(None, p, p, p, None, p, 1, 1, 1, 1, 4, 1.0, 0, 0, 0, 7) == 2

@@ -1,0 +1,153 @@
+"""GPU parity: dot_general GEMM through the C-ABI vs the float64 oracle on the
+same (already rounded) operands.  bf16/fp16: 2e-2 relative; fp32: 1e-5 relative,
+both with the floor max(tol, tol*|e|).  Integer-valued operands whose partial
+sums are exactly representable must come out bit-exact."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle
+from tests.util import NAME, TOL, as_f64, assert_close, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def _ab(M, N, K, dtype, seed, ta=False, tb=False, batch=()):
+    rng = np.random.default_rng(seed)
+    a = rng.uniform(-1, 1, batch + ((K, M) if ta else (M, K)))
+    b = rng.uniform(-1, 1, batch + ((N, K) if tb else (K, N)))
+    return to_dev(a, dtype), to_dev(b, dtype)
+
+
+# MFMA path: full tiles, ragged M/N/K (K tail not a multiple of 64), small-tile config
+SHAPES16 = [(256, 256, 256), (512, 768, 128), (300, 520, 136), (64, 8, 8), (1, 8, 64),
+            (1000, 264, 72), (2048, 2048, 512)]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=lambda d: NAME[d])
+@pytest.mark.parametrize("layout", [(False, False), (False, True), (True, False), (True, True)],
+                         ids=["nn", "nt", "tn", "tt"])
+@pytest.mark.parametrize("shape", SHAPES16, ids=lambda s: "x".join(map(str, s)))
+def test_gemm_16bit(shape, layout, dtype):
+    from metalhlo_amd import kernels
+    M, N, K = shape
+    ta, tb = layout
+    a, b = _ab(M, N, K, dtype, 21, ta, tb)
+    c = kernels.matmul(a, b, trans_a=ta, trans_b=tb)
+    assert c.shape == (M, N)
+    assert_close(c, oracle.gemm(as_f64(a), as_f64(b), ta, tb), TOL[dtype], f"gemm {shape} {layout}")
+
+
+@pytest.mark.parametrize("shape", [(4, 4, 4), (33, 17, 9), (64, 64, 64), (130, 70, 50)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_gemm_f32(shape):
+    # fp32 accumulation error grows like sqrt(K)*2^-24*|a||b|; these K keep it
+    # inside the reference's 1e-5 rule for uniform[-1,1] operands.
+    from metalhlo_amd import kernels
+    M, N, K = shape
+    for ta, tb in [(False, False), (True, True)]:
+        a, b = _ab(M, N, K, torch.float32, 22, ta, tb)
+        c = kernels.matmul(a, b, trans_a=ta, trans_b=tb)
+        assert_close(c, oracle.gemm(as_f64(a), as_f64(b), ta, tb), 1e-5, f"gemm f32 {shape}")
+
+
+def test_gemm_unaligned_falls_back():
+    """K or N not a multiple of 8 (e.g. vocab 50257) cannot use 16-byte loads."""
+    from metalhlo_amd import kernels
+    a, b = _ab(40, 50257 // 100, 100, torch.bfloat16, 23)          # N = 502
+    assert_close(kernels.matmul(a, b), oracle.gemm(as_f64(a), as_f64(b)), 2e-2, "N=502")
+    a, b = _ab(40, 64, 100 + 3, torch.bfloat16, 24)                # K = 103
+    assert_close(kernels.matmul(a, b), oracle.gemm(as_f64(a), as_f64(b)), 2e-2, "K=103")
+    # tied output head: x [T,768] . wte[50257,768]^T — k-contiguous, MFMA path, odd N
+    a, b = _ab(128, 50257, 768, torch.bfloat16, 25, tb=True)
+    assert_close(kernels.matmul(a, b, trans_b=True), oracle.gemm(as_f64(a), as_f64(b), False, True),
+                 2e-2, "logits")
+
+
+def test_gemm_exact_small_integers():
+    """Entries in {-2..2}: every product and partial sum is an integer far below
+    2^24, and |C| <= 4K = 256 is exact in bf16 -> result must be bit-exact."""
+    from metalhlo_amd import kernels
+    rng = np.random.default_rng(26)
+    M, N, K = 512, 384, 64
+    a = rng.integers(-2, 3, (M, K)).astype(np.float64)
+    b = rng.integers(-2, 3, (K, N)).astype(np.float64)
+    for dtype in (torch.bfloat16, torch.float16):
+        c = kernels.matmul(to_dev(a, dtype), to_dev(b, dtype))
+        assert np.array_equal(as_f64(c), a @ b)
+    # identity and all-ones closed forms
+    eye = to_dev(np.eye(256), torch.bfloat16)
+    x, _ = _ab(256, 256, 256, torch.bfloat16, 27)
+    assert torch.equal(kernels.matmul(x, eye), x)
+    assert torch.equal(kernels.matmul(eye, x), x)
+    ones = to_dev(np.ones((256, 256)), torch.bfloat16)
+    assert np.array_equal(as_f64(kernels.matmul(ones, ones)), np.full((256, 256), 256.0))
+
+
+def test_gemm_batched_bias_activation():
+    from metalhlo_amd import kernels
+    rng = np.random.default_rng(28)
+    a, b = _ab(96, 136, 72, torch.bfloat16, 29, batch=(5,))
+    c = kernels.matmul(a, b)
+    assert c.shape == (5, 96, 136)
+    assert_close(c, oracle.gemm(as_f64(a), as_f64(b)), 2e-2, "batched")
+    x, w = _ab(200, 264, 128, torch.bfloat16, 30)
+    bias = to_dev(rng.standard_normal(264) * 0.5, torch.bfloat16)
+    for act in ("none", "relu", "gelu", "silu", "tanh", "sigmoid"):
+        y = kernels.matmul(x, w, bias=bias, activation=act)
+        assert_close(y, oracle.matmul_bias_act(as_f64(x), as_f64(w), as_f64(bias), act), 2e-2, act)
+    xf, wf = _ab(20, 24, 16, torch.float32, 31)
+    bf = to_dev(rng.standard_normal(24), torch.float32)
+    assert_close(kernels.matmul(xf, wf, bias=bf, activation="gelu"),
+                 oracle.matmul_bias_act(as_f64(xf), as_f64(wf), as_f64(bf), "gelu"), 1e-5, "f32 gelu")
+
+
+def test_reference_dot_known_answers():
+    from metalhlo_amd import kernels
+    kat = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "kat.json")))
+    for case in kat["dot"]:
+        lhs, rhs = np.array(case["lhs"], dtype=np.float64), np.array(case["rhs"], dtype=np.float64)
+        lb, rb, lc, rc = (case[k] for k in ("lhs_batch", "rhs_batch", "lhs_contract", "rhs_contract"))
+        # canonicalise exactly like the host does: batch dims first, contracting last/first
+        lf = [i for i in range(lhs.ndim) if i not in lb and i not in lc]
+        rf = [i for i in range(rhs.ndim) if i not in rb and i not in rc]
+        a = np.transpose(lhs, lb + lf + lc)
+        b = np.transpose(rhs, rb + rc + rf)
+        bs = [lhs.shape[i] for i in lb]
+        B = int(np.prod(bs)) if bs else 1
+        M = int(np.prod([lhs.shape[i] for i in lf])) if lf else 1
+        K = int(np.prod([lhs.shape[i] for i in lc])) if lc else 1
+        N = int(np.prod([rhs.shape[i] for i in rf])) if rf else 1
+        c = kernels.matmul(to_dev(a.reshape(B, M, K), torch.float32), to_dev(b.reshape(B, K, N), torch.float32))
+        exp = np.array(case["y"], dtype=np.float64)
+        got = as_f64(c).reshape(exp.shape)
+        if case["tol"] == 0:
+            assert np.array_equal(got, exp), case["src"]
+        else:
+            assert np.all(np.abs(got - exp) <= case["tol"]), case["src"]
+
+
+def test_gemm_4096_sampled_rows():
+    """BASELINE GEMM config: 4096^3 bf16, uniform[-1,1] (seed 2). Oracle on 64 sampled rows."""
+    from metalhlo_amd import kernels
+    rng = np.random.default_rng(2)
+    a = to_dev(rng.uniform(-1, 1, (4096, 4096)), torch.bfloat16)
+    b = to_dev(rng.uniform(-1, 1, (4096, 4096)), torch.bfloat16)
+    c = kernels.matmul(a, b)
+    rows = np.r_[0, 1, 31, 32, 255, 256, 4095, rng.integers(0, 4096, 57)]
+    exp = as_f64(a[rows]) @ as_f64(b)
+    assert_close(c[rows], exp, 2e-2, "gemm 4096 sampled rows")
+    # linearity in A: (2A).B == 2(A.B) exactly (power-of-two scaling commutes with rounding)
+    assert torch.equal(kernels.matmul(a * 2, b), c * 2)
+
+
+def test_gemm_errors(lib):
+    assert lib.mhip_gemm(None, None, None, None, None, 4, 4, 4, 1, 0, 0, 0, 0, 0, 0, 3) == 1
+    x = torch.zeros(4, 4, dtype=torch.int32, device="cuda")
+    p = x.data_ptr()
+    assert lib.mhip_gemm(None, p, p, None, p, 4, 4, 4, 1, 0, 0, 0, 0, 0, 0, 7) == 2   # int32 unsupported
+    assert lib.mhip_gemm(None, p, p, None, p, 4, 4, 4, 1, 0, 0, 0, 0, 0, 99, 1) == 1  # bad activation
+    assert lib.mhip_gemm(None, p, p, None, p, 0, 4, 4, 1, 0, 0, 0, 0, 0, 0, 1) == 0   # empty is a no-op

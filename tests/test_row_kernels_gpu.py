@@ -1,0 +1,149 @@
+"""GPU parity: row operators (softmax, LayerNorm, RMSNorm, bias+GELU) through the
+C-ABI vs the float64 oracle.  Tolerances: fp32 1e-5, bf16/fp16 2e-2, relative
+with the same floor (max(tol, tol*|e|))."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle
+from tests.util import NAME, TOL, as_f64, assert_close, to_dev
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.bfloat16, torch.float16, torch.float32]
+# (rows, cols): register path at several vector counts, ragged rows, the
+# workgroup-per-row path (cols % 8 != 0, or too long for registers), tiny.
+SHAPES = [(7, 4096), (33, 768), (5, 100), (3, 8192), (2, 16384), (4, 8), (130, 1024), (1, 1), (9, 50257)]
+
+
+def _x(rows, cols, dtype, seed):
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((rows, cols)) * 2.0 + 0.5
+    return to_dev(x, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=lambda d: NAME[d])
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: f"{s[0]}x{s[1]}")
+def test_softmax(shape, dtype):
+    from metalhlo_amd import kernels
+    x = _x(*shape, dtype, 11)
+    y = kernels.softmax(x)
+    assert_close(y, oracle.softmax(as_f64(x)), TOL[dtype], "softmax")
+    s = as_f64(y).sum(-1)
+    assert np.allclose(s, 1.0, atol=2e-2 if dtype != torch.float32 else 1e-5)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=lambda d: NAME[d])
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: f"{s[0]}x{s[1]}")
+def test_layer_norm(shape, dtype):
+    from metalhlo_amd import kernels
+    rng = np.random.default_rng(12)
+    x = _x(*shape, dtype, 13)
+    g = to_dev(1.0 + 0.1 * rng.standard_normal(shape[1]), dtype)
+    b = to_dev(0.1 * rng.standard_normal(shape[1]), dtype)
+    if shape[1] == 1:
+        pytest.skip("variance of a single element is 0/eps: not a meaningful parity case")
+    y = kernels.layer_norm(x, g, b, eps=1e-5)
+    assert_close(y, oracle.layer_norm(as_f64(x), as_f64(g), as_f64(b), 1e-5), TOL[dtype] * (2 if dtype == torch.float32 else 1), "layer_norm")
+    y0 = kernels.layer_norm(x, None, None, eps=1e-5)
+    assert_close(y0, oracle.layer_norm(as_f64(x), None, None, 1e-5), TOL[dtype] * (2 if dtype == torch.float32 else 1), "layer_norm no affine")
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=lambda d: NAME[d])
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: f"{s[0]}x{s[1]}")
+def test_rms_norm(shape, dtype):
+    from metalhlo_amd import kernels
+    rng = np.random.default_rng(14)
+    x = _x(*shape, dtype, 15)
+    g = to_dev(1.0 + 0.1 * rng.standard_normal(shape[1]), dtype)
+    y = kernels.rms_norm(x, g, eps=1e-6)
+    assert_close(y, oracle.rms_norm(as_f64(x), as_f64(g), 1e-6), TOL[dtype], "rms_norm")
+    y0 = kernels.rms_norm(x, None, eps=1e-6)
+    assert_close(y0, oracle.rms_norm(as_f64(x), None, 1e-6), TOL[dtype], "rms_norm no gamma")
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=lambda d: NAME[d])
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: f"{s[0]}x{s[1]}")
+def test_bias_gelu(shape, dtype):
+    from metalhlo_amd import kernels
+    rng = np.random.default_rng(16)
+    x = _x(*shape, dtype, 17)
+    b = to_dev(0.02 * rng.standard_normal(shape[1]), dtype)
+    y = kernels.bias_gelu(x, b)
+    assert_close(y, oracle.bias_gelu(as_f64(x), as_f64(b)), TOL[dtype], "bias_gelu")
+    y0 = kernels.gelu(x)
+    assert_close(y0, oracle.gelu_tanh(as_f64(x)), TOL[dtype], "gelu")
+
+
+def test_reference_known_answers():
+    """Known answers the reference's own tests hold (tests/golden/kat.json)."""
+    import json, os
+    from metalhlo_amd import kernels
+    kat = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "kat.json")))
+    f32 = torch.float32
+    for case in kat["softmax"]:
+        y = kernels.softmax(to_dev(np.array(case["x"]), f32))
+        assert_close(y, np.array(case["y"]), case["tol"], "softmax KAT " + case["src"])
+    for case in kat["gelu"]:
+        y = kernels.gelu(to_dev(np.array(case["x"]), f32))
+        assert_close(y, np.array(case["y"]), case["tol"], "gelu KAT " + case["src"])
+    for case in kat["rms_norm"]:
+        x = to_dev(np.array(case["x"]), f32)
+        g = to_dev(np.array(case["gamma"]), f32)
+        assert_close(kernels.rms_norm(x, g, eps=case["eps"]), np.array(case["y"]), case["tol"],
+                     "rms KAT " + case["src"])
+    for case in kat["layer_norm"]:
+        x = to_dev(np.array(case["x"]), f32)
+        g = to_dev(np.array(case["gamma"]), f32)
+        b = to_dev(np.array(case["beta"]), f32)
+        y = kernels.layer_norm(x, g, b, eps=case["eps"])
+        if "y" in case:
+            assert_close(y, np.array(case["y"]), case["tol"], "ln KAT " + case["src"])
+        yy = as_f64(y)
+        assert np.all(np.abs(yy.mean(-1)) < case["tol"]) and np.all(np.abs(yy.std(-1) - 1) < 1e-3)
+
+
+def test_softmax_middle_axis():
+    from metalhlo_amd import kernels
+    x = _x(6 * 37, 24, torch.float32, 18).reshape(6, 37, 24)
+    assert_close(kernels.softmax(x, axis=1), oracle.softmax(as_f64(x), axis=1), 1e-5, "softmax axis=1")
+    xb = x.to(torch.bfloat16)
+    assert_close(kernels.softmax(xb, axis=0), oracle.softmax(as_f64(xb), axis=0), 2e-2, "softmax axis=0")
+
+
+def test_empty_and_errors(lib):
+    from metalhlo_amd import kernels, _lib
+    x = torch.empty(0, 128, dtype=torch.bfloat16, device="cuda")
+    assert kernels.softmax(x).shape == (0, 128)
+    # NULL pointer and unsupported dtype are reported, not launched
+    assert lib.mhip_softmax(None, None, None, 4, 4, 1) == 1
+    assert b"NULL" in lib.mhip_last_error()
+    xi = torch.zeros(4, 4, dtype=torch.int32, device="cuda")
+    with pytest.raises(_lib.MhipError):
+        kernels.softmax(xi)
+
+
+def test_invariants_full_size():
+    """BASELINE row-kernel shape [32768, 4096] bf16: size-independent properties."""
+    from metalhlo_amd import kernels
+    g = torch.Generator(device="cuda").manual_seed(3)
+    x = torch.randn(32768, 4096, generator=g, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+    y = kernels.softmax(x)
+    assert torch.allclose(y.float().sum(-1), torch.ones(32768, device="cuda"), atol=2e-2)
+    # shift invariance: softmax(x + c) == softmax(x) when x + c is exact in bf16
+    idx = [0, 1, 4097, 32767]
+    sub = x[idx]
+    assert_close(kernels.softmax(sub), oracle.softmax(as_f64(sub)), 2e-2, "softmax rows of full tensor")
+    assert_close(y[idx], oracle.softmax(as_f64(sub)), 2e-2, "softmax full launch, sampled rows")
+    gam = torch.ones(4096, device="cuda", dtype=torch.bfloat16)
+    r = kernels.rms_norm(x, gam, eps=1e-6)
+    ms = (r.float() ** 2).mean(-1)
+    assert torch.allclose(ms, torch.ones_like(ms), atol=2e-2)
+    # scale covariance: rms_norm(2x) == rms_norm(x) (power-of-two scale is exact in bf16)
+    r2 = kernels.rms_norm(x * 2, gam, eps=4e-6)
+    assert torch.equal(r2, r)
+    ln = kernels.layer_norm(x, gam, torch.zeros_like(gam), eps=1e-5)
+    assert ln.float().mean(-1).abs().max().item() < 2e-2
+    assert_close(ln[idx], oracle.layer_norm(as_f64(sub), 1.0, 0.0, 1e-5), 2e-2, "ln sampled rows")
+    ge = kernels.bias_gelu(x, torch.zeros_like(gam))
+    assert_close(ge[idx], oracle.gelu_tanh(as_f64(sub)), 2e-2, "gelu sampled rows")
