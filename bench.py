@@ -1,0 +1,212 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused-kernel hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--only]
+
+One "step" is one launch of the workload's kernel over one batch of synthetic
+input that already sits in HBM.  The headline workload is BASELINE.json
+configs[1] (bf16 GEMM 4096^3, fp32 accumulate); the other BASELINE kernels
+(flash attention, softmax, LayerNorm, RMSNorm, bias+GELU) are timed the same way
+and reported under "kernels" of the same JSON line unless --only is given.
+
+Timing: HIP events recorded on the stream the kernels are launched on, around
+exactly K launches, after W warm-up launches, bracketed by device
+synchronisation.  `roofline.achieved` = algorithmic FLOPs (or bytes) per launch
+divided by the mean launch duration from those events.
+`cpu_baseline` times the C restatement under oracle/ on the host cores, on a
+bounded sample of the same workload (never part of the measured GPU path).
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+
+
+def _time_launches(fn, steps, warmup, torch):
+    """Mean seconds per launch of fn(i) over `steps` launches (HIP events on the
+    current stream), after `warmup` untimed launches."""
+    for i in range(warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for i in range(steps):
+        fn(i)
+    stop.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return start.elapsed_time(stop) * 1e-3 / steps, wall / steps
+
+
+# ---------------------------------------------------------------- workloads
+def wl_gemm(torch, kernels, M=4096, N=4096, K=4096):
+    g = torch.Generator(device="cuda").manual_seed(2)
+    a = (torch.rand(M, K, generator=g, device="cuda") * 2 - 1).to(torch.bfloat16)
+    b = (torch.rand(K, N, generator=g, device="cuda") * 2 - 1).to(torch.bfloat16)
+    c = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    return dict(name=f"bf16 GEMM {M}x{N}x{K} (row-major A[M,K], B[K,N]; fp32 accumulate, bf16 out)",
+                fn=lambda i: kernels.matmul(a, b, out=c), flops=2.0 * M * N * K,
+                bytes=2.0 * (M * K + K * N + M * N), bound="mfma", kernel="gemm_mfma_kernel")
+
+
+def wl_attention(torch, kernels, B=4, H=32, S=4096, D=128, causal=True):
+    g = torch.Generator(device="cuda").manual_seed(4)
+    q, k, v = (torch.randn(B, H, S, D, generator=g, device="cuda").to(torch.bfloat16) for _ in range(3))
+    flops = 4.0 * B * H * S * S * D * (0.5 if causal else 1.0)
+    return dict(name=f"bf16 flash-attention fwd B{B} H{H} S{S} D{D} {'causal' if causal else 'full'}",
+                fn=lambda i: kernels.flash_attention(q, k, v, is_causal=causal), flops=flops,
+                bytes=4.0 * B * H * S * D * 2, bound="mfma", kernel="fa_fwd_kernel")
+
+
+def _rows(torch, rows=32768, cols=4096, nbuf=3):
+    # several input sets, visited round-robin, so that a launch cannot find its
+    # input still resident in the 256 MB last-level cache from the previous one
+    g = torch.Generator(device="cuda").manual_seed(3)
+    xs = [torch.randn(rows, cols, generator=g, device="cuda").to(torch.bfloat16) for _ in range(nbuf)]
+    gam = (1 + 0.1 * torch.randn(cols, generator=g, device="cuda")).to(torch.bfloat16)
+    bet = (0.1 * torch.randn(cols, generator=g, device="cuda")).to(torch.bfloat16)
+    bias = (0.02 * torch.randn(cols, generator=g, device="cuda")).to(torch.bfloat16)
+    return xs, gam, bet, bias
+
+
+def wl_rows(torch, kernels, op, rows=32768, cols=4096):
+    from metalhlo_amd import _lib
+    lib = _lib.load()
+    xs, gam, bet, bias = _rows(torch, rows, cols)
+    ys = [torch.empty_like(x) for x in xs]
+    st = lambda: torch.cuda.current_stream().cuda_stream
+    n = len(xs)
+    base = 2.0 * rows * cols * 2
+    if op == "softmax":
+        fn = lambda i: lib.mhip_softmax(st(), xs[i % n].data_ptr(), ys[i % n].data_ptr(), rows, cols, 3)
+        extra, kern = 0, "row_wave_kernel<bf16,softmax>"
+    elif op == "layer_norm":
+        fn = lambda i: lib.mhip_layer_norm(st(), xs[i % n].data_ptr(), gam.data_ptr(), bet.data_ptr(),
+                                           ys[i % n].data_ptr(), rows, cols, 1e-5, 3)
+        extra, kern = 2 * cols * 2, "row_wave_kernel<bf16,layer_norm>"
+    elif op == "rms_norm":
+        fn = lambda i: lib.mhip_rms_norm(st(), xs[i % n].data_ptr(), gam.data_ptr(), ys[i % n].data_ptr(),
+                                         rows, cols, 1e-6, 3)
+        extra, kern = cols * 2, "row_wave_kernel<bf16,rms_norm>"
+    elif op == "bias_gelu":
+        fn = lambda i: lib.mhip_bias_gelu(st(), xs[i % n].data_ptr(), bias.data_ptr(), ys[i % n].data_ptr(),
+                                          rows, cols, 3)
+        extra, kern = cols * 2, "bias_gelu_vec_kernel<bf16>"
+    else:
+        raise ValueError(op)
+    return dict(name=f"bf16 {op} [{rows},{cols}]", fn=fn, flops=0.0, bytes=base + extra, bound="hbm",
+                kernel=kern)
+
+
+def measure(wl, steps, warmup, torch):
+    sec, wall = _time_launches(wl["fn"], steps, warmup, torch)
+    if wl["bound"] == "mfma":
+        ach = wl["flops"] / sec / 1e12
+        roof = dict(bound="mfma", achieved=round(ach, 2), peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
+                    frac=round(ach / PEAK_BF16_TFLOPS, 4), traffic=None)
+        value, unit = ach, "TFLOP/s"
+    else:
+        ach = wl["bytes"] / sec / 1e9
+        roof = dict(bound="hbm", achieved=round(ach, 1), peak=PEAK_HBM_GBS, unit="GB/s",
+                    frac=round(ach / PEAK_HBM_GBS, 4), traffic=None)
+        value, unit = ach, "GB/s"
+    return dict(workload=wl["name"], kernel=wl["kernel"], value=round(value, 2), unit=unit,
+                us_per_launch=round(sec * 1e6, 2), wall_us_per_launch=round(wall * 1e6, 2), roofline=roof)
+
+
+# ---------------------------------------------------------------- CPU baseline (oracle port)
+def cpu_baseline_gemm(sample_rows=512, N=4096, K=4096):
+    import numpy as np
+    from oracle import oracle
+    lib = C.CDLL(os.path.join(ROOT, "oracle", "liboracle.so"))
+    lib.orc_num_threads.restype = C.c_int
+    rng = np.random.default_rng(2)
+    a = oracle.bf16_round_bits(rng.uniform(-1, 1, (sample_rows, K)).astype(np.float32))
+    b = oracle.bf16_round_bits(rng.uniform(-1, 1, (K, N)).astype(np.float32))
+    c = np.empty((sample_rows, N), np.uint16)
+    p = lambda x: x.ctypes.data_as(C.c_void_p)
+    args = (p(a), p(b), p(c), C.c_int64(sample_rows), C.c_int64(N), C.c_int64(K), 1)
+    lib.orc_gemm(*args)                     # warm-up
+    best = float("inf")
+    for _ in range(3):
+        t0 = time.perf_counter()
+        lib.orc_gemm(*args)
+        best = min(best, time.perf_counter() - t0)
+    return dict(value=round(2.0 * sample_rows * N * K / best / 1e12, 5), unit="TFLOP/s",
+                cores=int(lib.orc_num_threads()), kind="port",
+                sample=f"oracle/oracle_kernels.c orc_gemm on {sample_rows} of 4096 rows of A "
+                       f"(x full B), bf16 in / fp32 accumulate, best of 3; host has {os.cpu_count()} logical CPUs")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="gemm",
+                    choices=["gemm", "attention", "attention_full", "softmax", "layer_norm", "rms_norm", "bias_gelu"])
+    ap.add_argument("--only", action="store_true", help="time only --workload (for profiling runs)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on exactly one GPU (the reference is single-device and "
+                 "every workload here shards without communication); use --gpus 1")
+
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible; the kernels have no CPU path")
+    from metalhlo_amd import _lib, kernels
+    _lib.load()
+    torch.cuda.set_device(0)
+
+    def build(name):
+        if name == "gemm":
+            return wl_gemm(torch, kernels)
+        if name == "attention":
+            return wl_attention(torch, kernels, causal=True)
+        if name == "attention_full":
+            return wl_attention(torch, kernels, S=2048, causal=False)
+        return wl_rows(torch, kernels, name)
+
+    head = measure(build(args.workload), args.steps, args.warmup, torch)
+    others = {}
+    if not args.only:
+        for name in ["gemm", "attention", "attention_full", "softmax", "layer_norm", "rms_norm", "bias_gelu"]:
+            if name == args.workload:
+                continue
+            torch.cuda.empty_cache()
+            others[name] = measure(build(name), args.steps, args.warmup, torch)
+            print(f"[bench] {name}: {others[name]['value']} {others[name]['unit']} "
+                  f"({others[name]['roofline']['frac'] * 100:.1f}% of peak)", file=sys.stderr, flush=True)
+    cpu = None
+    if not args.no_cpu and args.workload == "gemm":
+        cpu = cpu_baseline_gemm()
+
+    line = {
+        "metric": "bf16 attn/GEMM TFLOP/s + norm/softmax GB/s (% roofline); GPT-2 fwd ms",
+        "value": head["value"], "unit": head["unit"], "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(head["us_per_launch"] / 1e3, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": head["workload"], "kernel": head["kernel"]},
+        "roofline": head["roofline"],
+        "cpu_baseline": cpu,
+        "kernels": others,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -35,7 +35,7 @@ SIGNATURES = {
     "mhip_transpose_0213": (_i32, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32]),
     "mhip_split_qkv_heads": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32]),
     "mhip_iota": (_i32, [_vp, _vp, _i64, _i64, _i64, _i32]),
-    "mhip_argmax": (_i32, [_vp, _vp, _vp, _i64, _i64, _i32, _i32]),
+    "mhip_argmax": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32]),
 }
 
 _lib = None

@@ -414,12 +414,12 @@ extern "C" int mhip_flash_attention(void* stream, const void* q, const void* k, 
                                     const void* mask, void* o, int64_t B, int64_t H, int64_t Sq,
                                     int64_t Skv, int64_t D, float scale, int is_causal,
                                     int64_t mask_stride_b, int64_t mask_stride_h, int dtype) {
-    if (!q || !k || !v || !o)
-        return fail(MHIP_ERR_INVALID_ARGUMENT, "mhip_flash_attention: NULL tensor pointer");
     if (B < 0 || H < 0 || Sq < 0 || Skv < 0 || D <= 0)
         return fail(MHIP_ERR_INVALID_ARGUMENT, "mhip_flash_attention: bad size");
     if (D > 256) return fail(MHIP_ERR_UNSUPPORTED, "mhip_flash_attention: head_dim %lld > 256", (long long)D);
     if (B == 0 || H == 0 || Sq == 0) return MHIP_OK;
+    if (!q || !o || (Skv > 0 && (!k || !v)))
+        return fail(MHIP_ERR_INVALID_ARGUMENT, "mhip_flash_attention: NULL tensor pointer");
     if (Sq > 0x7FFFFFFF || Skv > 0x7FFFFFFF || B * H > 0x7FFFFFFF)
         return fail(MHIP_ERR_UNSUPPORTED, "mhip_flash_attention: dimension exceeds 2^31-1");
     hipStream_t s = as_stream(stream);

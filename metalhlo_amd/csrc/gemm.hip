@@ -363,12 +363,12 @@ extern "C" int mhip_gemm(void* stream, const void* a, const void* b, const void*
                          int64_t M, int64_t N, int64_t K, int64_t batch, int64_t stride_a,
                          int64_t stride_b, int64_t stride_c, int trans_a, int trans_b,
                          int activation, int dtype) {
-    if (!a || !b || !c) return fail(MHIP_ERR_INVALID_ARGUMENT, "mhip_gemm: NULL matrix pointer");
     if (M < 0 || N < 0 || K < 0 || batch < 0)
         return fail(MHIP_ERR_INVALID_ARGUMENT, "mhip_gemm: negative size");
     if (activation < MHIP_ACT_NONE || activation > MHIP_ACT_SIGMOID)
         return fail(MHIP_ERR_INVALID_ARGUMENT, "mhip_gemm: unknown activation %d", activation);
     if (M == 0 || N == 0 || batch == 0) return MHIP_OK;
+    if (!a || !b || !c) return fail(MHIP_ERR_INVALID_ARGUMENT, "mhip_gemm: NULL matrix pointer");
     if (M > 0x7FFFFFFF || N > 0x7FFFFFFF || K > 0x7FFFFFFF)
         return fail(MHIP_ERR_UNSUPPORTED, "mhip_gemm: dimension exceeds 2^31-1");
     hipStream_t s = as_stream(stream);

@@ -311,9 +311,9 @@ static int launch_row(hipStream_t s, const void* x, const void* g, const void* b
 template <int OP>
 static int row_entry(const char* name, void* stream, const void* x, const void* g, const void* b,
                      void* y, int64_t rows, int64_t cols, float eps, int dtype) {
-    if (!x || !y) return fail(MHIP_ERR_INVALID_ARGUMENT, "%s: NULL tensor pointer", name);
     if (rows < 0 || cols < 0) return fail(MHIP_ERR_INVALID_ARGUMENT, "%s: negative size", name);
     if (rows == 0 || cols == 0) return MHIP_OK;
+    if (!x || !y) return fail(MHIP_ERR_INVALID_ARGUMENT, "%s: NULL tensor pointer", name);
     if (rows > 0x7FFFFFFFLL) return fail(MHIP_ERR_UNSUPPORTED, "%s: more than 2^31-1 rows", name);
     hipStream_t s = as_stream(stream);
     switch (dtype) {
@@ -370,9 +370,9 @@ extern "C" int mhip_rms_norm(void* stream, const void* x, const void* gamma, voi
 
 extern "C" int mhip_bias_gelu(void* stream, const void* x, const void* bias, void* y, int64_t rows,
                               int64_t cols, int dtype) {
-    if (!x || !y) return fail(MHIP_ERR_INVALID_ARGUMENT, "mhip_bias_gelu: NULL tensor pointer");
     if (rows < 0 || cols < 0) return fail(MHIP_ERR_INVALID_ARGUMENT, "mhip_bias_gelu: negative size");
     if (rows == 0 || cols == 0) return MHIP_OK;
+    if (!x || !y) return fail(MHIP_ERR_INVALID_ARGUMENT, "mhip_bias_gelu: NULL tensor pointer");
     hipStream_t s = as_stream(stream);
     switch (dtype) {
         case MHIP_F32: return launch_gelu<float>(s, x, bias, y, rows, cols);
@@ -384,10 +384,10 @@ extern "C" int mhip_bias_gelu(void* stream, const void* x, const void* bias, voi
 
 extern "C" int mhip_softmax_strided(void* stream, const void* x, void* y, int64_t outer,
                                     int64_t axis_len, int64_t inner, int dtype) {
-    if (!x || !y) return fail(MHIP_ERR_INVALID_ARGUMENT, "mhip_softmax_strided: NULL tensor pointer");
     if (outer < 0 || axis_len < 0 || inner < 0)
         return fail(MHIP_ERR_INVALID_ARGUMENT, "mhip_softmax_strided: negative size");
     if (outer == 0 || axis_len == 0 || inner == 0) return MHIP_OK;
+    if (!x || !y) return fail(MHIP_ERR_INVALID_ARGUMENT, "mhip_softmax_strided: NULL tensor pointer");
     if (inner == 1) return mhip_softmax(stream, x, y, outer, axis_len, dtype);
     const int64_t grid = (outer * inner + 255) / 256;
     if (grid > 0x7FFFFFFFLL) return fail(MHIP_ERR_UNSUPPORTED, "mhip_softmax_strided: too large");

@@ -1,0 +1,254 @@
+"""Pins the CPU oracle (oracle/oracle.py and the C restatement oracle/liboracle.so)
+against (1) the known answers the reference's own tests hold (tests/golden/kat.json),
+(2) independent library routines (torch CPU), and (3) what the mathematics
+fixes: invariants, closed forms, brute force on tiny inputs.  Runs without a GPU."""
+import ctypes as C
+import json
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle
+
+KAT = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "kat.json")))
+
+
+# ---------------------------------------------------------------- bf16 rounding
+def test_bf16_rne_matches_torch_everywhere():
+    # every bf16 value, its neighbours' midpoints (ties) and off-midpoint values
+    hi = np.arange(0, 1 << 16, dtype=np.uint32) << 16
+    for low in (0x0000, 0x0001, 0x7FFF, 0x8000, 0x8001, 0xFFFF):
+        bits = (hi | low).astype(np.uint32)
+        f = bits.view(np.float32)
+        ok = ~np.isnan(f)
+        exp = torch.from_numpy(f[ok].copy()).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+        assert np.array_equal(oracle.bf16_round_bits(f[ok]), exp)
+    assert oracle.bf16_round_bits(np.float32("nan"))[()] == 0x7FC0
+    # explicit ties: 1 + 2^-8 is halfway between 1.0 (even) and 1 + 2^-7
+    assert oracle.bf16_round_bits(np.float32(1.00390625))[()] == 0x3F80
+    assert oracle.bf16_round_bits(np.float32(1.01171875))[()] == 0x3F82
+    x = np.random.default_rng(0).standard_normal(1000).astype(np.float32)
+    assert np.array_equal(oracle.bf16_bits_to_f32(oracle.bf16_round_bits(x)),
+                          torch.from_numpy(x).to(torch.bfloat16).float().numpy())
+
+
+# ---------------------------------------------------------------- reference KATs
+def test_softmax_kat():
+    for c in KAT["softmax"]:
+        assert np.allclose(oracle.softmax(np.array(c["x"], float)), np.array(c["y"]), atol=1e-12), c["src"]
+
+
+def test_gelu_kat():
+    for c in KAT["gelu"]:
+        # the reference test's constant is 0.7978845608 (10 digits): 1e-9 apart
+        assert np.allclose(oracle.gelu_tanh(np.array(c["x"], float)), np.array(c["y"]), atol=1e-8)
+    assert oracle.gelu_tanh(0.0) == 0.0 and oracle.gelu_tanh(3.0) > 2.9
+
+
+def test_norm_kat():
+    for c in KAT["rms_norm"]:
+        y = oracle.rms_norm(np.array(c["x"], float), np.array(c["gamma"], float), c["eps"])
+        assert np.allclose(y, np.array(c["y"]), atol=c["tol"])
+    for c in KAT["layer_norm"]:
+        y = oracle.layer_norm(np.array(c["x"], float), np.array(c["gamma"], float),
+                              np.array(c["beta"], float), c["eps"])
+        assert np.all(np.abs(y.mean(-1)) < 1e-4) and np.all(np.abs(y.std(-1) - 1) < 1e-4)
+        if "y" in c:
+            assert np.allclose(y, np.array(c["y"]), atol=1e-12)
+
+
+def test_dot_kat():
+    for c in KAT["dot"]:
+        y = oracle.dot_general(np.array(c["lhs"]), np.array(c["rhs"]), c["lhs_batch"], c["rhs_batch"],
+                               c["lhs_contract"], c["rhs_contract"],
+                               dtype=np.int64 if c["tol"] == 0 else np.float64)
+        assert np.array_equal(y, np.array(c["y"])), c["src"]
+
+
+def test_dot_general_dims_follows_reference_rule():
+    # CodeGenerator.swift:5939-5970 examples: plain, batched, multi-head
+    assert oracle.dot_general_dims([2, 3], [3, 2]) == (2, 3, 2, 1)
+    assert oracle.dot_general_dims([2, 3, 4], [2, 4, 5], [0], [0], [2], [1]) == (3, 4, 5, 2)
+    assert oracle.dot_general_dims([4, 3], [5, 4], [], [], [0], [1]) == (3, 4, 5, 1)
+    assert oracle.dot_general_dims([8, 12, 64, 32], [8, 12, 32, 64], [0, 1], [0, 1], [3], [2]) == (64, 32, 64, 96)
+
+
+# ---------------------------------------------------------------- library cross-checks
+def test_against_torch_cpu():
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal((5, 37)) * 3
+    t = torch.from_numpy(x)
+    assert np.allclose(oracle.softmax(x), torch.softmax(t, -1).numpy(), atol=1e-14)
+    assert np.allclose(oracle.softmax(x.reshape(5, 37, 1), axis=1)[..., 0], oracle.softmax(x), atol=0)
+    g, b = rng.standard_normal(37), rng.standard_normal(37)
+    ln = torch.nn.functional.layer_norm(t, (37,), torch.from_numpy(g), torch.from_numpy(b), 1e-5)
+    assert np.allclose(oracle.layer_norm(x, g, b, 1e-5), ln.numpy(), atol=1e-12)
+    ge = torch.nn.functional.gelu(t, approximate="tanh")
+    assert np.allclose(oracle.gelu_tanh(x), ge.numpy(), atol=1e-12)
+    rms = t / torch.sqrt((t * t).mean(-1, keepdim=True) + 1e-6) * torch.from_numpy(g)
+    assert np.allclose(oracle.rms_norm(x, g, 1e-6), rms.numpy(), atol=1e-12)
+    q, k, v = (torch.from_numpy(rng.standard_normal((2, 3, 17, 8))) for _ in range(3))
+    for causal in (False, True):
+        ref = torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=causal)
+        assert np.allclose(oracle.attention(q.numpy(), k.numpy(), v.numpy(), is_causal=causal),
+                           ref.numpy(), atol=1e-12)
+    for act, fn in [("relu", torch.relu), ("silu", torch.nn.functional.silu), ("tanh", torch.tanh),
+                    ("sigmoid", torch.sigmoid)]:
+        assert np.allclose(oracle.ACTIVATIONS[act](x), fn(t).numpy(), atol=1e-12)
+
+
+# ---------------------------------------------------------------- what the maths fixes
+def test_attention_brute_force_and_invariants():
+    rng = np.random.default_rng(2)
+    q, k, v = rng.standard_normal((1, 1, 6, 4)), rng.standard_normal((1, 1, 9, 4)), rng.standard_normal((1, 1, 9, 4))
+    scale = 0.3
+    out = oracle.attention(q, k, v, scale=scale, is_causal=True)
+    for i in range(6):                       # scalar loops, no numpy broadcasting
+        w = [math.exp(scale * sum(q[0, 0, i, d] * k[0, 0, j, d] for d in range(4))) if j <= i else 0.0
+             for j in range(9)]
+        z = sum(w)
+        for d in range(4):
+            assert abs(out[0, 0, i, d] - sum(w[j] * v[0, 0, j, d] for j in range(9)) / z) < 1e-12
+    assert np.allclose(out[0, 0, 0], v[0, 0, 0])                              # causal row 0
+    vu = np.broadcast_to(v[:, :, :1], v.shape)
+    assert np.allclose(oracle.attention(q, k, vu), vu[:, :, :6][..., :], atol=1e-12)  # uniform V
+    m = np.where(np.arange(9)[None] > np.arange(6)[:, None], -np.inf, 0.0)
+    assert np.allclose(oracle.attention(q, k, v, scale=scale, mask=m), out, atol=1e-14)  # flag == mask
+    shift = rng.standard_normal((6, 1))                                       # row-constant shift
+    assert np.allclose(oracle.attention(q, k, v, mask=np.broadcast_to(shift, (6, 9))),
+                       oracle.attention(q, k, v), atol=1e-12)
+    dead = np.full((6, 9), 0.0); dead[2] = -np.inf
+    assert np.all(oracle.attention(q, k, v, mask=dead)[0, 0, 2] == 0)         # l_inv guard
+    rows = np.array([0, 3, 5])
+    assert np.allclose(oracle.attention_rows(q[0, 0], k[0, 0], v[0, 0], rows, scale, True), out[0, 0, rows])
+    assert np.allclose(oracle.attention(q, k, v), oracle.attention(q, k, v, scale=0.5))  # default 1/sqrt(4)
+
+
+def test_norm_invariants_and_gemm_brute_force():
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((4, 33))
+    assert np.allclose(oracle.layer_norm(3 * x + 7, eps=0), oracle.layer_norm(x, eps=0), atol=1e-12)
+    assert np.allclose(oracle.rms_norm(5 * x, eps=0), oracle.rms_norm(x, eps=0), atol=1e-12)
+    assert np.allclose((oracle.rms_norm(x, eps=0) ** 2).mean(-1), 1)
+    assert np.allclose(oracle.softmax(x + 11.5), oracle.softmax(x), atol=1e-14)
+    a, b = rng.standard_normal((5, 7)), rng.standard_normal((7, 3))
+    brute = [[sum(a[i, k] * b[k, j] for k in range(7)) for j in range(3)] for i in range(5)]
+    assert np.allclose(oracle.gemm(a, b), brute, atol=1e-13)
+    assert np.allclose(oracle.gemm(a.T, b.T, True, True), brute, atol=1e-13)
+    bias = rng.standard_normal(3)
+    assert np.allclose(oracle.matmul_bias_act(a, b, bias, "gelu"), oracle.gelu_tanh(np.array(brute) + bias))
+
+
+def test_custom_call_dispatch_contract():
+    rng = np.random.default_rng(4)
+    q, k, v = (rng.standard_normal((1, 2, 5, 4)) for _ in range(3))
+    cfg = json.dumps({"scale": 0.5, "has_mask": False, "is_causal": True})
+    assert np.allclose(oracle.custom_call("fused_scaled_dot_product_attention", [q, k, v], cfg),
+                       oracle.attention(q, k, v, scale=0.5, is_causal=True))
+    # no config -> scale 1.0 (handler default), garbage config -> {}
+    assert np.allclose(oracle.custom_call("fused_scaled_dot_product_attention", [q, k, v], "not json"),
+                       oracle.attention(q, k, v, scale=1.0))
+    m = rng.standard_normal((5, 5))
+    assert np.allclose(oracle.custom_call("fused_scaled_dot_product_attention", [q, k, v, m], '{"has_mask":true}'),
+                       oracle.attention(q, k, v, scale=1.0, mask=m))
+    # mask operand present but has_mask false -> ignored (CustomCallHandlers.swift:197-200)
+    assert np.allclose(oracle.custom_call("fused_scaled_dot_product_attention", [q, k, v, m], ""),
+                       oracle.attention(q, k, v, scale=1.0))
+    with pytest.raises(ValueError):
+        oracle.custom_call("fused_layer_norm", [q, k], "")
+    with pytest.raises(KeyError):
+        oracle.custom_call("fused_rope", [q], "")
+
+
+# ---------------------------------------------------------------- C restatement vs float64 closed forms
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def _bf16(a):
+    return oracle.bf16_round_bits(a.astype(np.float32))
+
+
+@pytest.mark.parametrize("et", [0, 1], ids=["f32", "bf16"])
+def test_c_oracle_matches_float64(oracle_c, et):
+    rng = np.random.default_rng(5)
+    i64, f32 = C.c_int64, C.c_float
+    tol = 1e-5 if et == 0 else 2e-2
+    enc = (lambda a: a.astype(np.float32)) if et == 0 else _bf16
+    dec = (lambda a: a.astype(np.float64)) if et == 0 else (lambda a: oracle.bf16_bits_to_f32(a).astype(np.float64))
+
+    def close(got, exp):
+        g = dec(got)
+        return np.all(np.abs(g - exp) <= np.maximum(tol, tol * np.abs(exp)))
+
+    rows, cols = 9, 203
+    x = enc(rng.standard_normal((rows, cols)) * 2)
+    g = enc(1 + 0.1 * rng.standard_normal(cols)); b = enc(0.1 * rng.standard_normal(cols))
+    y = np.empty_like(x)
+    oracle_c.orc_softmax(_p(x), _p(y), i64(rows), i64(cols), et)
+    assert close(y, oracle.softmax(dec(x)))
+    oracle_c.orc_layer_norm(_p(x), _p(g), _p(b), _p(y), i64(rows), i64(cols), f32(1e-5), et)
+    assert close(y, oracle.layer_norm(dec(x), dec(g), dec(b), 1e-5))
+    oracle_c.orc_rms_norm(_p(x), _p(g), _p(y), i64(rows), i64(cols), f32(1e-6), et)
+    assert close(y, oracle.rms_norm(dec(x), dec(g), 1e-6))
+    oracle_c.orc_bias_gelu(_p(x), _p(b), _p(y), i64(rows), i64(cols), et)
+    assert close(y, oracle.bias_gelu(dec(x), dec(b)))
+    M, N, K = 13, 21, 40
+    a = enc(rng.uniform(-1, 1, (M, K))); w = enc(rng.uniform(-1, 1, (K, N)))
+    c = np.empty((M, N), dtype=a.dtype)
+    oracle_c.orc_gemm(_p(a), _p(w), _p(c), i64(M), i64(N), i64(K), et)
+    assert close(c, oracle.gemm(dec(a), dec(w)))
+    B, H, Sq, Skv, D = 2, 3, 19, 23, 16
+    q = enc(rng.standard_normal((B, H, Sq, D))); k = enc(rng.standard_normal((B, H, Skv, D)))
+    v = enc(rng.standard_normal((B, H, Skv, D)))
+    o = np.empty_like(q)
+    for causal in (0, 1):
+        oracle_c.orc_flash_attention(_p(q), _p(k), _p(v), _p(o), i64(B), i64(H), i64(Sq), i64(Skv), i64(D),
+                                     f32(0.25), causal, et)
+        assert close(o, oracle.attention(dec(q), dec(k), dec(v), scale=0.25, is_causal=bool(causal)))
+
+
+def test_c_oracle_kats(oracle_c):
+    i64, f32 = C.c_int64, C.c_float
+    for c in KAT["softmax"]:
+        x = np.array(c["x"], np.float32); y = np.empty_like(x)
+        oracle_c.orc_softmax(_p(x), _p(y), i64(x.shape[0]), i64(x.shape[1]), 0)
+        assert np.allclose(y, np.array(c["y"]), atol=c["tol"])
+    c = KAT["rms_norm"][0]
+    x = np.array(c["x"], np.float32); g = np.array(c["gamma"], np.float32); y = np.empty_like(x)
+    oracle_c.orc_rms_norm(_p(x), _p(g), _p(y), i64(1), i64(4), f32(c["eps"]), 0)
+    assert np.allclose(y, np.array(c["y"]), atol=c["tol"])
+    c = KAT["gelu"][0]
+    x = np.array([c["x"]], np.float32); y = np.empty_like(x)
+    oracle_c.orc_bias_gelu(_p(x), None, _p(y), i64(1), i64(6), 0)
+    assert np.allclose(y[0], np.array(c["y"]), atol=c["tol"])
+    x = np.random.default_rng(6).standard_normal(999).astype(np.float32)
+    out = np.empty(999, np.uint16)
+    oracle_c.orc_f32_to_bf16(_p(x), _p(out), i64(999))
+    assert np.array_equal(out, oracle.bf16_round_bits(x))
+
+
+def test_gpt2_oracle_shapes_and_determinism():
+    rng = np.random.default_rng(7)
+    d, nh, L, V, S = 32, 4, 2, 61, 10
+
+    def lyr():
+        z = lambda *s: np.zeros(s)
+        return dict(ln1_g=np.ones(d), ln1_b=z(d), w_qkv=rng.normal(0, 0.02, (d, 3 * d)), b_qkv=z(3 * d),
+                    w_o=rng.normal(0, 0.02, (d, d)), b_o=z(d), ln2_g=np.ones(d), ln2_b=z(d),
+                    w_fc=rng.normal(0, 0.02, (d, 4 * d)), b_fc=z(4 * d),
+                    w_proj=rng.normal(0, 0.02, (4 * d, d)), b_proj=z(d))
+    params = dict(wte=rng.normal(0, 0.02, (V, d)), wpe=rng.normal(0, 0.02, (16, d)),
+                  layers=[lyr() for _ in range(L)], lnf_g=np.ones(d), lnf_b=np.zeros(d))
+    ids = rng.integers(0, V, (2, S))
+    lo = oracle.gpt2_forward(ids, params, nh, "f64")
+    assert lo.shape == (2, S, V) and np.isfinite(lo).all()
+    # causality: changing a later token never changes earlier logits
+    ids2 = ids.copy(); ids2[:, -1] = (ids2[:, -1] + 1) % V
+    lo2 = oracle.gpt2_forward(ids2, params, nh, "f64")
+    assert np.allclose(lo[:, :-1], lo2[:, :-1], atol=1e-12) and not np.allclose(lo[:, -1], lo2[:, -1])
+    lb = oracle.gpt2_forward(ids, params, nh, "bf16")
+    assert np.max(np.abs(lb - lo)) < 2e-2 * max(1.0, np.max(np.abs(lo)))

@@ -9,7 +9,7 @@ NAME = {torch.float32: "f32", torch.bfloat16: "bf16", torch.float16: "f16"}
 def to_dev(a: np.ndarray, dtype) -> torch.Tensor:
     """numpy (float64/float32/int) -> device tensor of `dtype`, RNE rounding."""
     t = torch.from_numpy(np.ascontiguousarray(a))
-    if t.dtype.is_floating_point:
+    if dtype.is_floating_point:
         t = t.to(torch.float32).to(dtype)
     return t.cuda()
 
