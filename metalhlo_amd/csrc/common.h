@@ -27,6 +27,13 @@ int fail(int code, const char* fmt, ...);
 // Checks the launch that was just issued.
 int check_launch(const char* what);
 
+// Compute units of the current device (queried once per device).
+int compute_units();
+
+// Integer launch-tuning knob from the environment (read on every call; unset or
+// unparsable -> `fallback`).
+int tune_int(const char* name, int fallback);
+
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 
 template <typename T> struct Elem;
@@ -59,16 +66,39 @@ template <typename T>
 __device__ inline void store16(T* p, const Vec16<T>& v) {
     *reinterpret_cast<Vec16<T>*>(p) = v;
 }
+// Streaming variants: data that is touched once should not displace the cache.
+template <typename T>
+__device__ inline Vec16<T> load16_stream(const T* p) {
+    const u32x4 r = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+    return __builtin_bit_cast(Vec16<T>, r);
+}
+template <typename T>
+__device__ inline void store16_stream(T* p, const Vec16<T>& v) {
+    __builtin_nontemporal_store(__builtin_bit_cast(u32x4, v), reinterpret_cast<u32x4*>(p));
+}
 
-__device__ inline float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o, kWave);
-    return v;
+// Wave-wide reductions on the DPP cross-lane network (no LDS traffic): four
+// steps inside each row of 16 lanes, two row broadcasts, result read from lane 63.
+struct SumOp { __device__ static float id() { return 0.f; } __device__ static float f(float a, float b) { return a + b; } };
+struct MaxOp { __device__ static float id() { return -__builtin_inff(); } __device__ static float f(float a, float b) { return fmaxf(a, b); } };
+
+template <int CTRL, int ROW_MASK>
+__device__ inline float dpp_move(float identity, float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, identity),
+                                                                 __builtin_bit_cast(int, v), CTRL,
+                                                                 ROW_MASK, 0xF, false));
 }
-__device__ inline float wave_max(float v) {
-#pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
-    return v;
+template <typename Op>
+__device__ inline float wave_reduce(float v) {
+    v = Op::f(v, dpp_move<0xB1, 0xF>(Op::id(), v));   // quad_perm [1,0,3,2]
+    v = Op::f(v, dpp_move<0x4E, 0xF>(Op::id(), v));   // quad_perm [2,3,0,1]
+    v = Op::f(v, dpp_move<0x141, 0xF>(Op::id(), v));  // row_half_mirror
+    v = Op::f(v, dpp_move<0x140, 0xF>(Op::id(), v));  // row_mirror
+    v = Op::f(v, dpp_move<0x142, 0xA>(Op::id(), v));  // row_bcast:15 into rows 1 and 3
+    v = Op::f(v, dpp_move<0x143, 0xC>(Op::id(), v));  // row_bcast:31 into rows 2 and 3
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
+__device__ inline float wave_sum(float v) { return wave_reduce<SumOp>(v); }
+__device__ inline float wave_max(float v) { return wave_reduce<MaxOp>(v); }
 
 }  // namespace mhip

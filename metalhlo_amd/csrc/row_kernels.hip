@@ -16,6 +16,26 @@ enum RowOp { kSoftmax = 0, kLayerNorm = 1, kRmsNorm = 2 };
 
 constexpr int kRowsPerBlock = 4;
 
+// Per-column parameters (gamma, beta, bias) are converted to fp32 once per
+// workgroup and parked in LDS, split into planes of four floats so that the
+// 64 lanes of a wave read 64 consecutive 16-byte slots (no bank conflicts);
+// each workgroup then walks many rows, so the parameters cost no HBM or L2
+// traffic per row.
+template <typename T>
+__device__ inline void stage_params(const T* __restrict__ p, f32x4* lds, int nvec) {
+    constexpr int E = Elem<T>::kPerVec;
+    for (int i = threadIdx.x; i < nvec; i += 256) {
+        const Vec16<T> t = load16(p + (int64_t)i * E);
+#pragma unroll
+        for (int q = 0; q < E / 4; q++) {
+            f32x4 w;
+#pragma unroll
+            for (int e = 0; e < 4; e++) w[e] = Elem<T>::to_f32(t.v[4 * q + e]);
+            lds[q * nvec + i] = w;
+        }
+    }
+}
+
 template <typename T, int OP, int NV>
 __global__ __launch_bounds__(256) void row_wave_kernel(const T* __restrict__ x,
                                                        const T* __restrict__ gamma,
@@ -23,109 +43,112 @@ __global__ __launch_bounds__(256) void row_wave_kernel(const T* __restrict__ x,
                                                        T* __restrict__ y, int64_t rows, int cols,
                                                        float eps) {
     constexpr int E = Elem<T>::kPerVec;
+    constexpr int P = E / 4;
+    extern __shared__ __attribute__((aligned(16))) f32x4 row_params[];
     const int lane = threadIdx.x & 63;
-    const int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
-    if (row >= rows) return;
-    const T* xr = x + row * cols;
-    T* yr = y + row * cols;
     const int nvec = cols / E;
-
-    float f[NV][E];
-#pragma unroll
-    for (int v = 0; v < NV; v++) {
-        const int idx = v * 64 + lane;
-        if (idx < nvec) {
-            Vec16<T> t = load16(xr + (int64_t)idx * E);
-#pragma unroll
-            for (int e = 0; e < E; e++) f[v][e] = Elem<T>::to_f32(t.v[e]);
-        } else {
-#pragma unroll
-            for (int e = 0; e < E; e++) f[v][e] = (OP == kSoftmax) ? -INFINITY : 0.f;
-        }
+    f32x4* gs = row_params;
+    f32x4* bs = row_params + (gamma ? P * nvec : 0);
+    if (OP != kSoftmax && (gamma || beta)) {
+        if (gamma) stage_params(gamma, gs, nvec);
+        if (OP == kLayerNorm && beta) stage_params(beta, bs, nvec);
+        __syncthreads();
     }
 
-    float a = 0.f, b = 0.f;  // per-row statistics; meaning depends on OP
-    if (OP == kSoftmax) {
-        float m = -INFINITY;
-#pragma unroll
-        for (int v = 0; v < NV; v++)
-#pragma unroll
-            for (int e = 0; e < E; e++) m = fmaxf(m, f[v][e]);
-        m = wave_max(m);
-        float s = 0.f;
-#pragma unroll
-        for (int v = 0; v < NV; v++)
-#pragma unroll
-            for (int e = 0; e < E; e++) {
-                float ex = (sizeof(T) == 4) ? expf(f[v][e] - m) : __expf(f[v][e] - m);
-                f[v][e] = ex;
-                s += ex;
-            }
-        s = wave_sum(s);
-        a = 1.f / s;
-    } else if (OP == kLayerNorm) {
-        float s = 0.f;
-#pragma unroll
-        for (int v = 0; v < NV; v++)
-#pragma unroll
-            for (int e = 0; e < E; e++) s += f[v][e];
-        const float mean = wave_sum(s) / (float)cols;
-        float q = 0.f;
+    for (int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6); row < rows;
+         row += (int64_t)gridDim.x * kRowsPerBlock) {
+        const T* xr = x + row * cols;
+        T* yr = y + row * cols;
+
+        float f[NV][E];
 #pragma unroll
         for (int v = 0; v < NV; v++) {
-            if (v * 64 + lane < nvec) {
+            const int idx = v * 64 + lane;
+            if (idx < nvec) {
+                Vec16<T> t = load16_stream(xr + (int64_t)idx * E);
 #pragma unroll
-                for (int e = 0; e < E; e++) {
-                    const float d = f[v][e] - mean;
-                    q += d * d;
-                }
+                for (int e = 0; e < E; e++) f[v][e] = Elem<T>::to_f32(t.v[e]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < E; e++) f[v][e] = (OP == kSoftmax) ? -INFINITY : 0.f;
             }
         }
-        const float var = wave_sum(q) / (float)cols;
-        a = mean;
-        b = 1.f / sqrtf(var + eps);
-    } else {
-        float q = 0.f;
-#pragma unroll
-        for (int v = 0; v < NV; v++)
-#pragma unroll
-            for (int e = 0; e < E; e++) q += f[v][e] * f[v][e];
-        a = 1.f / sqrtf(wave_sum(q) / (float)cols + eps);
-    }
 
+        float a = 0.f, b = 0.f;  // per-row statistics; meaning depends on OP
+        if (OP == kSoftmax) {
+            float m = -INFINITY;
 #pragma unroll
-    for (int v = 0; v < NV; v++) {
-        const int idx = v * 64 + lane;
-        if (idx < nvec) {
-            Vec16<T> o;
-            if (OP == kSoftmax) {
+            for (int v = 0; v < NV; v++)
 #pragma unroll
-                for (int e = 0; e < E; e++) o.v[e] = Elem<T>::from_f32(f[v][e] * a);
-            } else {
-                float g[E], bt[E];
-                if (gamma) {
-                    Vec16<T> t = load16(gamma + idx * E);
+                for (int e = 0; e < E; e++) m = fmaxf(m, f[v][e]);
+            m = wave_max(m);
+            float s = 0.f;
 #pragma unroll
-                    for (int e = 0; e < E; e++) g[e] = Elem<T>::to_f32(t.v[e]);
-                } else {
-#pragma unroll
-                    for (int e = 0; e < E; e++) g[e] = 1.f;
-                }
-                if (OP == kLayerNorm && beta) {
-                    Vec16<T> t = load16(beta + idx * E);
-#pragma unroll
-                    for (int e = 0; e < E; e++) bt[e] = Elem<T>::to_f32(t.v[e]);
-                } else {
-#pragma unroll
-                    for (int e = 0; e < E; e++) bt[e] = 0.f;
-                }
+            for (int v = 0; v < NV; v++)
 #pragma unroll
                 for (int e = 0; e < E; e++) {
-                    const float n = (OP == kLayerNorm) ? (f[v][e] - a) * b : f[v][e] * a;
-                    o.v[e] = Elem<T>::from_f32(n * g[e] + bt[e]);
+                    float ex = (sizeof(T) == 4) ? expf(f[v][e] - m)
+                                                : __builtin_amdgcn_exp2f((f[v][e] - m) * 1.4426950408889634f);
+                    f[v][e] = ex;
+                    s += ex;
+                }
+            s = wave_sum(s);
+            a = 1.f / s;
+        } else if (OP == kLayerNorm) {
+            float s = 0.f;
+#pragma unroll
+            for (int v = 0; v < NV; v++)
+#pragma unroll
+                for (int e = 0; e < E; e++) s += f[v][e];
+            const float mean = wave_sum(s) / (float)cols;
+            float q = 0.f;
+#pragma unroll
+            for (int v = 0; v < NV; v++) {
+                if (v * 64 + lane < nvec) {
+#pragma unroll
+                    for (int e = 0; e < E; e++) {
+                        const float d = f[v][e] - mean;
+                        q += d * d;
+                    }
                 }
             }
-            store16(yr + (int64_t)idx * E, o);
+            const float var = wave_sum(q) / (float)cols;
+            b = 1.f / sqrtf(var + eps);
+            a = -mean * b;
+        } else {
+            float q = 0.f;
+#pragma unroll
+            for (int v = 0; v < NV; v++)
+#pragma unroll
+                for (int e = 0; e < E; e++) q += f[v][e] * f[v][e];
+            a = 1.f / sqrtf(wave_sum(q) / (float)cols + eps);
+        }
+
+#pragma unroll
+        for (int v = 0; v < NV; v++) {
+            const int idx = v * 64 + lane;
+            if (idx < nvec) {
+                Vec16<T> o;
+                if (OP == kSoftmax) {
+#pragma unroll
+                    for (int e = 0; e < E; e++) o.v[e] = Elem<T>::from_f32(f[v][e] * a);
+                } else {
+#pragma unroll
+                    for (int q = 0; q < P; q++) {
+                        f32x4 g = {1.f, 1.f, 1.f, 1.f}, bt = {0.f, 0.f, 0.f, 0.f};
+                        if (gamma) g = gs[q * nvec + idx];
+                        if (OP == kLayerNorm && beta) bt = bs[q * nvec + idx];
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            const float xv = f[v][4 * q + e];
+                            // LayerNorm: (x - mean) * rstd == x * rstd + (-mean * rstd)
+                            const float n = (OP == kLayerNorm) ? fmaf(xv, b, a) : xv * a;
+                            o.v[4 * q + e] = Elem<T>::from_f32(fmaf(n, g[e], bt[e]));
+                        }
+                    }
+                }
+                store16_stream(yr + (int64_t)idx * E, o);
+            }
         }
     }
 }
@@ -215,49 +238,64 @@ __global__ __launch_bounds__(256) void softmax_strided_kernel(const T* __restric
 }
 
 // ---------------------------------------------------------------------------
-// bias + GELU(tanh): pure streaming, 4 x 128-bit vectors per thread.
+// bias + GELU(tanh): pure streaming; the bias sits in LDS as fp32 planes.
 // ---------------------------------------------------------------------------
 template <typename T>
 __device__ inline float gelu_tanh_f(float v) {
-    const float inner = 0.7978845608028654f * (v + 0.044715f * v * v * v);
-    if (sizeof(T) == 4) return 0.5f * v * (1.f + tanhf(inner));
-    // 0.5 (1 + tanh u) == 1 / (1 + exp(-2u)); ample for a 16-bit result.
-    return v * __frcp_rn(1.f + __expf(-2.f * inner));
+    if (sizeof(T) == 4) {
+        const float inner = 0.7978845608028654f * (v + 0.044715f * v * v * v);
+        return 0.5f * v * (1.f + tanhf(inner));
+    }
+    // 0.5 (1 + tanh u) == 1 / (1 + exp(-2u)) == 1 / (1 + 2^(-2 log2(e) u)); ample for
+    // a 16-bit result and three VALU + two transcendental operations.
+    constexpr float c0 = -2.f * 1.4426950408889634f * 0.7978845608028654f;
+    constexpr float c1 = c0 * 0.044715f;
+    const float t = v * fmaf(v * v, c1, c0);
+    return v * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(t));
 }
-
-constexpr int kGeluUnroll = 4;
 
 template <typename T>
 __global__ __launch_bounds__(256) void bias_gelu_vec_kernel(const T* __restrict__ x,
                                                             const T* __restrict__ bias,
                                                             T* __restrict__ y, int64_t nvec,
-                                                            int cols) {
+                                                            int nvec_row, int bias_in_lds) {
     constexpr int E = Elem<T>::kPerVec;
-    const int64_t base = (int64_t)blockIdx.x * (256 * kGeluUnroll) + threadIdx.x;
-    Vec16<T> in[kGeluUnroll];
-#pragma unroll
-    for (int u = 0; u < kGeluUnroll; u++) {
-        const int64_t i = base + u * 256;
-        if (i < nvec) in[u] = load16(x + i * E);
+    constexpr int P = E / 4;
+    extern __shared__ __attribute__((aligned(16))) f32x4 gelu_params[];
+    if (bias && bias_in_lds) {
+        stage_params(bias, gelu_params, nvec_row);
+        __syncthreads();
     }
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    for (int64_t i0 = (int64_t)blockIdx.x * 256 + threadIdx.x; i0 < nvec; i0 += 2 * stride) {
+        const int64_t i1 = i0 + stride;
+        const bool two = i1 < nvec;
+        Vec16<T> in0 = load16_stream(x + i0 * E), in1;
+        if (two) in1 = load16_stream(x + i1 * E);
 #pragma unroll
-    for (int u = 0; u < kGeluUnroll; u++) {
-        const int64_t i = base + u * 256;
-        if (i < nvec) {
+        for (int u = 0; u < 2; u++) {
+            if (u == 1 && !two) break;
+            const int64_t i = u ? i1 : i0;
+            const Vec16<T>& in = u ? in1 : in0;
             Vec16<T> o;
-            if (bias) {
-                const int col = (int)((i * E) % cols);
-                Vec16<T> bv = load16(bias + col);
+            const int cv = (int)(i % nvec_row);
 #pragma unroll
-                for (int e = 0; e < E; e++)
-                    o.v[e] = Elem<T>::from_f32(
-                        gelu_tanh_f<T>(Elem<T>::to_f32(in[u].v[e]) + Elem<T>::to_f32(bv.v[e])));
-            } else {
+            for (int q = 0; q < P; q++) {
+                f32x4 bv = {0.f, 0.f, 0.f, 0.f};
+                if (bias) {
+                    if (bias_in_lds) {
+                        bv = gelu_params[q * nvec_row + cv];
+                    } else {
 #pragma unroll
-                for (int e = 0; e < E; e++)
-                    o.v[e] = Elem<T>::from_f32(gelu_tanh_f<T>(Elem<T>::to_f32(in[u].v[e])));
+                        for (int e = 0; e < 4; e++) bv[e] = Elem<T>::to_f32(bias[(int64_t)cv * E + 4 * q + e]);
+                    }
+                }
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    o.v[4 * q + e] = Elem<T>::from_f32(
+                        gelu_tanh_f<T>(Elem<T>::to_f32(in.v[4 * q + e]) + bv[e]));
             }
-            store16(y + i * E, o);
+            store16_stream(y + i * E, o);
         }
     }
 }
@@ -291,15 +329,36 @@ static int launch_row(hipStream_t s, const void* x, const void* g, const void* b
                         aligned16(g) && aligned16(b);
     if (vec_ok) {
         const int nvec = (int)(cols / E);
-        const unsigned grid = (unsigned)((rows + kRowsPerBlock - 1) / kRowsPerBlock);
-#define MHIP_ROW_CASE(NV)                                                                  \
-    hipLaunchKernelGGL((row_wave_kernel<T, OP, NV>), dim3(grid), dim3(256), 0, s, xp, gp, \
-                       bp, yp, rows, (int)cols, eps)
-        if (nvec <= 64) MHIP_ROW_CASE(1);
-        else if (nvec <= 128) MHIP_ROW_CASE(2);
-        else if (nvec <= 256) MHIP_ROW_CASE(4);
-        else if (nvec <= 512) MHIP_ROW_CASE(8);
-        else MHIP_ROW_CASE(16);
+        // Persistent workgroups, exactly as many as the device holds at once for
+        // this kernel's register and LDS footprint: every CU stays full, and the
+        // LDS staging of the parameters is amortised over many rows.
+        const int64_t want = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
+        const size_t lds = (OP == kSoftmax) ? 0
+                                            : ((gp ? 1 : 0) + ((OP == kLayerNorm && bp) ? 1 : 0)) *
+                                                  (size_t)cols * sizeof(float);
+#define MHIP_ROW_CASE(NV)                                                                      \
+    {                                                                                          \
+        auto kern = row_wave_kernel<T, OP, NV>;                                                \
+        int per_cu = tune_int("MHIP_ROW_BLOCKS_PER_CU", 0);                                    \
+        if (per_cu == 0 &&                                                                     \
+            (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, 256, lds) !=          \
+                 hipSuccess || per_cu <= 0))                                                   \
+            per_cu = 4;                                                                        \
+        /* the occupancy query counts LDS to the last byte; keep a margin so that */          \
+        /* every workgroup of the grid really is resident at once */                          \
+        if (lds && per_cu > (int)((160 * 1024 - 4096) / (lds + 512)))                          \
+            per_cu = (int)((160 * 1024 - 4096) / (lds + 512));                                 \
+        if (per_cu < 1) per_cu = 1;                                                            \
+        const int64_t cap = (int64_t)compute_units() * per_cu;                                 \
+        const unsigned grid = (unsigned)(want < cap ? want : cap);                             \
+        hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, s, xp, gp, bp, yp, rows,          \
+                           (int)cols, eps);                                                    \
+    }
+        if (nvec <= 64) MHIP_ROW_CASE(1)
+        else if (nvec <= 128) MHIP_ROW_CASE(2)
+        else if (nvec <= 256) MHIP_ROW_CASE(4)
+        else if (nvec <= 512) MHIP_ROW_CASE(8)
+        else MHIP_ROW_CASE(16)
 #undef MHIP_ROW_CASE
     } else {
         hipLaunchKernelGGL((row_block_kernel<T, OP>), dim3((unsigned)rows), dim3(256), 0, s, xp,
@@ -333,12 +392,14 @@ static int launch_gelu(hipStream_t s, const void* x, const void* bias, void* y, 
                         aligned16(bias);
     if (vec_ok) {
         const int64_t nvec = n / E;
-        const int64_t per_block = 256 * kGeluUnroll;
-        const int64_t grid = (nvec + per_block - 1) / per_block;
-        if (grid > 0x7FFFFFFFLL) return fail(MHIP_ERR_UNSUPPORTED, "bias_gelu: tensor too large");
-        hipLaunchKernelGGL((bias_gelu_vec_kernel<T>), dim3((unsigned)grid), dim3(256), 0, s,
-                           static_cast<const T*>(x), static_cast<const T*>(bias),
-                           static_cast<T*>(y), nvec, (int)cols);
+        const int64_t want = (nvec + 511) / 512;
+        const int64_t cap = (int64_t)compute_units() * tune_int("MHIP_GELU_BLOCKS_PER_CU", 64);
+        const unsigned grid = (unsigned)(want < cap ? want : cap);
+        const bool in_lds = bias && cols * sizeof(float) <= 48 * 1024;
+        hipLaunchKernelGGL((bias_gelu_vec_kernel<T>), dim3(grid), dim3(256),
+                           in_lds ? (size_t)cols * sizeof(float) : 0, s, static_cast<const T*>(x),
+                           static_cast<const T*>(bias), static_cast<T*>(y), nvec, (int)(cols / E),
+                           in_lds ? 1 : 0);
     } else {
         const int64_t grid = (n + 255) / 256;
         if (grid > 0x7FFFFFFFLL) return fail(MHIP_ERR_UNSUPPORTED, "bias_gelu: tensor too large");

@@ -1,6 +1,7 @@
 // Library-level services of the C-ABI: version, thread-local error slot, device facts.
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include "common.h"
@@ -21,6 +22,27 @@ int check_launch(const char* what) {
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(MHIP_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
     return MHIP_OK;
+}
+
+int tune_int(const char* name, int fallback) {
+    const char* v = getenv(name);
+    if (!v || !*v) return fallback;
+    char* end = nullptr;
+    const long r = strtol(v, &end, 10);
+    return (end && *end == 0 && r > 0 && r < (1 << 20)) ? (int)r : fallback;
+}
+
+int compute_units() {
+    static int cached[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+            n = 256;
+        cached[dev] = n;
+    }
+    return cached[dev];
 }
 
 }  // namespace mhip
