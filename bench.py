@@ -32,6 +32,19 @@ sys.path.insert(0, ROOT)
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
+# HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by what the same
+# counter reads for the 'copy' workload (256 MiB in, 256 MiB out); see profiles/<workload>.txt.
+MEASURED_TRAFFIC = {
+    "gemm": 236982956,
+    "attention": 536931388,
+    "attention_full": 268556237,
+    "softmax": 536717179,
+    "layer_norm": 536879830,
+    "rms_norm": 536782397,
+    "bias_gelu": 536773400,
+    "copy": 536870912,
+}
+
 
 def _time_launches(fn, steps, warmup, torch):
     """Mean seconds per launch of fn(i) over `steps` launches (HIP events on the
@@ -110,17 +123,28 @@ def wl_rows(torch, kernels, op, rows=32768, cols=4096):
                 kernel=kern)
 
 
-def measure(wl, steps, warmup, torch):
+def wl_copy(torch, kernels, nbytes=256 << 20):
+    from metalhlo_amd import _lib
+    lib = _lib.load()
+    srcs = [torch.randint(0, 255, (nbytes,), dtype=torch.uint8, device="cuda") for _ in range(3)]
+    dsts = [torch.empty_like(x) for x in srcs]
+    st = lambda: torch.cuda.current_stream().cuda_stream
+    return dict(name=f"device copy of {nbytes} bytes (calibration)",
+                fn=lambda i: lib.mhip_copy(st(), srcs[i % 3].data_ptr(), dsts[i % 3].data_ptr(), nbytes),
+                flops=0.0, bytes=2.0 * nbytes, bound="hbm", kernel="copy_kernel")
+
+
+def measure(wl, steps, warmup, torch, key=None):
     sec, wall = _time_launches(wl["fn"], steps, warmup, torch)
     if wl["bound"] == "mfma":
         ach = wl["flops"] / sec / 1e12
         roof = dict(bound="mfma", achieved=round(ach, 2), peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
-                    frac=round(ach / PEAK_BF16_TFLOPS, 4), traffic=None)
+                    frac=round(ach / PEAK_BF16_TFLOPS, 4), traffic=MEASURED_TRAFFIC.get(key))
         value, unit = ach, "TFLOP/s"
     else:
         ach = wl["bytes"] / sec / 1e9
         roof = dict(bound="hbm", achieved=round(ach, 1), peak=PEAK_HBM_GBS, unit="GB/s",
-                    frac=round(ach / PEAK_HBM_GBS, 4), traffic=None)
+                    frac=round(ach / PEAK_HBM_GBS, 4), traffic=MEASURED_TRAFFIC.get(key))
         value, unit = ach, "GB/s"
     return dict(workload=wl["name"], kernel=wl["kernel"], value=round(value, 2), unit=unit,
                 us_per_launch=round(sec * 1e6, 2), wall_us_per_launch=round(wall * 1e6, 2), roofline=roof)
@@ -156,7 +180,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="gemm",
-                    choices=["gemm", "attention", "attention_full", "softmax", "layer_norm", "rms_norm", "bias_gelu"])
+                    choices=["gemm", "attention", "attention_full", "softmax", "layer_norm", "rms_norm", "bias_gelu", "copy"])
     ap.add_argument("--only", action="store_true", help="time only --workload (for profiling runs)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
@@ -178,16 +202,18 @@ def main():
             return wl_attention(torch, kernels, causal=True)
         if name == "attention_full":
             return wl_attention(torch, kernels, S=2048, causal=False)
+        if name == "copy":
+            return wl_copy(torch, kernels)
         return wl_rows(torch, kernels, name)
 
-    head = measure(build(args.workload), args.steps, args.warmup, torch)
+    head = measure(build(args.workload), args.steps, args.warmup, torch, args.workload)
     others = {}
     if not args.only:
         for name in ["gemm", "attention", "attention_full", "softmax", "layer_norm", "rms_norm", "bias_gelu"]:
             if name == args.workload:
                 continue
             torch.cuda.empty_cache()
-            others[name] = measure(build(name), args.steps, args.warmup, torch)
+            others[name] = measure(build(name), args.steps, args.warmup, torch, name)
             print(f"[bench] {name}: {others[name]['value']} {others[name]['unit']} "
                   f"({others[name]['roofline']['frac'] * 100:.1f}% of peak)", file=sys.stderr, flush=True)
     cpu = None

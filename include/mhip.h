@@ -150,6 +150,11 @@ int mhip_gather_rows(void* stream, const void* table, const void* indices, void*
                      int64_t n_idx, int64_t n_rows, int64_t row_elems, int table_dtype,
                      int idx_dtype);
 
+/* dst = src, `bytes` bytes, device to device, as one streaming kernel (reshape /
+ * copy; also the calibration kernel for the HBM traffic counters).
+ * Replaces the copy kernels of Compiler/CodeGenerator.swift:851-921. */
+int mhip_copy(void* stream, const void* src, void* dst, int64_t bytes);
+
 /* out[b, s, :] = convert(wte[ids[b, s], :] + wpe[s, :]) — token + position
  * embedding in one pass (gather :1133-1397, add :921, convert :1012-1078 of
  * Compiler/CodeGenerator.swift).  ids are I32 [B,S]; params F32 or the output

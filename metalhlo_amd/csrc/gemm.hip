@@ -10,57 +10,11 @@
 // way in (16-byte global loads either way).
 // Everything else (fp32, shapes that are not 16-byte friendly) goes through a
 // plain LDS-tiled kernel.
-#include <math.h>
-
 #include <mutex>
 
-#include "common.h"
+#include "gemm_common.h"
 
 namespace mhip {
-
-constexpr int kBK = 64;              // k extent of one LDS stage
-constexpr int kRowBytes = kBK * 2;   // bytes per LDS tile row (16-bit elements)
-constexpr uint32_t kOob = 0x80000000u;  // byte offset beyond any buffer: load returns 0
-
-struct GemmArgs {
-    const void* a;
-    const void* b;
-    const void* bias;
-    void* c;
-    int M, N, K;
-    int lda, ldb;           // leading dimensions in elements of the stored matrices
-    int64_t sa, sb, sc;     // batch strides in elements
-    int act;
-    int tiles_m, tiles_n;
-};
-
-template <typename T> struct Mfma32;
-template <> struct Mfma32<bf16_t> {
-    __device__ static f32x16 run(u32x4 a, u32x4 b, f32x16 c) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
-                                                       __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
-    }
-};
-template <> struct Mfma32<f16_t> {
-    __device__ static f32x16 run(u32x4 a, u32x4 b, f32x16 c) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
-                                                      __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
-    }
-};
-
-__device__ inline float apply_act(float v, int act) {
-    switch (act) {
-        case MHIP_ACT_RELU: return fmaxf(v, 0.f);
-        case MHIP_ACT_GELU: {
-            const float inner = 0.7978845608028654f * (v + 0.044715f * v * v * v);
-            return 0.5f * v * (1.f + tanhf(inner));
-        }
-        case MHIP_ACT_SILU: return v / (1.f + expf(-v));
-        case MHIP_ACT_TANH: return tanhf(v);
-        case MHIP_ACT_SIGMOID: return 1.f / (1.f + expf(-v));
-        default: return v;
-    }
-}
 
 // Swizzle of the 16-byte chunk index inside a 128-byte LDS row.  Rows r..r+15
 // (r % 16 == 0) map one chunk column onto 16 distinct bank groups.
@@ -102,75 +56,72 @@ struct KMajorLoader {
 };
 
 // ---- operand with k as the slow axis in memory: [K][ld] -------------------
-// A thread fetches a 4(k) x 8(mn) block with four 16-byte loads, transposes it
-// in registers and writes eight 8-byte k-runs into the k-major LDS tile.
+// The tile keeps the memory orientation in LDS, [64 k][ROWS mn] (16-byte global
+// loads, 16-byte LDS stores), and the MFMA operand is formed on the way OUT of
+// LDS with ds_read_b64_tr_b16, which transposes a 4(k) x 16(mn) block across
+// 16 lanes: lane i of a 16-lane group supplies the address of k-row i/4,
+// mn-columns 4*(i%4)..+3 and receives column i for the four k-rows.
+// Chunk swizzle: chunk' = chunk ^ (4 * (k % 4)) puts the four k-rows that one
+// transposing read touches on disjoint banks.
+template <int ROWS>
+__device__ inline uint32_t mn_off(int k, int chunk) {
+    return (uint32_t)(k * (ROWS * 2) + ((chunk ^ ((k & 3) << 2)) << 4));
+}
+
 template <int ROWS, int NT>
 struct MnMajorLoader {
-    static constexpr int kBlocks = 16 * (ROWS / 8);
-    static constexpr int kIters = kBlocks / NT;
-    static_assert(kBlocks % NT == 0, "tile does not split evenly over the workgroup");
-    u32x4 regs[kIters][4];
+    static constexpr int kCpr = ROWS / 8;               // 16-byte chunks per k-row
+    static constexpr int kIters = kBK * kCpr / NT;
+    static_assert((kBK * kCpr) % NT == 0, "tile does not split evenly over the workgroup");
+    u32x4 regs[kIters];
     __device__ void load(__amdgpu_buffer_rsrc_t rsrc, int col0, int k0, int cols_total, int K,
                          int ld) {
+        const int c = threadIdx.x % kCpr;
 #pragma unroll
         for (int i = 0; i < kIters; i++) {
-            const int blk = threadIdx.x + i * NT;
-            const int ng = blk % (ROWS / 8), kg = blk / (ROWS / 8);
-            const int gcol = col0 + ng * 8;
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const int gk = k0 + kg * 4 + j;
-                const uint32_t off = (gk < K && gcol < cols_total)
-                                         ? (uint32_t)(((int64_t)gk * ld + gcol) * 2)
-                                         : kOob;
-                regs[i][j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, 0);
-            }
+            const int k = threadIdx.x / kCpr + i * (NT / kCpr);
+            const int gk = k0 + k, gcol = col0 + c * 8;
+            const uint32_t off = (gk < K && gcol < cols_total)
+                                     ? (uint32_t)(((int64_t)gk * ld + gcol) * 2)
+                                     : kOob;
+            regs[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, 0);
         }
     }
     __device__ void store(char* tile) const {
+        const int c = threadIdx.x % kCpr;
 #pragma unroll
         for (int i = 0; i < kIters; i++) {
-            const int blk = threadIdx.x + i * NT;
-            const int ng = blk % (ROWS / 8), kg = blk / (ROWS / 8);
-#pragma unroll
-            for (int q = 0; q < 4; q++) {  // dword q of each row holds columns 2q, 2q+1
-                const uint32_t r0 = regs[i][0][q], r1 = regs[i][1][q];
-                const uint32_t r2 = regs[i][2][q], r3 = regs[i][3][q];
-                u32x2 even, odd;
-                even.x = __builtin_amdgcn_perm(r1, r0, 0x05040100);
-                even.y = __builtin_amdgcn_perm(r3, r2, 0x05040100);
-                odd.x = __builtin_amdgcn_perm(r1, r0, 0x07060302);
-                odd.y = __builtin_amdgcn_perm(r3, r2, 0x07060302);
-                const int row = ng * 8 + q * 2;
-                *reinterpret_cast<u32x2*>(tile + lds_off(row, kg >> 1) + (kg & 1) * 8) = even;
-                *reinterpret_cast<u32x2*>(tile + lds_off(row + 1, kg >> 1) + (kg & 1) * 8) = odd;
-            }
+            const int k = threadIdx.x / kCpr + i * (NT / kCpr);
+            *reinterpret_cast<u32x4*>(tile + mn_off<ROWS>(k, c)) = regs[i];
         }
     }
 };
 
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+
+// MFMA operand (32 mn x 16 k) for k-step `s` out of a k-major tile.
+__device__ inline u32x4 frag_kmajor(const char* tile, int row0, int s, int lane) {
+    return *reinterpret_cast<const u32x4*>(tile + lds_off(row0 + (lane & 31), 2 * s + (lane >> 5)));
+}
+// Same operand out of an mn-major tile via two transposing reads.
+template <int ROWS>
+__device__ inline u32x4 frag_mnmajor(const char* tile, int mn0, int s, int lane) {
+    const int i = lane & 15, g = lane >> 4;
+    const int mn = mn0 + 16 * (g & 1) + 4 * (i & 3);
+    const int k = 16 * s + 8 * (g >> 1) + (i >> 2);
+    const char* p0 = tile + mn_off<ROWS>(k, mn >> 3) + (mn & 7) * 2;
+    const char* p1 = tile + mn_off<ROWS>(k + 4, mn >> 3) + (mn & 7) * 2;
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)p0);
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)p1);
+    u32x4 r;
+    const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+    r.x = l2.x; r.y = l2.y; r.z = h2.x; r.w = h2.y;
+    return r;
+}
+
 template <int ROWS, int NT, bool KMAJOR> struct LoaderSel { using type = KMajorLoader<ROWS, NT>; };
 template <int ROWS, int NT> struct LoaderSel<ROWS, NT, false> { using type = MnMajorLoader<ROWS, NT>; };
-
-// Maps the linear workgroup id to a C tile.  Consecutive ids go to different
-// XCDs (round-robin dispatch), so ids are first regrouped so that each XCD's
-// share is a contiguous range, then walked in bands of kGroupM tile rows:
-// the workgroups resident on one XCD then share A row panels and B column
-// panels through that XCD's L2.
-constexpr int kXcds = 8;
-constexpr int kGroupM = 4;
-__device__ inline void tile_of(int pid, int grid, int tiles_m, int tiles_n, int& tm, int& tn) {
-    const int per = (grid + kXcds - 1) / kXcds;
-    const int tall = (grid % kXcds == 0) ? kXcds : grid % kXcds;
-    const int xcd = pid % kXcds, local = pid / kXcds;
-    const int lpid = (xcd < tall) ? xcd * per + local
-                                  : tall * per + (xcd - tall) * (per - 1) + local;
-    const int band = kGroupM * tiles_n;
-    const int g = lpid / band, first = g * kGroupM;
-    const int gsz = min(tiles_m - first, kGroupM);
-    tm = first + (lpid % band) % gsz;
-    tn = (lpid % band) / gsz;
-}
 
 template <typename T, int BM, int BN, int WGM, int WGN, bool TA, bool TB>
 __global__ __launch_bounds__(WGM* WGN * 64) void gemm_mfma_kernel(GemmArgs g) {
@@ -211,6 +162,17 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_mfma_kernel(GemmArgs g) {
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
+    auto read_frags = [&](int buf, int s, u32x4(&af)[TM], u32x4(&bf)[TN]) {
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+            af[i] = TA ? frag_mnmajor<BM>(a_tile(buf), wm * WTM + i * 32, s, lane)
+                       : frag_kmajor(a_tile(buf), wm * WTM + i * 32, s, lane);
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+            bf[j] = TB ? frag_kmajor(b_tile(buf), wn * WTN + j * 32, s, lane)
+                       : frag_mnmajor<BN>(b_tile(buf), wn * WTN + j * 32, s, lane);
+    };
+
     const int KT = (g.K + kBK - 1) / kBK;
     la.load(ra, m0, 0, g.M, g.K, g.lda);
     lb.load(rb, n0, 0, g.N, g.K, g.ldb);
@@ -224,21 +186,18 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_mfma_kernel(GemmArgs g) {
             la.load(ra, m0, (kt + 1) * kBK, g.M, g.K, g.lda);
             lb.load(rb, n0, (kt + 1) * kBK, g.N, g.K, g.ldb);
         }
+        // Fragments for k-step s+1 are fetched from LDS while the MFMAs of step
+        // s run (register double buffer).
+        u32x4 af[2][TM], bf[2][TN];
+        read_frags(cur, 0, af[0], bf[0]);
 #pragma unroll
         for (int s = 0; s < kBK / 16; s++) {
-            u32x4 af[TM], bf[TN];
-#pragma unroll
-            for (int i = 0; i < TM; i++)
-                af[i] = *reinterpret_cast<const u32x4*>(
-                    a_tile(cur) + lds_off(wm * WTM + i * 32 + lrow, 2 * s + lhalf));
-#pragma unroll
-            for (int j = 0; j < TN; j++)
-                bf[j] = *reinterpret_cast<const u32x4*>(
-                    b_tile(cur) + lds_off(wn * WTN + j * 32 + lrow, 2 * s + lhalf));
+            if (s + 1 < kBK / 16) read_frags(cur, s + 1, af[(s + 1) & 1], bf[(s + 1) & 1]);
 #pragma unroll
             for (int i = 0; i < TM; i++)
 #pragma unroll
-                for (int j = 0; j < TN; j++) acc[i][j] = Mfma32<T>::run(af[i], bf[j], acc[i][j]);
+                for (int j = 0; j < TN; j++)
+                    acc[i][j] = Mfma32<T>::run(bf[s & 1][j], af[s & 1][i], acc[i][j]);
         }
         if (kt + 1 < KT) {
             la.store(a_tile(cur ^ 1));
@@ -247,22 +206,74 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_mfma_kernel(GemmArgs g) {
         __syncthreads();
     }
 
-    // Epilogue: lane holds column n = lrow and rows 8*(r/4) + 4*lhalf + r%4 of
-    // every 32x32 accumulator tile.
+    // Epilogue.  The MFMAs were issued as (B-fragment, A-fragment), so each
+    // 32x32 accumulator tile is held transposed: a lane owns row m = lrow and,
+    // in register group q = r/4, the four consecutive columns 8q + 4*lhalf + r%4.
     const T* bias = static_cast<const T*>(g.bias);
+    const bool vec_store = (g.N % 8 == 0) && ((reinterpret_cast<uintptr_t>(c) & 15) == 0);
+    if (vec_store) {
+        // Stage the wave's sub-tile in LDS as rounded 16-bit rows (padded to 144
+        // bytes against bank conflicts), then write whole 128-byte row segments.
+        constexpr int kRowPad = WTN * 2 + 16;
+        char* stage = smem + wave * (WTM * kRowPad);
 #pragma unroll
-    for (int j = 0; j < TN; j++) {
-        const int n = n0 + wn * WTN + j * 32 + lrow;
-        if (n >= g.N) continue;
-        const float bv = bias ? Elem<T>::to_f32(bias[n]) : 0.f;
+        for (int j = 0; j < TN; j++) {
 #pragma unroll
-        for (int i = 0; i < TM; i++) {
-            const int mb = m0 + wm * WTM + i * 32 + 4 * lhalf;
+            for (int q = 0; q < 4; q++) {
+                const int nl = j * 32 + 8 * q + 4 * lhalf;          // column inside the wave tile
+                const int n = n0 + wn * WTN + nl;
+                float bv[4] = {0.f, 0.f, 0.f, 0.f};
+                if (bias && n < g.N) {
+                    const Pack4<T> t = __builtin_bit_cast(Pack4<T>, *reinterpret_cast<const u32x2*>(bias + n));
+#pragma unroll
+                    for (int e = 0; e < 4; e++) bv[e] = Elem<T>::to_f32(t.v[e]);
+                }
+#pragma unroll
+                for (int i = 0; i < TM; i++) {
+                    float v[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        v[e] = acc[i][j][4 * q + e] + bv[e];
+                        if (g.act != MHIP_ACT_NONE) v[e] = apply_act(v[e], g.act);
+                    }
+                    Pack4<T> o;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) o.v[e] = Elem<T>::from_f32(v[e]);
+                    *reinterpret_cast<u32x2*>(stage + (i * 32 + lrow) * kRowPad + nl * 2) =
+                        __builtin_bit_cast(u32x2, o);
+                }
+            }
+        }
+        // each wave only re-reads what it wrote itself
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        constexpr int kCpr = WTN / 8;                // 16-byte chunks per row
+        constexpr int kRowsPerPass = 64 / kCpr;
+        const int cc = lane % kCpr, rr = lane / kCpr;
+#pragma unroll
+        for (int p = 0; p < WTM / kRowsPerPass; p++) {
+            const int ml = p * kRowsPerPass + rr;
+            const int m = m0 + wm * WTM + ml;
+            const int n = n0 + wn * WTN + cc * 8;
+            if (m < g.M && n < g.N) {
+                const u32x4 w = *reinterpret_cast<const u32x4*>(stage + ml * kRowPad + cc * 16);
+                *reinterpret_cast<u32x4*>(c + (int64_t)m * g.N + n) = w;
+            }
+        }
+        return;
+    }
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+        const int m = m0 + wm * WTM + i * 32 + lrow;
+        if (m >= g.M) continue;
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                const int m = mb + 8 * (r >> 2) + (r & 3);
-                if (m < g.M) {
-                    float v = acc[i][j][r] + bv;
+                const int n = n0 + wn * WTN + j * 32 + 8 * (r >> 2) + 4 * lhalf + (r & 3);
+                if (n < g.N) {
+                    float v = acc[i][j][r] + (bias ? Elem<T>::to_f32(bias[n]) : 0.f);
                     if (g.act != MHIP_ACT_NONE) v = apply_act(v, g.act);
                     c[(int64_t)m * g.N + n] = Elem<T>::from_f32(v);
                 }
@@ -312,7 +323,10 @@ __global__ __launch_bounds__(256) void gemm_simple_kernel(GemmArgs g, int trans_
 template <typename T, int BM, int BN, int WGM, int WGN, bool TA, bool TB>
 static int launch_mfma(hipStream_t s, GemmArgs g, int64_t batch) {
     constexpr int NT = WGM * WGN * 64;
-    constexpr int kSmem = 2 * (BM + BN) * kRowBytes;
+    constexpr int kWaves = WGM * WGN;
+    constexpr int kStage = kWaves * (BM / WGM) * ((BN / WGN) * 2 + 16);   // epilogue staging
+    constexpr int kLoop = 2 * (BM + BN) * kRowBytes;
+    constexpr int kSmem = kLoop > kStage ? kLoop : kStage;
     auto kern = gemm_mfma_kernel<T, BM, BN, WGM, WGN, TA, TB>;
     static std::once_flag once;
     static hipError_t attr_err = hipSuccess;

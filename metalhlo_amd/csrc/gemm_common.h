@@ -1,0 +1,75 @@
+// Definitions shared by the GEMM kernels.
+#pragma once
+#include <math.h>
+
+#include "common.h"
+
+namespace mhip {
+
+constexpr int kBK = 64;              // k extent of one LDS stage
+constexpr int kRowBytes = kBK * 2;   // bytes per LDS tile row (16-bit elements)
+constexpr uint32_t kOob = 0x80000000u;  // byte offset beyond any buffer: load returns 0
+
+struct GemmArgs {
+    const void* a;
+    const void* b;
+    const void* bias;
+    void* c;
+    int M, N, K;
+    int lda, ldb;           // leading dimensions in elements of the stored matrices
+    int64_t sa, sb, sc;     // batch strides in elements
+    int act;
+    int tiles_m, tiles_n;
+};
+
+template <typename T> struct Mfma32;
+template <> struct Mfma32<bf16_t> {
+    __device__ static f32x16 run(u32x4 a, u32x4 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                       __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+};
+template <> struct Mfma32<f16_t> {
+    __device__ static f32x16 run(u32x4 a, u32x4 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
+                                                      __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+};
+
+template <typename T> struct alignas(8) Pack4 { T v[4]; };
+
+__device__ inline float apply_act(float v, int act) {
+    switch (act) {
+        case MHIP_ACT_RELU: return fmaxf(v, 0.f);
+        case MHIP_ACT_GELU: {
+            const float inner = 0.7978845608028654f * (v + 0.044715f * v * v * v);
+            return 0.5f * v * (1.f + tanhf(inner));
+        }
+        case MHIP_ACT_SILU: return v / (1.f + expf(-v));
+        case MHIP_ACT_TANH: return tanhf(v);
+        case MHIP_ACT_SIGMOID: return 1.f / (1.f + expf(-v));
+        default: return v;
+    }
+}
+
+// Maps the linear workgroup id to a C tile.  Consecutive ids go to different
+// XCDs (round-robin dispatch), so ids are first regrouped so that each XCD's
+// share is a contiguous range, then walked in bands of kGroupM tile rows:
+// the workgroups resident on one XCD then share A row panels and B column
+// panels through that XCD's L2.
+constexpr int kXcds = 8;
+constexpr int kGroupM = 4;
+__device__ inline void tile_of(int pid, int grid, int tiles_m, int tiles_n, int& tm, int& tn) {
+    const int per = (grid + kXcds - 1) / kXcds;
+    const int tall = (grid % kXcds == 0) ? kXcds : grid % kXcds;
+    const int xcd = pid % kXcds, local = pid / kXcds;
+    const int lpid = (xcd < tall) ? xcd * per + local
+                                  : tall * per + (xcd - tall) * (per - 1) + local;
+    const int band = kGroupM * tiles_n;
+    const int g = lpid / band, first = g * kGroupM;
+    const int gsz = min(tiles_m - first, kGroupM);
+    tm = first + (lpid % band) % gsz;
+    tn = (lpid % band) / gsz;
+}
+
+}  // namespace mhip

@@ -47,6 +47,19 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const char* __restrict
     }
 }
 
+// ---- plain device copy (16 bytes per lane, streaming) --------------------------
+__global__ __launch_bounds__(256) void copy_kernel(const u32x4* __restrict__ src,
+                                                   u32x4* __restrict__ dst, int64_t nvec) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < nvec) __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
+}
+__global__ __launch_bounds__(256) void copy_bytes_kernel(const char* __restrict__ src,
+                                                         char* __restrict__ dst, int64_t start,
+                                                         int64_t n) {
+    const int64_t i = start + (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) dst[i] = src[i];
+}
+
 // ---- token + position embedding --------------------------------------------
 template <typename P, typename O>
 __global__ __launch_bounds__(256) void embed_kernel(const int32_t* __restrict__ ids,
@@ -232,6 +245,26 @@ extern "C" int mhip_gather_rows(void* stream, const void* table, const void* ind
     else
         return fail(MHIP_ERR_UNSUPPORTED, "mhip_gather_rows: index dtype %d (need i32 or i64)", idx_dtype);
     return check_launch("gather_rows");
+}
+
+extern "C" int mhip_copy(void* stream, const void* src, void* dst, int64_t bytes) {
+    if (bytes < 0) return fail(MHIP_ERR_INVALID_ARGUMENT, "mhip_copy: negative size");
+    if (bytes == 0) return MHIP_OK;
+    if (!src || !dst) return fail(MHIP_ERR_INVALID_ARGUMENT, "mhip_copy: NULL pointer");
+    hipStream_t s = as_stream(stream);
+    const bool al = ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15) == 0;
+    const int64_t nvec = al ? bytes / 16 : 0;
+    unsigned grid;
+    if (nvec) {
+        if (grid_for(nvec, 256, &grid)) return MHIP_ERR_UNSUPPORTED;
+        hipLaunchKernelGGL(copy_kernel, dim3(grid), dim3(256), 0, s, (const u32x4*)src, (u32x4*)dst, nvec);
+    }
+    if (bytes - nvec * 16) {
+        if (grid_for(bytes - nvec * 16, 256, &grid)) return MHIP_ERR_UNSUPPORTED;
+        hipLaunchKernelGGL(copy_bytes_kernel, dim3(grid), dim3(256), 0, s, (const char*)src, (char*)dst,
+                           nvec * 16, bytes);
+    }
+    return check_launch("copy");
 }
 
 extern "C" int mhip_embed_tokens(void* stream, const void* ids, const void* wte, const void* wpe,
