@@ -68,29 +68,37 @@ __device__ inline __amdgpu_buffer_rsrc_t fa_rsrc(const void* p, uint32_t bytes) 
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
 }
 
-// K tile [64 keys][D] : 16-byte chunks XOR-swizzled inside each row.
+// K and V tiles sit in LDS as they lie in memory, [64 keys][D], 16-byte chunks
+// XOR-swizzled inside each row.  K is read as the A operand of S^T = K.Q^T with
+// ds_read_b128 (lane = key row, eight consecutive d); V is read as the A operand
+// of O^T += V^T.P^T with ds_read_b64_tr_b16, which hands lane i of a 16-lane
+// group column d = i of four consecutive key rows.
+template <int D>
+__device__ inline int k_swz(int row) { return (D == 128) ? (row & 15) : ((row >> 1) & 7); }
 template <int D>
 __device__ inline uint32_t k_off(int row, int chunk) {
-    const int s = (D == 128) ? (row & 15) : (((row >> 1) ^ (row >> 4)) & 7);
-    return (uint32_t)(row * (D * 2) + ((chunk ^ s) << 4));
+    return (uint32_t)(row * (D * 2) + ((chunk ^ k_swz<D>(row)) << 4));
 }
-// V^T tile [D][64 keys] : 128-byte rows.
-__device__ inline uint32_t vt_off(int row, int chunk) {
-    const int s = ((row >> 1) ^ (row >> 4)) & 7;
-    return (uint32_t)(row * 128 + ((chunk ^ s) << 4));
+// the four key rows that one transposing read touches must fall on disjoint banks
+template <int D>
+__device__ inline int v_swz(int row) { return (D == 128) ? ((row & 3) << 2) : (((row >> 1) & 1) << 2); }
+template <int D>
+__device__ inline uint32_t v_off(int row, int chunk) {
+    return (uint32_t)(row * (D * 2) + ((chunk ^ v_swz<D>(row)) << 4));
 }
 
+typedef short fa_s16x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) fa_s16x4 fa_lds_s16x4;
+typedef __attribute__((address_space(3))) void fa_lds_void;
+
 template <typename T, int D, bool CAUSAL, bool HAS_MASK>
-__global__ __launch_bounds__(256) void fa_fwd_kernel(FaArgs a) {
-    constexpr int CPR = D / 8;                  // 16-byte chunks per K row
-    constexpr int kKTile = kBKV * D * 2;        // bytes
-    constexpr int kVTile = D * 128;             // bytes
-    constexpr int kKIters = kBKV * CPR / 128;   // K chunks per loading thread
-    constexpr int kVBlocks = 8 * (D / 8);       // 8x8 blocks of the V tile
+__global__ __launch_bounds__(256, 2) void fa_fwd_kernel(FaArgs a) {
+    constexpr int CPR = D / 8;                  // 16-byte chunks per row
+    constexpr int kTile = kBKV * D * 2;         // bytes of one K (or V) tile
+    constexpr int kRowsPerInst = 64 / CPR;      // tile rows one wave-wide LDS-DMA load fills
+    constexpr int kInst = kBKV / kRowsPerInst / 4;   // such loads per wave per tile
     constexpr int ND = D / 32, NS = D / 16;
-    __shared__ __attribute__((aligned(16))) char smem[2 * (kKTile + kVTile)];
-    auto k_tile = [&](int buf) { return smem + buf * kKTile; };
-    auto v_tile = [&](int buf) { return smem + 2 * kKTile + buf * kVTile; };
+    __shared__ __attribute__((aligned(1024))) char smem[4 * kTile];   // K0 K1 V0 V1
 
     // ---- which (batch*head, query block) -----------------------------------
     int bh, qb;
@@ -126,8 +134,8 @@ __global__ __launch_bounds__(256) void fa_fwd_kernel(FaArgs a) {
         const uint32_t off = qpos < a.Sq ? (uint32_t)((qpos * D + 16 * s + 8 * lhalf) * 2) : kOobA;
         qf[s] = __builtin_amdgcn_raw_buffer_load_b128(rq, off, 0, 0);
         if (a.negate_q) {
-            const uint32_t flip = sizeof(T) == 2 ? 0x80008000u : 0u;
-            qf[s].x ^= flip; qf[s].y ^= flip; qf[s].z ^= flip; qf[s].w ^= flip;
+            qf[s].x ^= 0x80008000u; qf[s].y ^= 0x80008000u;
+            qf[s].z ^= 0x80008000u; qf[s].w ^= 0x80008000u;
         }
     }
 
@@ -137,80 +145,51 @@ __global__ __launch_bounds__(256) void fa_fwd_kernel(FaArgs a) {
         nkv = min(nkv, last_q / kBKV + 1);
     }
 
-    // ---- staging registers: waves 0,1 fetch K, waves 2,3 fetch + transpose V
-    u32x4 stage[8];
-    auto load_tile = [&](int kv0) {
-        if (wave < 2) {
+    // ---- global -> LDS without a register stop: every wave-wide load fills 1 KB
+    // of a tile (lane l lands at byte 16*l of that KB); the swizzle is applied by
+    // choosing which global chunk each lane fetches.  Keys past the end read 0.
+    const int ld_row = lane / CPR, ld_pos = lane % CPR;
+    auto load_tile = [&](int kv0, int buf) {
 #pragma unroll
-            for (int i = 0; i < kKIters; i++) {
-                const int idx = tid + i * 128;
-                const int row = idx / CPR, c = idx % CPR;
-                const int key = kv0 + row;
-                const uint32_t off = key < a.Skv ? (uint32_t)((key * D + c * 8) * 2) : kOobA;
-                stage[i] = __builtin_amdgcn_raw_buffer_load_b128(rk, off, 0, 0);
-            }
-        } else {
-            const int blk = tid - 128;
-            if (blk < kVBlocks) {
-                const int dg = blk % (D / 8), ch = blk / (D / 8);
-                const int u = ch >> 1, h = ch & 1;
-#pragma unroll
-                for (int j = 0; j < 8; j++) {
-                    const int key = kv0 + 16 * u + 8 * (j >> 2) + 4 * h + (j & 3);
-                    const uint32_t off = key < a.Skv ? (uint32_t)((key * D + dg * 8) * 2) : kOobA;
-                    stage[j] = __builtin_amdgcn_raw_buffer_load_b128(rv, off, 0, 0);
-                }
-            }
+        for (int i = 0; i < kInst; i++) {
+            const int blk = i * 4 + wave;                 // which KB of the tile
+            const int row = blk * kRowsPerInst + ld_row;
+            const int key = kv0 + row;
+            const uint32_t koff = key < a.Skv ? (uint32_t)((key * D + ((ld_pos ^ k_swz<D>(row)) << 3)) * 2) : kOobA;
+            const uint32_t voff = key < a.Skv ? (uint32_t)((key * D + ((ld_pos ^ v_swz<D>(row)) << 3)) * 2) : kOobA;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, (fa_lds_void*)(smem + buf * kTile + blk * 1024), 16, koff, 0, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, (fa_lds_void*)(smem + (2 + buf) * kTile + blk * 1024), 16, voff, 0, 0, 0);
         }
     };
-    auto store_tile = [&](int buf) {
-        if (wave < 2) {
-#pragma unroll
-            for (int i = 0; i < kKIters; i++) {
-                const int idx = tid + i * 128;
-                const int row = idx / CPR, c = idx % CPR;
-                *reinterpret_cast<u32x4*>(k_tile(buf) + k_off<D>(row, c)) = stage[i];
-            }
-        } else {
-            const int blk = tid - 128;
-            if (blk < kVBlocks) {
-                const int dg = blk % (D / 8), ch = blk / (D / 8);
-#pragma unroll
-                for (int q = 0; q < 4; q++) {   // dword q of a key row holds d = 2q, 2q+1
-                    u32x4 even, odd;
-                    even.x = __builtin_amdgcn_perm(stage[1][q], stage[0][q], 0x05040100);
-                    even.y = __builtin_amdgcn_perm(stage[3][q], stage[2][q], 0x05040100);
-                    even.z = __builtin_amdgcn_perm(stage[5][q], stage[4][q], 0x05040100);
-                    even.w = __builtin_amdgcn_perm(stage[7][q], stage[6][q], 0x05040100);
-                    odd.x = __builtin_amdgcn_perm(stage[1][q], stage[0][q], 0x07060302);
-                    odd.y = __builtin_amdgcn_perm(stage[3][q], stage[2][q], 0x07060302);
-                    odd.z = __builtin_amdgcn_perm(stage[5][q], stage[4][q], 0x07060302);
-                    odd.w = __builtin_amdgcn_perm(stage[7][q], stage[6][q], 0x07060302);
-                    const int d = dg * 8 + 2 * q;
-                    *reinterpret_cast<u32x4*>(v_tile(buf) + vt_off(d, ch)) = even;
-                    *reinterpret_cast<u32x4*>(v_tile(buf) + vt_off(d + 1, ch)) = odd;
-                }
-            }
-        }
+    auto tiles_ready = [&]() {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
     };
+
+    // V^T fragment addresses: lane i of a 16-lane group supplies key row i/4 and
+    // d columns 4*(i%4)..+3 of its group's 16-column block.
+    const int ti = lane & 15, tg = lane >> 4;
+    const int v_row0 = 4 * (tg >> 1) + (ti >> 2);                   // + 16u (+ 8)
+    const int v_d0 = 16 * (tg & 1) + 4 * (ti & 3);                  // + 32 dt
 
     f32x16 oacc[ND];
 #pragma unroll
     for (int i = 0; i < ND; i++)
 #pragma unroll
         for (int r = 0; r < 16; r++) oacc[i][r] = 0.f;
-    float m_run = -INFINITY, l_run = 0.f;
+    float m_run = -INFINITY, l_run = 0.f;   // running max in the log2 domain, running sum
 
-    load_tile(0);
-    store_tile(0);
-    __syncthreads();
+    load_tile(0, 0);
+    tiles_ready();
 
     for (int it = 0; it < nkv; it++) {
         const int cur = it & 1, kv0 = it * kBKV;
-        if (it + 1 < nkv) load_tile(kv0 + kBKV);
+        if (it + 1 < nkv) load_tile(kv0 + kBKV, cur ^ 1);
 
         const bool wave_active = !CAUSAL || kv0 <= qw + 31;
         if (wave_active) {
+            const char* kt = smem + cur * kTile;
+            const char* vt = smem + (2 + cur) * kTile;
             // ---- S^T = K . Q^T ---------------------------------------------
             f32x16 sacc[2];
 #pragma unroll
@@ -221,55 +200,74 @@ __global__ __launch_bounds__(256) void fa_fwd_kernel(FaArgs a) {
             for (int s = 0; s < NS; s++) {
 #pragma unroll
                 for (int t = 0; t < 2; t++) {
-                    const u32x4 kf = *reinterpret_cast<const u32x4*>(
-                        k_tile(cur) + k_off<D>(32 * t + lrow, 2 * s + lhalf));
+                    const u32x4 kf = *reinterpret_cast<const u32x4*>(kt + k_off<D>(32 * t + lrow, 2 * s + lhalf));
                     sacc[t] = Mfma32A<T>::run(kf, qf[s], sacc[t]);
                 }
             }
-            // ---- to the log2 domain, additive mask, causal / tail masking ---
             float sv[32];
 #pragma unroll
             for (int t = 0; t < 2; t++)
 #pragma unroll
-                for (int r = 0; r < 16; r++) sv[t * 16 + r] = sacc[t][r] * a.c;
-            if (HAS_MASK) {
-                const T* mp = static_cast<const T*>(a.mask) + (int64_t)(bh / a.H) * a.mask_sb +
-                              (int64_t)(bh % a.H) * a.mask_sh;
-#pragma unroll
-                for (int i = 0; i < 32; i++) {
-                    const int key = kv0 + 32 * (i >> 4) + 8 * ((i & 15) >> 2) + 4 * lhalf + (i & 3);
-                    if (qpos < a.Sq && key < a.Skv)
-                        sv[i] += Elem<T>::to_f32(mp[(int64_t)qpos * a.Skv + key]) * kLog2e;
-                }
-            }
+                for (int r = 0; r < 16; r++) sv[t * 16 + r] = sacc[t][r];
+            // Register i of the pair (t = i/16, r = i%16) is key
+            // kv0 + 32t + 8(r/4) + 4*lhalf + r%4 of query column qpos.
             const bool boundary = (CAUSAL && kv0 + kBKV - 1 > qw) || kv0 + kBKV > a.Skv;
-            if (boundary) {
+            float m_new;
+            if (HAS_MASK || boundary) {
+                // general form: scores to the log2 domain first, then mask
 #pragma unroll
-                for (int i = 0; i < 32; i++) {
-                    const int key = kv0 + 32 * (i >> 4) + 8 * ((i & 15) >> 2) + 4 * lhalf + (i & 3);
-                    if ((CAUSAL && key > qpos) || key >= a.Skv) sv[i] = -INFINITY;
+                for (int i = 0; i < 32; i++) sv[i] *= a.c;
+                if (HAS_MASK) {
+                    const T* mp = static_cast<const T*>(a.mask) + (int64_t)(bh / a.H) * a.mask_sb +
+                                  (int64_t)(bh % a.H) * a.mask_sh;
+#pragma unroll
+                    for (int i = 0; i < 32; i++) {
+                        const int key = kv0 + 32 * (i >> 4) + 8 * ((i & 15) >> 2) + 4 * lhalf + (i & 3);
+                        if (qpos < a.Sq && key < a.Skv)
+                            sv[i] += Elem<T>::to_f32(mp[(int64_t)qpos * a.Skv + key]) * kLog2e;
+                    }
                 }
-            }
-            // ---- online softmax ---------------------------------------------
-            float mloc = sv[0];
+                if (boundary) {
 #pragma unroll
-            for (int i = 1; i < 32; i++) mloc = fmaxf(mloc, sv[i]);
-            mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
-            const float m_new = fmaxf(m_run, mloc);
-            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-            const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
+                    for (int i = 0; i < 32; i++) {
+                        const int key = kv0 + 32 * (i >> 4) + 8 * ((i & 15) >> 2) + 4 * lhalf + (i & 3);
+                        if ((CAUSAL && key > qpos) || key >= a.Skv) sv[i] = -INFINITY;
+                    }
+                }
+                float mloc = sv[0];
+#pragma unroll
+                for (int i = 1; i < 32; i++) mloc = fmaxf(mloc, sv[i]);
+                mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
+                m_new = fmaxf(m_run, mloc);
+                const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+#pragma unroll
+                for (int i = 0; i < 32; i++) sv[i] = __builtin_amdgcn_exp2f(sv[i] - m_use);
+            } else {
+                // interior block: max over raw scores (the scale is positive), and
+                // scale + shift folded into one fma in front of the exp2
+                float mloc = sv[0];
+#pragma unroll
+                for (int i = 1; i < 32; i++) mloc = fmaxf(mloc, sv[i]);
+                mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
+                m_new = fmaxf(m_run, mloc * a.c);
+                const float neg_m = -m_new;     // finite: an interior block has no masked score
+#pragma unroll
+                for (int i = 0; i < 32; i++) sv[i] = __builtin_amdgcn_exp2f(fmaf(sv[i], a.c, neg_m));
+            }
+            const float m_use2 = (m_new == -INFINITY) ? 0.f : m_new;
+            const float alpha = __builtin_amdgcn_exp2f(m_run - m_use2);
             m_run = m_new;
             float lsum = 0.f;
 #pragma unroll
-            for (int i = 0; i < 32; i++) {
-                sv[i] = __builtin_amdgcn_exp2f(sv[i] - m_use);
-                lsum += sv[i];
-            }
+            for (int i = 0; i < 32; i++) lsum += sv[i];
             l_run = l_run * alpha + lsum;
+            // the accumulator only needs rescaling when some row's maximum moved
+            if (__any(alpha != 1.f)) {
 #pragma unroll
-            for (int i = 0; i < ND; i++)
+                for (int i = 0; i < ND; i++)
 #pragma unroll
-                for (int r = 0; r < 16; r++) oacc[i][r] *= alpha;
+                    for (int r = 0; r < 16; r++) oacc[i][r] *= alpha;
+            }
             // ---- P^T as B operand: slot j of step u is register 8u + j ------
             u32x4 pb[4];
 #pragma unroll
@@ -279,19 +277,25 @@ __global__ __launch_bounds__(256) void fa_fwd_kernel(FaArgs a) {
                 pb[u].z = Mfma32A<T>::pack2(sv[8 * u + 4], sv[8 * u + 5]);
                 pb[u].w = Mfma32A<T>::pack2(sv[8 * u + 6], sv[8 * u + 7]);
             }
-            // ---- O^T += V^T . P^T -------------------------------------------
+            // ---- O^T += V^T . P^T: A operand slot j of step u is key
+            // 16u + 8(j/4) + 4*lhalf + j%4, i.e. two transposing reads 8 keys apart
 #pragma unroll
             for (int u = 0; u < 4; u++) {
 #pragma unroll
                 for (int dt = 0; dt < ND; dt++) {
-                    const u32x4 vf = *reinterpret_cast<const u32x4*>(
-                        v_tile(cur) + vt_off(32 * dt + lrow, 2 * u + lhalf));
+                    const int row = 16 * u + v_row0;
+                    const int d0 = 32 * dt + v_d0;
+                    const char* p0 = vt + v_off<D>(row, d0 >> 3) + (d0 & 7) * 2;
+                    const char* p1 = vt + v_off<D>(row + 8, d0 >> 3) + (d0 & 7) * 2;
+                    const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((fa_lds_s16x4*)p0));
+                    const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((fa_lds_s16x4*)p1));
+                    u32x4 vf;
+                    vf.x = lo.x; vf.y = lo.y; vf.z = hi.x; vf.w = hi.y;
                     oacc[dt] = Mfma32A<T>::run(vf, pb[u], oacc[dt]);
                 }
             }
         }
-        if (it + 1 < nkv) store_tile(cur ^ 1);
-        __syncthreads();
+        if (it + 1 < nkv) tiles_ready();
     }
 
     // ---- normalise and store: lane holds 4 consecutive d per register group -
