@@ -134,6 +134,17 @@ def wl_copy(torch, kernels, nbytes=256 << 20):
                 flops=0.0, bytes=2.0 * nbytes, bound="hbm", kernel="copy_kernel")
 
 
+def wl_gpt2(torch, kernels, B=8, S=1024):
+    from metalhlo_amd.gpt2 import GPT2, GPT2Config, init_params
+    cfg = GPT2Config()
+    model = GPT2(cfg, init_params(cfg, seed=5))
+    g = torch.Generator(device="cuda").manual_seed(5)
+    ids = torch.randint(0, cfg.vocab, (B, S), generator=g, device="cuda", dtype=torch.int32)
+    return dict(name=f"GPT-2-small forward B{B} S{S}, bf16 compute / fp32 params (converted every step)",
+                fn=lambda i: model.forward(ids), flops=GPT2.flops(cfg, B, S), bytes=0.0, bound="mfma",
+                kernel="fused pipeline (12 x [LN, GEMM+bias, attention, GEMM+bias, add, LN, GEMM+bias+GELU, GEMM+bias, add])")
+
+
 def measure(wl, steps, warmup, torch, key=None):
     sec, wall = _time_launches(wl["fn"], steps, warmup, torch)
     if wl["bound"] == "mfma":
@@ -180,7 +191,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="gemm",
-                    choices=["gemm", "attention", "attention_full", "softmax", "layer_norm", "rms_norm", "bias_gelu", "copy"])
+                    choices=["gemm", "attention", "attention_full", "softmax", "layer_norm", "rms_norm", "bias_gelu", "copy", "gpt2"])
     ap.add_argument("--only", action="store_true", help="time only --workload (for profiling runs)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
@@ -204,16 +215,21 @@ def main():
             return wl_attention(torch, kernels, S=2048, causal=False)
         if name == "copy":
             return wl_copy(torch, kernels)
+        if name == "gpt2":
+            return wl_gpt2(torch, kernels)
         return wl_rows(torch, kernels, name)
 
     head = measure(build(args.workload), args.steps, args.warmup, torch, args.workload)
     others = {}
     if not args.only:
-        for name in ["gemm", "attention", "attention_full", "softmax", "layer_norm", "rms_norm", "bias_gelu"]:
+        for name in ["gemm", "attention", "attention_full", "softmax", "layer_norm", "rms_norm", "bias_gelu", "gpt2"]:
             if name == args.workload:
                 continue
             torch.cuda.empty_cache()
-            others[name] = measure(build(name), args.steps, args.warmup, torch, name)
+            k_steps = min(args.steps, 10) if name == "gpt2" else args.steps
+            others[name] = measure(build(name), k_steps, min(args.warmup, 3) if name == "gpt2" else args.warmup, torch, name)
+            if name == "gpt2":
+                others[name]["fwd_ms"] = round(others[name]["us_per_launch"] / 1e3, 3)
             print(f"[bench] {name}: {others[name]['value']} {others[name]['unit']} "
                   f"({others[name]['roofline']['frac'] * 100:.1f}% of peak)", file=sys.stderr, flush=True)
     cpu = None

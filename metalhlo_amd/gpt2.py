@@ -1,0 +1,87 @@
+"""GPT-2 forward through the fused kernels (BASELINE config 5).
+
+The op sequence is the one the reference's fusion passes produce for a pre-LN
+GPT-2 block — fused_layer_norm, fused_matmul_bias_activation (bias only, and
+bias + tanh-GELU), fused_scaled_dot_product_attention with is_causal, residual
+adds, token + position gather, tied output head — issued in order on one HIP
+stream like the reference's integrated executor does
+(Sources/MetalHLOCore/Runtime/IntegratedExecutor.swift:208-232), but with no
+host synchronisation between launches.  Architecture constants:
+Sources/GPT2EndToEnd/main.swift:35-40.
+
+Parameters are held in fp32; every forward converts them to the compute type at
+use (the `convert` ops of the fp32-params / bf16-compute graph), computes each
+fused op with fp32 accumulation and rounds once at its output.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, List
+
+import numpy as np
+import torch
+
+from . import kernels
+
+
+@dataclass
+class GPT2Config:
+    n_layer: int = 12
+    d_model: int = 768
+    n_head: int = 12
+    d_ff: int = 3072
+    vocab: int = 50257
+    n_pos: int = 1024
+
+
+def init_params(cfg: GPT2Config, seed: int = 5) -> Dict:
+    """Random-init N(0, 0.02) weights, zero biases, LN gamma 1 / beta 0 (numpy fp32)."""
+    rng = np.random.default_rng(seed)
+    d, f = cfg.d_model, cfg.d_ff
+    w = lambda *s: rng.normal(0.0, 0.02, s).astype(np.float32)
+    z = lambda *s: np.zeros(s, np.float32)
+    o = lambda *s: np.ones(s, np.float32)
+    layers = [dict(ln1_g=o(d), ln1_b=z(d), w_qkv=w(d, 3 * d), b_qkv=z(3 * d), w_o=w(d, d), b_o=z(d),
+                   ln2_g=o(d), ln2_b=z(d), w_fc=w(d, f), b_fc=z(f), w_proj=w(f, d), b_proj=z(d))
+              for _ in range(cfg.n_layer)]
+    return dict(wte=w(cfg.vocab, d), wpe=w(cfg.n_pos, d), layers=layers, lnf_g=o(d), lnf_b=z(d))
+
+
+class GPT2:
+    def __init__(self, cfg: GPT2Config, params: Dict, compute_dtype=torch.bfloat16, device="cuda"):
+        self.cfg, self.dtype = cfg, compute_dtype
+        dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)
+        self.p32 = dict(wte=dev(params["wte"]), wpe=dev(params["wpe"]),
+                        lnf_g=dev(params["lnf_g"]), lnf_b=dev(params["lnf_b"]),
+                        layers=[{k: dev(v) for k, v in l.items()} for l in params["layers"]])
+
+    def _cast(self, t: torch.Tensor) -> torch.Tensor:
+        return t if t.dtype == self.dtype else kernels.convert(t, self.dtype)
+
+    def forward(self, ids: torch.Tensor) -> torch.Tensor:
+        """ids int32 [B,S] on the device -> logits [B,S,vocab] in the compute type."""
+        cfg, c = self.cfg, self._cast
+        B, S = ids.shape
+        d, H = cfg.d_model, cfg.n_head
+        p = self.p32
+        x = kernels.embed_tokens(ids, p["wte"], p["wpe"], self.dtype).reshape(B * S, d)
+        for l in p["layers"]:
+            h = kernels.layer_norm(x, c(l["ln1_g"]), c(l["ln1_b"]), eps=1e-5)
+            qkv = kernels.matmul(h, c(l["w_qkv"]), bias=c(l["b_qkv"]))
+            q, k, v = kernels.split_qkv_heads(qkv.reshape(B, S, 3 * d), H)
+            a = kernels.flash_attention(q, k, v, is_causal=True)
+            a = kernels.transpose_0213(a).reshape(B * S, d)
+            x = kernels.add(x, kernels.matmul(a, c(l["w_o"]), bias=c(l["b_o"])))
+            h = kernels.layer_norm(x, c(l["ln2_g"]), c(l["ln2_b"]), eps=1e-5)
+            u = kernels.matmul(h, c(l["w_fc"]), bias=c(l["b_fc"]), activation="gelu")
+            x = kernels.add(x, kernels.matmul(u, c(l["w_proj"]), bias=c(l["b_proj"])))
+        x = kernels.layer_norm(x, c(p["lnf_g"]), c(p["lnf_b"]), eps=1e-5)
+        logits = kernels.matmul(x, c(p["wte"]), trans_b=True)       # tied head: x . wte^T
+        return logits.reshape(B, S, cfg.vocab)
+
+    @staticmethod
+    def flops(cfg: GPT2Config, B: int, S: int) -> float:
+        d, f = cfg.d_model, cfg.d_ff
+        per_tok = cfg.n_layer * (d * 3 * d + d * d + 2 * d * f) + d * cfg.vocab
+        attn = cfg.n_layer * 2 * B * cfg.n_head * S * S * (d // cfg.n_head)   # causal: half of 4BHS^2D
+        return 2.0 * per_tok * B * S + attn

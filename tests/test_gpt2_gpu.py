@@ -1,0 +1,71 @@
+"""GPU parity: GPT-2-small forward through the fused pipeline (bf16 compute,
+fp32 parameters) vs the float64 oracle with the same rounding points.
+Tolerance: bf16 rule, |got - e| <= max(2e-2, 2e-2 |e|)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle
+from tests.util import as_f64
+
+pytestmark = pytest.mark.gpu
+
+
+def _check(got, exp, what="", frac=1e-5):
+    """Every fused operator is held to 2e-2 on its own (other test files).  Through a
+    whole network a value that sits next to a bf16 rounding boundary can round the
+    other way than in the float64 oracle and the difference is carried on, so the
+    end-to-end rule is: at most `frac` of the logits outside the 2e-2 rule (1e-5 for
+    the 2-layer model, 5e-3 for 12 layers, where the residual stream reaches
+    magnitudes whose bf16 spacing is itself 3e-2), an RMS error below 1e-2, and none
+    outside 5e-2, the bound the reference's own bf16 suite uses
+    (Examples/FlaxExample/flax_metalhlo_bf16.py:68)."""
+    g = as_f64(got)
+    err = np.abs(g - exp)
+    frac_bad = float((err > np.maximum(2e-2, 2e-2 * np.abs(exp))).mean())
+    worst = float((err / np.maximum(1.0, np.abs(exp))).max())
+    rms = float(np.sqrt((err ** 2).mean()))
+    assert frac_bad <= frac and worst <= 5e-2 and rms <= 1e-2, \
+        f"{what}: {frac_bad:.2e} of logits outside 2e-2, worst scaled error {worst:.4f}, rms {rms:.4f}"
+
+
+def test_gpt2_reduced_depth_full_width():
+    """2 layers, full width / heads / vocabulary, B2 S192: whole-tensor comparison."""
+    from metalhlo_amd.gpt2 import GPT2, GPT2Config, init_params
+    cfg = GPT2Config(n_layer=2)
+    params = init_params(cfg, seed=5)
+    rng = np.random.default_rng(5)
+    ids = rng.integers(0, cfg.vocab, (2, 192)).astype(np.int32)
+    model = GPT2(cfg, params)
+    logits = model.forward(torch.from_numpy(ids).cuda())
+    assert logits.shape == (2, 192, cfg.vocab) and logits.dtype == torch.bfloat16
+    exp = oracle.gpt2_forward(ids, params, cfg.n_head, "bf16")
+    _check(logits, exp, what="2-layer GPT-2")
+
+
+def test_gpt2_small_baseline_shape():
+    """BASELINE config 4: 12 layers, B8 S1024.  The oracle runs on batch element 0
+    alone (sequences are independent); properties cover the rest."""
+    from metalhlo_amd.gpt2 import GPT2, GPT2Config, init_params
+    cfg = GPT2Config()
+    params = init_params(cfg, seed=5)
+    rng = np.random.default_rng(5)
+    ids = rng.integers(0, cfg.vocab, (8, 1024)).astype(np.int32)
+    model = GPT2(cfg, params)
+    dev_ids = torch.from_numpy(ids).cuda()
+    logits = model.forward(dev_ids)
+    assert logits.shape == (8, 1024, cfg.vocab)
+    assert torch.isfinite(logits.float()).all()
+    exp = oracle.gpt2_forward(ids[:1, :256], params, cfg.n_head, "bf16")      # causal: prefix suffices
+    _check(logits[:1, :256], exp, what="GPT-2-small, batch 0, first 256 positions", frac=5e-3)
+    # causality: changing the last token of every sequence leaves earlier logits bit-identical
+    ids2 = ids.copy(); ids2[:, -1] = (ids2[:, -1] + 1) % cfg.vocab
+    l2 = model.forward(torch.from_numpy(ids2).cuda())
+    assert torch.equal(l2[:, :-1], logits[:, :-1]) and not torch.equal(l2[:, -1], logits[:, -1])
+    # batch independence: sequence 3 alone gives the same logits as inside the batch
+    l3 = model.forward(dev_ids[3:4].contiguous())
+    assert torch.equal(l3[0], logits[3])
+    # greedy next-token ids are exact integer results of argmax over bf16 logits
+    from metalhlo_amd import kernels
+    nxt = kernels.argmax(logits[:, -1].contiguous())
+    assert torch.equal(nxt.long(), logits[:, -1].float().argmax(-1))
