@@ -191,6 +191,49 @@ int mhip_iota(void* stream, void* y, int64_t outer, int64_t n, int64_t inner, in
 int mhip_argmax(void* stream, const void* x, void* out_idx, void* out_val, int64_t rows,
                 int64_t cols, int dtype, int idx_dtype);
 
+/* Unfused StableHLO glue for a host executor ------------------------------- */
+
+typedef enum { MHIP_UN_EXP = 0, MHIP_UN_TANH, MHIP_UN_RSQRT, MHIP_UN_SQRT, MHIP_UN_NEG,
+               MHIP_UN_LOGISTIC, MHIP_UN_ABS, MHIP_UN_LOG, MHIP_UN_ERF } mhip_unary_op;
+typedef enum { MHIP_BIN_ADD = 0, MHIP_BIN_SUB, MHIP_BIN_MUL, MHIP_BIN_DIV, MHIP_BIN_MAX,
+               MHIP_BIN_MIN, MHIP_BIN_POW } mhip_binary_op;
+typedef enum { MHIP_CMP_EQ = 0, MHIP_CMP_NE, MHIP_CMP_LT, MHIP_CMP_LE, MHIP_CMP_GT,
+               MHIP_CMP_GE } mhip_compare_dir;
+typedef enum { MHIP_RED_SUM = 0, MHIP_RED_MAX, MHIP_RED_MIN, MHIP_RED_PROD } mhip_reduce_op;
+
+/* y = op(x) elementwise (unary kernels, Compiler/CodeGenerator.swift:851-920).
+ * F32/F16/BF16 (fp32 math, one rounding); NEG and ABS also on I32/I64. */
+int mhip_unary(void* stream, int op, const void* x, void* y, int64_t n, int dtype);
+
+/* y = a op b elementwise, equal shapes (binary kernels, CodeGenerator.swift:921-1010).
+ * Floats: fp32 math, one rounding, max/min propagate NaN; integers wrap. */
+int mhip_binary(void* stream, int op, const void* a, const void* b, void* y, int64_t n, int dtype);
+
+/* y[i] = (a[i] <dir> b[i]) as one byte 0/1 (stablehlo.compare, CodeGenerator.swift:1101). */
+int mhip_compare(void* stream, int direction, const void* a, const void* b, void* y, int64_t n,
+                 int dtype);
+
+/* y[i] = pred[i] ? a[i] : b[i]; pred is bytes, or one byte when scalar_pred
+ * (stablehlo.select, CodeGenerator.swift:2008). elem_size in {1,2,4,8}. */
+int mhip_select(void* stream, const void* pred, const void* a, const void* b, void* y, int64_t n,
+                int elem_size, int scalar_pred);
+
+/* y[o] = x[in_offset + sum_d idx_d(o) * in_strides[d]] over a dense row-major
+ * output of `out_shape` (rank <= 8; stride 0 broadcasts).  One kernel for
+ * broadcast_in_dim (:3057), transpose (:2840-3056) and slice of
+ * Compiler/CodeGenerator.swift. */
+int mhip_strided_copy(void* stream, const void* x, void* y, int rank, const int64_t* out_shape,
+                      const int64_t* in_strides, int64_t in_offset, int elem_size);
+
+/* y[o, i] = reduce_l x[o, l, i] starting from `init`, in index order
+ * (stablehlo.reduce with add / maximum / minimum / multiply bodies,
+ * Parser/Parser.swift:657-730). F32/F16/BF16/I32/I64. */
+int mhip_reduce(void* stream, int op, const void* x, void* y, int64_t outer, int64_t len,
+                int64_t inner, double init, int dtype);
+
+/* y[i] = the low elem_size bytes of `pattern`, n elements (splat constants). */
+int mhip_fill(void* stream, void* y, int64_t n, uint64_t pattern, int elem_size);
+
 #ifdef __cplusplus
 }
 #endif

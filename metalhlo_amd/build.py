@@ -14,7 +14,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 ROOT = os.path.dirname(HERE)
 
-HIP_SOURCES = ["runtime.hip", "row_kernels.hip", "gemm.hip", "attention.hip", "glue_kernels.hip"]
+HIP_SOURCES = ["runtime.hip", "row_kernels.hip", "gemm.hip", "attention.hip", "glue_kernels.hip", "elementwise.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=fast",
@@ -74,9 +74,10 @@ def build_host(verbose: bool = True) -> list:
     if not srcs:
         return outs
     out = os.path.join(LIBDIR, "libCMetalHLO.so")
-    _run([hipcc(), "-O2", "-std=c++17", "-fPIC", "-shared", "-D__HIP_PLATFORM_AMD__",
-          "-I", os.path.join(ROOT, "include"), "-I", "/opt/rocm/include", "-o", out, *srcs,
-          "-L", LIBDIR, "-lmetalhlo_hip", "-Wl,-rpath,$ORIGIN"])
+    _run([hipcc(), "-x", "c++", "-O2", "-std=c++17", "-fPIC", "-D__HIP_PLATFORM_AMD__", "-Wall",
+          "-I", os.path.join(ROOT, "include"), "-I", "/opt/rocm/include", *srcs,
+          "-shared", "-o", out, "-L", LIBDIR, "-lmetalhlo_hip", "-L", "/opt/rocm/lib", "-lamdhip64",
+          "-Wl,-rpath,$ORIGIN", "-Wl,-rpath,/opt/rocm/lib"])
     if verbose:
         print("  link ", os.path.relpath(out, ROOT), flush=True)
     outs.append(out)

@@ -211,43 +211,48 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_mfma_kernel(GemmArgs g) {
     // in register group q = r/4, the four consecutive columns 8q + 4*lhalf + r%4.
     const T* bias = static_cast<const T*>(g.bias);
     const bool vec_store = (g.N % 8 == 0) && ((reinterpret_cast<uintptr_t>(c) & 15) == 0);
-    if (vec_store) {
-        // Stage the wave's sub-tile in LDS as rounded 16-bit rows (padded to 144
-        // bytes against bank conflicts), then write whole 128-byte row segments.
-        constexpr int kRowPad = WTN * 2 + 16;
-        char* stage = smem + wave * (WTM * kRowPad);
+    // Stage the wave's sub-tile in LDS as rounded 16-bit rows (padded by 16 bytes
+    // against bank conflicts); the rows then go out with lanes running along n, so
+    // every store instruction writes whole contiguous row segments.
+    constexpr int kRowPad = WTN * 2 + 16;
+    char* stage = smem + wave * (WTM * kRowPad);
 #pragma unroll
-        for (int j = 0; j < TN; j++) {
+    for (int j = 0; j < TN; j++) {
 #pragma unroll
-            for (int q = 0; q < 4; q++) {
-                const int nl = j * 32 + 8 * q + 4 * lhalf;          // column inside the wave tile
-                const int n = n0 + wn * WTN + nl;
-                float bv[4] = {0.f, 0.f, 0.f, 0.f};
-                if (bias && n < g.N) {
+        for (int q = 0; q < 4; q++) {
+            const int nl = j * 32 + 8 * q + 4 * lhalf;          // column inside the wave tile
+            const int n = n0 + wn * WTN + nl;
+            float bv[4] = {0.f, 0.f, 0.f, 0.f};
+            if (bias) {
+                if (vec_store && n < g.N) {
                     const Pack4<T> t = __builtin_bit_cast(Pack4<T>, *reinterpret_cast<const u32x2*>(bias + n));
 #pragma unroll
                     for (int e = 0; e < 4; e++) bv[e] = Elem<T>::to_f32(t.v[e]);
-                }
+                } else {
 #pragma unroll
-                for (int i = 0; i < TM; i++) {
-                    float v[4];
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        v[e] = acc[i][j][4 * q + e] + bv[e];
-                        if (g.act != MHIP_ACT_NONE) v[e] = apply_act(v[e], g.act);
-                    }
-                    Pack4<T> o;
-#pragma unroll
-                    for (int e = 0; e < 4; e++) o.v[e] = Elem<T>::from_f32(v[e]);
-                    *reinterpret_cast<u32x2*>(stage + (i * 32 + lrow) * kRowPad + nl * 2) =
-                        __builtin_bit_cast(u32x2, o);
+                    for (int e = 0; e < 4; e++)
+                        if (n + e < g.N) bv[e] = Elem<T>::to_f32(bias[n + e]);
                 }
             }
+#pragma unroll
+            for (int i = 0; i < TM; i++) {
+                Pack4<T> o;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    float v = acc[i][j][4 * q + e] + bv[e];
+                    if (g.act != MHIP_ACT_NONE) v = apply_act(v, g.act);
+                    o.v[e] = Elem<T>::from_f32(v);
+                }
+                *reinterpret_cast<u32x2*>(stage + (i * 32 + lrow) * kRowPad + nl * 2) =
+                    __builtin_bit_cast(u32x2, o);
+            }
         }
-        // each wave only re-reads what it wrote itself
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+    // each wave only re-reads what it wrote itself
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    if (vec_store) {
         constexpr int kCpr = WTN / 8;                // 16-byte chunks per row
         constexpr int kRowsPerPass = 64 / kCpr;
         const int cc = lane % kCpr, rr = lane / kCpr;
@@ -261,22 +266,20 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_mfma_kernel(GemmArgs g) {
                 *reinterpret_cast<u32x4*>(c + (int64_t)m * g.N + n) = w;
             }
         }
-        return;
-    }
+    } else {
+        // rows of C are not 16-byte aligned (odd N): one element per lane, 64
+        // consecutive columns per store instruction
+        const uint16_t* st16 = reinterpret_cast<const uint16_t*>(stage);
+        uint16_t* c16 = reinterpret_cast<uint16_t*>(c);
+#pragma unroll 4
+        for (int ml = 0; ml < WTM; ml++) {
+            const int m = m0 + wm * WTM + ml;
+            if (m >= g.M) break;
 #pragma unroll
-    for (int i = 0; i < TM; i++) {
-        const int m = m0 + wm * WTM + i * 32 + lrow;
-        if (m >= g.M) continue;
-#pragma unroll
-        for (int j = 0; j < TN; j++) {
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int n = n0 + wn * WTN + j * 32 + 8 * (r >> 2) + 4 * lhalf + (r & 3);
-                if (n < g.N) {
-                    float v = acc[i][j][r] + (bias ? Elem<T>::to_f32(bias[n]) : 0.f);
-                    if (g.act != MHIP_ACT_NONE) v = apply_act(v, g.act);
-                    c[(int64_t)m * g.N + n] = Elem<T>::from_f32(v);
-                }
+            for (int cb = 0; cb < WTN / 64; cb++) {
+                const int nl = cb * 64 + lane;
+                const int n = n0 + wn * WTN + nl;
+                if (n < g.N) c16[(int64_t)m * g.N + n] = st16[ml * (kRowPad / 2) + nl];
             }
         }
     }
@@ -348,7 +351,8 @@ static int launch_mfma(hipStream_t s, GemmArgs g, int64_t batch) {
 template <typename T, bool TA, bool TB>
 static int pick_tile(hipStream_t s, const GemmArgs& g, int64_t batch) {
     const int64_t big = (int64_t)((g.M + 255) / 256) * ((g.N + 255) / 256) * batch;
-    if (big >= 192) return launch_mfma<T, 256, 256, 2, 4, TA, TB>(s, g, batch);
+    const int force = tune_int("MHIP_GEMM_TILE", 0);
+    if (force == 256 || (force != 128 && big >= 192)) return launch_mfma<T, 256, 256, 2, 4, TA, TB>(s, g, batch);
     return launch_mfma<T, 128, 128, 2, 2, TA, TB>(s, g, batch);
 }
 

@@ -131,6 +131,23 @@ __global__ __launch_bounds__(256) void convert_kernel(const S* __restrict__ x, D
     }
 }
 
+// fp32 -> 16-bit float, eight elements per lane (two 16-byte loads, one 16-byte store)
+template <typename D>
+__global__ __launch_bounds__(256) void narrow_vec_kernel(const float* __restrict__ x,
+                                                         D* __restrict__ y, int64_t nvec) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= nvec) return;
+    const f32x4 a = *reinterpret_cast<const f32x4*>(x + i * 8);
+    const f32x4 b = *reinterpret_cast<const f32x4*>(x + i * 8 + 4);
+    Vec16<D> o;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        o.v[e] = Elem<D>::from_f32(a[e]);
+        o.v[4 + e] = Elem<D>::from_f32(b[e]);
+    }
+    store16(y + i * 8, o);
+}
+
 // ---- [d0,d1,d2,d3] -> [d0,d2,d1,d3] ------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void transpose_0213_kernel(const T* __restrict__ x,
@@ -363,6 +380,20 @@ extern "C" int mhip_convert(void* stream, const void* x, void* y, int64_t n, int
     if (n < 0) return fail(MHIP_ERR_INVALID_ARGUMENT, "mhip_convert: negative size");
     if (n == 0) return MHIP_OK;
     hipStream_t s = as_stream(stream);
+    if (src_dtype == MHIP_F32 && (dst_dtype == MHIP_BF16 || dst_dtype == MHIP_F16) && n >= 8 &&
+        ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15) == 0) {
+        const int64_t nvec = n / 8;
+        unsigned grid;
+        if (grid_for(nvec, 256, &grid)) return MHIP_ERR_UNSUPPORTED;
+        if (dst_dtype == MHIP_BF16)
+            hipLaunchKernelGGL((narrow_vec_kernel<bf16_t>), dim3(grid), dim3(256), 0, s, (const float*)x, (bf16_t*)y, nvec);
+        else
+            hipLaunchKernelGGL((narrow_vec_kernel<f16_t>), dim3(grid), dim3(256), 0, s, (const float*)x, (f16_t*)y, nvec);
+        const int64_t done = nvec * 8;
+        if (done == n) return check_launch("convert");
+        const int es = 2;
+        return mhip_convert(stream, (const char*)x + done * 4, (char*)y + done * es, n - done, src_dtype, dst_dtype);
+    }
     switch (src_dtype) {
         case MHIP_F32: return convert_from<float>(s, x, y, n, dst_dtype);
         case MHIP_F64: return convert_from<double>(s, x, y, n, dst_dtype);

@@ -1,0 +1,516 @@
+#include "executor.h"
+
+#include <math.h>
+#include <string.h>
+
+#include <algorithm>
+#include <chrono>
+#include <map>
+
+#include "../../../include/mhip.h"
+
+namespace mhlo {
+
+// ---------------------------------------------------------------- memory
+DevicePool::~DevicePool() {
+    for (auto& kv : free_) (void)hipFree(kv.second);
+}
+
+static size_t bucket(size_t bytes) {
+    size_t b = 256;
+    while (b < bytes) b <<= 1;
+    return bytes > (64u << 20) ? ((bytes + (2u << 20) - 1) & ~((size_t)(2u << 20) - 1)) : b;
+}
+
+void* DevicePool::alloc(size_t bytes) {
+    const size_t b = bucket(bytes ? bytes : 1);
+    {
+        std::lock_guard<std::mutex> g(mu_);
+        auto it = free_.find(b);
+        if (it != free_.end()) {
+            void* p = it->second;
+            free_.erase(it);
+            return p;
+        }
+    }
+    void* p = nullptr;
+    hipError_t e = hipMalloc(&p, b);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        {   // give cached blocks back and retry once
+            std::lock_guard<std::mutex> g(mu_);
+            for (auto& kv : free_) (void)hipFree(kv.second);
+            free_.clear();
+        }
+        e = hipMalloc(&p, b);
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            throw BufferError(std::string("hipMalloc of ") + std::to_string(b) + " bytes failed: " + hipGetErrorString(e));
+        }
+    }
+    return p;
+}
+
+void DevicePool::release(void* p, size_t bytes) {
+    std::lock_guard<std::mutex> g(mu_);
+    free_.emplace(bucket(bytes ? bytes : 1), p);
+}
+
+DeviceTensor Client::allocate(const TensorType& t) {
+    if (device < 0) throw NoDevice("no HIP device: buffers cannot be created");
+    DeviceTensor d;
+    d.type = t;
+    d.mem = std::make_shared<DeviceMem>();
+    d.mem->pool = &pool;
+    d.mem->bytes = t.bytes();
+    d.mem->ptr = pool.alloc(d.mem->bytes);
+    return d;
+}
+
+// ---------------------------------------------------------------- op tables
+static const std::map<std::string, int> kUnary = {
+    {"exponential", MHIP_UN_EXP}, {"tanh", MHIP_UN_TANH}, {"rsqrt", MHIP_UN_RSQRT}, {"sqrt", MHIP_UN_SQRT},
+    {"negate", MHIP_UN_NEG}, {"logistic", MHIP_UN_LOGISTIC}, {"abs", MHIP_UN_ABS}, {"log", MHIP_UN_LOG},
+    {"erf", MHIP_UN_ERF}};
+static const std::map<std::string, int> kBinary = {
+    {"add", MHIP_BIN_ADD}, {"subtract", MHIP_BIN_SUB}, {"multiply", MHIP_BIN_MUL}, {"divide", MHIP_BIN_DIV},
+    {"maximum", MHIP_BIN_MAX}, {"minimum", MHIP_BIN_MIN}, {"power", MHIP_BIN_POW}};
+static const std::map<std::string, int> kCompare = {{"EQ", MHIP_CMP_EQ}, {"NE", MHIP_CMP_NE}, {"LT", MHIP_CMP_LT},
+                                                    {"LE", MHIP_CMP_LE}, {"GT", MHIP_CMP_GT}, {"GE", MHIP_CMP_GE}};
+static const std::map<std::string, int> kReduce = {{"add", MHIP_RED_SUM}, {"maximum", MHIP_RED_MAX},
+                                                   {"minimum", MHIP_RED_MIN}, {"multiply", MHIP_RED_PROD}};
+static const std::map<std::string, int> kActivation = {{"none", MHIP_ACT_NONE}, {"relu", MHIP_ACT_RELU},
+                                                       {"gelu", MHIP_ACT_GELU}, {"silu", MHIP_ACT_SILU},
+                                                       {"tanh", MHIP_ACT_TANH}, {"sigmoid", MHIP_ACT_SIGMOID}};
+// custom_call targets served by a kernel (Compiler/CustomCallHandlers.swift:75-89)
+static const char* kTargets[] = {"fused_scaled_dot_product_attention", "fused_layer_norm", "fused_rms_norm",
+                                 "fused_softmax", "fused_gelu", "fused_matmul_bias_activation"};
+
+static std::string where(const Op& op) { return "line " + std::to_string(op.line) + " (stablehlo." + op.name + "): "; }
+
+static bool is_kernel_float(int dt) { return dt == F32 || dt == F16 || dt == BF16; }
+
+// Shapes/dtypes of every value, filled while validating.
+static std::vector<TensorType> value_types(const Function& fn) {
+    std::vector<TensorType> t(fn.num_values);
+    for (size_t i = 0; i < fn.arg_ids.size(); i++) t[fn.arg_ids[i]] = fn.arg_types[i];
+    for (auto& op : fn.ops) t[op.result] = op.out;
+    return t;
+}
+
+struct DotPlan {
+    int64_t B = 1, M = 1, N = 1, K = 1;
+    bool lhs_copy = false, rhs_copy = false;   // need a transposing copy into canonical order
+    bool trans_a = false, trans_b = false;
+    std::vector<int64_t> lhs_perm, rhs_perm;   // canonical orders [batch, free, contract] / [batch, contract, free]
+};
+
+static bool is_identity_after(const std::vector<int64_t>& perm) {
+    for (size_t i = 0; i < perm.size(); i++) if (perm[i] != (int64_t)i) return false;
+    return true;
+}
+
+static DotPlan plan_dot(const Op& op, const TensorType& lt, const TensorType& rt) {
+    DotPlan p;
+    std::vector<int64_t> lb = op.lhs_batch, rb = op.rhs_batch, lc = op.lhs_contract, rc = op.rhs_contract;
+    if (op.name == "dot") {
+        lc = {(int64_t)lt.shape.size() - 1};
+        rc = {0};
+    }
+    auto in = [](const std::vector<int64_t>& v, int64_t d) { return std::find(v.begin(), v.end(), d) != v.end(); };
+    std::vector<int64_t> lf, rf;
+    for (int64_t d = 0; d < (int64_t)lt.shape.size(); d++) if (!in(lb, d) && !in(lc, d)) lf.push_back(d);
+    for (int64_t d = 0; d < (int64_t)rt.shape.size(); d++) if (!in(rb, d) && !in(rc, d)) rf.push_back(d);
+    if (lb.size() != rb.size() || lc.size() != rc.size()) throw ParseError(where(op) + "mismatched dimension numbers");
+    for (size_t i = 0; i < lb.size(); i++) {
+        if (lt.shape.at(lb[i]) != rt.shape.at(rb[i])) throw ParseError(where(op) + "batch sizes differ");
+        p.B *= lt.shape[lb[i]];
+    }
+    for (size_t i = 0; i < lc.size(); i++) {
+        if (lt.shape.at(lc[i]) != rt.shape.at(rc[i])) throw ParseError(where(op) + "contracting sizes differ");
+        p.K *= lt.shape[lc[i]];
+    }
+    for (auto d : lf) p.M *= lt.shape[d];
+    for (auto d : rf) p.N *= rt.shape[d];
+    auto cat = [](std::vector<int64_t> a, const std::vector<int64_t>& b, const std::vector<int64_t>& c) {
+        a.insert(a.end(), b.begin(), b.end());
+        a.insert(a.end(), c.begin(), c.end());
+        return a;
+    };
+    // lhs: [batch, free, contract] is A[M,K]; [batch, contract, free] is A stored [K,M]
+    if (is_identity_after(cat(lb, lf, lc))) p.trans_a = false;
+    else if (is_identity_after(cat(lb, lc, lf))) p.trans_a = true;
+    else { p.lhs_copy = true; p.lhs_perm = cat(lb, lf, lc); }
+    // rhs: [batch, contract, free] is B[K,N]; [batch, free, contract] is B stored [N,K]
+    if (is_identity_after(cat(rb, rc, rf))) p.trans_b = false;
+    else if (is_identity_after(cat(rb, rf, rc))) p.trans_b = true;
+    else { p.rhs_copy = true; p.rhs_perm = cat(rb, rc, rf); }
+    return p;
+}
+
+// Reduced dims must form one contiguous block [a, b]; gives outer/len/inner.
+static bool reduce_block(const std::vector<int64_t>& shape, std::vector<int64_t> dims, int64_t& outer, int64_t& len,
+                         int64_t& inner) {
+    std::sort(dims.begin(), dims.end());
+    for (size_t i = 1; i < dims.size(); i++) if (dims[i] != dims[i - 1] + 1) return false;
+    outer = len = inner = 1;
+    for (int64_t d = 0; d < (int64_t)shape.size(); d++) {
+        if (dims.empty() || d < dims.front()) outer *= shape[d];
+        else if (d > dims.back()) inner *= shape[d];
+        else len *= shape[d];
+    }
+    return true;
+}
+
+static double scalar_constant(const Op& c) {
+    if (!c.splat && c.constant.empty()) throw UnsupportedOp(where(c) + "reduce init must be a scalar constant");
+    uint64_t bits = c.splat_bits;
+    if (!c.splat) memcpy(&bits, c.constant.data(), std::min<size_t>(8, c.constant.size()));
+    switch (c.out.dtype) {
+        case F32: { float f; memcpy(&f, &bits, 4); return f; }
+        case F64: { double d; memcpy(&d, &bits, 8); return d; }
+        case BF16: { uint32_t w = (uint32_t)(bits & 0xFFFF) << 16; float f; memcpy(&f, &w, 4); return f; }
+        case F16: {
+            const uint32_t h = bits & 0xFFFF, s = (h >> 15) & 1, e = (h >> 10) & 31, m = h & 1023;
+            double v = e == 0 ? ldexp((double)m, -24) : e == 31 ? (m ? NAN : INFINITY) : ldexp((double)(m | 1024), (int)e - 25);
+            return s ? -v : v;
+        }
+        case I32: { int32_t v; memcpy(&v, &bits, 4); return v; }
+        case I64: { int64_t v; memcpy(&v, &bits, 8); return (double)v; }
+        default: return (double)(int64_t)bits;
+    }
+}
+
+// ---------------------------------------------------------------- validation
+void compile(Executable& exe) {
+    Function& fn = exe.fn;
+    std::vector<TensorType> vt = value_types(fn);
+    std::map<int, const Op*> producer;
+    for (auto& op : fn.ops) producer[op.result] = &op;
+    exe.constants.assign(fn.ops.size(), DeviceTensor());
+    for (size_t oi = 0; oi < fn.ops.size(); oi++) {
+        Op& op = fn.ops[oi];
+        auto in = [&](size_t i) -> const TensorType& {
+            if (i >= op.operands.size()) throw ParseError(where(op) + "expected at least " + std::to_string(i + 1) + " operands");
+            return vt[op.operands[i]];
+        };
+        const std::string& n = op.name;
+        if (n == "constant") {
+            if (exe.client && exe.client->device >= 0) {
+                DeviceTensor d = exe.client->allocate(op.out);
+                if (op.splat) {
+                    if (mhip_fill(exe.client->stream, d.data(), op.out.numel(), op.splat_bits, dtype_bytes(op.out.dtype)) != MHIP_OK)
+                        throw ExecError(std::string("constant fill failed: ") + mhip_last_error());
+                } else if (!op.constant.empty()) {
+                    if (hipMemcpy(d.data(), op.constant.data(), op.constant.size(), hipMemcpyHostToDevice) != hipSuccess)
+                        throw BufferError("constant upload failed");
+                }
+                exe.constants[oi] = d;
+            }
+        } else if (kUnary.count(n)) {
+            if (!(in(0) == op.out)) throw ParseError(where(op) + "operand and result types differ");
+            const bool int_ok = (n == "negate" || n == "abs") && (op.out.dtype == I32 || op.out.dtype == I64);
+            if (!is_kernel_float(op.out.dtype) && !int_ok) throw UnsupportedOp(where(op) + "element type not supported");
+        } else if (kBinary.count(n)) {
+            if (!(in(0) == op.out) || !(in(1) == op.out)) throw ParseError(where(op) + "operand and result types differ");
+            if (op.out.dtype == F64 || op.out.dtype == I1 || op.out.dtype == I16 || op.out.dtype == UI16)
+                throw UnsupportedOp(where(op) + "element type not supported");
+            if (n == "power" && !is_kernel_float(op.out.dtype)) throw UnsupportedOp(where(op) + "integer power is not supported");
+        } else if (n == "convert") {
+            if (in(0).shape != op.out.shape) throw ParseError(where(op) + "convert changes the shape");
+        } else if (n == "reshape") {
+            if (in(0).numel() != op.out.numel() || in(0).dtype != op.out.dtype) throw ParseError(where(op) + "reshape changes the element count or type");
+        } else if (n == "transpose") {
+            if (op.dims.size() != in(0).shape.size() || op.dims.size() > 8) throw ParseError(where(op) + "bad permutation");
+            for (size_t d = 0; d < op.dims.size(); d++)
+                if (op.dims[d] < 0 || op.dims[d] >= (int64_t)op.dims.size() || op.out.shape.at(d) != in(0).shape[op.dims[d]])
+                    throw ParseError(where(op) + "permutation does not match the result shape");
+        } else if (n == "broadcast_in_dim") {
+            if (op.dims.size() != in(0).shape.size() || op.out.shape.size() > 8) throw ParseError(where(op) + "bad broadcast dims");
+            for (size_t d = 0; d < op.dims.size(); d++) {
+                if (op.dims[d] < 0 || op.dims[d] >= (int64_t)op.out.shape.size()) throw ParseError(where(op) + "broadcast dim out of range");
+                const int64_t a = in(0).shape[d], b = op.out.shape[op.dims[d]];
+                if (a != b && a != 1) throw ParseError(where(op) + "operand dim is neither 1 nor the result dim");
+            }
+        } else if (n == "slice") {
+            const size_t r = in(0).shape.size();
+            if (op.starts.size() != r || op.limits.size() != r || op.strides.size() != r || r > 8) throw ParseError(where(op) + "bad slice indices");
+            for (size_t d = 0; d < r; d++) {
+                if (op.strides[d] <= 0 || op.starts[d] < 0 || op.limits[d] > in(0).shape[d] || op.starts[d] > op.limits[d])
+                    throw ParseError(where(op) + "slice range outside the operand");
+                if ((op.limits[d] - op.starts[d] + op.strides[d] - 1) / op.strides[d] != op.out.shape.at(d))
+                    throw ParseError(where(op) + "slice range does not match the result shape");
+            }
+        } else if (n == "reduce") {
+            if (!kReduce.count(op.reducer)) throw UnsupportedOp(where(op) + "reducer body is not add / maximum / minimum / multiply");
+            auto it = producer.find(op.operands.at(1));
+            if (it == producer.end() || it->second->name != "constant") throw UnsupportedOp(where(op) + "init value must be a constant");
+            if (!is_kernel_float(in(0).dtype) && in(0).dtype != I32 && in(0).dtype != I64) throw UnsupportedOp(where(op) + "element type not supported");
+            for (auto d : op.dims) if (d < 0 || d >= (int64_t)in(0).shape.size()) throw ParseError(where(op) + "dimension out of range");
+        } else if (n == "dot" || n == "dot_general") {
+            if (!is_kernel_float(in(0).dtype) || in(0).dtype != in(1).dtype || op.out.dtype != in(0).dtype)
+                throw UnsupportedOp(where(op) + "dot needs f32 / f16 / bf16 operands and a result of the same type");
+            (void)plan_dot(op, in(0), in(1));
+        } else if (n == "iota") {
+            if (op.iota_dim < 0 || op.iota_dim >= (int64_t)op.out.shape.size()) throw ParseError(where(op) + "iota dim out of range");
+        } else if (n == "compare") {
+            if (!(in(0) == in(1)) || op.out.dtype != I1 || op.out.shape != in(0).shape) throw ParseError(where(op) + "bad compare types");
+            if (in(0).dtype == F64 || in(0).dtype == I16 || in(0).dtype == UI16) throw UnsupportedOp(where(op) + "element type not supported");
+        } else if (n == "select") {
+            if (!(in(1) == op.out) || !(in(2) == op.out) || in(0).dtype != I1) throw ParseError(where(op) + "bad select types");
+            if (in(0).numel() != 1 && in(0).shape != op.out.shape) throw ParseError(where(op) + "predicate shape mismatch");
+        } else if (n == "gather") {
+            // whole-row gather only: operand [rows, d], one collapsed / mapped dim 0
+            if (in(0).shape.size() != 2 || op.dims != std::vector<int64_t>{0} || op.starts != std::vector<int64_t>{0} ||
+                op.limits != std::vector<int64_t>{1, in(0).shape[1]} || (in(1).dtype != I32 && in(1).dtype != I64))
+                throw UnsupportedOp(where(op) + "only whole-row gathers (embedding lookups) are supported");
+        } else if (n == "custom_call") {
+            bool ok = false;
+            for (auto t : kTargets) ok |= op.target == t;
+            if (!ok) throw UnsupportedOp(where(op) + "Unsupported custom call target: " + op.target);
+            const size_t need = op.target == "fused_scaled_dot_product_attention" || op.target == "fused_layer_norm" ? 3
+                              : op.target == "fused_rms_norm" || op.target == "fused_matmul_bias_activation" ? 2 : 1;
+            if (op.operands.size() < need)
+                throw ParseError(where(op) + "Invalid input count: expected " + std::to_string(need) + ", got " + std::to_string(op.operands.size()));
+            if (!is_kernel_float(in(0).dtype)) throw UnsupportedOp(where(op) + "element type not supported");
+            if (op.target == "fused_matmul_bias_activation" &&
+                !kActivation.count(parse_config(op.backend_config).get_string("activation", "none")))
+                throw UnsupportedOp(where(op) + "unknown activation");
+        } else {
+            throw UnsupportedOp(where(op) + "operation is outside the supported subset");
+        }
+    }
+    for (int r : fn.returns) (void)r;
+    if (exe.client && exe.client->device >= 0) (void)hipStreamSynchronize(exe.client->stream);
+}
+
+// ---------------------------------------------------------------- execution
+static void check(int st, const Op& op) {
+    if (st != MHIP_OK) throw ExecError(where(op) + mhip_last_error());
+}
+
+static std::vector<int64_t> dense_strides(const std::vector<int64_t>& shape) {
+    std::vector<int64_t> s(shape.size(), 1);
+    for (int i = (int)shape.size() - 2; i >= 0; i--) s[i] = s[i + 1] * shape[i + 1];
+    return s;
+}
+
+static DeviceTensor permuted_copy(Client& c, const DeviceTensor& x, const std::vector<int64_t>& perm, const Op& op) {
+    TensorType t;
+    t.dtype = x.type.dtype;
+    const auto st = dense_strides(x.type.shape);
+    std::vector<int64_t> in_str;
+    for (auto d : perm) { t.shape.push_back(x.type.shape[d]); in_str.push_back(st[d]); }
+    DeviceTensor y = c.allocate(t);
+    check(mhip_strided_copy(c.stream, x.data(), y.data(), (int)perm.size(), t.shape.data(), in_str.data(), 0,
+                            dtype_bytes(t.dtype)), op);
+    return y;
+}
+
+std::vector<DeviceTensor> execute(Executable& exe, const std::vector<DeviceTensor>& inputs, double* encode_s,
+                                  double* gpu_s) {
+    Client& c = *exe.client;
+    if (c.device < 0) throw NoDevice("no HIP device: cannot execute");
+    const Function& fn = exe.fn;
+    if (inputs.size() != fn.arg_types.size())
+        throw InputMismatch("Expected " + std::to_string(fn.arg_types.size()) + " inputs, got " + std::to_string(inputs.size()));
+    for (size_t i = 0; i < inputs.size(); i++)
+        if (!(inputs[i].type == fn.arg_types[i]))
+            throw InputMismatch("Input " + std::to_string(i) + " has the wrong shape or element type");
+    const auto t0 = std::chrono::steady_clock::now();
+    std::vector<DeviceTensor> val(fn.num_values);
+    for (size_t i = 0; i < inputs.size(); i++) val[fn.arg_ids[i]] = inputs[i];
+    // last use of every value, so that intermediates return to the pool early
+    std::vector<int> last(fn.num_values, -1);
+    for (size_t oi = 0; oi < fn.ops.size(); oi++) for (int v : fn.ops[oi].operands) last[v] = (int)oi;
+    for (int r : fn.returns) last[r] = (int)fn.ops.size();
+    std::map<int, const Op*> producer;
+    for (auto& op : fn.ops) producer[op.result] = &op;
+    void* s = c.stream;
+
+    for (size_t oi = 0; oi < fn.ops.size(); oi++) {
+        const Op& op = fn.ops[oi];
+        const std::string& n = op.name;
+        auto in = [&](size_t i) -> const DeviceTensor& { return val[op.operands.at(i)]; };
+        DeviceTensor out;
+        if (n == "constant") {
+            out = exe.constants[oi];
+        } else if (n == "reshape") {
+            out = in(0);
+            out.type = op.out;
+        } else {
+            out = c.allocate(op.out);
+            const int dt = op.out.dtype;
+            const int64_t cnt = op.out.numel();
+            if (kUnary.count(n)) {
+                check(mhip_unary(s, kUnary.at(n), in(0).data(), out.data(), cnt, dt), op);
+            } else if (kBinary.count(n)) {
+                check(mhip_binary(s, kBinary.at(n), in(0).data(), in(1).data(), out.data(), cnt, dt), op);
+            } else if (n == "convert") {
+                if (in(0).type.dtype == dt) check(mhip_copy(s, in(0).data(), out.data(), (int64_t)op.out.bytes()), op);
+                else check(mhip_convert(s, in(0).data(), out.data(), cnt, in(0).type.dtype, dt), op);
+            } else if (n == "transpose") {
+                const auto st = dense_strides(in(0).type.shape);
+                std::vector<int64_t> is;
+                for (auto d : op.dims) is.push_back(st[d]);
+                check(mhip_strided_copy(s, in(0).data(), out.data(), (int)op.dims.size(), op.out.shape.data(), is.data(), 0,
+                                        dtype_bytes(dt)), op);
+            } else if (n == "broadcast_in_dim") {
+                const auto st = dense_strides(in(0).type.shape);
+                std::vector<int64_t> is(op.out.shape.size(), 0);
+                for (size_t d = 0; d < op.dims.size(); d++)
+                    is[op.dims[d]] = in(0).type.shape[d] == 1 ? 0 : st[d];
+                check(mhip_strided_copy(s, in(0).data(), out.data(), (int)op.out.shape.size(), op.out.shape.data(), is.data(),
+                                        0, dtype_bytes(dt)), op);
+            } else if (n == "slice") {
+                const auto st = dense_strides(in(0).type.shape);
+                std::vector<int64_t> is;
+                int64_t off = 0;
+                for (size_t d = 0; d < st.size(); d++) { is.push_back(st[d] * op.strides[d]); off += st[d] * op.starts[d]; }
+                check(mhip_strided_copy(s, in(0).data(), out.data(), (int)st.size(), op.out.shape.data(), is.data(), off,
+                                        dtype_bytes(dt)), op);
+            } else if (n == "reduce") {
+                const double init = scalar_constant(*producer.at(op.operands.at(1)));
+                int64_t outer, len, inner;
+                DeviceTensor x = in(0);
+                if (!reduce_block(x.type.shape, op.dims, outer, len, inner)) {
+                    // move the reduced dims to the end, then reduce the trailing block
+                    std::vector<int64_t> perm, red = op.dims;
+                    std::sort(red.begin(), red.end());
+                    for (int64_t d = 0; d < (int64_t)x.type.shape.size(); d++)
+                        if (std::find(red.begin(), red.end(), d) == red.end()) perm.push_back(d);
+                    const size_t kept = perm.size();
+                    perm.insert(perm.end(), red.begin(), red.end());
+                    x = permuted_copy(c, x, perm, op);
+                    outer = len = 1;
+                    inner = 1;
+                    for (size_t d = 0; d < perm.size(); d++) (d < kept ? outer : len) *= x.type.shape[d];
+                }
+                check(mhip_reduce(s, kReduce.at(op.reducer), x.data(), out.data(), outer, len, inner, init, dt), op);
+            } else if (n == "dot" || n == "dot_general") {
+                DotPlan p = plan_dot(op, in(0).type, in(1).type);
+                DeviceTensor a = in(0), b = in(1);
+                if (p.lhs_copy) a = permuted_copy(c, a, p.lhs_perm, op);
+                if (p.rhs_copy) b = permuted_copy(c, b, p.rhs_perm, op);
+                check(mhip_gemm(s, a.data(), b.data(), nullptr, out.data(), p.M, p.N, p.K, p.B, p.M * p.K, p.K * p.N,
+                                p.M * p.N, p.trans_a, p.trans_b, MHIP_ACT_NONE, dt), op);
+            } else if (n == "iota") {
+                int64_t outer = 1, inner = 1;
+                for (int64_t d = 0; d < (int64_t)op.out.shape.size(); d++) {
+                    if (d < op.iota_dim) outer *= op.out.shape[d];
+                    else if (d > op.iota_dim) inner *= op.out.shape[d];
+                }
+                check(mhip_iota(s, out.data(), outer, op.out.shape[op.iota_dim], inner, dt), op);
+            } else if (n == "compare") {
+                check(mhip_compare(s, kCompare.at(op.direction), in(0).data(), in(1).data(), out.data(), cnt, in(0).type.dtype), op);
+            } else if (n == "select") {
+                check(mhip_select(s, in(0).data(), in(1).data(), in(2).data(), out.data(), cnt, dtype_bytes(dt),
+                                  in(0).type.numel() == 1 && cnt != 1), op);
+            } else if (n == "gather") {
+                check(mhip_gather_rows(s, in(0).data(), in(1).data(), out.data(), in(1).type.numel(), in(0).type.shape[0],
+                                       in(0).type.shape[1], in(0).type.dtype, in(1).type.dtype), op);
+            } else if (n == "custom_call") {
+                const Config cfg = parse_config(op.backend_config);
+                const TensorType& xt = in(0).type;
+                const int64_t cols = xt.shape.empty() ? 1 : xt.shape.back();
+                const int64_t rows = cols ? xt.numel() / cols : 0;
+                if (op.target == "fused_softmax") {
+                    int64_t axis = cfg.get_int("axis", -1);
+                    if (axis < 0) axis += (int64_t)xt.shape.size();
+                    if (axis < 0 || axis >= (int64_t)xt.shape.size()) throw ExecError(where(op) + "softmax axis out of range");
+                    int64_t outer = 1, inner = 1;
+                    outer = inner = 1;
+                    for (int64_t d = 0; d < axis; d++) outer *= xt.shape[d];
+                    for (int64_t d = axis + 1; d < (int64_t)xt.shape.size(); d++) inner *= xt.shape[d];
+                    check(mhip_softmax_strided(s, in(0).data(), out.data(), outer, xt.shape[axis], inner, dt), op);
+                } else if (op.target == "fused_gelu") {
+                    check(mhip_bias_gelu(s, in(0).data(), nullptr, out.data(), rows, cols, dt), op);
+                } else if (op.target == "fused_layer_norm" || op.target == "fused_rms_norm") {
+                    const auto axes = cfg.get_int_array("axes", {-1});
+                    if (axes.size() != 1 || (axes[0] != -1 && axes[0] != (int64_t)xt.shape.size() - 1))
+                        throw ExecError(where(op) + "only normalisation over the last axis is supported");
+                    const float eps = (float)cfg.get_float("eps", 1e-5);
+                    if (in(1).type.numel() != cols || in(1).type.dtype != dt) throw ExecError(where(op) + "gamma must be [cols] of the input type");
+                    if (op.target == "fused_layer_norm") {
+                        if (in(2).type.numel() != cols || in(2).type.dtype != dt) throw ExecError(where(op) + "beta must be [cols] of the input type");
+                        check(mhip_layer_norm(s, in(0).data(), in(1).data(), in(2).data(), out.data(), rows, cols, eps, dt), op);
+                    } else {
+                        check(mhip_rms_norm(s, in(0).data(), in(1).data(), out.data(), rows, cols, eps, dt), op);
+                    }
+                } else if (op.target == "fused_matmul_bias_activation") {
+                    const bool ta = cfg.get_bool("trans_a", false), tb = cfg.get_bool("trans_b", false);
+                    const TensorType& wt = in(1).type;
+                    if (wt.shape.size() != 2 || xt.shape.size() < 2 || (ta && xt.shape.size() != 2))
+                        throw ExecError(where(op) + "expected x [.., M, K] and w [K, N]");
+                    const int64_t K = ta ? xt.shape[0] : cols, M = ta ? xt.shape[1] : rows;
+                    const int64_t Kb = tb ? wt.shape[1] : wt.shape[0], N = tb ? wt.shape[0] : wt.shape[1];
+                    if (K != Kb || op.out.numel() != M * N) throw ExecError(where(op) + "operand shapes do not contract");
+                    const void* bias = op.operands.size() > 2 ? in(2).data() : nullptr;
+                    if (bias && (in(2).type.numel() != N || in(2).type.dtype != dt)) throw ExecError(where(op) + "bias must be [N] of the input type");
+                    check(mhip_gemm(s, in(0).data(), in(1).data(), bias, out.data(), M, N, K, 1, 0, 0, 0, ta, tb,
+                                    kActivation.at(cfg.get_string("activation", "none")), dt), op);
+                } else {   // fused_scaled_dot_product_attention
+                    const TensorType& kt = in(1).type;
+                    if (xt.shape.size() < 2 || kt.shape.size() != xt.shape.size() || !(in(2).type == kt) || kt.dtype != dt)
+                        throw ExecError(where(op) + "expected q [.., Sq, D] and k, v [.., Skv, D]");
+                    const size_t r = xt.shape.size();
+                    const int64_t D = xt.shape[r - 1], Sq = xt.shape[r - 2], Skv = kt.shape[r - 2];
+                    const int64_t H = r >= 3 ? xt.shape[r - 3] : 1;
+                    int64_t B = 1;
+                    for (size_t d = 0; d + 3 < r; d++) B *= xt.shape[d];
+                    const float scale = (float)cfg.get_float("scale", 1.0);
+                    const bool has_mask = cfg.get_bool("has_mask", false) && op.operands.size() > 3;
+                    const void* mask = nullptr;
+                    int64_t msb = 0, msh = 0;
+                    if (has_mask) {
+                        const TensorType& mt = in(3).type;
+                        const size_t mr = mt.shape.size();
+                        if (mr < 2 || mt.shape[mr - 1] != Skv || mt.shape[mr - 2] != Sq || mt.dtype != dt)
+                            throw ExecError(where(op) + "mask must end in [Sq, Skv] and have the input type");
+                        const int64_t mh = mr >= 3 ? mt.shape[mr - 3] : 1;
+                        int64_t mb = 1;
+                        for (size_t d = 0; d + 3 < mr; d++) mb *= mt.shape[d];
+                        if ((mh != 1 && mh != H) || (mb != 1 && mb != B)) throw ExecError(where(op) + "mask does not broadcast to [B, H, Sq, Skv]");
+                        msh = mh == H && H != 1 ? Sq * Skv : 0;
+                        msb = mb == B && B != 1 ? mh * Sq * Skv : 0;
+                        mask = in(3).data();
+                    }
+                    check(mhip_flash_attention(s, in(0).data(), in(1).data(), in(2).data(), mask, out.data(), B, H, Sq, Skv, D,
+                                               scale, cfg.get_bool("is_causal", false), msb, msh, dt), op);
+                }
+            }
+        }
+        val[op.result] = out;
+        for (int v : op.operands)
+            if (last[v] == (int)oi) val[v] = DeviceTensor();
+    }
+    const auto t1 = std::chrono::steady_clock::now();
+    if (hipStreamSynchronize(c.stream) != hipSuccess) {
+        const hipError_t e = hipGetLastError();
+        throw ExecError(std::string("execution failed: ") + hipGetErrorString(e));
+    }
+    const auto t2 = std::chrono::steady_clock::now();
+    if (encode_s) *encode_s = std::chrono::duration<double>(t1 - t0).count();
+    if (gpu_s) *gpu_s = std::chrono::duration<double>(t2 - t0).count();
+    std::vector<DeviceTensor> outs;
+    std::map<int, size_t> first_out;
+    for (size_t i = 0; i < fn.returns.size(); i++) {
+        const int r = fn.returns[i];
+        DeviceTensor o = first_out.count(r) ? outs[first_out[r]] : std::move(val[r]);
+        if (!first_out.count(r)) { val[r] = DeviceTensor(); first_out[r] = i; }
+        if (!o.mem) throw ExecError("a returned value was never produced");
+        // an output must own its storage: inputs, constants, aliases and repeated
+        // results are copied out
+        const bool shared = o.mem.use_count() > 1;
+        if (shared) {
+            DeviceTensor cpy = c.allocate(o.type);
+            if (mhip_copy(c.stream, o.data(), cpy.data(), (int64_t)o.type.bytes()) != MHIP_OK) throw ExecError(mhip_last_error());
+            (void)hipStreamSynchronize(c.stream);
+            o = cpy;
+        }
+        outs.push_back(o);
+    }
+    return outs;
+}
+
+}  // namespace mhlo

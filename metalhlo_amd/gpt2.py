@@ -50,33 +50,56 @@ def init_params(cfg: GPT2Config, seed: int = 5) -> Dict:
 class GPT2:
     def __init__(self, cfg: GPT2Config, params: Dict, compute_dtype=torch.bfloat16, device="cuda"):
         self.cfg, self.dtype = cfg, compute_dtype
-        dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)
-        self.p32 = dict(wte=dev(params["wte"]), wpe=dev(params["wpe"]),
-                        lnf_g=dev(params["lnf_g"]), lnf_b=dev(params["lnf_b"]),
-                        layers=[{k: dev(v) for k, v in l.items()} for l in params["layers"]])
+        # All parameters live in ONE fp32 device buffer (each tensor starts on a
+        # 16-byte boundary), so the per-step fp32 -> compute-type conversion is a
+        # single streaming launch; the named entries are views into the buffers.
+        flat, self._slots = [], []
 
-    def _cast(self, t: torch.Tensor) -> torch.Tensor:
-        return t if t.dtype == self.dtype else kernels.convert(t, self.dtype)
+        def put(path, a):
+            a = np.ascontiguousarray(a, dtype=np.float32)
+            off = sum(x.size for x in flat)
+            pad = (-a.size) % 8
+            flat.append(np.concatenate([a.reshape(-1), np.zeros(pad, np.float32)]))
+            self._slots.append((path, off, a.shape))
+
+        for name in ("wte", "wpe", "lnf_g", "lnf_b"):
+            put((name,), params[name])
+        for i, l in enumerate(params["layers"]):
+            for k, v in l.items():
+                put(("layers", i, k), v)
+        self.flat32 = torch.from_numpy(np.concatenate(flat)).to(device)
+        self.p32 = self._views(self.flat32)
+
+    def _views(self, flat: torch.Tensor) -> Dict:
+        out: Dict = {"layers": [dict() for _ in range(self.cfg.n_layer)]}
+        for path, off, shape in self._slots:
+            v = flat[off:off + int(np.prod(shape))].view(*shape)
+            if path[0] == "layers":
+                out["layers"][path[1]][path[2]] = v
+            else:
+                out[path[0]] = v
+        return out
 
     def forward(self, ids: torch.Tensor) -> torch.Tensor:
         """ids int32 [B,S] on the device -> logits [B,S,vocab] in the compute type."""
-        cfg, c = self.cfg, self._cast
+        cfg = self.cfg
         B, S = ids.shape
         d, H = cfg.d_model, cfg.n_head
-        p = self.p32
-        x = kernels.embed_tokens(ids, p["wte"], p["wpe"], self.dtype).reshape(B * S, d)
+        # the graph's `convert` ops: fp32 parameters -> compute type, every step
+        p = self.p32 if self.dtype == torch.float32 else self._views(kernels.convert(self.flat32, self.dtype))
+        x = kernels.embed_tokens(ids, self.p32["wte"], self.p32["wpe"], self.dtype).reshape(B * S, d)
         for l in p["layers"]:
-            h = kernels.layer_norm(x, c(l["ln1_g"]), c(l["ln1_b"]), eps=1e-5)
-            qkv = kernels.matmul(h, c(l["w_qkv"]), bias=c(l["b_qkv"]))
+            h = kernels.layer_norm(x, l["ln1_g"], l["ln1_b"], eps=1e-5)
+            qkv = kernels.matmul(h, l["w_qkv"], bias=l["b_qkv"])
             q, k, v = kernels.split_qkv_heads(qkv.reshape(B, S, 3 * d), H)
             a = kernels.flash_attention(q, k, v, is_causal=True)
             a = kernels.transpose_0213(a).reshape(B * S, d)
-            x = kernels.add(x, kernels.matmul(a, c(l["w_o"]), bias=c(l["b_o"])))
-            h = kernels.layer_norm(x, c(l["ln2_g"]), c(l["ln2_b"]), eps=1e-5)
-            u = kernels.matmul(h, c(l["w_fc"]), bias=c(l["b_fc"]), activation="gelu")
-            x = kernels.add(x, kernels.matmul(u, c(l["w_proj"]), bias=c(l["b_proj"])))
-        x = kernels.layer_norm(x, c(p["lnf_g"]), c(p["lnf_b"]), eps=1e-5)
-        logits = kernels.matmul(x, c(p["wte"]), trans_b=True)       # tied head: x . wte^T
+            x = kernels.add(x, kernels.matmul(a, l["w_o"], bias=l["b_o"]))
+            h = kernels.layer_norm(x, l["ln2_g"], l["ln2_b"], eps=1e-5)
+            u = kernels.matmul(h, l["w_fc"], bias=l["b_fc"], activation="gelu")
+            x = kernels.add(x, kernels.matmul(u, l["w_proj"], bias=l["b_proj"]))
+        x = kernels.layer_norm(x, p["lnf_g"], p["lnf_b"], eps=1e-5)
+        logits = kernels.matmul(x, p["wte"], trans_b=True)       # tied head: x . wte^T
         return logits.reshape(B, S, cfg.vocab)
 
     @staticmethod
