@@ -216,6 +216,8 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_mfma_kernel(GemmArgs g) {
     // every store instruction writes whole contiguous row segments.
     constexpr int kRowPad = WTN * 2 + 16;
     char* stage = smem + wave * (WTM * kRowPad);
+    dispatch_act(g.act, [&](auto act_tag) {
+    constexpr int ACT = decltype(act_tag)::value;
 #pragma unroll
     for (int j = 0; j < TN; j++) {
 #pragma unroll
@@ -240,7 +242,7 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_mfma_kernel(GemmArgs g) {
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
                     float v = acc[i][j][4 * q + e] + bv[e];
-                    if (g.act != MHIP_ACT_NONE) v = apply_act(v, g.act);
+                    v = apply_act_c<ACT>(v);
                     o.v[e] = Elem<T>::from_f32(v);
                 }
                 *reinterpret_cast<u32x2*>(stage + (i * 32 + lrow) * kRowPad + nl * 2) =
@@ -248,6 +250,7 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_mfma_kernel(GemmArgs g) {
             }
         }
     }
+    });
     // each wave only re-reads what it wrote itself
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -348,10 +351,17 @@ static int launch_mfma(hipStream_t s, GemmArgs g, int64_t batch) {
     return check_launch("gemm_mfma");
 }
 
+// gemm256.hip: 4-wave 256x256 kernel with a hand-scheduled main loop.
+bool gemm256_eligible(const GemmArgs& g, int64_t batch, int dtype);
+int launch_gemm256(hipStream_t s, const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype);
+
 template <typename T, bool TA, bool TB>
 static int pick_tile(hipStream_t s, const GemmArgs& g, int64_t batch) {
     const int64_t big = (int64_t)((g.M + 255) / 256) * ((g.N + 255) / 256) * batch;
     const int force = tune_int("MHIP_GEMM_TILE", 0);
+    constexpr int dt = std::is_same<T, bf16_t>::value ? MHIP_BF16 : MHIP_F16;
+    if ((force == 0 || force == 2560) && gemm256_eligible(g, batch, dt))
+        return launch_gemm256(s, g, batch, TA, TB, dt);
     if (force == 256 || (force != 128 && big >= 192)) return launch_mfma<T, 256, 256, 2, 4, TA, TB>(s, g, batch);
     return launch_mfma<T, 128, 128, 2, 2, TA, TB>(s, g, batch);
 }

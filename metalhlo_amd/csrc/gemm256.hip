@@ -1,0 +1,244 @@
+// Large-problem GEMM for gfx950: 256x256 C tile, K step 64, four waves (one per
+// SIMD), each wave a 128x128 sub-tile = 4x4 v_mfma_f32_32x32x16 accumulators that
+// fill the AGPR file.  The main loop is generated, hand-scheduled inline assembly
+// (gen_gemm256_loop.py -> gemm256_loop.inc: schedule and register map are
+// documented there); this file computes the per-thread addresses it consumes and
+// holds the epilogue.
+//
+// LDS (128 KB in the loop): [A buf0][A buf1][B buf0][B buf1], 32 KB each.  An
+// operand whose k axis is contiguous in memory is stored [256 rows][64 k] with the
+// 16-byte chunks of a row XOR-swizzled by (row >> 1) & 7 and read with
+// ds_read_b128; an operand whose k axis is the slow one is stored as it lies,
+// [64 k][256 mn], chunks swizzled by (k & 3) << 2, and transposed on the way out
+// with ds_read_b64_tr_b16.  Global loads are bounds-checked buffer loads: rows or
+// columns beyond the matrix read as zero, so ragged M and N need no special path.
+#include <mutex>
+#include <type_traits>
+#include <utility>
+
+#include "gemm_common.h"
+
+namespace mhip {
+
+#include "gemm256_loop.inc"
+
+namespace {
+
+constexpr uint32_t kTileBytes = 32 * 1024;
+
+template <typename F, int... I>
+__device__ inline void static_for_impl(F& f, std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ inline void static_for(F&& f) {
+    static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+// ---- operand with k contiguous in memory --------------------------------------
+// thread -> 16-byte chunk c = tid & 7 (8 k), row r = tid >> 3 (+ 32 per pass), 8 passes.
+struct KMajor {
+    __device__ static uint32_t goff(int tid, int row0, int ld, int cols_total) {
+        (void)cols_total;
+        return (uint32_t)((((int64_t)row0 + (tid >> 3)) * ld + (tid & 7) * 8) * 2);
+    }
+    __device__ static uint32_t pass_stride(int ld) { return (uint32_t)(32 * ld * 2); }
+    __device__ static uint32_t tile_stride(int ld) { (void)ld; return 128u; }
+    __device__ static uint32_t woff(int tid) {
+        const int r = tid >> 3, c = tid & 7;
+        return (uint32_t)(r * 128 + ((c ^ ((r >> 1) & 7)) << 4));   // + 4096 per pass
+    }
+    // read addresses: element s = k-step s of row block 0; + 4096 per row block of 32
+    __device__ static u32x4 raddr(int lane, int row_block0, uint32_t base) {
+        const int lrow = lane & 31, lhalf = lane >> 5;
+        const uint32_t b = base + (uint32_t)((row_block0 + lrow) * 128 + ((lhalf ^ ((lrow >> 1) & 7)) << 4));
+        u32x4 r;
+        r.x = b; r.y = b ^ 32u; r.z = b ^ 64u; r.w = b ^ 96u;
+        return r;
+    }
+};
+
+// ---- operand with k as the slow memory axis -------------------------------------
+// thread -> chunk c = tid & 31 (8 mn), k row = tid >> 5 (+ 8 per pass), 8 passes.
+struct MnMajor {
+    __device__ static uint32_t goff(int tid, int col0, int ld, int cols_total) {
+        const int col = col0 + (tid & 31) * 8;
+        return col < cols_total ? (uint32_t)((((int64_t)(tid >> 5)) * ld + col) * 2) : kOob;
+    }
+    __device__ static uint32_t pass_stride(int ld) { return (uint32_t)(8 * ld * 2); }
+    __device__ static uint32_t tile_stride(int ld) { return (uint32_t)(64 * ld * 2); }
+    __device__ static uint32_t woff(int tid) {
+        const int k = tid >> 5, c = tid & 31;
+        return (uint32_t)(k * 512 + ((c ^ ((k & 3) << 2)) << 4));   // + 4096 per pass
+    }
+    // read addresses: element j = mn block j at k-step 0; + 8192 per k-step, + 2048 for
+    // the upper four k of a fragment
+    __device__ static u32x4 raddr(int lane, int mn_block0, uint32_t base) {
+        const int i = lane & 15, gq = lane >> 4;
+        const int xr = (i >> 2) & 3;
+        const int mn = mn_block0 + 16 * (gq & 1) + 4 * (i & 3);
+        const uint32_t b = base + (uint32_t)((8 * (gq >> 1) + (i >> 2)) * 512 + ((mn >> 3) << 4) + (mn & 7) * 2);
+        u32x4 r;
+        r.x = b + (uint32_t)((0 ^ xr) << 6); r.y = b + (uint32_t)((1 ^ xr) << 6);
+        r.z = b + (uint32_t)((2 ^ xr) << 6); r.w = b + (uint32_t)((3 ^ xr) << 6);
+        return r;
+    }
+};
+
+template <typename T, bool TA, bool TB>
+__device__ inline void main_loop(f32x16 (&acc)[16], u32x4 ra, u32x4 rb, u32x4& misc,
+                                 __amdgpu_buffer_rsrc_t rsa, __amdgpu_buffer_rsrc_t rsb, uint32_t pa,
+                                 uint32_t pb, uint32_t ta, uint32_t tb, uint32_t kt) {
+    constexpr bool bf = std::is_same<T, bf16_t>::value;
+    if constexpr (bf && !TA && !TB) gemm256_loop_nn_bf16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, kt);
+    if constexpr (bf && !TA && TB) gemm256_loop_nt_bf16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, kt);
+    if constexpr (bf && TA && !TB) gemm256_loop_tn_bf16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, kt);
+    if constexpr (bf && TA && TB) gemm256_loop_tt_bf16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, kt);
+    if constexpr (!bf && !TA && !TB) gemm256_loop_nn_f16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, kt);
+    if constexpr (!bf && !TA && TB) gemm256_loop_nt_f16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, kt);
+    if constexpr (!bf && TA && !TB) gemm256_loop_tn_f16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, kt);
+    if constexpr (!bf && TA && TB) gemm256_loop_tt_f16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, kt);
+}
+
+template <typename T, bool TA, bool TB>
+__global__ __launch_bounds__(256) void gemm256_kernel(GemmArgs g) {
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    using LA = typename std::conditional<TA, MnMajor, KMajor>::type;
+    using LB = typename std::conditional<TB, KMajor, MnMajor>::type;
+
+    int tm, tn;
+    tile_of(blockIdx.x, gridDim.x, g.tiles_m, g.tiles_n, tm, tn);
+    const int m0 = tm * 256, n0 = tn * 256;
+    const int64_t batch = blockIdx.y;
+    const char* a = reinterpret_cast<const char*>(static_cast<const T*>(g.a) + batch * g.sa);
+    const char* b = reinterpret_cast<const char*>(static_cast<const T*>(g.b) + batch * g.sb);
+    T* c = static_cast<T*>(g.c) + batch * g.sc;
+    const uint32_t a_bytes = (uint32_t)((int64_t)(TA ? g.K : g.M) * g.lda * 2);
+    const uint32_t b_bytes = (uint32_t)((int64_t)(TB ? g.N : g.K) * g.ldb * 2);
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int lrow = lane & 31, lhalf = lane >> 5;
+    // LDS byte address of the dynamic segment
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
+
+    const u32x4 ra = LA::raddr(lane, wm * 128, lds0);
+    const u32x4 rb = LB::raddr(lane, wn * 128, lds0 + 2 * kTileBytes);
+    u32x4 misc;
+    misc.x = lds0 + LA::woff(tid);
+    misc.y = lds0 + 2 * kTileBytes + LB::woff(tid);
+    misc.z = LA::goff(tid, m0, g.lda, g.M);
+    misc.w = LB::goff(tid, n0, g.ldb, g.N);
+    const __amdgpu_buffer_rsrc_t rsa =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(a), 0, a_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsb =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(b), 0, b_bytes, 0x00020000);
+
+    f32x16 acc[16];
+    main_loop<T, TA, TB>(acc, ra, rb, misc, rsa, rsb, LA::pass_stride(g.lda), LB::pass_stride(g.ldb),
+                         LA::tile_stride(g.lda), LB::tile_stride(g.ldb), (uint32_t)(g.K / 64));
+
+    // Waves still read (unused) prefetched fragments of a tile past the end; the
+    // staging area below overlaps those buffers, which is harmless, but every wave
+    // must have left the loop's last real reads behind: the loop's final barrier
+    // guarantees that.
+    //
+    // Accumulator tiles are transposed: lane = row m (lrow), register group
+    // q = r / 4 holds columns 8q + 4*lhalf + r % 4 of the 32-column block.
+    const T* bias = static_cast<const T*>(g.bias);
+    constexpr int kRowPad = 128 * 2 + 16;
+    char* stage = smem + wave * (128 * kRowPad);
+    dispatch_act(g.act, [&](auto act_tag) {
+    constexpr int ACT = decltype(act_tag)::value;
+    static_for<16>([&](auto jq_tag) {
+        constexpr int j = decltype(jq_tag)::value >> 2, q = decltype(jq_tag)::value & 3;
+        const int nl = j * 32 + 8 * q + 4 * lhalf;
+        const int n = n0 + wn * 128 + nl;
+        float bv[4] = {0.f, 0.f, 0.f, 0.f};
+        if (bias && n < g.N) {
+            const Pack4<T> t = __builtin_bit_cast(Pack4<T>, *reinterpret_cast<const u32x2*>(bias + n));
+#pragma unroll
+            for (int e = 0; e < 4; e++) bv[e] = Elem<T>::to_f32(t.v[e]);
+        }
+        static_for<4>([&](auto i_tag) {
+            constexpr int i = decltype(i_tag)::value;
+            Pack4<T> o;
+            static_for<4>([&](auto e_tag) {
+                constexpr int e = decltype(e_tag)::value;
+                float v = acc[i * 4 + j][4 * q + e] + bv[e];
+                v = apply_act_c<ACT>(v);
+                o.v[e] = Elem<T>::from_f32(v);
+            });
+            *reinterpret_cast<u32x2*>(stage + (i * 32 + lrow) * kRowPad + nl * 2) =
+                __builtin_bit_cast(u32x2, o);
+        });
+        // one register group at a time: do not let 256 accumulator reads pile up
+        __builtin_amdgcn_sched_barrier(0);
+    });
+    });
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // a wave re-reads only its own rows
+    const int cc = lane & 15, rr = lane >> 4;
+#pragma unroll 4
+    for (int p = 0; p < 32; p++) {
+        const int ml = p * 4 + rr;
+        const int m = m0 + wm * 128 + ml;
+        const int n = n0 + wn * 128 + cc * 8;
+        if (m < g.M && n < g.N) {
+            const u32x4 w = *reinterpret_cast<const u32x4*>(stage + ml * kRowPad + cc * 16);
+            *reinterpret_cast<u32x4*>(c + (int64_t)m * g.N + n) = w;
+        }
+    }
+}
+
+template <typename T, bool TA, bool TB>
+int launch256(hipStream_t s, GemmArgs g, int64_t batch) {
+    constexpr int kSmem = 4 * 128 * (128 * 2 + 16);   // epilogue staging (136 KB) >= 4 tiles (128 KB)
+    auto kern = gemm256_kernel<T, TA, TB>;
+    static std::once_flag once;
+    static hipError_t attr_err = hipSuccess;
+    std::call_once(once, [&] {
+        attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kSmem);
+    });
+    if (attr_err != hipSuccess)
+        return fail(MHIP_ERR_LAUNCH, "gemm256: cannot reserve %d bytes of LDS: %s", kSmem,
+                    hipGetErrorString(attr_err));
+    g.tiles_m = (g.M + 255) / 256;
+    g.tiles_n = (g.N + 255) / 256;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(g.tiles_m * g.tiles_n), (unsigned)batch), dim3(256),
+                       kSmem, s, g);
+    return check_launch("gemm256");
+}
+
+template <typename T>
+int layout256(hipStream_t s, const GemmArgs& g, int64_t batch, int ta, int tb) {
+    if (!ta && !tb) return launch256<T, false, false>(s, g, batch);
+    if (!ta && tb) return launch256<T, false, true>(s, g, batch);
+    if (ta && !tb) return launch256<T, true, false>(s, g, batch);
+    return launch256<T, true, true>(s, g, batch);
+}
+
+}  // namespace
+
+// The kernel needs whole K tiles, 16-byte-aligned operand rows (checked by the
+// caller), an output it can store 16 bytes at a time, operands small enough for
+// 32-bit byte offsets including the prefetch overrun of three K tiles, and enough
+// 256x256 tiles to occupy the device.
+bool gemm256_eligible(const GemmArgs& g, int64_t batch, int dtype) {
+    if (dtype != MHIP_BF16 && dtype != MHIP_F16) return false;
+    if (g.K % 64 != 0 || g.K < 64) return false;
+    if (g.N % 8 != 0 || (reinterpret_cast<uintptr_t>(g.c) & 15) != 0 || g.sc % 8 != 0) return false;
+    if (g.bias && (reinterpret_cast<uintptr_t>(g.bias) & 7) != 0) return false;
+    const int64_t a_bytes = (int64_t)g.M * g.K * 2, b_bytes = (int64_t)g.N * g.K * 2;
+    if (a_bytes >= 0x70000000LL || b_bytes >= 0x70000000LL) return false;
+    const int64_t tiles = (int64_t)((g.M + 255) / 256) * ((g.N + 255) / 256) * batch;
+    return tiles >= 192 && tiles <= 0x7FFFFFFF && batch <= 65535;
+}
+
+int launch_gemm256(hipStream_t s, const GemmArgs& g, int64_t batch, int trans_a, int trans_b,
+                   int dtype) {
+    if (dtype == MHIP_BF16) return layout256<bf16_t>(s, g, batch, trans_a, trans_b);
+    return layout256<f16_t>(s, g, batch, trans_a, trans_b);
+}
+
+}  // namespace mhip

@@ -2,6 +2,8 @@
 #pragma once
 #include <math.h>
 
+#include <type_traits>
+
 #include "common.h"
 
 namespace mhip {
@@ -49,6 +51,26 @@ __device__ inline float apply_act(float v, int act) {
         case MHIP_ACT_TANH: return tanhf(v);
         case MHIP_ACT_SIGMOID: return 1.f / (1.f + expf(-v));
         default: return v;
+    }
+}
+
+// Activation known at compile time (the switch folds away), and a dispatcher that
+// turns the runtime code into such a constant ONCE per kernel: an epilogue that
+// tests the code per element unrolls into hundreds of branchy copies, far larger
+// than the instruction cache.
+template <int ACT>
+__device__ inline float apply_act_c(float v) {
+    return ACT == MHIP_ACT_NONE ? v : apply_act(v, ACT);
+}
+template <typename F>
+__device__ inline void dispatch_act(int act, F&& f) {
+    switch (act) {
+        case MHIP_ACT_RELU: f(std::integral_constant<int, MHIP_ACT_RELU>{}); break;
+        case MHIP_ACT_GELU: f(std::integral_constant<int, MHIP_ACT_GELU>{}); break;
+        case MHIP_ACT_SILU: f(std::integral_constant<int, MHIP_ACT_SILU>{}); break;
+        case MHIP_ACT_TANH: f(std::integral_constant<int, MHIP_ACT_TANH>{}); break;
+        case MHIP_ACT_SIGMOID: f(std::integral_constant<int, MHIP_ACT_SIGMOID>{}); break;
+        default: f(std::integral_constant<int, MHIP_ACT_NONE>{}); break;
     }
 }
 
