@@ -1,17 +1,21 @@
-// Large-problem GEMM for gfx950: 256x256 C tile, K step 64, four waves (one per
-// SIMD), each wave a 128x128 sub-tile = 4x4 v_mfma_f32_32x32x16 accumulators that
-// fill the AGPR file.  The main loop is generated, hand-scheduled inline assembly
+// Large-problem GEMM for gfx950: 256x256 C tile, four waves (one per SIMD), each
+// wave a 128x128 sub-tile = 4x4 v_mfma_f32_32x32x16 accumulators that fill the
+// AGPR file.  The main loop is generated, hand-scheduled inline assembly
 // (gen_gemm256_loop.py -> gemm256_loop.inc: schedule and register map are
 // documented there); this file computes the per-thread addresses it consumes and
 // holds the epilogue.
 //
-// LDS (128 KB in the loop): [A buf0][A buf1][B buf0][B buf1], 32 KB each.  An
-// operand whose k axis is contiguous in memory is stored [256 rows][64 k] with the
-// 16-byte chunks of a row XOR-swizzled by (row >> 1) & 7 and read with
+// K is consumed in stages of 32 through a ring of four 32 KB LDS buffers
+// ([A tile 16 KB][B tile 16 KB]) filled by buffer loads that write LDS directly:
+// a wave's load instruction deposits 64 x 16 bytes contiguously, so the LDS
+// layout is fixed by which 16-byte chunk of global memory each lane asks for.
+// An operand whose k axis is contiguous in memory is stored [256 rows][32 k]
+// (64-byte rows, chunk c of row r at position c ^ ((r >> 2) & 3)) and read with
 // ds_read_b128; an operand whose k axis is the slow one is stored as it lies,
-// [64 k][256 mn], chunks swizzled by (k & 3) << 2, and transposed on the way out
-// with ds_read_b64_tr_b16.  Global loads are bounds-checked buffer loads: rows or
-// columns beyond the matrix read as zero, so ragged M and N need no special path.
+// [32 k][256 mn] (chunk c of k-row k at position c ^ ((k & 3) << 2)), and
+// transposed on the way out with ds_read_b64_tr_b16.  The loads are
+// bounds-checked buffer loads: rows or columns beyond the matrix read as zero, so
+// ragged M and N need no special path.
 #include <mutex>
 #include <type_traits>
 #include <utility>
@@ -24,7 +28,7 @@ namespace mhip {
 
 namespace {
 
-constexpr uint32_t kTileBytes = 32 * 1024;
+constexpr uint32_t kStageBytes = 32 * 1024, kOperBytes = 16 * 1024, kHalfRing = 64 * 1024;
 
 template <typename F, int... I>
 __device__ inline void static_for_impl(F& f, std::integer_sequence<int, I...>) {
@@ -36,68 +40,79 @@ __device__ inline void static_for(F&& f) {
 }
 
 // ---- operand with k contiguous in memory --------------------------------------
-// thread -> 16-byte chunk c = tid & 7 (8 k), row r = tid >> 3 (+ 32 per pass), 8 passes.
+// One load instruction of wave w in pass p fills rows 64p + 16w .. +15 (64 bytes
+// each): lane -> row (lane >> 2), position (lane & 3).
 struct KMajor {
-    __device__ static uint32_t goff(int tid, int row0, int ld, int cols_total) {
+    __device__ static uint32_t goff(int lane, int wave, int row0, int ld, int cols_total) {
         (void)cols_total;
-        return (uint32_t)((((int64_t)row0 + (tid >> 3)) * ld + (tid & 7) * 8) * 2);
+#ifdef GEMM256_FULLLINE_EXP   // timing experiment only: whole 128-byte lines, wrong data
+        return (uint32_t)(((int64_t)(row0 + 8 * wave + (lane >> 3)) * ld + (lane & 7) * 8) * 2);
+#endif
+        const int row = row0 + 16 * wave + (lane >> 2);
+        const int c = (lane & 3) ^ ((lane >> 4) & 3);
+        return (uint32_t)(((int64_t)row * ld + c * 8) * 2);
     }
+#ifdef GEMM256_FULLLINE_EXP
     __device__ static uint32_t pass_stride(int ld) { return (uint32_t)(32 * ld * 2); }
-    __device__ static uint32_t tile_stride(int ld) { (void)ld; return 128u; }
-    __device__ static uint32_t woff(int tid) {
-        const int r = tid >> 3, c = tid & 7;
-        return (uint32_t)(r * 128 + ((c ^ ((r >> 1) & 7)) << 4));   // + 4096 per pass
-    }
-    // read addresses: element s = k-step s of row block 0; + 4096 per row block of 32
-    __device__ static u32x4 raddr(int lane, int row_block0, uint32_t base) {
+    __device__ static uint32_t stage_stride(int ld) { (void)ld; return 128u; }
+#else
+    __device__ static uint32_t pass_stride(int ld) { return (uint32_t)(64 * ld * 2); }
+    __device__ static uint32_t stage_stride(int ld) { (void)ld; return 64u; }
+#endif
+    // read addresses: element 2h + s = k-step s of row block 0 in ring half h;
+    // + 2048 per row block of 32, + 32768 for the odd buffer of the half
+    __device__ static u32x8 raddr(int lane, int row_block0, uint32_t base) {
         const int lrow = lane & 31, lhalf = lane >> 5;
-        const uint32_t b = base + (uint32_t)((row_block0 + lrow) * 128 + ((lhalf ^ ((lrow >> 1) & 7)) << 4));
-        u32x4 r;
-        r.x = b; r.y = b ^ 32u; r.z = b ^ 64u; r.w = b ^ 96u;
+        const uint32_t b = base + (uint32_t)((row_block0 + lrow) * 64 + ((lhalf ^ ((lrow >> 2) & 3)) << 4));
+        u32x8 r;
+        r[0] = b; r[1] = b ^ 32u; r[2] = b + kHalfRing; r[3] = (b ^ 32u) + kHalfRing;
+        r[4] = r[5] = r[6] = r[7] = 0;
         return r;
     }
 };
 
 // ---- operand with k as the slow memory axis -------------------------------------
-// thread -> chunk c = tid & 31 (8 mn), k row = tid >> 5 (+ 8 per pass), 8 passes.
+// One load instruction of wave w in pass p fills k rows 8p + 2w, 8p + 2w + 1
+// (512 bytes each): lane -> k row (lane >> 5), position (lane & 31).
 struct MnMajor {
-    __device__ static uint32_t goff(int tid, int col0, int ld, int cols_total) {
-        const int col = col0 + (tid & 31) * 8;
-        return col < cols_total ? (uint32_t)((((int64_t)(tid >> 5)) * ld + col) * 2) : kOob;
+    __device__ static uint32_t goff(int lane, int wave, int col0, int ld, int cols_total) {
+        const int k = 2 * wave + (lane >> 5);
+        const int c = (lane & 31) ^ ((k & 3) << 2);
+        const int col = col0 + c * 8;
+        return col < cols_total ? (uint32_t)(((int64_t)k * ld + col) * 2) : kOob;
     }
     __device__ static uint32_t pass_stride(int ld) { return (uint32_t)(8 * ld * 2); }
-    __device__ static uint32_t tile_stride(int ld) { return (uint32_t)(64 * ld * 2); }
-    __device__ static uint32_t woff(int tid) {
-        const int k = tid >> 5, c = tid & 31;
-        return (uint32_t)(k * 512 + ((c ^ ((k & 3) << 2)) << 4));   // + 4096 per pass
-    }
-    // read addresses: element j = mn block j at k-step 0; + 8192 per k-step, + 2048 for
-    // the upper four k of a fragment
-    __device__ static u32x4 raddr(int lane, int mn_block0, uint32_t base) {
+    __device__ static uint32_t stage_stride(int ld) { return (uint32_t)(32 * ld * 2); }
+    // read addresses: element 4h + j = mn block j at k-step 0 in ring half h; + 8192 per
+    // k-step, + 2048 for the upper four k of a fragment, + 32768 for the odd buffer
+    __device__ static u32x8 raddr(int lane, int mn_block0, uint32_t base) {
         const int i = lane & 15, gq = lane >> 4;
         const int xr = (i >> 2) & 3;
         const int mn = mn_block0 + 16 * (gq & 1) + 4 * (i & 3);
         const uint32_t b = base + (uint32_t)((8 * (gq >> 1) + (i >> 2)) * 512 + ((mn >> 3) << 4) + (mn & 7) * 2);
-        u32x4 r;
-        r.x = b + (uint32_t)((0 ^ xr) << 6); r.y = b + (uint32_t)((1 ^ xr) << 6);
-        r.z = b + (uint32_t)((2 ^ xr) << 6); r.w = b + (uint32_t)((3 ^ xr) << 6);
+        u32x8 r;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            r[j] = b + (uint32_t)((j ^ xr) << 6);
+            r[4 + j] = r[j] + kHalfRing;
+        }
         return r;
     }
 };
 
 template <typename T, bool TA, bool TB>
-__device__ inline void main_loop(f32x16 (&acc)[16], u32x4 ra, u32x4 rb, u32x4& misc,
+__device__ inline void main_loop(f32x16 (&acc)[16], u32x8 ra, u32x8 rb, u32x2& misc,
                                  __amdgpu_buffer_rsrc_t rsa, __amdgpu_buffer_rsrc_t rsb, uint32_t pa,
-                                 uint32_t pb, uint32_t ta, uint32_t tb, uint32_t kt) {
+                                 uint32_t pb, uint32_t ta, uint32_t tb, uint32_t m0b, uint32_t kt, uint32_t wv) {
     constexpr bool bf = std::is_same<T, bf16_t>::value;
-    if constexpr (bf && !TA && !TB) gemm256_loop_nn_bf16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, kt);
-    if constexpr (bf && !TA && TB) gemm256_loop_nt_bf16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, kt);
-    if constexpr (bf && TA && !TB) gemm256_loop_tn_bf16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, kt);
-    if constexpr (bf && TA && TB) gemm256_loop_tt_bf16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, kt);
-    if constexpr (!bf && !TA && !TB) gemm256_loop_nn_f16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, kt);
-    if constexpr (!bf && !TA && TB) gemm256_loop_nt_f16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, kt);
-    if constexpr (!bf && TA && !TB) gemm256_loop_tn_f16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, kt);
-    if constexpr (!bf && TA && TB) gemm256_loop_tt_f16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, kt);
+    if constexpr (bf && !TA && !TB) gemm256_loop_nn_bf16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt, wv);
+    if constexpr (bf && !TA && TB) gemm256_loop_nt_bf16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt, wv);
+    if constexpr (bf && TA && !TB) gemm256_loop_tn_bf16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt, wv);
+    if constexpr (bf && TA && TB) gemm256_loop_tt_bf16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt, wv);
+    if constexpr (!bf && !TA && !TB) gemm256_loop_nn_f16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt, wv);
+    if constexpr (!bf && !TA && TB) gemm256_loop_nt_f16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt, wv);
+    if constexpr (!bf && TA && !TB) gemm256_loop_tn_f16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt, wv);
+    if constexpr (!bf && TA && TB) gemm256_loop_tt_f16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt, wv);
 }
 
 template <typename T, bool TA, bool TB>
@@ -122,13 +137,13 @@ __global__ __launch_bounds__(256) void gemm256_kernel(GemmArgs g) {
     // LDS byte address of the dynamic segment
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
 
-    const u32x4 ra = LA::raddr(lane, wm * 128, lds0);
-    const u32x4 rb = LB::raddr(lane, wn * 128, lds0 + 2 * kTileBytes);
-    u32x4 misc;
-    misc.x = lds0 + LA::woff(tid);
-    misc.y = lds0 + 2 * kTileBytes + LB::woff(tid);
-    misc.z = LA::goff(tid, m0, g.lda, g.M);
-    misc.w = LB::goff(tid, n0, g.ldb, g.N);
+    const u32x8 ra = LA::raddr(lane, wm * 128, lds0);
+    const u32x8 rb = LB::raddr(lane, wn * 128, lds0 + kOperBytes);
+    u32x2 misc;
+    misc.x = LA::goff(lane, wave, m0, g.lda, g.M);
+    misc.y = LB::goff(lane, wave, n0, g.ldb, g.N);
+    // LDS address of this wave's 1 KB slot in pass 0 of buffer 0 (wave-uniform)
+    const uint32_t m0b = __builtin_amdgcn_readfirstlane(lds0 + (uint32_t)wave * 1024u);
     const __amdgpu_buffer_rsrc_t rsa =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(a), 0, a_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t rsb =
@@ -136,12 +151,12 @@ __global__ __launch_bounds__(256) void gemm256_kernel(GemmArgs g) {
 
     f32x16 acc[16];
     main_loop<T, TA, TB>(acc, ra, rb, misc, rsa, rsb, LA::pass_stride(g.lda), LB::pass_stride(g.ldb),
-                         LA::tile_stride(g.lda), LB::tile_stride(g.ldb), (uint32_t)(g.K / 64));
+                         LA::stage_stride(g.lda), LB::stage_stride(g.ldb), m0b, (uint32_t)(g.K / 32),
+                         __builtin_amdgcn_readfirstlane((uint32_t)wave));
 
-    // Waves still read (unused) prefetched fragments of a tile past the end; the
-    // staging area below overlaps those buffers, which is harmless, but every wave
-    // must have left the loop's last real reads behind: the loop's final barrier
-    // guarantees that.
+    // The loop ends with every wave's outstanding loads landed and a barrier, so the
+    // ring may be reused as the staging area below.  Waves may still have (unused)
+    // fragment reads of a stage past the end in flight; overwriting those is harmless.
     //
     // Accumulator tiles are transposed: lane = row m (lrow), register group
     // q = r / 4 holds columns 8q + 4*lhalf + r % 4 of the 32-column block.
@@ -220,13 +235,13 @@ int layout256(hipStream_t s, const GemmArgs& g, int64_t batch, int ta, int tb) {
 
 }  // namespace
 
-// The kernel needs whole K tiles, 16-byte-aligned operand rows (checked by the
+// The kernel needs whole K stages, 16-byte-aligned operand rows (checked by the
 // caller), an output it can store 16 bytes at a time, operands small enough for
-// 32-bit byte offsets including the prefetch overrun of three K tiles, and enough
+// 32-bit byte offsets including the prefetch overrun of four K stages, and enough
 // 256x256 tiles to occupy the device.
 bool gemm256_eligible(const GemmArgs& g, int64_t batch, int dtype) {
     if (dtype != MHIP_BF16 && dtype != MHIP_F16) return false;
-    if (g.K % 64 != 0 || g.K < 64) return false;
+    if (g.K % 32 != 0 || g.K < 32) return false;
     if (g.N % 8 != 0 || (reinterpret_cast<uintptr_t>(g.c) & 15) != 0 || g.sc % 8 != 0) return false;
     if (g.bias && (reinterpret_cast<uintptr_t>(g.bias) & 7) != 0) return false;
     const int64_t a_bytes = (int64_t)g.M * g.K * 2, b_bytes = (int64_t)g.N * g.K * 2;

@@ -144,6 +144,51 @@ def test_gemm_4096_sampled_rows():
     assert torch.equal(kernels.matmul(a * 2, b), c * 2)
 
 
+# Shapes with >= 192 tiles of 256x256: served by the four-wave kernel with the
+# hand-scheduled main loop (K stages of 32: single stage, exit after each position of the
+# unrolled ring, ragged M / N, every operand layout).
+BIG = [(4096, 3072, 32), (3585, 3848, 96), (4000, 3608, 160), (3600, 4104, 448), (8192, 2304, 768)]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=lambda d: NAME[d])
+@pytest.mark.parametrize("layout", [(False, False), (False, True), (True, False), (True, True)],
+                         ids=["nn", "nt", "tn", "tt"])
+@pytest.mark.parametrize("shape", BIG, ids=lambda s: "x".join(map(str, s)))
+def test_gemm_large_tiles(shape, layout, dtype):
+    from metalhlo_amd import kernels
+    M, N, K = shape
+    ta, tb = layout
+    a, b = _ab(M, N, K, dtype, 27, ta, tb)
+    rng = np.random.default_rng(28)
+    bias = to_dev(rng.standard_normal(N) * 0.5, dtype)
+    c = kernels.matmul(a, b, bias, "relu", trans_a=ta, trans_b=tb)
+    assert c.shape == (M, N)
+    rows = np.unique(np.r_[0, 127, 128, 255, 256, M - 1, rng.integers(0, M, 42)])
+    A = as_f64(a).T if ta else as_f64(a)
+    B = as_f64(b).T if tb else as_f64(b)
+    exp = np.maximum(A[rows] @ B + as_f64(bias)[None, :], 0.0)
+    assert_close(c[rows], exp, TOL[dtype], f"gemm {shape} {layout}")
+    # the other kernel (128x128 tiles) accumulates each k-block in the same order
+    os.environ["MHIP_GEMM_TILE"] = "128"
+    try:
+        c128 = kernels.matmul(a, b, bias, "relu", trans_a=ta, trans_b=tb)
+    finally:
+        del os.environ["MHIP_GEMM_TILE"]
+    assert torch.equal(c, c128)
+
+
+def test_gemm_large_exact_small_integers():
+    """Integer-valued operands with exactly representable partial sums: bit-exact."""
+    from metalhlo_amd import kernels
+    rng = np.random.default_rng(29)
+    a = to_dev(rng.integers(-3, 4, (4096, 512)).astype(np.float64), torch.bfloat16)
+    b = to_dev(rng.integers(-3, 4, (512, 4096)).astype(np.float64), torch.bfloat16)
+    c = kernels.matmul(a, b)
+    exp = (a.double() @ b.double())
+    assert torch.equal(c.double(), exp.to(torch.bfloat16).double())
+    assert torch.equal(kernels.matmul(a, b.t().contiguous(), trans_b=True), c)
+
+
 def test_gemm_errors(lib):
     assert lib.mhip_gemm(None, None, None, None, None, 4, 4, 4, 1, 0, 0, 0, 0, 0, 0, 3) == 1
     x = torch.zeros(4, 4, dtype=torch.int32, device="cuda")
