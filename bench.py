@@ -35,13 +35,13 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by what the same
 # counter reads for the 'copy' workload (256 MiB in, 256 MiB out); see profiles/<workload>.txt.
 MEASURED_TRAFFIC = {
-    "gemm": 236982956,
-    "attention": 536931388,
-    "attention_full": 268556237,
-    "softmax": 536717179,
-    "layer_norm": 536879830,
-    "rms_norm": 536782397,
-    "bias_gelu": 536773400,
+    "gemm": 238938188,
+    "attention": 540499858,
+    "attention_full": 268510134,
+    "softmax": 536807759,
+    "layer_norm": 536968239,
+    "rms_norm": 536871699,
+    "bias_gelu": 536863287,
     "copy": 536870912,
 }
 
@@ -71,7 +71,7 @@ def wl_gemm(torch, kernels, M=4096, N=4096, K=4096):
     c = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
     return dict(name=f"bf16 GEMM {M}x{N}x{K} (row-major A[M,K], B[K,N]; fp32 accumulate, bf16 out)",
                 fn=lambda i: kernels.matmul(a, b, out=c), flops=2.0 * M * N * K,
-                bytes=2.0 * (M * K + K * N + M * N), bound="mfma", kernel="gemm_mfma_kernel")
+                bytes=2.0 * (M * K + K * N + M * N), bound="mfma", kernel="gemm256_kernel")
 
 
 def wl_attention(torch, kernels, B=4, H=32, S=4096, D=128, causal=True):

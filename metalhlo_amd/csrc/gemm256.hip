@@ -45,20 +45,12 @@ __device__ inline void static_for(F&& f) {
 struct KMajor {
     __device__ static uint32_t goff(int lane, int wave, int row0, int ld, int cols_total) {
         (void)cols_total;
-#ifdef GEMM256_FULLLINE_EXP   // timing experiment only: whole 128-byte lines, wrong data
-        return (uint32_t)(((int64_t)(row0 + 8 * wave + (lane >> 3)) * ld + (lane & 7) * 8) * 2);
-#endif
         const int row = row0 + 16 * wave + (lane >> 2);
         const int c = (lane & 3) ^ ((lane >> 4) & 3);
         return (uint32_t)(((int64_t)row * ld + c * 8) * 2);
     }
-#ifdef GEMM256_FULLLINE_EXP
-    __device__ static uint32_t pass_stride(int ld) { return (uint32_t)(32 * ld * 2); }
-    __device__ static uint32_t stage_stride(int ld) { (void)ld; return 128u; }
-#else
     __device__ static uint32_t pass_stride(int ld) { return (uint32_t)(64 * ld * 2); }
     __device__ static uint32_t stage_stride(int ld) { (void)ld; return 64u; }
-#endif
     // read addresses: element 2h + s = k-step s of row block 0 in ring half h;
     // + 2048 per row block of 32, + 32768 for the odd buffer of the half
     __device__ static u32x8 raddr(int lane, int row_block0, uint32_t base) {
