@@ -91,6 +91,18 @@ typedef short fa_s16x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) fa_s16x4 fa_lds_s16x4;
 typedef __attribute__((address_space(3))) void fa_lds_void;
 
+// The value held by lane ^ 32, through the register-file lane swap of gfx950 instead
+// of a round trip through LDS.  The swap exchanges the upper half of its first
+// operand with the lower half of its second; picking the result by the lane's own
+// half is right whether or not the two operands share a register.
+__device__ inline float other_half(float x) {
+    const unsigned u = __builtin_bit_cast(unsigned, x);
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return __builtin_bit_cast(float, (threadIdx.x & 32) ? r[0] : r[1]);
+}
+__device__ inline float half_max(float x) { return fmaxf(x, other_half(x)); }
+__device__ inline float half_sum(float x) { return x + other_half(x); }
+
 template <typename T, int D, bool CAUSAL, bool HAS_MASK>
 __global__ __launch_bounds__(256, 2) void fa_fwd_kernel(FaArgs a) {
     constexpr int CPR = D / 8;                  // 16-byte chunks per row
@@ -196,6 +208,9 @@ __global__ __launch_bounds__(256, 2) void fa_fwd_kernel(FaArgs a) {
             for (int t = 0; t < 2; t++)
 #pragma unroll
                 for (int r = 0; r < 16; r++) sacc[t][r] = 0.f;
+            // two workgroups share a SIMD: let a wave in a matrix phase issue ahead of
+            // the other wave's softmax arithmetic
+            __builtin_amdgcn_s_setprio(2);
 #pragma unroll
             for (int s = 0; s < NS; s++) {
 #pragma unroll
@@ -204,6 +219,7 @@ __global__ __launch_bounds__(256, 2) void fa_fwd_kernel(FaArgs a) {
                     sacc[t] = Mfma32A<T>::run(kf, qf[s], sacc[t]);
                 }
             }
+            __builtin_amdgcn_s_setprio(0);
             float sv[32];
 #pragma unroll
             for (int t = 0; t < 2; t++)
@@ -237,7 +253,7 @@ __global__ __launch_bounds__(256, 2) void fa_fwd_kernel(FaArgs a) {
                 float mloc = sv[0];
 #pragma unroll
                 for (int i = 1; i < 32; i++) mloc = fmaxf(mloc, sv[i]);
-                mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
+                mloc = half_max(mloc);
                 m_new = fmaxf(m_run, mloc);
                 const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
 #pragma unroll
@@ -248,7 +264,7 @@ __global__ __launch_bounds__(256, 2) void fa_fwd_kernel(FaArgs a) {
                 float mloc = sv[0];
 #pragma unroll
                 for (int i = 1; i < 32; i++) mloc = fmaxf(mloc, sv[i]);
-                mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
+                mloc = half_max(mloc);
                 m_new = fmaxf(m_run, mloc * a.c);
                 const float neg_m = -m_new;     // finite: an interior block has no masked score
 #pragma unroll
@@ -277,6 +293,7 @@ __global__ __launch_bounds__(256, 2) void fa_fwd_kernel(FaArgs a) {
                 pb[u].z = Mfma32A<T>::pack2(sv[8 * u + 4], sv[8 * u + 5]);
                 pb[u].w = Mfma32A<T>::pack2(sv[8 * u + 6], sv[8 * u + 7]);
             }
+            __builtin_amdgcn_s_setprio(2);
             // ---- O^T += V^T . P^T: A operand slot j of step u is key
             // 16u + 8(j/4) + 4*lhalf + j%4, i.e. two transposing reads 8 keys apart
 #pragma unroll
@@ -294,12 +311,13 @@ __global__ __launch_bounds__(256, 2) void fa_fwd_kernel(FaArgs a) {
                     oacc[dt] = Mfma32A<T>::run(vf, pb[u], oacc[dt]);
                 }
             }
+            __builtin_amdgcn_s_setprio(0);
         }
         if (it + 1 < nkv) tiles_ready();
     }
 
     // ---- normalise and store: lane holds 4 consecutive d per register group -
-    const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+    const float l_tot = half_sum(l_run);
     const float inv = l_tot > 1e-10f ? 1.f / l_tot : 0.f;
     if (qpos < a.Sq) {
         T* orow = op + (int64_t)qpos * D;
