@@ -5,7 +5,7 @@
 // documented there); this file computes the per-thread addresses it consumes and
 // holds the epilogue.
 //
-// K is consumed in stages of 32 through a ring of four 32 KB LDS buffers
+// K is consumed in stages of 32 through a ring of five 32 KB LDS buffers
 // ([A tile 16 KB][B tile 16 KB]) filled by buffer loads that write LDS directly:
 // a wave's load instruction deposits 64 x 16 bytes contiguously, so the LDS
 // layout is fixed by which 16-byte chunk of global memory each lane asks for.
@@ -28,7 +28,7 @@ namespace mhip {
 
 namespace {
 
-constexpr uint32_t kStageBytes = 32 * 1024, kOperBytes = 16 * 1024, kHalfRing = 64 * 1024;
+constexpr uint32_t kOperBytes = 16 * 1024;   // B tile offset inside a 32 KB stage buffer
 
 template <typename F, int... I>
 __device__ inline void static_for_impl(F& f, std::integer_sequence<int, I...>) {
@@ -51,14 +51,14 @@ struct KMajor {
     }
     __device__ static uint32_t pass_stride(int ld) { return (uint32_t)(64 * ld * 2); }
     __device__ static uint32_t stage_stride(int ld) { (void)ld; return 64u; }
-    // read addresses: element 2h + s = k-step s of row block 0 in ring half h;
-    // + 2048 per row block of 32, + 32768 for the odd buffer of the half
-    __device__ static u32x8 raddr(int lane, int row_block0, uint32_t base) {
+    // read addresses of ring buffers 0 and 1: element s = k-step s of row block 0
+    // (+ 2048 per row block of 32, + 32768 for buffer 1); the loop derives the other
+    // buffers' addresses
+    __device__ static u32x4 raddr(int lane, int row_block0, uint32_t base) {
         const int lrow = lane & 31, lhalf = lane >> 5;
         const uint32_t b = base + (uint32_t)((row_block0 + lrow) * 64 + ((lhalf ^ ((lrow >> 2) & 3)) << 4));
-        u32x8 r;
-        r[0] = b; r[1] = b ^ 32u; r[2] = b + kHalfRing; r[3] = (b ^ 32u) + kHalfRing;
-        r[4] = r[5] = r[6] = r[7] = 0;
+        u32x4 r;
+        r.x = b; r.y = b ^ 32u; r.z = 0; r.w = 0;
         return r;
     }
 };
@@ -75,36 +75,34 @@ struct MnMajor {
     }
     __device__ static uint32_t pass_stride(int ld) { return (uint32_t)(8 * ld * 2); }
     __device__ static uint32_t stage_stride(int ld) { return (uint32_t)(32 * ld * 2); }
-    // read addresses: element 4h + j = mn block j at k-step 0 in ring half h; + 8192 per
-    // k-step, + 2048 for the upper four k of a fragment, + 32768 for the odd buffer
-    __device__ static u32x8 raddr(int lane, int mn_block0, uint32_t base) {
+    // read addresses of ring buffers 0 and 1: element j = mn block j at k-step 0
+    // (+ 8192 per k-step, + 2048 for the upper four k of a fragment, + 32768 for
+    // buffer 1); the loop derives the other buffers' addresses
+    __device__ static u32x4 raddr(int lane, int mn_block0, uint32_t base) {
         const int i = lane & 15, gq = lane >> 4;
         const int xr = (i >> 2) & 3;
         const int mn = mn_block0 + 16 * (gq & 1) + 4 * (i & 3);
         const uint32_t b = base + (uint32_t)((8 * (gq >> 1) + (i >> 2)) * 512 + ((mn >> 3) << 4) + (mn & 7) * 2);
-        u32x8 r;
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            r[j] = b + (uint32_t)((j ^ xr) << 6);
-            r[4 + j] = r[j] + kHalfRing;
-        }
+        u32x4 r;
+        r.x = b + (uint32_t)((0 ^ xr) << 6); r.y = b + (uint32_t)((1 ^ xr) << 6);
+        r.z = b + (uint32_t)((2 ^ xr) << 6); r.w = b + (uint32_t)((3 ^ xr) << 6);
         return r;
     }
 };
 
 template <typename T, bool TA, bool TB>
-__device__ inline void main_loop(f32x16 (&acc)[16], u32x8 ra, u32x8 rb, u32x2& misc,
+__device__ inline void main_loop(f32x16 (&acc)[16], u32x4 ra, u32x4 rb, u32x2& misc,
                                  __amdgpu_buffer_rsrc_t rsa, __amdgpu_buffer_rsrc_t rsb, uint32_t pa,
-                                 uint32_t pb, uint32_t ta, uint32_t tb, uint32_t m0b, uint32_t kt, uint32_t wv) {
+                                 uint32_t pb, uint32_t ta, uint32_t tb, uint32_t m0b, uint32_t kt) {
     constexpr bool bf = std::is_same<T, bf16_t>::value;
-    if constexpr (bf && !TA && !TB) gemm256_loop_nn_bf16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt, wv);
-    if constexpr (bf && !TA && TB) gemm256_loop_nt_bf16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt, wv);
-    if constexpr (bf && TA && !TB) gemm256_loop_tn_bf16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt, wv);
-    if constexpr (bf && TA && TB) gemm256_loop_tt_bf16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt, wv);
-    if constexpr (!bf && !TA && !TB) gemm256_loop_nn_f16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt, wv);
-    if constexpr (!bf && !TA && TB) gemm256_loop_nt_f16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt, wv);
-    if constexpr (!bf && TA && !TB) gemm256_loop_tn_f16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt, wv);
-    if constexpr (!bf && TA && TB) gemm256_loop_tt_f16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt, wv);
+    if constexpr (bf && !TA && !TB) gemm256_loop_nn_bf16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt);
+    if constexpr (bf && !TA && TB) gemm256_loop_nt_bf16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt);
+    if constexpr (bf && TA && !TB) gemm256_loop_tn_bf16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt);
+    if constexpr (bf && TA && TB) gemm256_loop_tt_bf16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt);
+    if constexpr (!bf && !TA && !TB) gemm256_loop_nn_f16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt);
+    if constexpr (!bf && !TA && TB) gemm256_loop_nt_f16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt);
+    if constexpr (!bf && TA && !TB) gemm256_loop_tn_f16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt);
+    if constexpr (!bf && TA && TB) gemm256_loop_tt_f16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt);
 }
 
 template <typename T, bool TA, bool TB>
@@ -129,8 +127,8 @@ __global__ __launch_bounds__(256) void gemm256_kernel(GemmArgs g) {
     // LDS byte address of the dynamic segment
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
 
-    const u32x8 ra = LA::raddr(lane, wm * 128, lds0);
-    const u32x8 rb = LB::raddr(lane, wn * 128, lds0 + kOperBytes);
+    const u32x4 ra = LA::raddr(lane, wm * 128, lds0);
+    const u32x4 rb = LB::raddr(lane, wn * 128, lds0 + kOperBytes);
     u32x2 misc;
     misc.x = LA::goff(lane, wave, m0, g.lda, g.M);
     misc.y = LB::goff(lane, wave, n0, g.ldb, g.N);
@@ -143,8 +141,7 @@ __global__ __launch_bounds__(256) void gemm256_kernel(GemmArgs g) {
 
     f32x16 acc[16];
     main_loop<T, TA, TB>(acc, ra, rb, misc, rsa, rsb, LA::pass_stride(g.lda), LB::pass_stride(g.ldb),
-                         LA::stage_stride(g.lda), LB::stage_stride(g.ldb), m0b, (uint32_t)(g.K / 32),
-                         __builtin_amdgcn_readfirstlane((uint32_t)wave));
+                         LA::stage_stride(g.lda), LB::stage_stride(g.ldb), m0b, (uint32_t)(g.K / 32));
 
     // The loop ends with every wave's outstanding loads landed and a barrier, so the
     // ring may be reused as the staging area below.  Waves may still have (unused)
@@ -199,7 +196,7 @@ __global__ __launch_bounds__(256) void gemm256_kernel(GemmArgs g) {
 
 template <typename T, bool TA, bool TB>
 int launch256(hipStream_t s, GemmArgs g, int64_t batch) {
-    constexpr int kSmem = 4 * 128 * (128 * 2 + 16);   // epilogue staging (136 KB) >= 4 tiles (128 KB)
+    constexpr int kSmem = 5 * 32 * 1024;   // ring of five stage buffers; the epilogue staging (136 KB) reuses it
     auto kern = gemm256_kernel<T, TA, TB>;
     static std::once_flag once;
     static hipError_t attr_err = hipSuccess;
@@ -229,7 +226,7 @@ int layout256(hipStream_t s, const GemmArgs& g, int64_t batch, int ta, int tb) {
 
 // The kernel needs whole K stages, 16-byte-aligned operand rows (checked by the
 // caller), an output it can store 16 bytes at a time, operands small enough for
-// 32-bit byte offsets including the prefetch overrun of four K stages, and enough
+// 32-bit byte offsets including the prefetch overrun of five K stages, and enough
 // 256x256 tiles to occupy the device.
 bool gemm256_eligible(const GemmArgs& g, int64_t batch, int dtype) {
     if (dtype != MHIP_BF16 && dtype != MHIP_F16) return false;

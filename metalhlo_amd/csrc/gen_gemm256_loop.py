@@ -7,25 +7,34 @@ One workgroup = 4 waves (one per SIMD); each wave owns a 128x128 sub-tile =
 SIMD nothing hides a stall except the wave's own instruction stream, so the
 order of every instruction is fixed here instead of being left to the compiler.
 
-K is consumed in stages of 32 (two k-steps of 16).  LDS holds a ring of four stage
+K is consumed in stages of 32 (two k-steps of 16).  LDS holds a ring of five stage
 buffers (32 KB each: A tile 16 KB, B tile 16 KB) that is filled by buffer loads
 that write LDS directly (no staging registers, no LDS store instructions).
 Fragments are read from LDS two k-steps (= one stage) before the MFMAs that use
 them, into a rotation of four fragment register sets, so a wait for fragments
-never follows their reads closely.  Stage t (buffer t % 4):
+never follows their reads closely.  Stage t (buffer t % 5):
 
   k-step 0 : 16 MFMAs; reads of stage t+1 k-step 0 fragments;
-             second half of the direct-to-LDS loads of stage t+3
-  wait: k-step 1 fragments there (= all own reads of buffer t % 4 done), own
-        loads of stage t+2 landed;  workgroup barrier
+             second half of the loads triggered by the previous stage's barrier
+  wait: k-step 1 fragments there (= all own reads of buffer t % 5 done), own
+        loads of stage t+2 landed;  workgroup barrier (buffer t % 5 is free)
   k-step 1 : 16 MFMAs; reads of stage t+1 k-step 1 fragments;
-             first half of the loads of stage t+4 into buffer t % 4
+             first half of the loads this barrier triggers:
+               operand with k as the slow axis: stage t+5 into buffer t % 5;
+               operand with k contiguous, t even: stages t+4 AND t+5 together.
+A stage of a k-contiguous operand is 64 bytes of each row = half a cache line; asking
+for both halves in adjacent instructions fetches every line from L2 once instead of
+twice (the L2 -> L1 fill path, 64 bytes per clock per CU, is what the loop is
+short of).
 
 Register map (VGPR):
   fragment set n (n = 0..3, k-step 2t+s uses set (2t+s) % 4):
       A fragments v[32n : 32n+15], B fragments v[32n+16 : 32n+31]
-  v[192:199] A fragment read addresses, v[200:207] B fragment read addresses
-  v208 / v209 A / B global byte offsets of this thread's 16-byte chunk
+  v[192:203] A fragment read addresses, v[204:215] B fragment read addresses
+      (k-contiguous operand: element 2h + s = k-step s, ring buffers 2h and 2h+1;
+       other operand: element 4h + j = mn block j, ring buffers 2h and 2h+1)
+  v216 / v217 A / B global byte offset of this thread's 16-byte chunk,
+  v218 / v219 the same + 64 (second half line of a k-contiguous operand)
 AGPR: accumulator (i, j) = a[16*(4*i+j) : +15]
 SGPR: s[72:74] = 1..3 x A pass stride, s[76:78] = 1..3 x B pass stride, s80 = stage counter,
       s81 = caller's M0 (restored at the end)
@@ -33,22 +42,24 @@ SGPR: s[72:74] = 1..3 x A pass stride, s[76:78] = 1..3 x B pass stride, s80 = st
 An operand is either "K" (k is the contiguous axis in memory: stage tile stored
 [256 rows][32 k], fragments read with ds_read_b128) or "MN" (k is the slow axis:
 tile stored as it lies, [32 k][256 mn], fragments transposed on the way out with
-ds_read_b64_tr_b16).  Fragment read addresses: "K": element 2*h + s = k-step s in
-ring half h (buffers 2h, 2h+1); "MN": element 4*h + j = mn block j in ring half h.
+ds_read_b64_tr_b16).
 
 Run:  python3 gen_gemm256_loop.py > gemm256_loop.inc
 """
 import os
 
-EXP = os.environ.get("GEMM256_EXP", "")   # timing experiments only: noload, nomfma, noread
+EXP = os.environ.get("GEMM256_EXP", "")   # timing experiments only: noload, nomfma, noread, nobarrier
 
-NST = 4               # ring stages
+NST = 5               # ring stages
+UNROLL = 10           # stages per loop body: lcm(ring, pair issue, fragment set rotation)
 STAGE = 32768         # bytes per stage buffer
 OPER = 16384          # bytes per operand tile
 SET = {n: (32 * n, 32 * n + 16) for n in range(4)}   # fragment set -> (A base vgpr, B base vgpr)
-RA, RB = 192, 200
-GA, GB = 208, 209
-SPA, SPB, ST = 72, 76, 80
+RA, RB = 192, 204
+GOFF = {"A": 216, "B": 217}
+GOFF2 = {"A": 218, "B": 219}
+SP = {"A": 72, "B": 76}
+ST = 80
 
 
 def vr(base, n):
@@ -72,44 +83,48 @@ def frag_reads(kind, which, g, s, fset):
     return out
 
 
-def all_frag_reads(ka, kb, g, s, fset):
-    a, b = frag_reads(ka, "A", g, s, fset), frag_reads(kb, "B", g, s, fset)
+def all_frag_reads(kinds, g, s, fset):
+    a, b = frag_reads(kinds["A"], "A", g, s, fset), frag_reads(kinds["B"], "B", g, s, fset)
     out = []
     for i in range(max(len(a), len(b))):
         out += a[i:i + 1] + b[i:i + 1]
     return out
 
 
-def stage_loads(g, passes=range(4), advance=True):
-    """Direct-to-LDS loads of one stage into ring buffer `g`: 4 passes per operand; the
-    wave's 1 KB LDS slot of pass p is M0 = wave base + buffer + operand + p * 4096."""
-    out = []
-    for p in passes:
-        so_a = "0" if p == 0 else f"s{SPA + p - 1}"
-        so_b = "0" if p == 0 else f"s{SPB + p - 1}"
-        out.append(f"s_add_u32 m0, %[m0b], {g * STAGE + p * 4096}")
-        out.append("s_nop 0")
-        out.append(f"buffer_load_dwordx4 v{GA}, %[rsa], {so_a} offen lds")
-        out.append(f"s_add_u32 m0, %[m0b], {g * STAGE + OPER + p * 4096}")
-        out.append("s_nop 0")
-        out.append(f"buffer_load_dwordx4 v{GB}, %[rsb], {so_b} offen lds")
-    if advance:
-        out.append(f"v_add_u32 v{GA}, %[ta], v{GA}")
-        out.append(f"v_add_u32 v{GB}, %[tb], v{GB}")
-    return out
+def load_instr(which, stage, p, second_half=False):
+    """One direct-to-LDS load (kept together with its M0 set-up) of pass `p` of `stage`:
+    the wave's 1 KB LDS slot is M0 = wave base + buffer + operand + p * 4096."""
+    g = stage % NST
+    m0 = g * STAGE + (OPER if which == "B" else 0) + p * 4096
+    so = "0" if p == 0 else f"s{SP[which] + p - 1}"
+    voff = (GOFF2 if second_half else GOFF)[which]
+    rs = "%[rsa]" if which == "A" else "%[rsb]"
+    return dict(stage=stage, lines=[f"s_add_u32 m0, %[m0b], {m0}", "s_nop 0",
+                                    f"buffer_load_dwordx4 v{voff}, {rs}, {so} offen lds"])
 
 
-def group3(lines):
-    """Keeps each (s_add m0, s_nop, buffer_load) triple together when interleaving."""
-    out, i = [], 0
-    while i < len(lines):
-        if lines[i].startswith("s_add_u32 m0"):
-            out.append(lines[i:i + 3])
-            i += 3
+def trigger_group(kinds, t):
+    """Loads triggered by the barrier of stage t (buffer t % 5 has just become free)."""
+    grp = []
+    for which in ("A", "B"):
+        if kinds[which] == "K":
+            if t % 2 == 0:
+                for p in range(4):
+                    grp.append(load_instr(which, t + 4, p))
+                    grp.append(load_instr(which, t + 5, p, second_half=True))
+                grp.append(dict(stage=None, lines=[f"v_add_u32 v{GOFF[which]}, 128, v{GOFF[which]}",
+                                                   f"v_add_u32 v{GOFF2[which]}, 128, v{GOFF2[which]}"]))
         else:
-            out.append([lines[i]])
-            i += 1
-    return out
+            for p in range(4):
+                grp.append(load_instr(which, t + 5, p))
+            step = "%[ta]" if which == "A" else "%[tb]"
+            grp.append(dict(stage=None, lines=[f"v_add_u32 v{GOFF[which]}, {step}, v{GOFF[which]}"]))
+    return grp
+
+
+def halves(grp):
+    n = (len(grp) + 1) // 2
+    return grp[:n], grp[n:]
 
 
 def mfmas(mnem, fset):
@@ -123,44 +138,82 @@ def mfmas(mnem, fset):
     return out
 
 
-def interleave(main, reads, loads, wave):
-    """The four waves of a workgroup run in lockstep between barriers and share one
-    LDS and one texture addresser, so each wave gets its own slots: wave w issues its
-    fragment reads behind MFMAs 4w .. 4w+3 and its global loads behind MFMAs
-    w, w+4, w+8, w+12 of a k-step.  A load group is a list of lines kept together."""
-    loads = [[x] if isinstance(x, str) else x for x in loads]
+def interleave(main, reads, loads):
+    """Fragment reads behind the first four MFMAs of a k-step (they are not needed before
+    the k-step after the next), loads spread evenly over the k-step.  `loads` are dicts
+    whose lines stay together."""
     per = (len(reads) + 3) // 4
+    every = max(1, len(main) // max(len(loads), 1))
     out, kl = [], 0
     for idx, m in enumerate(main):
         out.append(m)
-        rel = idx - 4 * wave
-        if 0 <= rel < 4:
-            out += reads[rel * per:(rel + 1) * per]
-        if idx % 4 == wave and kl < len(loads):
-            out += loads[kl]
+        if idx < 4:
+            out += reads[idx * per:(idx + 1) * per]
+        if kl < len(loads) and idx % every == 0:
+            out += loads[kl]["lines"]
             kl += 1
-    for grp in loads[kl:]:
-        out += grp
+    for ld in loads[kl:]:
+        out += ld["lines"]
     return out
+
+
+class Tracker:
+    """Program-order list of issued loads, to size the vmcnt waits: a wait in front of the
+    barrier of stage t needs every load of stages <= t+2 landed, i.e. may leave
+    outstanding only the loads issued after the last of those."""
+
+    def __init__(self):
+        self.order = []
+
+    def issue(self, loads):
+        for ld in loads:
+            if ld["stage"] is not None:
+                self.order.append(ld["stage"])
+
+    def allowed(self, need_stage):
+        last = max(i for i, s in enumerate(self.order) if s <= need_stage)
+        return len(self.order) - 1 - last
+
+
+def simulate(kinds):
+    """vmcnt for the barrier of each body position (minimum over the first iterations and
+    the steady state) and for the prologue."""
+    tr = Tracker()
+    for t in range(-NST, -1):
+        tr.issue(trigger_group(kinds, t))
+    first, second = halves(trigger_group(kinds, -1))
+    tr.issue(first)
+    pro = tr.allowed(1)
+    pending = second
+    counts = {}
+    for t in range(4 * UNROLL):
+        tr.issue(pending)                       # k-step 0
+        c = tr.allowed(t + 2)
+        counts[t % UNROLL] = min(counts.get(t % UNROLL, 63), c)
+        first, pending = halves(trigger_group(kinds, t))
+        tr.issue(first)                         # k-step 1
+    return pro, counts
 
 
 def drop(lines, prefix):
     return [l for l in lines if not l.startswith(prefix)]
 
 
-def stage_iteration(mnem, ka, kb, g, wave):
-    nxt, prv = (g + 1) % NST, (g - 1) % NST
-    r0 = all_frag_reads(ka, kb, nxt, 0, (2 * g + 2) % 4)
-    r1 = all_frag_reads(ka, kb, nxt, 1, (2 * g + 3) % 4)
+def stage_iteration(mnem, kinds, t, vmcnt):
+    g, nxt = t % NST, (t + 1) % NST
+    r0 = all_frag_reads(kinds, nxt, 0, (2 * t + 2) % 4)
+    r1 = all_frag_reads(kinds, nxt, 1, (2 * t + 3) % 4)
+    _, prev_second = halves(trigger_group(kinds, t - 1))
+    this_first, _ = halves(trigger_group(kinds, t))
     out = []
     # k-step 0: its fragments were read one stage ago; only the previous k-step's reads
     # (LDS operations retire in order) may still be outstanding
     out.append(f"s_waitcnt lgkmcnt({min(len(r1), 15)})")
-    out += interleave(mfmas(mnem, (2 * g) % 4), r0, group3(stage_loads(prv, (2, 3))), wave)
+    out += interleave(mfmas(mnem, (2 * t) % 4), r0, prev_second)
     # k-step 1
-    out.append(f"s_waitcnt vmcnt(8) lgkmcnt({min(len(r0), 15)})")
+    out.append(f"s_waitcnt vmcnt({min(vmcnt, 63)}) lgkmcnt({min(len(r0), 15)})")
     out.append("s_barrier")
-    out += interleave(mfmas(mnem, (2 * g + 1) % 4), r1, group3(stage_loads(g, (0, 1), advance=False)), wave)
+    out += interleave(mfmas(mnem, (2 * t + 1) % 4), r1, this_first)
     if "noload" in EXP:
         out = [l for l in drop(drop(out, "buffer_load"), "s_add_u32 m0") if l != "s_nop 0"]
     if "nomfma" in EXP:
@@ -172,41 +225,45 @@ def stage_iteration(mnem, ka, kb, g, wave):
     return out
 
 
-def body(mnem, ka, kb):
+def body(mnem, kinds):
+    pro_vmcnt, vmcnts = simulate(kinds)
     out = []
     for r in range(256):
         out.append(f"v_accvgpr_write_b32 a{r}, 0")
-    for i in range(1, 4):
-        out.append(f"s_mul_i32 s{SPA + i - 1}, %[pa], {i}")
-        out.append(f"s_mul_i32 s{SPB + i - 1}, %[pb], {i}")
+    for which, pin in (("A", "%[pa]"), ("B", "%[pb]")):
+        for i in range(1, 4):
+            out.append(f"s_mul_i32 s{SP[which] + i - 1}, {pin}, {i}")
     out.append(f"s_mov_b32 s{ST}, 0")
     out.append(f"s_mov_b32 s{ST + 1}, m0")
-    for g in range(NST - 1):
-        out += stage_loads(g)
-    out += stage_loads(NST - 1, (0, 1), advance=False)
-    out.append("s_waitcnt vmcnt(12)")           # stages 0 and 1 landed
+    # fragment read addresses of ring buffers 2..4 from those of buffers 0 and 1
+    for which, base in (("A", RA), ("B", RB)):
+        n = 2 if kinds[which] == "K" else 4
+        for h in (1, 2):
+            for e in range(n):
+                out.append(f"v_add_u32 v{base + n * h + e}, {h * 2 * STAGE}, v{base + e}")
+        out.append(f"v_add_u32 v{GOFF2[which]}, 64, v{GOFF[which]}")
+    # the loads the barriers of stages -5 .. -1 would have triggered
+    for t in range(-NST, -1):
+        for ld in trigger_group(kinds, t):
+            out += ld["lines"]
+    first, _ = halves(trigger_group(kinds, -1))
+    for ld in first:
+        out += ld["lines"]
+    out.append(f"s_waitcnt vmcnt({pro_vmcnt})")           # stages 0 and 1 landed
     out.append("s_barrier")
-    out += all_frag_reads(ka, kb, 0, 0, 0)
-    out += all_frag_reads(ka, kb, 0, 1, 1)
+    out += all_frag_reads(kinds, 0, 0, 0)
+    out += all_frag_reads(kinds, 0, 1, 1)
     out.append("s_waitcnt lgkmcnt(0)")
-    # one copy of the loop per wave of the workgroup (different slot assignment)
-    nvar = 1 if "nostagger" in EXP else 4
-    for w in range(1, nvar):
-        out.append(f"s_cmp_eq_u32 %[wv], {w}")
-        out.append(f"s_cbranch_scc1 L_gemm256_loop{w}_%=")
-    for w in range(nvar):
-        out.append(f"L_gemm256_loop{w}_%=:")
-        for g in range(NST):
-            out += stage_iteration(mnem, ka, kb, g, w)
-            out.append(f"s_add_u32 s{ST}, s{ST}, 1")
-            if g < NST - 1:
-                out.append(f"s_cmp_ge_u32 s{ST}, %[kt]")
-                out.append("s_cbranch_scc1 L_gemm256_done_%=")
-            else:
-                out.append(f"s_cmp_lt_u32 s{ST}, %[kt]")
-                out.append(f"s_cbranch_scc1 L_gemm256_loop{w}_%=")
-        if w < nvar - 1:
-            out.append("s_branch L_gemm256_done_%=")
+    out.append("L_gemm256_loop_%=:")
+    for t in range(UNROLL):
+        out += stage_iteration(mnem, kinds, t, vmcnts[t])
+        out.append(f"s_add_u32 s{ST}, s{ST}, 1")
+        if t < UNROLL - 1:
+            out.append(f"s_cmp_ge_u32 s{ST}, %[kt]")
+            out.append("s_cbranch_scc1 L_gemm256_done_%=")
+        else:
+            out.append(f"s_cmp_lt_u32 s{ST}, %[kt]")
+            out.append("s_cbranch_scc1 L_gemm256_loop_%=")
     out.append("L_gemm256_done_%=:")
     # drain: loads of stages past the end still write LDS, which the caller reuses;
     # the last MFMA results must be readable by ordinary instructions
@@ -218,21 +275,22 @@ def body(mnem, ka, kb):
 
 
 def emit(name, mnem, ka, kb):
-    lines = body(mnem, ka, kb)
+    lines = body(mnem, {"A": ka, "B": kb})
     print(f"// {name}: A operand {ka}-major, B operand {kb}-major, {mnem}")
-    print(f"__device__ __forceinline__ void {name}(f32x16 (&acc)[16], u32x8 ra, u32x8 rb, u32x2& goff,")
+    print(f"__device__ __forceinline__ void {name}(f32x16 (&acc)[16], u32x4 ra, u32x4 rb, u32x2& goff,")
     print("        __amdgpu_buffer_rsrc_t rsa, __amdgpu_buffer_rsrc_t rsb, uint32_t pa, uint32_t pb,")
-    print("        uint32_t ta, uint32_t tb, uint32_t m0b, uint32_t kt, uint32_t wv) {")
+    print("        uint32_t ta, uint32_t tb, uint32_t m0b, uint32_t kt) {")
     print("    asm volatile(")
     for ln in lines:
         print(f'        "{ln}\\n"')
     outs = ", ".join(f'"={{a[{16 * i}:{16 * i + 15}]}}"(acc[{i}])' for i in range(16))
     print(f"        : {outs},")
-    print(f'          "+{{v[{GA}:{GB}]}}"(goff)')
-    print(f'        : "{{v[{RA}:{RA + 7}]}}"(ra), "{{v[{RB}:{RB + 7}]}}"(rb),')
+    print(f'          "+{{v[{GOFF["A"]}:{GOFF["B"]}]}}"(goff)')
+    print(f'        : "{{v[{RA}:{RA + 3}]}}"(ra), "{{v[{RB}:{RB + 3}]}}"(rb),')
     print('          [rsa] "s"(rsa), [rsb] "s"(rsb), [pa] "s"(pa), [pb] "s"(pb), [ta] "s"(ta), [tb] "s"(tb),')
-    print('          [m0b] "s"(m0b), [kt] "s"(kt), [wv] "s"(wv)')
-    clob = [f'"v{i}"' for i in range(128)] + [f'"s{i}"' for i in range(SPA, ST + 2)] + ['"scc"', '"memory"']
+    print('          [m0b] "s"(m0b), [kt] "s"(kt)')
+    vclob = list(range(128)) + list(range(RA + 4, RB)) + list(range(RB + 4, GOFF["A"])) + [GOFF2["A"], GOFF2["B"]]
+    clob = [f'"v{i}"' for i in vclob] + [f'"s{i}"' for i in range(SP["A"], ST + 2)] + ['"scc"', '"memory"']
     print("        : " + ", ".join(clob) + ");")
     print("}\n")
 
