@@ -355,14 +355,22 @@ static int launch_mfma(hipStream_t s, GemmArgs g, int64_t batch) {
 bool gemm256_eligible(const GemmArgs& g, int64_t batch, int dtype);
 int launch_gemm256(hipStream_t s, const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype);
 
+// Which kernel serves a 16-bit problem (MHIP_GEMM_TILE = 128 | 256 | 2560 forces one):
+//   * the four-wave 256x256 kernel (gemm256.hip) when it is eligible and K is long
+//     enough (>= 1024) to amortise its one-workgroup-per-CU prologue and epilogue;
+//   * the eight-wave 256x256 kernel for large problems it cannot take whose rows of C
+//     are not 16-byte aligned (odd N): its eight waves hide the narrow stores;
+//   * otherwise 128x128 tiles, two workgroups per CU (short K, few tiles).
 template <typename T, bool TA, bool TB>
 static int pick_tile(hipStream_t s, const GemmArgs& g, int64_t batch) {
     const int64_t big = (int64_t)((g.M + 255) / 256) * ((g.N + 255) / 256) * batch;
     const int force = tune_int("MHIP_GEMM_TILE", 0);
     constexpr int dt = std::is_same<T, bf16_t>::value ? MHIP_BF16 : MHIP_F16;
-    if ((force == 0 || force == 2560) && gemm256_eligible(g, batch, dt))
-        return launch_gemm256(s, g, batch, TA, TB, dt);
-    if (force == 256 || (force != 128 && big >= 192)) return launch_mfma<T, 256, 256, 2, 4, TA, TB>(s, g, batch);
+    if (force == 2560 || (force == 0 && g.K >= 1024)) {
+        if (gemm256_eligible(g, batch, dt)) return launch_gemm256(s, g, batch, TA, TB, dt);
+    }
+    const bool want256 = force == 256 || (force != 128 && big >= 192 && (g.K >= 1024 || g.N % 8 != 0));
+    if (want256) return launch_mfma<T, 256, 256, 2, 4, TA, TB>(s, g, batch);
     return launch_mfma<T, 128, 128, 2, 2, TA, TB>(s, g, batch);
 }
 

@@ -36,6 +36,15 @@ __device__ inline void stage_params(const T* __restrict__ p, f32x4* lds, int nve
     }
 }
 
+// The same, kept in the storage type (one 16-byte vector per 16 bytes of LDS): half the
+// LDS of the fp32 planes for 16-bit types, so more workgroups fit on a CU, and one LDS
+// read per vector instead of two; the widening to fp32 happens at the use.
+template <typename T>
+__device__ inline void stage_params_raw(const T* __restrict__ p, Vec16<T>* lds, int nvec) {
+    constexpr int E = Elem<T>::kPerVec;
+    for (int i = threadIdx.x; i < nvec; i += 256) lds[i] = load16(p + (int64_t)i * E);
+}
+
 template <typename T, int OP, int NV>
 __global__ __launch_bounds__(256) void row_wave_kernel(const T* __restrict__ x,
                                                        const T* __restrict__ gamma,
@@ -43,15 +52,14 @@ __global__ __launch_bounds__(256) void row_wave_kernel(const T* __restrict__ x,
                                                        T* __restrict__ y, int64_t rows, int cols,
                                                        float eps) {
     constexpr int E = Elem<T>::kPerVec;
-    constexpr int P = E / 4;
-    extern __shared__ __attribute__((aligned(16))) f32x4 row_params[];
+    extern __shared__ __attribute__((aligned(16))) char row_params[];
     const int lane = threadIdx.x & 63;
     const int nvec = cols / E;
-    f32x4* gs = row_params;
-    f32x4* bs = row_params + (gamma ? P * nvec : 0);
+    Vec16<T>* gs = reinterpret_cast<Vec16<T>*>(row_params);
+    Vec16<T>* bs = gs + (gamma ? nvec : 0);
     if (OP != kSoftmax && (gamma || beta)) {
-        if (gamma) stage_params(gamma, gs, nvec);
-        if (OP == kLayerNorm && beta) stage_params(beta, bs, nvec);
+        if (gamma) stage_params_raw(gamma, gs, nvec);
+        if (OP == kLayerNorm && beta) stage_params_raw(beta, bs, nvec);
         __syncthreads();
     }
 
@@ -133,18 +141,17 @@ __global__ __launch_bounds__(256) void row_wave_kernel(const T* __restrict__ x,
 #pragma unroll
                     for (int e = 0; e < E; e++) o.v[e] = Elem<T>::from_f32(f[v][e] * a);
                 } else {
+                    Vec16<T> gv, bv;
+                    if (gamma) gv = gs[idx];
+                    if (OP == kLayerNorm && beta) bv = bs[idx];
 #pragma unroll
-                    for (int q = 0; q < P; q++) {
-                        f32x4 g = {1.f, 1.f, 1.f, 1.f}, bt = {0.f, 0.f, 0.f, 0.f};
-                        if (gamma) g = gs[q * nvec + idx];
-                        if (OP == kLayerNorm && beta) bt = bs[q * nvec + idx];
-#pragma unroll
-                        for (int e = 0; e < 4; e++) {
-                            const float xv = f[v][4 * q + e];
-                            // LayerNorm: (x - mean) * rstd == x * rstd + (-mean * rstd)
-                            const float n = (OP == kLayerNorm) ? fmaf(xv, b, a) : xv * a;
-                            o.v[4 * q + e] = Elem<T>::from_f32(fmaf(n, g[e], bt[e]));
-                        }
+                    for (int e = 0; e < E; e++) {
+                        const float g = gamma ? Elem<T>::to_f32(gv.v[e]) : 1.f;
+                        const float bt = (OP == kLayerNorm && beta) ? Elem<T>::to_f32(bv.v[e]) : 0.f;
+                        const float xv = f[v][e];
+                        // LayerNorm: (x - mean) * rstd == x * rstd + (-mean * rstd)
+                        const float n = (OP == kLayerNorm) ? fmaf(xv, b, a) : xv * a;
+                        o.v[e] = Elem<T>::from_f32(fmaf(n, g, bt));
                     }
                 }
                 store16_stream(yr + (int64_t)idx * E, o);
@@ -335,7 +342,7 @@ static int launch_row(hipStream_t s, const void* x, const void* g, const void* b
         const int64_t want = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
         const size_t lds = (OP == kSoftmax) ? 0
                                             : ((gp ? 1 : 0) + ((OP == kLayerNorm && bp) ? 1 : 0)) *
-                                                  (size_t)cols * sizeof(float);
+                                                  (size_t)cols * sizeof(T);
 #define MHIP_ROW_CASE(NV)                                                                      \
     {                                                                                          \
         auto kern = row_wave_kernel<T, OP, NV>;                                                \

@@ -102,9 +102,42 @@ class GPT2:
         logits = kernels.matmul(x, p["wte"], trans_b=True)       # tied head: x . wte^T
         return logits.reshape(B, S, cfg.vocab)
 
+    def capture(self, ids: torch.Tensor) -> "GraphedForward":
+        """Records one forward pass for ids of this shape into a HIP graph.  Every launch
+        of the pass goes to the stream handed to the kernel library, so the whole
+        pipeline (about 135 launches) replays with one submission instead of one host
+        call per kernel."""
+        static_ids = ids.clone()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):           # first calls set kernel attributes; keep them out of the capture
+            for _ in range(2):
+                self.forward(static_ids)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            logits = self.forward(static_ids)
+        return GraphedForward(graph, static_ids, logits)
+
     @staticmethod
     def flops(cfg: GPT2Config, B: int, S: int) -> float:
         d, f = cfg.d_model, cfg.d_ff
         per_tok = cfg.n_layer * (d * 3 * d + d * d + 2 * d * f) + d * cfg.vocab
         attn = cfg.n_layer * 2 * B * cfg.n_head * S * S * (d // cfg.n_head)   # causal: half of 4BHS^2D
         return 2.0 * per_tok * B * S + attn
+
+
+class GraphedForward:
+    """A captured forward pass: copy new token ids in, replay, read `logits` (a buffer
+    owned by the graph, overwritten by the next replay)."""
+
+    def __init__(self, graph, ids: torch.Tensor, logits: torch.Tensor):
+        self.graph, self.ids, self.logits = graph, ids, logits
+
+    def __call__(self, ids: torch.Tensor) -> torch.Tensor:
+        if ids.shape != self.ids.shape or ids.dtype != self.ids.dtype:
+            raise ValueError("captured for ids of shape %s" % (tuple(self.ids.shape),))
+        self.ids.copy_(ids)
+        self.graph.replay()
+        return self.logits

@@ -144,10 +144,11 @@ def test_gemm_4096_sampled_rows():
     assert torch.equal(kernels.matmul(a * 2, b), c * 2)
 
 
-# Shapes with >= 192 tiles of 256x256: served by the four-wave kernel with the
-# hand-scheduled main loop (K stages of 32: single stage, exit after each position of the
-# unrolled ring, ragged M / N, every operand layout).
-BIG = [(4096, 3072, 32), (3585, 3848, 96), (4000, 3608, 160), (3600, 4104, 448), (8192, 2304, 768)]
+# Shapes with >= 192 tiles of 256x256 for the four-wave kernel with the hand-scheduled
+# main loop (K stages of 32: a single stage, exits at several positions of the unrolled
+# ring of ten stages, more than one trip through it, ragged M / N, every operand layout).
+BIG = [(4096, 3072, 32), (3585, 3848, 96), (4000, 3608, 160), (3600, 4104, 448), (8192, 2304, 768),
+       (4096, 4096, 1056)]
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=lambda d: NAME[d])
@@ -161,7 +162,11 @@ def test_gemm_large_tiles(shape, layout, dtype):
     a, b = _ab(M, N, K, dtype, 27, ta, tb)
     rng = np.random.default_rng(28)
     bias = to_dev(rng.standard_normal(N) * 0.5, dtype)
-    c = kernels.matmul(a, b, bias, "relu", trans_a=ta, trans_b=tb)
+    os.environ["MHIP_GEMM_TILE"] = "2560"      # this kernel also where the default picks another (short K)
+    try:
+        c = kernels.matmul(a, b, bias, "relu", trans_a=ta, trans_b=tb)
+    finally:
+        del os.environ["MHIP_GEMM_TILE"]
     assert c.shape == (M, N)
     rows = np.unique(np.r_[0, 127, 128, 255, 256, M - 1, rng.integers(0, M, 42)])
     A = as_f64(a).T if ta else as_f64(a)

@@ -69,3 +69,22 @@ def test_gpt2_small_baseline_shape():
     from metalhlo_amd import kernels
     nxt = kernels.argmax(logits[:, -1].contiguous())
     assert torch.equal(nxt.long(), logits[:, -1].float().argmax(-1))
+
+
+def test_gpt2_graph_replay_matches_eager():
+    """A captured forward pass replayed several times, with eager work and
+    synchronisations between the replays, reproduces the eager logits bit for bit."""
+    from metalhlo_amd.gpt2 import GPT2, GPT2Config, init_params
+    cfg = GPT2Config(n_layer=2, d_model=128, n_head=4, d_ff=512, vocab=1000, n_pos=64)
+    model = GPT2(cfg, init_params(cfg, seed=11))
+    rng = np.random.default_rng(12)
+    ids = [torch.from_numpy(rng.integers(0, cfg.vocab, (2, 64)).astype(np.int32)).cuda() for _ in range(4)]
+    graphed = model.capture(ids[0])
+    for k in (0, 1, 2, 3, 1):
+        eager = model.forward(ids[k]).clone()
+        torch.cuda.synchronize()
+        got = graphed(ids[k]).clone()
+        torch.cuda.synchronize()
+        assert torch.equal(got, eager), f"replay for ids[{k}] differs from the eager pass"
+    with pytest.raises(ValueError):
+        graphed(ids[0][:1])
