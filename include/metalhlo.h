@@ -182,6 +182,11 @@ MHLOStatusCode mhlo_execute_with_profile(MHLOExecutableRef executable,
 /* metalhlo.h:397 */
 void mhlo_free_string(const char* str);
 
+/* Extension, not part of the reference's header: the operations an executable runs
+ * after pattern recognition, in program order, comma-separated (custom calls by their
+ * target name).  Returns a malloc'd string; release with mhlo_free_string. */
+char* mhlo_ext_executable_ops(MHLOExecutableRef executable);
+
 #ifdef __cplusplus
 }
 #endif

@@ -66,6 +66,7 @@ SIGNATURES = {
     "mhlo_execute_with_profile": (C.c_int, [_vp, C.POINTER(_vp), _i32, C.POINTER(_vp), C.POINTER(_i32),
                                             C.POINTER(ExecutionProfile)]),
     "mhlo_free_string": (None, [_vp]),
+    "mhlo_ext_executable_ops": (_vp, [_vp]),     # extension: op list after pattern recognition
 }
 
 _lib = None
@@ -109,10 +110,24 @@ class Session:
             self.lib.mhlo_client_destroy(self.client)
             self.client = _vp()
 
-    def compile(self, mlir: str):
+    def compile(self, mlir: str, opt_level: int = None):
         exe = _vp()
-        _check(self.lib.mhlo_compile(self.client, mlir.encode(), C.byref(exe)))
+        if opt_level is None:
+            _check(self.lib.mhlo_compile(self.client, mlir.encode(), C.byref(exe)))
+        else:
+            cfg = CompileConfig()
+            self.lib.mhlo_compile_config_init(C.byref(cfg))
+            cfg.optimization_level = opt_level
+            _check(self.lib.mhlo_compile_with_config(self.client, mlir.encode(), C.byref(cfg), C.byref(exe)))
         return exe
+
+    def ops(self, exe):
+        """Names of the operations the executable runs (custom calls by target)."""
+        p = self.lib.mhlo_ext_executable_ops(exe)
+        try:
+            return C.string_at(p).decode().split(",") if p else []
+        finally:
+            self.lib.mhlo_free_string(p)
 
     def buffer(self, array: np.ndarray, element_type: str):
         a = np.ascontiguousarray(array)

@@ -56,6 +56,9 @@ MHLOStatusCode compile_text(MHLOClientRef client, const std::string& text, const
         exe->client = static_cast<Client*>(client);
         exe->opt_level = cfg ? (int)cfg->optimization_level : (int)MHLO_OPT_O2;
         exe->fn = parse_module(text);
+        // O0 runs the module as written; every other level recognises the fused patterns
+        // (Sources/MetalHLO/CompilationConfig.swift:232-263 enables the fusion passes from O1)
+        if (exe->opt_level >= (int)MHLO_OPT_O1) fuse_patterns(exe->fn);
         compile(*exe);
     });
     if (st != MHLO_OK) { delete exe; return st; }
@@ -358,5 +361,20 @@ MHLOStatusCode mhlo_execute_with_profile(MHLOExecutableRef executable, const MHL
 }
 
 void mhlo_free_string(const char* str) { free(const_cast<char*>(str)); }
+
+// Extension (no counterpart in the reference's header): the operations an
+// executable runs after pattern recognition, in program order, separated by
+// commas; custom calls appear as their target name.  Caller frees with
+// mhlo_free_string.
+char* mhlo_ext_executable_ops(MHLOExecutableRef executable) {
+    if (!executable) { set_error(MHLO_ERROR_INVALID_ARGUMENT, "executable is null"); return nullptr; }
+    const Executable* exe = static_cast<const Executable*>(executable);
+    std::string out;
+    for (const Op& op : exe->fn.ops) {
+        if (!out.empty()) out += ",";
+        out += op.name == "custom_call" ? op.target : op.name;
+    }
+    return strdup(out.c_str());
+}
 
 }  // extern "C"

@@ -1,0 +1,592 @@
+// Pattern recogniser: rewrites decomposed StableHLO subgraphs into the fused
+// custom_calls the kernels serve -- the job of the reference's SoftmaxPattern /
+// GELUPattern / LayerNormPattern / RMSNormPattern / AttentionPattern
+// (Sources/MetalHLOCore/Optimizer/FusionPatterns.swift:18-1142) and of its
+// MatMulBiasActFusionPass (Compiler/PassManager.swift:1436-1570).
+//
+// A match is only rewritten when every interior value is used inside the pattern
+// alone (the reference's rule, Analyzer.swift:1715-1721): that is what makes the
+// rewrite semantics-preserving.  Matching is structural and strict: constants
+// must have the right values, reductions the right axis and neutral element, and
+// commutative operands are accepted in either order.  Forms the kernels would
+// answer differently (erf GELU, attention with dropout, ...) are left unfused.
+#include <math.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <algorithm>
+#include <set>
+
+#include "hlo.h"
+
+namespace mhlo {
+namespace {
+
+struct Rewriter {
+    Function& fn;
+    std::map<int, size_t> def;          // value id -> index of the op that defines it
+    std::map<int, TensorType> type;     // value id -> type
+    std::vector<bool> dead;
+    int fused = 0;
+
+    explicit Rewriter(Function& f) : fn(f) { reindex(); }
+
+    void reindex() {
+        def.clear();
+        type.clear();
+        for (size_t i = 0; i < fn.arg_ids.size(); i++) type[fn.arg_ids[i]] = fn.arg_types[i];
+        for (size_t i = 0; i < fn.ops.size(); i++) {
+            def[fn.ops[i].result] = i;
+            type[fn.ops[i].result] = fn.ops[i].out;
+        }
+        dead.assign(fn.ops.size(), false);
+    }
+
+    const Op* op_of(int v) const {
+        auto it = def.find(v);
+        return (it == def.end() || dead[it->second]) ? nullptr : &fn.ops[it->second];
+    }
+    const Op* op_named(int v, const char* name) const {
+        const Op* o = op_of(v);
+        return (o && o->name == name) ? o : nullptr;
+    }
+    size_t index_of(const Op* o) const { return (size_t)(o - fn.ops.data()); }
+
+    // every use of the values defined by `interior` ops (root excluded) lies inside the pattern
+    bool closed(const std::set<size_t>& interior, size_t root) const {
+        std::set<int> vals;
+        for (size_t i : interior)
+            if (i != root) vals.insert(fn.ops[i].result);
+        for (int r : fn.returns)
+            if (vals.count(r)) return false;
+        for (size_t i = 0; i < fn.ops.size(); i++) {
+            if (dead[i] || interior.count(i)) continue;
+            for (int v : fn.ops[i].operands)
+                if (vals.count(v)) return false;
+        }
+        return true;
+    }
+
+    static bool decode(const Op& c, double& out) {
+        if (c.name != "constant" || (!c.splat && c.out.numel() != 1)) return false;
+        uint64_t bits = c.splat_bits;
+        if (!c.splat) {
+            if (c.constant.empty()) return false;
+            bits = 0;
+            memcpy(&bits, c.constant.data(), std::min<size_t>(8, c.constant.size()));
+        }
+        switch (c.out.dtype) {
+            case F32: { float f; memcpy(&f, &bits, 4); out = f; return true; }
+            case F64: { memcpy(&out, &bits, 8); return true; }
+            case BF16: { uint32_t w = (uint32_t)(bits & 0xFFFF) << 16; float f; memcpy(&f, &w, 4); out = f; return true; }
+            case F16: {
+                const uint32_t h = bits & 0xFFFF, s = (h >> 15) & 1, e = (h >> 10) & 31, m = h & 1023;
+                double v = e == 0 ? ldexp((double)m, -24) : e == 31 ? (m ? NAN : INFINITY) : ldexp((double)(m | 1024), (int)e - 25);
+                out = s ? -v : v;
+                return true;
+            }
+            case I32: { int32_t v; memcpy(&v, &bits, 4); out = v; return true; }
+            case I64: { int64_t v; memcpy(&v, &bits, 8); out = (double)v; return true; }
+            default: return false;
+        }
+    }
+
+    // the single value a tensor is filled with: a splat constant, possibly behind
+    // broadcast_in_dim / reshape / convert
+    bool splat_value(int v, double& out, std::set<size_t>* via = nullptr) const {
+        for (int hop = 0; hop < 4; hop++) {
+            const Op* o = op_of(v);
+            if (!o) return false;
+            if (o->name == "constant") return decode(*o, out);
+            if (o->name != "broadcast_in_dim" && o->name != "reshape" && o->name != "convert") return false;
+            if (via) via->insert(index_of(o));
+            v = o->operands.at(0);
+        }
+        return false;
+    }
+
+    static bool near(double a, double b, double tol) { return fabs(a - b) <= tol; }
+
+    // dims of a broadcast_in_dim that puts an operand of rank r-1 back over every axis but `axis`
+    static bool dims_skip_axis(const std::vector<int64_t>& dims, size_t rank, int64_t axis) {
+        if (dims.size() + 1 != rank) return false;
+        int64_t d = 0;
+        for (int64_t got : dims) {
+            if (d == axis) d++;
+            if (got != d++) return false;
+        }
+        return true;
+    }
+
+    // reduce of `x` over the single axis `axis` with `reducer`; the neutral element is checked
+    const Op* reduce_over(int v, const char* reducer, int64_t& axis, int& x) const {
+        const Op* r = op_named(v, "reduce");
+        if (!r || r->reducer != reducer || r->dims.size() != 1 || r->operands.size() != 2) return nullptr;
+        double init;
+        if (!splat_value(r->operands[1], init)) return nullptr;
+        if (!strcmp(reducer, "add") ? init != 0.0 : !(init <= -1e30)) return nullptr;
+        axis = r->dims[0];
+        x = r->operands[0];
+        return r;
+    }
+
+    void replace(size_t root, const std::set<size_t>& interior, const std::string& target,
+                 const std::vector<int>& operands, const std::string& config) {
+        Op& o = fn.ops[root];
+        o.name = "custom_call";
+        o.target = target;
+        o.backend_config = config;
+        o.operands = operands;
+        o.in_types.clear();
+        for (int v : operands) o.in_types.push_back(type.at(v));
+        o.attrs.clear();
+        o.dims.clear();
+        for (size_t i : interior)
+            if (i != root) dead[i] = true;
+        fused++;
+    }
+
+    // ------------------------------------------------------------------ softmax
+    // divide(e, bcast(reduce_add(e))), e = exp(subtract(x, bcast(reduce_max(x))))
+    bool softmax(size_t ri) {
+        const Op& root = fn.ops[ri];
+        if (root.name != "divide" || !dtype_is_float(root.out.dtype)) return false;
+        const Op* e = op_named(root.operands[0], "exponential");
+        const Op* sb = op_named(root.operands[1], "broadcast_in_dim");
+        if (!e || !sb) return false;
+        int64_t ax_s, ax_m;
+        int e_in, x;
+        const Op* s = reduce_over(sb->operands[0], "add", ax_s, e_in);
+        if (!s || e_in != e->result) return false;
+        const size_t rank = root.out.shape.size();
+        if (!dims_skip_axis(sb->dims, rank, ax_s)) return false;
+        const Op* sh = op_named(e->operands[0], "subtract");
+        if (!sh) return false;
+        const Op* mb = op_named(sh->operands[1], "broadcast_in_dim");
+        if (!mb) return false;
+        const Op* m = reduce_over(mb->operands[0], "maximum", ax_m, x);
+        if (!m || ax_m != ax_s || x != sh->operands[0] || !dims_skip_axis(mb->dims, rank, ax_m)) return false;
+        if (!(type.at(x) == root.out)) return false;
+        std::set<size_t> in = {ri, index_of(e), index_of(sb), index_of(s), index_of(sh), index_of(mb), index_of(m)};
+        if (!closed(in, ri)) return false;
+        char cfg[64];
+        snprintf(cfg, sizeof cfg, "{\"axis\": %lld}", (long long)ax_s);
+        replace(ri, in, "fused_softmax", {x}, cfg);
+        return true;
+    }
+
+    // ------------------------------------------------------------------ GELU (tanh form)
+    // leaves of a product: nested multiplies are opened while their value has no other use
+    void product_leaves(int v, bool is_root, std::vector<int>& leaves, std::set<size_t>& nodes) const {
+        const Op* o = op_named(v, "multiply");
+        if (o && (is_root || uses(v) == 1)) {
+            nodes.insert(index_of(o));
+            product_leaves(o->operands[0], false, leaves, nodes);
+            product_leaves(o->operands[1], false, leaves, nodes);
+        } else {
+            leaves.push_back(v);
+        }
+    }
+    int uses(int v) const {
+        int n = 0;
+        for (int r : fn.returns) n += r == v;
+        for (size_t i = 0; i < fn.ops.size(); i++)
+            if (!dead[i])
+                for (int u : fn.ops[i].operands) n += u == v;
+        return n;
+    }
+    // add(const c, other) in either order
+    const Op* add_const(int v, double c, double tol, int& other, std::set<size_t>& nodes) const {
+        const Op* a = op_named(v, "add");
+        if (!a) return nullptr;
+        for (int k = 0; k < 2; k++) {
+            double got;
+            if (splat_value(a->operands[k], got) && near(got, c, tol)) {
+                other = a->operands[1 - k];
+                nodes.insert(index_of(a));
+                return a;
+            }
+        }
+        return nullptr;
+    }
+
+    bool gelu(size_t ri) {
+        const Op& root = fn.ops[ri];
+        if (root.name != "multiply" || !dtype_is_float(root.out.dtype)) return false;
+        std::vector<int> leaves;
+        std::set<size_t> in;
+        product_leaves(root.result, true, leaves, in);
+        if (leaves.size() != 3) return false;
+        int x = -1, opt = -1, halves = 0, t = -1;
+        for (int v : leaves) {
+            double c;
+            int inner;
+            std::set<size_t> tmp;
+            if (splat_value(v, c) && near(c, 0.5, 1e-6)) halves++;
+            else if (add_const(v, 1.0, 1e-6, inner, tmp) && op_named(inner, "tanh")) { opt = v; t = inner; in.insert(tmp.begin(), tmp.end()); }
+            else x = v;
+        }
+        if (halves != 1 || x < 0 || opt < 0) return false;
+        const Op* th = op_named(t, "tanh");
+        in.insert(index_of(th));
+        // tanh argument: sqrt(2/pi) * (x + 0.044715 x^3)
+        std::vector<int> l2;
+        product_leaves(th->operands[0], true, l2, in);
+        if (l2.size() != 2) return false;
+        int inner = -1, ks = 0;
+        for (int v : l2) {
+            double c;
+            if (splat_value(v, c) && near(c, 0.7978845608028654, 0.01)) ks++;
+            else inner = v;
+        }
+        if (ks != 1 || inner < 0) return false;
+        const Op* ia = op_named(inner, "add");
+        if (!ia) return false;
+        in.insert(index_of(ia));
+        int cubic = ia->operands[0] == x ? ia->operands[1] : ia->operands[1] == x ? ia->operands[0] : -1;
+        if (cubic < 0) return false;
+        std::vector<int> l3;
+        product_leaves(cubic, true, l3, in);
+        int xs = 0, cs = 0;
+        for (int v : l3) {
+            double c;
+            if (v == x) xs++;
+            else if (splat_value(v, c) && near(c, 0.044715, 0.005)) cs++;
+            else return false;
+        }
+        if (xs != 3 || cs != 1 || !(type.at(x) == root.out)) return false;
+        if (!closed(in, ri)) return false;
+        replace(ri, in, "fused_gelu", {x}, "{\"approximate\": true}");
+        return true;
+    }
+
+    // ------------------------------------------------------------------ LayerNorm / RMSNorm
+    // mean over the last axis: reduce_add(u) / N  or  reduce_add(u) * (1/N)
+    bool mean_last(int v, int& u, std::set<size_t>& nodes) const {
+        const Op* o = op_of(v);
+        if (!o || (o->name != "divide" && o->name != "multiply")) return false;
+        for (int k = 0; k < 2; k++) {
+            if (o->name == "divide" && k == 1) break;
+            double c;
+            int64_t axis;
+            int src;
+            std::set<size_t> via;
+            const Op* r = reduce_over(o->operands[k], "add", axis, src);
+            if (!r || !splat_value(o->operands[1 - k], c, &via)) continue;
+            const auto& shp = type.at(src).shape;
+            if (shp.empty() || axis != (int64_t)shp.size() - 1) continue;
+            const double n = (double)shp.back();
+            if (o->name == "divide" ? !near(c, n, 1e-6 * n) : !near(c * n, 1.0, 1e-5)) continue;
+            u = src;
+            nodes.insert(index_of(o));
+            nodes.insert(index_of(r));
+            return true;
+        }
+        return false;
+    }
+    // v = broadcast over the last axis of a [.., 1]-less statistic
+    const Op* bcast_stat(int v, size_t rank) const {
+        const Op* b = op_named(v, "broadcast_in_dim");
+        return (b && dims_skip_axis(b->dims, rank, (int64_t)rank - 1)) ? b : nullptr;
+    }
+    // v = c * bcast(rsqrt(mean(c*c) + eps)); centred: c = x - bcast(mean(x))
+    bool norm_core(int v, int& x, double& eps, bool& centred, std::set<size_t>& nodes) const {
+        const Op* m = op_named(v, "multiply");
+        if (!m) return false;
+        const size_t rank = m->out.shape.size();
+        if (rank < 1) return false;
+        for (int k = 0; k < 2; k++) {
+            const Op* rb = bcast_stat(m->operands[k], rank);
+            if (!rb) continue;
+            const int c = m->operands[1 - k];
+            const Op* rs = op_named(rb->operands[0], "rsqrt");
+            if (!rs) continue;
+            const Op* ve = op_named(rs->operands[0], "add");
+            if (!ve) continue;
+            std::set<size_t> tmp = {index_of(m), index_of(rb), index_of(rs), index_of(ve)};
+            for (int j = 0; j < 2; j++) {
+                double e;
+                int sq;
+                std::set<size_t> t2 = tmp;
+                if (!splat_value(ve->operands[j], e) || !(e > 0 && e < 1e-1)) continue;
+                if (!mean_last(ve->operands[1 - j], sq, t2)) continue;
+                const Op* sqo = op_named(sq, "multiply");
+                if (!sqo || sqo->operands[0] != c || sqo->operands[1] != c) continue;
+                t2.insert(index_of(sqo));
+                const Op* sub = op_named(c, "subtract");
+                const Op* mb = sub ? bcast_stat(sub->operands[1], rank) : nullptr;
+                int mx;
+                std::set<size_t> t3 = t2;
+                if (sub && mb && mean_last(mb->operands[0], mx, t3) && mx == sub->operands[0]) {
+                    t3.insert(index_of(sub));
+                    t3.insert(index_of(mb));
+                    x = mx;
+                    centred = true;
+                    nodes.insert(t3.begin(), t3.end());
+                } else {
+                    x = c;
+                    centred = false;
+                    nodes.insert(t2.begin(), t2.end());
+                }
+                eps = e;
+                return true;
+            }
+        }
+        return false;
+    }
+    // v = bcast of a [cols] vector along the last axis
+    bool param_vector(int v, size_t rank, int64_t cols, int dtype, int& vec, std::set<size_t>& nodes) const {
+        const Op* b = op_named(v, "broadcast_in_dim");
+        if (!b || b->dims != std::vector<int64_t>{(int64_t)rank - 1}) return false;
+        const TensorType& t = type.at(b->operands[0]);
+        if (t.shape != std::vector<int64_t>{cols} || t.dtype != dtype) return false;
+        vec = b->operands[0];
+        nodes.insert(index_of(b));
+        return true;
+    }
+
+    bool norm(size_t ri) {
+        const Op& root = fn.ops[ri];
+        if (!dtype_is_float(root.out.dtype) || root.out.dtype == F64 || root.out.shape.empty()) return false;
+        const size_t rank = root.out.shape.size();
+        const int64_t cols = root.out.shape.back();
+        int x, gamma = -1, beta = -1;
+        double eps;
+        bool centred;
+        std::set<size_t> in = {ri};
+        if (root.name == "add") {            // (core * gamma) + beta
+            for (int k = 0; k < 2; k++) {
+                std::set<size_t> t = {ri};
+                int b;
+                if (!param_vector(root.operands[k], rank, cols, root.out.dtype, b, t)) continue;
+                const Op* y = op_named(root.operands[1 - k], "multiply");
+                if (!y) continue;
+                for (int j = 0; j < 2; j++) {
+                    std::set<size_t> t2 = t;
+                    int g;
+                    t2.insert(index_of(y));
+                    if (!param_vector(y->operands[j], rank, cols, root.out.dtype, g, t2)) continue;
+                    if (!norm_core(y->operands[1 - j], x, eps, centred, t2) || !centred) continue;
+                    if (!closed(t2, ri)) continue;
+                    char cfg[96];
+                    snprintf(cfg, sizeof cfg, "{\"eps\": %.9g, \"axes\": [-1]}", eps);
+                    replace(ri, t2, "fused_layer_norm", {x, g, b}, cfg);
+                    return true;
+                }
+            }
+            return false;
+        }
+        if (root.name != "multiply") return false;
+        // core * gamma (RMSNorm)
+        for (int j = 0; j < 2; j++) {
+            std::set<size_t> t2 = {ri};
+            int g;
+            if (!param_vector(root.operands[j], rank, cols, root.out.dtype, g, t2)) continue;
+            if (!norm_core(root.operands[1 - j], x, eps, centred, t2) || centred) continue;
+            if (!closed(t2, ri)) continue;
+            char cfg[96];
+            snprintf(cfg, sizeof cfg, "{\"eps\": %.9g, \"axes\": [-1]}", eps);
+            replace(ri, t2, "fused_rms_norm", {x, g}, cfg);
+            return true;
+        }
+        (void)gamma; (void)beta; (void)in;
+        return false;
+    }
+
+    // ------------------------------------------------------------------ attention
+    static bool iota_prefix(const std::vector<int64_t>& v, size_t n) {
+        if (v.size() != n) return false;
+        for (size_t i = 0; i < n; i++)
+            if (v[i] != (int64_t)i) return false;
+        return true;
+    }
+    bool attention(size_t ri) {
+        const Op& pv = fn.ops[ri];
+        if (pv.name != "dot_general" || !dtype_is_float(pv.out.dtype) || pv.out.dtype == F64) return false;
+        const size_t r = pv.out.shape.size();
+        if (r < 2 || r > 4) return false;
+        const std::vector<int64_t> last = {(int64_t)r - 1}, prev = {(int64_t)r - 2};
+        if (!iota_prefix(pv.lhs_batch, r - 2) || !iota_prefix(pv.rhs_batch, r - 2) || pv.lhs_contract != last ||
+            pv.rhs_contract != prev)
+            return false;
+        const Op* p = op_named(pv.operands[0], "custom_call");
+        if (!p || p->target != "fused_softmax") return false;
+        const long long axis = parse_config(p->backend_config).get_int("axis", -1);
+        if (axis != -1 && axis != (long long)r - 1) return false;
+        std::set<size_t> in = {ri, index_of(p)};
+        int cur = p->operands[0], mask = -1;
+        double scale = 1.0;
+        if (const Op* a = op_named(cur, "add")) {          // scores + mask
+            const bool lhs_scores = op_named(a->operands[0], "multiply") || op_named(a->operands[0], "divide") ||
+                                    op_named(a->operands[0], "dot_general");
+            mask = a->operands[lhs_scores ? 1 : 0];
+            cur = a->operands[lhs_scores ? 0 : 1];
+            in.insert(index_of(a));
+        }
+        if (const Op* m = op_named(cur, "multiply")) {      // scores * scale
+            double c;
+            int k = splat_value(m->operands[1], c) ? 1 : splat_value(m->operands[0], c) ? 0 : -1;
+            if (k < 0) return false;
+            scale = c;
+            cur = m->operands[1 - k];
+            in.insert(index_of(m));
+        } else if (const Op* d = op_named(cur, "divide")) { // scores / sqrt(D)
+            double c;
+            if (!splat_value(d->operands[1], c) || c == 0.0) return false;
+            scale = 1.0 / c;
+            cur = d->operands[0];
+            in.insert(index_of(d));
+        }
+        const Op* qk = op_named(cur, "dot_general");
+        if (!qk || !iota_prefix(qk->lhs_batch, r - 2) || !iota_prefix(qk->rhs_batch, r - 2) || qk->lhs_contract != last)
+            return false;
+        in.insert(index_of(qk));
+        const int q = qk->operands[0], v = pv.operands[1];
+        int k = qk->operands[1];
+        if (qk->rhs_contract == prev) {                     // explicit transpose of K
+            const Op* t = op_named(k, "transpose");
+            if (!t || t->dims.size() != r) return false;
+            for (size_t i = 0; i + 2 < r; i++)
+                if (t->dims[i] != (int64_t)i) return false;
+            if (t->dims[r - 2] != (int64_t)r - 1 || t->dims[r - 1] != (int64_t)r - 2) return false;
+            in.insert(index_of(t));
+            k = t->operands[0];
+        } else if (qk->rhs_contract != last) {
+            return false;
+        }
+        const TensorType &qt = type.at(q), &kt = type.at(k), &vt = type.at(v);
+        if (qt.dtype != pv.out.dtype || !(kt == vt) || kt.dtype != qt.dtype || qt.shape.size() != r || kt.shape.size() != r)
+            return false;
+        if (qt.shape[r - 1] != kt.shape[r - 1]) return false;
+        for (size_t i = 0; i + 2 < r; i++)
+            if (qt.shape[i] != kt.shape[i]) return false;
+        if (mask >= 0) {
+            // a mask broadcast along leading axes only need not be materialised
+            if (const Op* mbc = op_named(mask, "broadcast_in_dim")) {
+                const size_t mr0 = type.at(mbc->operands[0]).shape.size();
+                bool trailing = mbc->dims.size() == mr0 && mr0 >= 2 && mr0 <= r;
+                for (size_t i = 0; trailing && i < mr0; i++) trailing = mbc->dims[i] == (int64_t)(r - mr0 + i);
+                if (trailing && uses(mask) == 1) {
+                    in.insert(index_of(mbc));
+                    mask = mbc->operands[0];
+                }
+            }
+        }
+        if (mask >= 0) {                                    // must end in [Sq, Skv] and broadcast over batch / heads
+            const TensorType& mt = type.at(mask);
+            const size_t mr = mt.shape.size();
+            const int64_t Sq = qt.shape[r - 2], Skv = kt.shape[r - 2];
+            if (mt.dtype != qt.dtype || mr < 2 || mr > r || mt.shape[mr - 1] != Skv || mt.shape[mr - 2] != Sq) return false;
+            const int64_t H = r >= 3 ? qt.shape[r - 3] : 1;
+            int64_t B = 1, mb = 1;
+            for (size_t i = 0; i + 3 < r; i++) B *= qt.shape[i];
+            const int64_t mh = mr >= 3 ? mt.shape[mr - 3] : 1;
+            for (size_t i = 0; i + 3 < mr; i++) mb *= mt.shape[i];
+            if ((mh != 1 && mh != H) || (mb != 1 && mb != B)) return false;
+        }
+        if (!closed(in, ri)) return false;
+        char cfg[128];
+        snprintf(cfg, sizeof cfg, "{\"scale\": %.9g, \"has_mask\": %s, \"is_causal\": false}", scale, mask >= 0 ? "true" : "false");
+        std::vector<int> ops = {q, k, v};
+        if (mask >= 0) ops.push_back(mask);
+        replace(ri, in, "fused_scaled_dot_product_attention", ops, cfg);
+        return true;
+    }
+
+    // ------------------------------------------------------------------ matmul + bias (+ activation)
+    bool plain_matmul(const Op* d) const {
+        if (!d || (d->name != "dot" && d->name != "dot_general") || d->operands.size() != 2) return false;
+        const TensorType &xt = type.at(d->operands[0]), &wt = type.at(d->operands[1]);
+        if (wt.shape.size() != 2 || xt.shape.size() < 2 || !dtype_is_float(xt.dtype) || xt.dtype == F64 || wt.dtype != xt.dtype)
+            return false;
+        if (d->name == "dot") return xt.shape.size() == 2;
+        if (d->name != "dot_general") return false;
+        return d->lhs_batch.empty() && d->rhs_batch.empty() &&
+               d->lhs_contract == std::vector<int64_t>{(int64_t)xt.shape.size() - 1} &&
+               d->rhs_contract == std::vector<int64_t>{0};
+    }
+    bool matmul_bias_act(size_t ri) {
+        const Op& root = fn.ops[ri];
+        std::string act = "none";
+        std::set<size_t> in = {ri};
+        const Op* add = nullptr;
+        if (root.name == "add") {
+            add = &root;
+        } else {
+            int src = -1;
+            if (root.name == "tanh") { act = "tanh"; src = root.operands[0]; }
+            else if (root.name == "logistic") { act = "sigmoid"; src = root.operands[0]; }
+            else if (root.name == "custom_call" && root.target == "fused_gelu") { act = "gelu"; src = root.operands[0]; }
+            else if (root.name == "maximum") {
+                double c;
+                for (int k = 0; k < 2; k++)
+                    if (splat_value(root.operands[k], c) && c == 0.0) { act = "relu"; src = root.operands[1 - k]; }
+            }
+            if (src < 0) return false;
+            add = op_named(src, "add");
+            if (!add) return false;
+            in.insert(index_of(add));
+        }
+        const size_t rank = add->out.shape.size();
+        if (rank < 2) return false;
+        for (int k = 0; k < 2; k++) {
+            std::set<size_t> t = in;
+            int bias;
+            if (!param_vector(add->operands[k], rank, add->out.shape.back(), add->out.dtype, bias, t)) continue;
+            const Op* d = op_of(add->operands[1 - k]);
+            if (!plain_matmul(d)) continue;
+            t.insert(index_of(d));
+            if (!closed(t, ri)) continue;
+            const std::vector<int> ops = {d->operands[0], d->operands[1], bias};
+            replace(ri, t, "fused_matmul_bias_activation", ops, "{\"activation\": \"" + act + "\"}");
+            return true;
+        }
+        return false;
+    }
+
+    // drop rewritten ops and everything that has become unused
+    void sweep() {
+        bool changed = true;
+        while (changed) {
+            changed = false;
+            for (size_t i = fn.ops.size(); i-- > 0;) {
+                if (dead[i]) continue;
+                if (uses(fn.ops[i].result) == 0) { dead[i] = true; changed = true; }
+            }
+        }
+        std::vector<Op> keep;
+        for (size_t i = 0; i < fn.ops.size(); i++)
+            if (!dead[i]) keep.push_back(std::move(fn.ops[i]));
+        fn.ops = std::move(keep);
+        reindex();
+    }
+
+    template <typename F>
+    void pass(F&& try_at) {
+        for (size_t i = fn.ops.size(); i-- > 0;)
+            if (!dead[i]) try_at(i);
+        sweep();
+    }
+};
+
+}  // namespace
+
+int fuse_patterns(Function& fn) {
+    // malformed operations are reported by the validation that follows; do not look inside them
+    static const std::map<std::string, size_t> kArity = {
+        {"add", 2}, {"subtract", 2}, {"multiply", 2}, {"divide", 2}, {"maximum", 2}, {"minimum", 2}, {"dot", 2},
+        {"dot_general", 2}, {"reduce", 2}, {"exponential", 1}, {"tanh", 1}, {"rsqrt", 1}, {"logistic", 1},
+        {"broadcast_in_dim", 1}, {"reshape", 1}, {"convert", 1}, {"transpose", 1}};
+    for (const Op& op : fn.ops) {
+        auto it = kArity.find(op.name);
+        if (it != kArity.end() && op.operands.size() != it->second) return 0;
+        for (int v : op.operands)
+            if (v < 0 || v >= fn.num_values) return 0;
+    }
+    Rewriter rw(fn);
+    rw.pass([&](size_t i) { rw.softmax(i) || rw.gelu(i) || rw.norm(i); });
+    rw.pass([&](size_t i) { rw.attention(i) || rw.matmul_bias_act(i); });
+    return rw.fused;
+}
+
+}  // namespace mhlo

@@ -73,6 +73,11 @@ struct Function {
 // (`main` when present, else the first).  Throws ParseError / UnsupportedOp.
 Function parse_module(const std::string& text);
 
+// Rewrites decomposed softmax / GELU(tanh) / LayerNorm / RMSNorm / attention /
+// matmul+bias+activation subgraphs into the fused custom_calls (fusion.cpp); returns the
+// number of rewrites.  Values used outside a pattern are never absorbed.
+int fuse_patterns(Function& fn);
+
 // Flat JSON object {"k": number | bool | "string" | [numbers]} as used by
 // backend_config (Compiler/CustomCallHandlers.swift:102-168).  Anything that
 // does not parse yields an empty config.

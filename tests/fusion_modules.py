@@ -1,0 +1,153 @@
+"""Decomposed StableHLO modules (the forms JAX-style lowering produces, which the
+reference's pattern detectors accept: Optimizer/FusionPatterns.swift:18-1142) shared by
+the CPU and GPU fusion tests."""
+
+SOFTMAX = """func.func @main(%x: tensor<8x32xf32>) -> tensor<8x32xf32> {
+  %ninf = stablehlo.constant dense<0xFF800000> : tensor<f32>
+  %m = stablehlo.reduce(%x init: %ninf) applies stablehlo.maximum across dimensions = [1] : (tensor<8x32xf32>, tensor<f32>) -> tensor<8xf32>
+  %mb = stablehlo.broadcast_in_dim %m, dims = [0] : (tensor<8xf32>) -> tensor<8x32xf32>
+  %sh = stablehlo.subtract %x, %mb : tensor<8x32xf32>
+  %e = stablehlo.exponential %sh : tensor<8x32xf32>
+  %zero = stablehlo.constant dense<0.0> : tensor<f32>
+  %s = stablehlo.reduce(%e init: %zero) applies stablehlo.add across dimensions = [1] : (tensor<8x32xf32>, tensor<f32>) -> tensor<8xf32>
+  %sb = stablehlo.broadcast_in_dim %s, dims = [0] : (tensor<8xf32>) -> tensor<8x32xf32>
+  %r = stablehlo.divide %e, %sb : tensor<8x32xf32>
+  return %r : tensor<8x32xf32> }"""
+
+# the same chain, but the exponentials are also returned: an interior value escapes
+SOFTMAX_ESCAPING = SOFTMAX.replace("-> tensor<8x32xf32> {", "-> (tensor<8x32xf32>, tensor<8x32xf32>) {") \
+                          .replace("return %r : tensor<8x32xf32>", "return %r, %e : tensor<8x32xf32>, tensor<8x32xf32>")
+
+SOFTMAX_AXIS0 = """func.func @main(%x: tensor<8x32xf32>) -> tensor<8x32xf32> {
+  %ninf = stablehlo.constant dense<0xFF800000> : tensor<f32>
+  %m = stablehlo.reduce(%x init: %ninf) applies stablehlo.maximum across dimensions = [0] : (tensor<8x32xf32>, tensor<f32>) -> tensor<32xf32>
+  %mb = stablehlo.broadcast_in_dim %m, dims = [1] : (tensor<32xf32>) -> tensor<8x32xf32>
+  %sh = stablehlo.subtract %x, %mb : tensor<8x32xf32>
+  %e = stablehlo.exponential %sh : tensor<8x32xf32>
+  %zero = stablehlo.constant dense<0.0> : tensor<f32>
+  %s = stablehlo.reduce(%e init: %zero) applies stablehlo.add across dimensions = [0] : (tensor<8x32xf32>, tensor<f32>) -> tensor<32xf32>
+  %sb = stablehlo.broadcast_in_dim %s, dims = [1] : (tensor<32xf32>) -> tensor<8x32xf32>
+  %r = stablehlo.divide %e, %sb : tensor<8x32xf32>
+  return %r : tensor<8x32xf32> }"""
+
+GELU = """func.func @main(%x: tensor<4x64xf32>) -> tensor<4x64xf32> {
+  %half = stablehlo.constant dense<0.5> : tensor<4x64xf32>
+  %one = stablehlo.constant dense<1.0> : tensor<4x64xf32>
+  %coeff = stablehlo.constant dense<0.044715> : tensor<4x64xf32>
+  %k = stablehlo.constant dense<0.7978845608> : tensor<4x64xf32>
+  %x2 = stablehlo.multiply %x, %x : tensor<4x64xf32>
+  %x3 = stablehlo.multiply %x2, %x : tensor<4x64xf32>
+  %cx3 = stablehlo.multiply %coeff, %x3 : tensor<4x64xf32>
+  %inner = stablehlo.add %x, %cx3 : tensor<4x64xf32>
+  %sc = stablehlo.multiply %k, %inner : tensor<4x64xf32>
+  %t = stablehlo.tanh %sc : tensor<4x64xf32>
+  %opt = stablehlo.add %one, %t : tensor<4x64xf32>
+  %hx = stablehlo.multiply %half, %x : tensor<4x64xf32>
+  %r = stablehlo.multiply %hx, %opt : tensor<4x64xf32>
+  return %r : tensor<4x64xf32> }"""
+
+# wrong cubic coefficient: not GELU, must stay as written
+NOT_GELU = GELU.replace("0.044715", "0.144715")
+
+LAYER_NORM = """func.func @main(%x: tensor<16x64xf32>, %g: tensor<64xf32>, %b: tensor<64xf32>) -> tensor<16x64xf32> {
+  %zero = stablehlo.constant dense<0.0> : tensor<f32>
+  %n = stablehlo.constant dense<64.0> : tensor<16xf32>
+  %eps = stablehlo.constant dense<1.0e-5> : tensor<16xf32>
+  %s = stablehlo.reduce(%x init: %zero) applies stablehlo.add across dimensions = [1] : (tensor<16x64xf32>, tensor<f32>) -> tensor<16xf32>
+  %mean = stablehlo.divide %s, %n : tensor<16xf32>
+  %mb = stablehlo.broadcast_in_dim %mean, dims = [0] : (tensor<16xf32>) -> tensor<16x64xf32>
+  %c = stablehlo.subtract %x, %mb : tensor<16x64xf32>
+  %sq = stablehlo.multiply %c, %c : tensor<16x64xf32>
+  %s2 = stablehlo.reduce(%sq init: %zero) applies stablehlo.add across dimensions = [1] : (tensor<16x64xf32>, tensor<f32>) -> tensor<16xf32>
+  %var = stablehlo.divide %s2, %n : tensor<16xf32>
+  %ve = stablehlo.add %var, %eps : tensor<16xf32>
+  %r = stablehlo.rsqrt %ve : tensor<16xf32>
+  %rb = stablehlo.broadcast_in_dim %r, dims = [0] : (tensor<16xf32>) -> tensor<16x64xf32>
+  %xn = stablehlo.multiply %c, %rb : tensor<16x64xf32>
+  %gb = stablehlo.broadcast_in_dim %g, dims = [1] : (tensor<64xf32>) -> tensor<16x64xf32>
+  %bb = stablehlo.broadcast_in_dim %b, dims = [1] : (tensor<64xf32>) -> tensor<16x64xf32>
+  %y = stablehlo.multiply %xn, %gb : tensor<16x64xf32>
+  %z = stablehlo.add %y, %bb : tensor<16x64xf32>
+  return %z : tensor<16x64xf32> }"""
+
+RMS_NORM = """func.func @main(%x: tensor<16x64xf32>, %g: tensor<64xf32>) -> tensor<16x64xf32> {
+  %zero = stablehlo.constant dense<0.0> : tensor<f32>
+  %rn = stablehlo.constant dense<0.015625> : tensor<16xf32>
+  %eps = stablehlo.constant dense<1.0e-6> : tensor<16xf32>
+  %sq = stablehlo.multiply %x, %x : tensor<16x64xf32>
+  %s2 = stablehlo.reduce(%sq init: %zero) applies stablehlo.add across dimensions = [1] : (tensor<16x64xf32>, tensor<f32>) -> tensor<16xf32>
+  %ms = stablehlo.multiply %s2, %rn : tensor<16xf32>
+  %ve = stablehlo.add %ms, %eps : tensor<16xf32>
+  %r = stablehlo.rsqrt %ve : tensor<16xf32>
+  %rb = stablehlo.broadcast_in_dim %r, dims = [0] : (tensor<16xf32>) -> tensor<16x64xf32>
+  %xn = stablehlo.multiply %x, %rb : tensor<16x64xf32>
+  %gb = stablehlo.broadcast_in_dim %g, dims = [1] : (tensor<64xf32>) -> tensor<16x64xf32>
+  %y = stablehlo.multiply %gb, %xn : tensor<16x64xf32>
+  return %y : tensor<16x64xf32> }"""
+
+
+def attention(B=2, H=3, S=64, D=32, with_mask=False, transpose_k=True, divide=False, dtype="f32"):
+    t = f"tensor<{B}x{H}x{S}x{D}x{dtype}>"
+    st = f"tensor<{B}x{H}x{S}x{S}x{dtype}>"
+    rt = f"tensor<{B}x{H}x{S}x{dtype}>"
+    args = f"%q: {t}, %k: {t}, %v: {t}" + (f", %mask: tensor<{S}x{S}x{dtype}>" if with_mask else "")
+    lines = [f"func.func @main({args}) -> {t} {{"]
+    if transpose_k:
+        kt = f"tensor<{B}x{H}x{D}x{S}x{dtype}>"
+        lines.append(f"  %kt = stablehlo.transpose %k, dims = [0, 1, 3, 2] : ({t}) -> {kt}")
+        lines.append(f"  %s0 = stablehlo.dot_general %q, %kt, batching_dims = [0, 1] x [0, 1], contracting_dims = [3] x [2] : ({t}, {kt}) -> {st}")
+    else:
+        lines.append(f"  %s0 = stablehlo.dot_general %q, %k, batching_dims = [0, 1] x [0, 1], contracting_dims = [3] x [3] : ({t}, {t}) -> {st}")
+    if divide:
+        lines.append(f"  %sc = stablehlo.constant dense<{D ** 0.5!r}> : {st}")
+        lines.append(f"  %s1 = stablehlo.divide %s0, %sc : {st}")
+    else:
+        lines.append(f"  %sc = stablehlo.constant dense<{D ** -0.5!r}> : {st}")
+        lines.append(f"  %s1 = stablehlo.multiply %s0, %sc : {st}")
+    cur = "%s1"
+    if with_mask:
+        lines.append(f"  %mbc = stablehlo.broadcast_in_dim %mask, dims = [2, 3] : (tensor<{S}x{S}x{dtype}>) -> {st}")
+        lines.append(f"  %s2 = stablehlo.add %s1, %mbc : {st}")
+        cur = "%s2"
+    neg = {"f32": "0xFF800000", "bf16": "0xFF80", "f16": "0xFC00"}[dtype]
+    lines += [
+        f"  %ninf = stablehlo.constant dense<{neg}> : tensor<{dtype}>",
+        f"  %zero = stablehlo.constant dense<0.0> : tensor<{dtype}>",
+        f"  %m = stablehlo.reduce({cur} init: %ninf) applies stablehlo.maximum across dimensions = [3] : ({st}, tensor<{dtype}>) -> {rt}",
+        f"  %mb = stablehlo.broadcast_in_dim %m, dims = [0, 1, 2] : ({rt}) -> {st}",
+        f"  %sh = stablehlo.subtract {cur}, %mb : {st}",
+        f"  %e = stablehlo.exponential %sh : {st}",
+        f"  %s = stablehlo.reduce(%e init: %zero) applies stablehlo.add across dimensions = [3] : ({st}, tensor<{dtype}>) -> {rt}",
+        f"  %sb = stablehlo.broadcast_in_dim %s, dims = [0, 1, 2] : ({rt}) -> {st}",
+        f"  %p = stablehlo.divide %e, %sb : {st}",
+        f"  %o = stablehlo.dot_general %p, %v, batching_dims = [0, 1] x [0, 1], contracting_dims = [3] x [2] : ({st}, {t}) -> {t}",
+        f"  return %o : {t} }}"]
+    return "\n".join(lines)
+
+
+FFN_UP = """func.func @main(%x: tensor<32x64xf32>, %w: tensor<64x128xf32>, %b: tensor<128xf32>) -> tensor<32x128xf32> {
+  %d = stablehlo.dot_general %x, %w, contracting_dims = [1] x [0] : (tensor<32x64xf32>, tensor<64x128xf32>) -> tensor<32x128xf32>
+  %bb = stablehlo.broadcast_in_dim %b, dims = [1] : (tensor<128xf32>) -> tensor<32x128xf32>
+  %h = stablehlo.add %d, %bb : tensor<32x128xf32>
+  %half = stablehlo.constant dense<0.5> : tensor<32x128xf32>
+  %one = stablehlo.constant dense<1.0> : tensor<32x128xf32>
+  %coeff = stablehlo.constant dense<0.044715> : tensor<32x128xf32>
+  %k = stablehlo.constant dense<0.7978845608> : tensor<32x128xf32>
+  %h2 = stablehlo.multiply %h, %h : tensor<32x128xf32>
+  %h3 = stablehlo.multiply %h, %h2 : tensor<32x128xf32>
+  %ch3 = stablehlo.multiply %h3, %coeff : tensor<32x128xf32>
+  %inner = stablehlo.add %ch3, %h : tensor<32x128xf32>
+  %sc = stablehlo.multiply %inner, %k : tensor<32x128xf32>
+  %t = stablehlo.tanh %sc : tensor<32x128xf32>
+  %opt = stablehlo.add %t, %one : tensor<32x128xf32>
+  %xo = stablehlo.multiply %h, %opt : tensor<32x128xf32>
+  %r = stablehlo.multiply %half, %xo : tensor<32x128xf32>
+  return %r : tensor<32x128xf32> }"""
+
+MATMUL_BIAS_RELU = """func.func @main(%x: tensor<32x64xf32>, %w: tensor<64x128xf32>, %b: tensor<128xf32>) -> tensor<32x128xf32> {
+  %d = stablehlo.dot %x, %w : (tensor<32x64xf32>, tensor<64x128xf32>) -> tensor<32x128xf32>
+  %bb = stablehlo.broadcast_in_dim %b, dims = [1] : (tensor<128xf32>) -> tensor<32x128xf32>
+  %h = stablehlo.add %bb, %d : tensor<32x128xf32>
+  %zero = stablehlo.constant dense<0.0> : tensor<32x128xf32>
+  %r = stablehlo.maximum %h, %zero : tensor<32x128xf32>
+  return %r : tensor<32x128xf32> }"""

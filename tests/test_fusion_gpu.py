@@ -1,0 +1,105 @@
+"""GPU: modules compiled with pattern recognition (the default) and as written (O0) agree
+with each other and with the float64 oracle; fp32 tolerance 1e-5, bf16 2e-2, with the
+floor max(tol, tol*|e|)."""
+import numpy as np
+import pytest
+
+from oracle import oracle
+from tests import fusion_modules as M
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def sess():
+    from metalhlo_amd import capi
+    s = capi.Session()
+    yield s
+    s.close()
+
+
+def close(got, exp, tol):
+    exp = np.asarray(exp, dtype=np.float64)
+    got = np.asarray(got, dtype=np.float64)
+    assert got.shape == exp.shape
+    assert np.all(np.abs(got - exp) <= np.maximum(tol, tol * np.abs(exp))), np.abs(got - exp).max()
+
+
+def both(sess, text, inputs, expect_op):
+    fused, plain = sess.compile(text), sess.compile(text, 0)
+    assert expect_op in sess.ops(fused) and expect_op not in sess.ops(plain)
+    (a,), (b,) = sess.run(fused, inputs), sess.run(plain, inputs)
+    sess.lib.mhlo_executable_destroy(fused)
+    sess.lib.mhlo_executable_destroy(plain)
+    return a, b
+
+
+def test_softmax_gelu_norms(sess):
+    rng = np.random.default_rng(81)
+    x = rng.standard_normal((8, 32)).astype(np.float32)
+    a, b = both(sess, M.SOFTMAX, [(x, "f32")], "fused_softmax")
+    close(a, oracle.softmax(x.astype(np.float64)), 1e-5)
+    close(b, oracle.softmax(x.astype(np.float64)), 1e-5)
+    a, b = both(sess, M.SOFTMAX_AXIS0, [(x, "f32")], "fused_softmax")
+    close(a, oracle.softmax(x.astype(np.float64), axis=0), 1e-5)
+    close(b, a, 1e-5)
+    x = rng.uniform(-4, 4, (4, 64)).astype(np.float32)
+    a, b = both(sess, M.GELU, [(x, "f32")], "fused_gelu")
+    close(a, oracle.gelu_tanh(x.astype(np.float64)), 1e-5)
+    close(b, oracle.gelu_tanh(x.astype(np.float64)), 1e-5)
+    x = (3 + 2 * rng.standard_normal((16, 64))).astype(np.float32)
+    g = (1 + 0.1 * rng.standard_normal(64)).astype(np.float32)
+    bt = (0.1 * rng.standard_normal(64)).astype(np.float32)
+    a, b = both(sess, M.LAYER_NORM, [(x, "f32"), (g, "f32"), (bt, "f32")], "fused_layer_norm")
+    exp = oracle.layer_norm(x.astype(np.float64), g.astype(np.float64), bt.astype(np.float64), 1e-5)
+    close(a, exp, 1e-5)
+    close(b, exp, 2e-5)      # the decomposed form subtracts the mean in fp32 before squaring
+    a, b = both(sess, M.RMS_NORM, [(x, "f32"), (g, "f32")], "fused_rms_norm")
+    exp = oracle.rms_norm(x.astype(np.float64), g.astype(np.float64), 1e-6)
+    close(a, exp, 1e-5)
+    close(b, exp, 1e-5)
+
+
+@pytest.mark.parametrize("with_mask,transpose_k,divide", [(False, True, False), (True, False, True), (True, True, False)])
+def test_attention_chain(sess, with_mask, transpose_k, divide):
+    B, H, S, D = 2, 3, 64, 32
+    rng = np.random.default_rng(82)
+    q, k, v = (rng.standard_normal((B, H, S, D)).astype(np.float32) for _ in range(3))
+    inputs = [(q, "f32"), (k, "f32"), (v, "f32")]
+    mask = None
+    if with_mask:
+        mask = np.where(np.arange(S)[None, :] > np.arange(S)[:, None], -np.inf, 0.0).astype(np.float32)
+        inputs.append((mask, "f32"))
+    text = M.attention(B, H, S, D, with_mask=with_mask, transpose_k=transpose_k, divide=divide)
+    a, b = both(sess, text, inputs, "fused_scaled_dot_product_attention")
+    exp = oracle.attention(q, k, v, scale=D ** -0.5, mask=mask)
+    close(a, exp, 1e-5)
+    close(b, exp, 1e-5)
+
+
+def test_attention_chain_bf16(sess):
+    B, H, S, D = 1, 4, 128, 64
+    rng = np.random.default_rng(83)
+    bits = [oracle.bf16_round_bits(rng.standard_normal((B, H, S, D)).astype(np.float32)) for _ in range(3)]
+    text = M.attention(B, H, S, D, dtype="bf16")
+    fused = sess.compile(text)
+    assert sess.ops(fused) == ["fused_scaled_dot_product_attention"]
+    (o,) = sess.run(fused, [(x, "bf16") for x in bits])
+    q, k, v = (oracle.bf16_bits_to_f32(x).astype(np.float64) for x in bits)
+    close(oracle.bf16_bits_to_f32(o), oracle.attention(q, k, v, scale=D ** -0.5), 2e-2)
+
+
+def test_matmul_bias_activation(sess):
+    rng = np.random.default_rng(84)
+    x = rng.uniform(-1, 1, (32, 64)).astype(np.float32)
+    w = rng.uniform(-1, 1, (64, 128)).astype(np.float32)
+    bias = rng.standard_normal(128).astype(np.float32)
+    ins = [(x, "f32"), (w, "f32"), (bias, "f32")]
+    a, b = both(sess, M.FFN_UP, ins, "fused_matmul_bias_activation")
+    exp = oracle.matmul_bias_act(x.astype(np.float64), w.astype(np.float64), bias.astype(np.float64), "gelu")
+    close(a, exp, 1e-5)
+    close(b, exp, 1e-5)
+    a, b = both(sess, M.MATMUL_BIAS_RELU, ins, "fused_matmul_bias_activation")
+    exp = oracle.matmul_bias_act(x.astype(np.float64), w.astype(np.float64), bias.astype(np.float64), "relu")
+    close(a, exp, 1e-5)
+    close(b, exp, 1e-5)

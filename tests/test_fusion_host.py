@@ -1,0 +1,60 @@
+"""CPU: the pattern recogniser of the C++ host rewrites decomposed subgraphs into the
+fused custom calls, and refuses when that would change the program (interior value used
+elsewhere, wrong constants).  Checked through the operation list an executable reports."""
+import os
+
+import pytest
+
+os.environ.setdefault("METALHLO_ALLOW_NO_DEVICE", "1")
+from metalhlo_amd import capi   # noqa: E402
+from tests import fusion_modules as M   # noqa: E402
+
+
+@pytest.fixture(scope="module")
+def sess():
+    s = capi.Session()
+    yield s
+    s.close()
+
+
+def ops(sess, text, level=None):
+    exe = sess.compile(text, level)
+    try:
+        return sess.ops(exe)
+    finally:
+        sess.lib.mhlo_executable_destroy(exe)
+
+
+def test_softmax_chain_becomes_one_call(sess):
+    assert ops(sess, M.SOFTMAX) == ["fused_softmax"]
+    assert ops(sess, M.SOFTMAX_AXIS0) == ["fused_softmax"]
+    # O0 runs the module as written
+    assert "fused_softmax" not in ops(sess, M.SOFTMAX, 0) and "reduce" in ops(sess, M.SOFTMAX, 0)
+    # the exponentials are a result of the function too: nothing may be absorbed
+    assert "fused_softmax" not in ops(sess, M.SOFTMAX_ESCAPING)
+
+
+def test_gelu_only_with_the_right_constants(sess):
+    assert ops(sess, M.GELU) == ["fused_gelu"]
+    assert "fused_gelu" not in ops(sess, M.NOT_GELU) and "tanh" in ops(sess, M.NOT_GELU)
+
+
+def test_norms(sess):
+    assert ops(sess, M.LAYER_NORM) == ["fused_layer_norm"]
+    assert ops(sess, M.RMS_NORM) == ["fused_rms_norm"]
+    # a LayerNorm over rows of 64 whose divisor is 63 is something else
+    assert "fused_layer_norm" not in ops(sess, M.LAYER_NORM.replace("dense<64.0>", "dense<63.0>"))
+
+
+@pytest.mark.parametrize("with_mask", [False, True])
+@pytest.mark.parametrize("transpose_k", [False, True])
+@pytest.mark.parametrize("divide", [False, True])
+def test_attention_absorbs_scale_mask_and_transpose(sess, with_mask, transpose_k, divide):
+    got = ops(sess, M.attention(with_mask=with_mask, transpose_k=transpose_k, divide=divide))
+    want = ["fused_scaled_dot_product_attention"]
+    assert got == want, got
+
+
+def test_matmul_bias_activation(sess):
+    assert ops(sess, M.FFN_UP) == ["fused_matmul_bias_activation"]
+    assert ops(sess, M.MATMUL_BIAS_RELU) == ["fused_matmul_bias_activation"]
