@@ -234,6 +234,27 @@ int mhip_reduce(void* stream, int op, const void* x, void* y, int64_t outer, int
 /* y[i] = the low elem_size bytes of `pattern`, n elements (splat constants). */
 int mhip_fill(void* stream, void* y, int64_t n, uint64_t pattern, int elem_size);
 
+/* Autotuner ----------------------------------------------------------------- */
+
+/* Times every GEMM kernel variant that can serve this 16-bit problem (128x128 tiles /
+ * 4 waves, 256x256 / 8 waves, 256x256 / 4 waves with the five-stage LDS ring) with
+ * `iters` launches each on `stream`, stores the fastest in the process-wide tuning
+ * table that mhip_gemm consults before its heuristic, and reports it (variant code
+ * 128 | 256 | 2560, microseconds per launch).  Overwrites c; synchronises with the
+ * stream.  (Tuning/AutoTuner.swift:301-458.) */
+int mhip_gemm_autotune(void* stream, const void* a, const void* b, const void* bias, void* c,
+                       int64_t M, int64_t N, int64_t K, int64_t batch, int64_t stride_a,
+                       int64_t stride_b, int64_t stride_c, int trans_a, int trans_b, int activation,
+                       int dtype, int iters, int* out_variant, float* out_us);
+
+/* The tuning table as text, one "gemm M N K batch trans_a trans_b dtype variant us" line
+ * per entry (Tuning/TuningDatabase.swift:109-150).  Loading merges into the table; the
+ * file named by the environment variable MHIP_TUNING_DB is loaded at first use. */
+int mhip_tuning_save(const char* path);
+int mhip_tuning_load(const char* path);
+void mhip_tuning_clear(void);
+int mhip_tuning_count(void);
+
 #ifdef __cplusplus
 }
 #endif

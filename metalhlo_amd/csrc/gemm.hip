@@ -354,6 +354,8 @@ static int launch_mfma(hipStream_t s, GemmArgs g, int64_t batch) {
 // gemm256.hip: 4-wave 256x256 kernel with a hand-scheduled main loop.
 bool gemm256_eligible(const GemmArgs& g, int64_t batch, int dtype);
 int launch_gemm256(hipStream_t s, const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype);
+// tuning.hip: variant prescribed by the tuning table for this problem, 0 = none.
+int tuned_gemm_variant(const GemmArgs& g, int64_t batch, int ta, int tb, int dtype);
 
 // Which kernel serves a 16-bit problem (MHIP_GEMM_TILE = 128 | 256 | 2560 forces one):
 //   * the four-wave 256x256 kernel (gemm256.hip) when it is eligible and K is long
@@ -361,11 +363,13 @@ int launch_gemm256(hipStream_t s, const GemmArgs& g, int64_t batch, int trans_a,
 //   * the eight-wave 256x256 kernel for large problems it cannot take whose rows of C
 //     are not 16-byte aligned (odd N): its eight waves hide the narrow stores;
 //   * otherwise 128x128 tiles, two workgroups per CU (short K, few tiles).
+// An entry of the tuning table (mhip_gemm_autotune) for the problem overrides the heuristic.
 template <typename T, bool TA, bool TB>
 static int pick_tile(hipStream_t s, const GemmArgs& g, int64_t batch) {
     const int64_t big = (int64_t)((g.M + 255) / 256) * ((g.N + 255) / 256) * batch;
-    const int force = tune_int("MHIP_GEMM_TILE", 0);
     constexpr int dt = std::is_same<T, bf16_t>::value ? MHIP_BF16 : MHIP_F16;
+    int force = tune_int("MHIP_GEMM_TILE", 0);
+    if (force == 0) force = tuned_gemm_variant(g, batch, TA, TB, dt);   // tuning table / running tuner
     if (force == 2560 || (force == 0 && g.K >= 1024)) {
         if (gemm256_eligible(g, batch, dt)) return launch_gemm256(s, g, batch, TA, TB, dt);
     }

@@ -10,6 +10,7 @@ layer_norm, rms_norm, gelu, flash_attention, plus matmul.
 """
 from __future__ import annotations
 
+import ctypes as C
 import math
 from typing import Optional
 
@@ -261,3 +262,38 @@ def argmax(x, index_dtype=torch.int32, return_values: bool = False):
     _lib.check(lib.mhip_argmax(_stream(), x.data_ptr(), idx.data_ptr(), _ptr(val),
                                x.numel() // cols, cols, _code(x), DTYPE_CODE[index_dtype]))
     return (idx, val) if return_values else idx
+
+
+def autotune_matmul(a, b, bias=None, activation: str = "none", trans_a: bool = False,
+                    trans_b: bool = False, iters: int = 10):
+    """Times the GEMM kernel variants for this 2-D problem and stores the fastest in the
+    library's tuning table (used by every later matmul of the same shape, layout and
+    type).  Returns (variant code 128 | 256 | 2560, microseconds per launch)."""
+    _dev(a, b, bias)
+    lib = _lib.load()
+    if a.dim() != 2 or b.dim() != 2 or a.dtype != b.dtype:
+        raise ValueError("autotune_matmul takes two 2-D operands of one dtype")
+    M, K = (a.shape[1], a.shape[0]) if trans_a else (a.shape[0], a.shape[1])
+    N = b.shape[0] if trans_b else b.shape[1]
+    out = torch.empty((M, N), dtype=a.dtype, device=a.device)
+    variant, us = C.c_int(0), C.c_float(0.0)
+    _lib.check(lib.mhip_gemm_autotune(_stream(), a.data_ptr(), b.data_ptr(), _ptr(bias), out.data_ptr(), M, N, K, 1,
+                                      0, 0, M * N, int(trans_a), int(trans_b), ACTIVATION_CODE[activation], _code(a),
+                                      int(iters), C.byref(variant), C.byref(us)))
+    return variant.value, us.value
+
+
+def tuning_save(path: str) -> None:
+    _lib.check(_lib.load().mhip_tuning_save(str(path).encode()))
+
+
+def tuning_load(path: str) -> None:
+    _lib.check(_lib.load().mhip_tuning_load(str(path).encode()))
+
+
+def tuning_clear() -> None:
+    _lib.load().mhip_tuning_clear()
+
+
+def tuning_count() -> int:
+    return _lib.load().mhip_tuning_count()
