@@ -14,7 +14,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 ROOT = os.path.dirname(HERE)
 
-HIP_SOURCES = ["runtime.hip", "row_kernels.hip", "gemm.hip", "gemm256.hip", "tuning.hip", "attention.hip", "glue_kernels.hip", "elementwise.hip"]
+HIP_SOURCES = ["runtime.hip", "row_kernels.hip", "gemm.hip", "gemm256.hip", "tuning.hip", "attention.hip", "attention_pipe.hip", "glue_kernels.hip", "elementwise.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=fast",
@@ -43,19 +43,19 @@ def hipcc() -> str:
 
 
 def generate_sources(verbose: bool = True) -> None:
-    """Regenerates the hand-scheduled main loops included by gemm256.hip."""
-    gen = os.path.join(CSRC, "gen_gemm256_loop.py")
-    r = subprocess.run([sys.executable, gen], capture_output=True, text=True)
-    if r.returncode != 0:
-        sys.stderr.write(r.stderr)
-        raise RuntimeError("build step failed: gen_gemm256_loop.py")
-    out = os.path.join(CSRC, "gemm256_loop.inc")
-    old = open(out).read() if os.path.exists(out) else None
-    if old != r.stdout:
-        with open(out, "w") as f:
-            f.write(r.stdout)
-    if verbose:
-        print("  gen   gemm256_loop.inc", flush=True)
+    """Regenerates the hand-scheduled loops included by gemm256.hip and attention_pipe.hip."""
+    for script, target in (("gen_gemm256_loop.py", "gemm256_loop.inc"), ("gen_fa_loop.py", "fa_loop.inc")):
+        r = subprocess.run([sys.executable, os.path.join(CSRC, script)], capture_output=True, text=True)
+        if r.returncode != 0:
+            sys.stderr.write(r.stderr)
+            raise RuntimeError("build step failed: " + script)
+        out = os.path.join(CSRC, target)
+        old = open(out).read() if os.path.exists(out) else None
+        if old != r.stdout:
+            with open(out, "w") as f:
+                f.write(r.stdout)
+        if verbose:
+            print("  gen   " + target, flush=True)
 
 
 def build_kernels(verbose: bool = True) -> str:

@@ -1,0 +1,92 @@
+// Definitions shared by the flash-attention kernels.
+#pragma once
+#include <math.h>
+
+#include "common.h"
+
+namespace mhip {
+
+constexpr uint32_t kOobA = 0x80000000u;
+constexpr int kBQ = 128;   // query rows per workgroup (two-workgroups-per-CU kernel)
+constexpr int kBKV = 64;   // keys per LDS stage
+constexpr float kLog2e = 1.4426950408889634f;
+
+struct FaArgs {
+    const void* q;
+    const void* k;
+    const void* v;
+    const void* mask;
+    void* o;
+    int B, H, Sq, Skv;
+    float c;          // |scale| * log2(e)
+    int negate_q;     // scale < 0: flip the sign of Q instead
+    int is_causal;    // read by the scalar path (the MFMA path is templated on it)
+    int64_t mask_sb, mask_sh;
+    int nqb;          // query blocks per (batch, head)
+    int xcd_map;      // 1: (batch*head) % 8 == 0, use the XCD-aware block order
+};
+
+template <typename T> struct Mfma32A;
+template <> struct Mfma32A<bf16_t> {
+    __device__ static f32x16 run(u32x4 a, u32x4 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                       __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+    __device__ static uint32_t pack2(float lo, float hi) {
+        typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+        bf16x2 t = {(__bf16)lo, (__bf16)hi};
+        return __builtin_bit_cast(uint32_t, t);
+    }
+};
+template <> struct Mfma32A<f16_t> {
+    __device__ static f32x16 run(u32x4 a, u32x4 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
+                                                      __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+    __device__ static uint32_t pack2(float lo, float hi) {
+        typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+        f16x2 t = {(_Float16)lo, (_Float16)hi};
+        return __builtin_bit_cast(uint32_t, t);
+    }
+};
+
+__device__ inline __amdgpu_buffer_rsrc_t fa_rsrc(const void* p, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
+}
+
+// K and V tiles sit in LDS as they lie in memory, [64 keys][D], 16-byte chunks
+// XOR-swizzled inside each row.  K is read as the A operand of S^T = K.Q^T with
+// ds_read_b128 (lane = key row, eight consecutive d); V is read as the A operand
+// of O^T += V^T.P^T with ds_read_b64_tr_b16, which hands lane i of a 16-lane
+// group column d = i of four consecutive key rows.
+template <int D>
+__device__ inline int k_swz(int row) { return (D == 128) ? (row & 15) : ((row >> 1) & 7); }
+template <int D>
+__device__ inline uint32_t k_off(int row, int chunk) {
+    return (uint32_t)(row * (D * 2) + ((chunk ^ k_swz<D>(row)) << 4));
+}
+// the four key rows that one transposing read touches must fall on disjoint banks
+template <int D>
+__device__ inline int v_swz(int row) { return (D == 128) ? ((row & 3) << 2) : (((row >> 1) & 1) << 2); }
+template <int D>
+__device__ inline uint32_t v_off(int row, int chunk) {
+    return (uint32_t)(row * (D * 2) + ((chunk ^ v_swz<D>(row)) << 4));
+}
+
+typedef short fa_s16x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) fa_s16x4 fa_lds_s16x4;
+typedef __attribute__((address_space(3))) void fa_lds_void;
+
+// The value held by lane ^ 32, through the register-file lane swap of gfx950 instead
+// of a round trip through LDS.  The swap exchanges the upper half of its first
+// operand with the lower half of its second; picking the result by the lane's own
+// half is right whether or not the two operands share a register.
+__device__ inline float other_half(float x) {
+    const unsigned u = __builtin_bit_cast(unsigned, x);
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return __builtin_bit_cast(float, (threadIdx.x & 32) ? r[0] : r[1]);
+}
+__device__ inline float half_max(float x) { return fmaxf(x, other_half(x)); }
+__device__ inline float half_sum(float x) { return x + other_half(x); }
+
+}  // namespace mhip
