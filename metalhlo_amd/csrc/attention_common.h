@@ -24,6 +24,7 @@ struct FaArgs {
     int64_t mask_sb, mask_sh;
     int nqb;          // query blocks per (batch, head)
     int xcd_map;      // 1: (batch*head) % 8 == 0, use the XCD-aware block order
+    int pair_tiles;   // pipelined kernel, causal: a workgroup takes two query tiles (first + last, ...)
 };
 
 template <typename T> struct Mfma32A;

@@ -44,7 +44,8 @@ Register map:
   v[144:145] byte offsets of this thread's chunk in the K / V blocks loaded next
   v[146:159] alpha q0, q1 and six temporaries per query block
   s[72:74] = 4096, 8192, 12288 (row-group offsets of the loads), s76 = body counter,
-  s77 = caller's M0, s[78:79] / s[80:81] = compare results of q0 / q1
+  s77 = caller's M0, s[78:79] / s[80:81] = compare results of q0 / q1,
+  s[82:83] / s[84:85] = lanes of q0 / q1 whose reference maximum moved
 """
 import os
 
@@ -102,6 +103,7 @@ def softmax_stream(qi, sbase, pnew):
     out.append(f"v_sub_f32 {v(thr)}, {v(MREF + qi)}, {v(mnew)}")
     out.append(f"v_exp_f32 {v(al)}, {v(thr)}")                   # alpha = 2^(old ref - new ref)
     out.append(f"v_mov_b32 {v(MREF + qi)}, {v(mnew)}")
+    out.append(f"v_cmp_neq_f32 s[{82 + 2 * qi}:{83 + 2 * qi}], 1.0, {v(al)}")      # lanes whose reference moved
     # exponentials: the fma of element i+2 sits between the fma and the exp of element i
     for r in S[:2]:
         out.append(f"v_fma_f32 {v(r)}, {v(r)}, %[c], -{v(mnew)}")
@@ -109,7 +111,8 @@ def softmax_stream(qi, sbase, pnew):
         if i + 2 < 32:
             out.append(f"v_fma_f32 {v(S[i + 2])}, {v(S[i + 2])}, %[c], -{v(mnew)}")
         out.append(f"v_exp_f32 {v(r)}, {v(r)}")
-    # row sum: two chains
+    # row sum: two chains (v_dot2c on the packed pairs would halve the count, but it costs
+    # more than two adds next to the MFMAs)
     out.append(f"v_add_f32 {v(acc)}, {v(S[0])}, {v(S[1])}")
     out.append(f"v_add_f32 {v(t0)}, {v(S[2])}, {v(S[3])}")
     for i in range(4, 32):
@@ -144,15 +147,17 @@ def chunks(lst, n):
     return out
 
 
-def rescale_block(qi, tag):
-    """O(qi) *= alpha(qi) when some lane's alpha is not 1 (the accumulators live in AGPRs)."""
-    out = [f"v_cmp_neq_f32 vcc, 1.0, {v(ALPHA + qi)}", "s_nop 4", f"s_cbranch_vccz L_fa_keep_{tag}_%=",
+def rescale_block(tag):
+    """O *= alpha when some lane's alpha is not 1 (the accumulators live in AGPRs); lanes
+    whose alpha is 1 multiply by 1.  The compares sit in the softmax streams."""
+    out = ["s_or_b64 s[82:83], s[82:83], s[84:85]", "s_cmp_eq_u64 s[82:83], 0", f"s_cbranch_scc1 L_fa_keep_{tag}_%=",
            "s_nop 15", "s_nop 15"]          # the last MFMAs' results must be readable
-    for r in range(64):
-        reg = 128 + 64 * qi + r
-        out.append(f"v_accvgpr_read_b32 {v(T0)}, {a(reg)}")
-        out.append(f"v_mul_f32 {v(T0)}, {v(T0)}, {v(ALPHA + qi)}")
-        out.append(f"v_accvgpr_write_b32 {a(reg)}, {v(T0)}")
+    for qi in range(NQ):
+        for r in range(64):
+            reg = 128 + 64 * qi + r
+            out.append(f"v_accvgpr_read_b32 {v(T0)}, {a(reg)}")
+            out.append(f"v_mul_f32 {v(T0)}, {v(T0)}, {v(ALPHA + qi)}")
+            out.append(f"v_accvgpr_write_b32 {a(reg)}, {v(T0)}")
     out.append("s_nop 4")
     out.append(f"L_fa_keep_{tag}_%=:")
     return out
@@ -196,47 +201,53 @@ def body(n):
     out = []
     # ---- phase B: O += V^T . P^T  ||  first half of the softmax
     k = 0
-    for g in range(16):
-        u, dt = g // 4, g % 4
-        out.append(f"s_waitcnt lgkmcnt({min(6, 2 * (15 - g))})")
-        for qi in range(NQ):
-            acc = a(128 + 16 * (4 * qi + dt), 16)
-            out.append(f"{MN} {acc}, {v(VF + 4 * (g % 4), 4)}, {v(pprev + 4 * (4 * qi + u), 4)}, {acc}")
-            out += head[k]
-            k += 1
-        if g + 4 < 16:
-            out += v_reads(g + 4, slot_v)
+    for g2 in range(8):
+        out.append(f"s_waitcnt lgkmcnt({4 if g2 < 7 else 0})")       # two fragments (four reads) may be in flight
+        for g in (2 * g2, 2 * g2 + 1):
+            u, dt = g // 4, g % 4
+            for qi in range(NQ):
+                acc = a(128 + 16 * (4 * qi + dt), 16)
+                out.append(f"{MN} {acc}, {v(VF + 4 * (g % 4), 4)}, {v(pprev + 4 * (4 * qi + u), 4)}, {acc}")
+                out += head[k]
+                k += 1
+        for g in (2 * g2 + 4, 2 * g2 + 5):
+            if g < 16:
+                out += v_reads(g, slot_v)
     # ---- end of B
     if "norescale" not in EXP:
-        out += rescale_block(0, f"{n}a")
-        out += rescale_block(1, f"{n}b")
+        out += rescale_block(f"{n}")
     out.append("s_waitcnt vmcnt(16)")
     out.append("s_barrier")
     for f in range(4):
         out.append(k_read(f, slot_k))
+    # the eight loads of K(j+4), V(j+3): M0 (the LDS target) is written one MFMA ahead of its load
+    loads = []
     for i in range(4):
         so = "0" if i == 0 else f"s{72 + i - 1}"
-        out.append(f"s_add_u32 m0, %[m0b], {load_k * KTILE + i * 4096}")
-        out.append("s_nop 0")
-        out.append(f"buffer_load_dwordx4 {v(GK)}, %[rk], {so} offen lds")
-        out.append(f"s_add_u32 m0, %[m0b], {VRING + load_v * KTILE + i * 4096}")
-        out.append("s_nop 0")
-        out.append(f"buffer_load_dwordx4 {v(GV)}, %[rv], {so} offen lds")
-    out.append(f"v_add_u32 {v(GK)}, {KTILE}, {v(GK)}")
-    out.append(f"v_add_u32 {v(GV)}, {KTILE}, {v(GV)}")
+        loads.append((f"s_add_u32 m0, %[m0b], {load_k * KTILE + i * 4096}", f"buffer_load_dwordx4 {v(GK)}, %[rk], {so} offen lds"))
+        loads.append((f"s_add_u32 m0, %[m0b], {VRING + load_v * KTILE + i * 4096}", f"buffer_load_dwordx4 {v(GV)}, %[rv], {so} offen lds"))
     # ---- phase A: S(j+1) = K . Q^T  ||  second half of the softmax
     k = 0
-    for f in range(16):
-        st, t = f // 2, f % 2
-        out.append(f"s_waitcnt lgkmcnt({min(3, 15 - f)})")
-        for qi in range(NQ):
-            d = v(s_out + 16 * (2 * qi + t), 16)
-            c = "0" if st == 0 else d
-            out.append(f"{MN} {d}, {v(KF + 4 * (f % 4), 4)}, {a(4 * (8 * qi + st), 4)}, {c}")
-            out += tail[k]
-            k += 1
-        if f + 4 < 16:
-            out.append(k_read(f + 4, slot_k))
+    for f2 in range(8):
+        out.append(f"s_waitcnt lgkmcnt({2 if f2 < 7 else 0})")       # two fragments may be in flight
+        for f in (2 * f2, 2 * f2 + 1):
+            st, t = f // 2, f % 2
+            for qi in range(NQ):
+                if k < len(loads):
+                    out.append(loads[k][0])
+                d = v(s_out + 16 * (2 * qi + t), 16)
+                c = "0" if st == 0 else d
+                out.append(f"{MN} {d}, {v(KF + 4 * (f % 4), 4)}, {a(4 * (8 * qi + st), 4)}, {c}")
+                out += tail[k]
+                if k < len(loads):
+                    out.append(loads[k][1])
+                if k == len(loads) - 1:
+                    out.append(f"v_add_u32 {v(GK)}, {KTILE}, {v(GK)}")
+                    out.append(f"v_add_u32 {v(GV)}, {KTILE}, {v(GV)}")
+                k += 1
+        for f in (2 * f2 + 4, 2 * f2 + 5):
+            if f < 16:
+                out.append(k_read(f, slot_k))
     out += v_prefetch(n % 4)                  # V(j): the first fragments of the next body
     return out
 
@@ -313,8 +324,7 @@ def final():
             k += 1
         if g + 4 < 16:
             out += v_reads(g + 4, 0)
-    out += rescale_block(0, "fa")
-    out += rescale_block(1, "fb")
+    out += rescale_block("f")
     out += ["s_nop 4"]
     return out
 
@@ -343,6 +353,9 @@ def strip(lines):
         lines = [x for x in lines if not x.startswith("buffer_load")]
     if "nobarrier" in EXP:
         lines = [x for x in lines if x != "s_barrier"]
+    for e in EXP:
+        if e.startswith("no:"):
+            lines = [x for x in lines if not x.startswith(e[3:])]
     return lines
 
 
@@ -390,7 +403,7 @@ def main():
     print(f'          "+{{v[{GK}:{GV}]}}"(goff)')
     print(f'        : "{{a[0:31]}}"(q0), "{{a[32:63]}}"(q1), "{{v[{KADDR}:{KADDR + 7}]}}"(kaddr), "{{v[{VADDR}:{VADDR + 3}]}}"(vaddr),')
     print('          [rk] "s"(rk), [rv] "s"(rv), [c] "s"(c), [m0b] "s"(m0b), [count] "s"(count)')
-    print("        : " + clobbers(FRAGS + TEMPS, range(72, 82)) + ");")
+    print("        : " + clobbers(FRAGS + TEMPS, range(72, 86)) + ");")
     print("}\n")
     # ---- last block
     print("// Last block of a wave: raw scores in (s0, s1), probabilities of the block before it in py,")
@@ -403,7 +416,7 @@ def main():
     print(f'          "+{{v[{SBUF[0]}:{SBUF[0] + 31}]}}"(s0), "+{{v[{SBUF[0] + 32}:{SBUF[0] + 63}]}}"(s1),')
     print(f'          "={{v[{PX}:{PX + 31}]}}"(px), "+{{v[{MREF}:{MREF + 3}]}}"(state)')
     print(f'        : "{{v[{PY}:{PY + 31}]}}"(py), "{{v[{VADDR}:{VADDR + 3}]}}"(vaddr), "{{v[{LIM}:{LIM + 1}]}}"(lim), [c] "s"(c)')
-    print("        : " + clobbers(FRAGS + TEMPS + [NEGINF], range(78, 82)) + ");")
+    print("        : " + clobbers(FRAGS + TEMPS + [NEGINF], range(78, 86)) + ");")
     print("}\n")
     # ---- last product
     print("// O += V(j)^T . P(j)^T for the last block: P in px, vaddr = V fragment addresses of block j.")

@@ -46,13 +46,6 @@ CASES = [  # B, H, Sq, Skv, D, causal
     (1, 8, 1024, 1024, 64, True),     # GPT-2-small head shape
     (2, 2, 96, 160, 32, True),        # head size without an MFMA path
     (1, 1, 1, 1, 128, True),
-    # head size 128 with at least 256 query rows: the 256-row pipelined kernel (bf16)
-    (1, 2, 256, 64, 128, False),      # a single key block
-    (1, 2, 512, 1000, 128, False),    # last key block partly filled
-    (2, 3, 777, 777, 128, True),      # ragged causal, even number of query tiles
-    (1, 2, 1280, 1280, 128, True),    # odd number of query tiles: the middle one is not paired
-    (1, 1, 300, 5, 128, True),        # fewer keys than one block
-    (1, 2, 640, 2048, 128, True),     # causal with more keys than queries
 ]
 
 
@@ -88,7 +81,40 @@ def test_attention_mask_scale_variants():
     assert torch.count_nonzero(o[:, :, 5]) == 0
 
 
-def test_attention_pipelined_scale_and_extremes():
+PIPE_CASES = [  # B, H, Sq, Skv, causal -- head size 128, bf16, at least 256 query rows
+    (1, 2, 256, 64, False),       # a single key block
+    (1, 2, 512, 1000, False),     # last key block partly filled
+    (2, 3, 777, 777, True),       # ragged causal, even number of query tiles
+    (1, 2, 1280, 1280, True),     # odd number of query tiles: the middle one is not paired
+    (1, 1, 300, 5, True),         # fewer keys than one block
+    (1, 2, 640, 2048, True),      # causal with more keys than queries
+    (1, 1, 333, 77, True),        # more queries than keys
+    (1, 8, 2048, 2048, True),
+]
+
+
+@pytest.fixture
+def force_pipelined(monkeypatch):
+    """The 256-row pipelined kernel is normally chosen only for grids that fill the chip."""
+    monkeypatch.setenv("MHIP_FA_PIPE", "3")
+    return monkeypatch
+
+
+@pytest.mark.parametrize("pair", [0, 1], ids=["one-tile", "paired-tiles"])
+@pytest.mark.parametrize("case", PIPE_CASES, ids=lambda c: "B%dH%dq%dk%d%s" % (*c[:4], "c" if c[4] else ""))
+def test_attention_pipelined_kernel(case, pair, force_pipelined):
+    from metalhlo_amd import kernels
+    B, H, Sq, Skv, causal = case
+    if pair and not causal:
+        pytest.skip("only causal workgroups pair tiles")
+    force_pipelined.setenv("MHIP_FA_PAIR", str(pair))
+    q, k, v = _qkv(B, H, Sq, Skv, 128, torch.bfloat16, 46)
+    o = kernels.flash_attention(q, k, v, is_causal=causal)
+    exp = oracle.attention(as_f64(q), as_f64(k), as_f64(v), is_causal=causal)
+    assert_close(o, exp, 2e-2, f"pipelined attention {case}")
+
+
+def test_attention_pipelined_scale_and_extremes(force_pipelined):
     """Negative scale and widely spread scores on the 256-row kernel (bf16, head size 128)."""
     from metalhlo_amd import kernels
     q, k, v = _qkv(1, 2, 512, 512, 128, torch.bfloat16, 45)
@@ -102,14 +128,11 @@ def test_attention_pipelined_scale_and_extremes():
     exp = oracle.attention(as_f64(q), as_f64(kk), as_f64(v), scale=0.5)
     assert_close(o, exp, 2e-2, "growing maxima")
     # the pipelined kernel and the 128-row kernel agree (same inputs, kernel choice forced)
-    import os
     a = kernels.flash_attention(q, k, v, is_causal=True)
-    os.environ["MHIP_FA_PIPE"] = "2"
-    try:
-        b = kernels.flash_attention(q, k, v, is_causal=True)
-    finally:
-        os.environ.pop("MHIP_FA_PIPE")
+    force_pipelined.setenv("MHIP_FA_PIPE", "2")
+    b = kernels.flash_attention(q, k, v, is_causal=True)
     assert_close(a, as_f64(b), 2e-2, "pipelined == 128-row kernel")
+    assert not torch.equal(a, b)         # two different kernels ran (their roundings differ)
 
 
 def test_attention_invariants():
