@@ -61,7 +61,8 @@ ALPHA = 146
 T0 = 148          # temporaries: six per query block
 KTILE = 16384
 VRING = 65536
-MN = "v_mfma_f32_32x32x16_bf16"
+MN = "v_mfma_f32_32x32x16_bf16"     # main() sets both per element type
+CVT = "v_cvt_pk_bf16_f32"
 
 
 def v(i, n=1):
@@ -120,10 +121,10 @@ def softmax_stream(qi, sbase, pnew):
         out.append(f"v_add_f32 {v(t)}, {v(t)}, {v(S[i])}")
     out.append(f"v_add_f32 {v(acc)}, {v(acc)}, {v(t0)}")
     for p in range(8):
-        out.append(f"v_cvt_pk_bf16_f32 {v(pnew + 16 * qi + p)}, {v(S[2 * p])}, {v(S[2 * p + 1])}")
+        out.append(f"{CVT} {v(pnew + 16 * qi + p)}, {v(S[2 * p])}, {v(S[2 * p + 1])}")
     out.append(f"v_fma_f32 {v(LSUM + qi)}, {v(LSUM + qi)}, {v(al)}, {v(acc)}")
     for p in range(8, 16):
-        out.append(f"v_cvt_pk_bf16_f32 {v(pnew + 16 * qi + p)}, {v(S[2 * p])}, {v(S[2 * p + 1])}")
+        out.append(f"{CVT} {v(pnew + 16 * qi + p)}, {v(S[2 * p])}, {v(S[2 * p + 1])}")
     return out
 
 
@@ -346,7 +347,7 @@ def pv_tail():
 
 def strip(lines):
     if "nomfma" in EXP:
-        lines = [x for x in lines if not x.startswith(MN)]
+        lines = [x for x in lines if not x.startswith("v_mfma")]
     if "nolds" in EXP:
         lines = [x for x in lines if not x.startswith("ds_read")]
     if "noload" in EXP:
@@ -374,13 +375,10 @@ FRAGS = list(range(KF, KF + 16))
 TEMPS = list(range(ALPHA, ALPHA + 14))
 
 
-def main():
-    print("// Generated by gen_fa_loop.py -- do not edit by hand.")
-    print("// Hand-scheduled pieces of the pipelined flash-attention kernel; the generator documents")
-    print("// the schedule and the register map.\n")
+def emit_all(dt):
     # ---- scores of block 0
     print("// S(0) = K(0) . Q^T into (s0, s1).")
-    print("__device__ __forceinline__ void fa_pipe_scores0_bf16(f32x32& s0, f32x32& s1, u32x32 q0, u32x32 q1, u32x8 kaddr) {")
+    print(f"__device__ __forceinline__ void fa_pipe_scores0_{dt}(f32x32& s0, f32x32& s1, u32x32 q0, u32x32 q1, u32x8 kaddr) {{")
     emit(scores0())
     print(f'        : "={{v[{SBUF[0]}:{SBUF[0] + 31}]}}"(s0), "={{v[{SBUF[0] + 32}:{SBUF[0] + 63}]}}"(s1)')
     print(f'        : "{{a[0:31]}}"(q0), "{{a[32:63]}}"(q1), "{{v[{KADDR}:{KADDR + 7}]}}"(kaddr)')
@@ -391,7 +389,7 @@ def main():
     print("// in (s0, s1) and zeros in py; after `count` bodies the raw scores of block `count` are in")
     print("// (s0, s1) when count is even, else in (s2, s3), and the probabilities of block count-1 in")
     print("// py when count is even, else in px.")
-    print("__device__ __forceinline__ void fa_pipe_loop_bf16(f32x32& o0, f32x32& o1, f32x32& o2, f32x32& o3,")
+    print(f"__device__ __forceinline__ void fa_pipe_loop_{dt}(f32x32& o0, f32x32& o1, f32x32& o2, f32x32& o3,")
     print("        f32x32& s0, f32x32& s1, f32x32& s2, f32x32& s3, u32x32& px, u32x32& py, f32x4& state, u32x2& goff,")
     print("        u32x32 q0, u32x32 q1, u32x8 kaddr, u32x4 vaddr,")
     print("        __amdgpu_buffer_rsrc_t rk, __amdgpu_buffer_rsrc_t rv, float c, uint32_t m0b, uint32_t count) {")
@@ -409,7 +407,7 @@ def main():
     print("// Last block of a wave: raw scores in (s0, s1), probabilities of the block before it in py,")
     print("// lim = per-lane index of the last key of the block that is kept (minus 4 in the upper 32")
     print("// lanes), vaddr = V fragment addresses of the block before it.  Leaves P in px.")
-    print("__device__ __forceinline__ void fa_pipe_final_bf16(f32x32& o0, f32x32& o1, f32x32& o2, f32x32& o3,")
+    print(f"__device__ __forceinline__ void fa_pipe_final_{dt}(f32x32& o0, f32x32& o1, f32x32& o2, f32x32& o3,")
     print("        f32x32& s0, f32x32& s1, u32x32& px, u32x32 py, f32x4& state, u32x4 vaddr, u32x2 lim, float c) {")
     emit(final())
     print("        : " + O_OPS + ",")
@@ -420,12 +418,25 @@ def main():
     print("}\n")
     # ---- last product
     print("// O += V(j)^T . P(j)^T for the last block: P in px, vaddr = V fragment addresses of block j.")
-    print("__device__ __forceinline__ void fa_pipe_pv_bf16(f32x32& o0, f32x32& o1, f32x32& o2, f32x32& o3, u32x32 px, u32x4 vaddr) {")
+    print(f"__device__ __forceinline__ void fa_pipe_pv_{dt}(f32x32& o0, f32x32& o1, f32x32& o2, f32x32& o3, u32x32 px, u32x4 vaddr) {{")
     emit(pv_tail())
     print("        : " + O_OPS)
     print(f'        : "{{v[{PX}:{PX + 31}]}}"(px), "{{v[{VADDR}:{VADDR + 3}]}}"(vaddr)')
     print("        : " + clobbers(FRAGS) + ");")
     print("}")
+
+
+
+def main():
+    global MN, CVT
+    print("// Generated by gen_fa_loop.py -- do not edit by hand.")
+    print("// Hand-scheduled pieces of the pipelined flash-attention kernel; the generator documents")
+    print("// the schedule and the register map.\n")
+    for dt in ("bf16", "f16"):
+        MN = f"v_mfma_f32_32x32x16_{dt}"
+        CVT = f"v_cvt_pk_{dt}_f32"
+        print(f"// ---- {dt} ----\n")
+        emit_all(dt)
 
 
 if __name__ == "__main__":

@@ -100,18 +100,19 @@ def force_pipelined(monkeypatch):
     return monkeypatch
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=lambda d: NAME[d])
 @pytest.mark.parametrize("pair", [0, 1], ids=["one-tile", "paired-tiles"])
 @pytest.mark.parametrize("case", PIPE_CASES, ids=lambda c: "B%dH%dq%dk%d%s" % (*c[:4], "c" if c[4] else ""))
-def test_attention_pipelined_kernel(case, pair, force_pipelined):
+def test_attention_pipelined_kernel(case, pair, dtype, force_pipelined):
     from metalhlo_amd import kernels
     B, H, Sq, Skv, causal = case
     if pair and not causal:
         pytest.skip("only causal workgroups pair tiles")
     force_pipelined.setenv("MHIP_FA_PAIR", str(pair))
-    q, k, v = _qkv(B, H, Sq, Skv, 128, torch.bfloat16, 46)
+    q, k, v = _qkv(B, H, Sq, Skv, 128, dtype, 46)
     o = kernels.flash_attention(q, k, v, is_causal=causal)
     exp = oracle.attention(as_f64(q), as_f64(k), as_f64(v), is_causal=causal)
-    assert_close(o, exp, 2e-2, f"pipelined attention {case}")
+    assert_close(o, exp, TOL[dtype], f"pipelined attention {case}")
 
 
 def test_attention_pipelined_scale_and_extremes(force_pipelined):
