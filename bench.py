@@ -35,13 +35,13 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by what the same
 # counter reads for the 'copy' workload (256 MiB in, 256 MiB out); see profiles/<workload>.txt.
 MEASURED_TRAFFIC = {
-    "gemm": 238938188,
-    "attention": 540499858,
-    "attention_full": 268510134,
-    "softmax": 536807759,
-    "layer_norm": 536968239,
-    "rms_norm": 536871699,
-    "bias_gelu": 536863287,
+    "gemm": 238902106,
+    "attention": 775878327,
+    "attention_full": 268950097,
+    "softmax": 536720377,
+    "layer_norm": 536913493,
+    "rms_norm": 536798961,
+    "bias_gelu": 536775641,
     "copy": 536870912,
 }
 
@@ -80,7 +80,7 @@ def wl_attention(torch, kernels, B=4, H=32, S=4096, D=128, causal=True):
     flops = 4.0 * B * H * S * S * D * (0.5 if causal else 1.0)
     return dict(name=f"bf16 flash-attention fwd B{B} H{H} S{S} D{D} {'causal' if causal else 'full'}",
                 fn=lambda i: kernels.flash_attention(q, k, v, is_causal=causal), flops=flops,
-                bytes=4.0 * B * H * S * D * 2, bound="mfma", kernel="fa_fwd_kernel")
+                bytes=4.0 * B * H * S * D * 2, bound="mfma", kernel="fa_pipe_kernel")
 
 
 def _rows(torch, rows=32768, cols=4096, nbuf=3):
