@@ -370,7 +370,9 @@ static int pick_tile(hipStream_t s, const GemmArgs& g, int64_t batch) {
     constexpr int dt = std::is_same<T, bf16_t>::value ? MHIP_BF16 : MHIP_F16;
     int force = tune_int("MHIP_GEMM_TILE", 0);
     if (force == 0) force = tuned_gemm_variant(g, batch, TA, TB, dt);   // tuning table / running tuner
-    if (force == 2560 || (force == 0 && g.K >= 1024)) {
+    // the four-wave ring kernel: long K always; short K (its five-stage prologue weighs more)
+    // when there are clearly more 256x256 tiles than CUs
+    if (force == 2560 || (force == 0 && (g.K >= 1024 || (g.K >= 512 && big >= 320)))) {
         if (gemm256_eligible(g, batch, dt)) return launch_gemm256(s, g, batch, TA, TB, dt);
     }
     const bool want256 = force == 256 || (force != 128 && big >= 192 && (g.K >= 1024 || g.N % 8 != 0));

@@ -58,9 +58,25 @@ __device__ inline float apply_act(float v, int act) {
 // turns the runtime code into such a constant ONCE per kernel: an epilogue that
 // tests the code per element unrolls into hundreds of branchy copies, far larger
 // than the instruction cache.
+// The same functions for results that are rounded to 16 bits (the MFMA kernels): exp2 and the
+// hardware reciprocal (about 1 ulp each) instead of the library's tanhf / expf, which cost
+// an epilogue of 256 accumulators per lane more than the K loop of a short GEMM.
+//   0.5 (1 + tanh u) = 1 / (1 + 2^(-2 log2(e) u)),  tanh u = 1 - 2 / (1 + 2^(2 log2(e) u))
 template <int ACT>
 __device__ inline float apply_act_c(float v) {
-    return ACT == MHIP_ACT_NONE ? v : apply_act(v, ACT);
+    constexpr float kLog2e = 1.4426950408889634f;
+    if (ACT == MHIP_ACT_NONE) return v;
+    if (ACT == MHIP_ACT_RELU) return fmaxf(v, 0.f);
+    if (ACT == MHIP_ACT_GELU) {
+        constexpr float c0 = -2.f * kLog2e * 0.7978845608028654f;
+        constexpr float c1 = c0 * 0.044715f;
+        const float t = v * fmaf(v * v, c1, c0);
+        return v * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(t));
+    }
+    if (ACT == MHIP_ACT_SILU) return v * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-kLog2e * v));
+    if (ACT == MHIP_ACT_SIGMOID) return __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-kLog2e * v));
+    if (ACT == MHIP_ACT_TANH) return 1.f - 2.f * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(2.f * kLog2e * v));
+    return v;
 }
 template <typename F>
 __device__ inline void dispatch_act(int act, F&& f) {

@@ -62,7 +62,13 @@ class GPT2:
             flat.append(np.concatenate([a.reshape(-1), np.zeros(pad, np.float32)]))
             self._slots.append((path, off, a.shape))
 
-        for name in ("wte", "wpe", "lnf_g", "lnf_b"):
+        # the tied output head multiplies by wte^T: rows padded with zeros to a multiple of 64
+        # keep that GEMM on the aligned kernels; "wte" is the view of the real rows
+        wte = np.asarray(params["wte"], dtype=np.float32)
+        self.vocab_pad = -(-wte.shape[0] // 64) * 64
+        put(("wte_pad",), np.concatenate([wte, np.zeros((self.vocab_pad - wte.shape[0], wte.shape[1]), np.float32)]))
+        self._slots.append((("wte",), self._slots[-1][1], wte.shape))
+        for name in ("wpe", "lnf_g", "lnf_b"):
             put((name,), params[name])
         for i, l in enumerate(params["layers"]):
             for k, v in l.items():
@@ -99,8 +105,8 @@ class GPT2:
             u = kernels.matmul(h, l["w_fc"], bias=l["b_fc"], activation="gelu")
             x = kernels.add(x, kernels.matmul(u, l["w_proj"], bias=l["b_proj"]))
         x = kernels.layer_norm(x, p["lnf_g"], p["lnf_b"], eps=1e-5)
-        logits = kernels.matmul(x, p["wte"], trans_b=True)       # tied head: x . wte^T
-        return logits.reshape(B, S, cfg.vocab)
+        logits = kernels.matmul(x, p["wte_pad"], trans_b=True)   # tied head: x . wte^T (padded columns are 0)
+        return logits.reshape(B, S, self.vocab_pad)[..., :cfg.vocab]
 
     def capture(self, ids: torch.Tensor) -> "GraphedForward":
         """Records one forward pass for ids of this shape into a HIP graph.  Every launch
