@@ -98,6 +98,25 @@ def build_host(verbose: bool = True) -> list:
     if verbose:
         print("  link ", os.path.relpath(out, ROOT), flush=True)
     outs.append(out)
+    # the PJRT plugin: same parser / executor, its own boundary file instead of the mhlo_* one
+    pjrt = os.path.join(CSRC, "pjrt", "pjrt.cpp")
+    if os.path.exists(pjrt):
+        out = os.path.join(LIBDIR, "libPJRTMetalHLO.so")
+        _run([hipcc(), "-x", "c++", "-O2", "-std=c++17", "-fPIC", "-D__HIP_PLATFORM_AMD__", "-Wall",
+              "-I", os.path.join(ROOT, "include"), "-I", "/opt/rocm/include", pjrt,
+              *[f for f in srcs if os.path.basename(f) != "capi.cpp"],
+              "-shared", "-o", out, "-L", LIBDIR, "-lmetalhlo_hip", "-L", "/opt/rocm/lib", "-lamdhip64",
+              "-Wl,-rpath,$ORIGIN", "-Wl,-rpath,/opt/rocm/lib"])
+        if verbose:
+            print("  link ", os.path.relpath(out, ROOT), flush=True)
+        outs.append(out)
+        # the test program that drives the plugin through its function table (tests/test_pjrt_*.py)
+        drv_src = os.path.join(ROOT, "tests", "pjrt", "pjrt_driver.cpp")
+        if os.path.exists(drv_src):
+            drv = os.path.join(ROOT, "tests", "pjrt", "pjrt_driver")
+            _run(["g++", "-O1", "-std=c++17", "-Wall", "-I", os.path.join(ROOT, "include"), drv_src, "-o", drv, "-ldl"])
+            if verbose:
+                print("  link ", os.path.relpath(drv, ROOT), flush=True)
     return outs
 
 

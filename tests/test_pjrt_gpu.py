@@ -1,0 +1,20 @@
+"""PJRT plugin on the GPU: host <-> device round trips, events, compile + execute, serialize ->
+deserialize -> execute, a fused kernel through the plugin (tests/pjrt/pjrt_driver.cpp, gpu mode)."""
+import os
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+PLUGIN = os.path.join(ROOT, "metalhlo_amd", "lib", "libPJRTMetalHLO.so")
+DRIVER = os.path.join(ROOT, "tests", "pjrt", "pjrt_driver")
+
+pytestmark = pytest.mark.gpu
+
+
+def test_driver_gpu_cases():
+    assert os.path.exists(PLUGIN) and os.path.exists(DRIVER), "plugin / driver not built"
+    r = subprocess.run([DRIVER, PLUGIN, "gpu"], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stdout[-3000:] + r.stderr[-3000:]
+    for case in ("table", "errors", "platform", "compile", "round_trip", "execute", "all"):
+        assert f"ok {case}\n" in r.stdout, r.stdout
