@@ -139,6 +139,20 @@ int mhip_flash_attention(void* stream, const void* q, const void* k, const void*
                          int64_t D, float scale, int is_causal, int64_t mask_stride_b,
                          int64_t mask_stride_h, int dtype);
 
+/* The same operator on tensors that are views: `strides` holds twelve element strides,
+ * {batch, head, row} for q, k, v, o in that order (NULL = packed, as above); the head
+ * dimension itself is contiguous.  This lets attention read Q, K, V straight out of a
+ * fused QKV projection [B,S,3,H,D] and write O as [B,S,H,D], in place of the
+ * transpose / reshape / slice operations the reference materialises around its attention
+ * call (it has no strided variant: MetalExecutor.swift:502-564 binds packed buffers).
+ * Strided layouts need bf16 / f16, D in {64, 128}, 16-byte aligned pointers and strides
+ * that are multiples of 8 elements; anything else returns 2 (unsupported). */
+int mhip_flash_attention_strided(void* stream, const void* q, const void* k, const void* v,
+                                 const void* mask, void* o, int64_t B, int64_t H, int64_t Sq,
+                                 int64_t Skv, int64_t D, float scale, int is_causal,
+                                 int64_t mask_stride_b, int64_t mask_stride_h, int dtype,
+                                 const int64_t* strides);
+
 /* Glue operators (index / data movement; integer results are bit-exact) ---- */
 
 /* out[i, :] = table[clamp(idx[i], 0, n_rows-1), :], rows of `row_elems` elements.

@@ -28,6 +28,8 @@ SIGNATURES = {
                          _i32, _i32, _i32, _i32]),
     "mhip_flash_attention": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64,
                                     _f32, _i32, _i64, _i64, _i32]),
+    "mhip_flash_attention_strided": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64,
+                                            _f32, _i32, _i64, _i64, _i32, _vp]),
     "mhip_copy": (_i32, [_vp, _vp, _vp, _i64]),
     "mhip_gather_rows": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _i32]),
     "mhip_embed_tokens": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32, _i32]),

@@ -46,19 +46,21 @@ __global__ __launch_bounds__(256, 2) void fa_fwd_kernel(FaArgs a) {
     const int qw = qblk0 + wave * 32;          // first query row of this wave
     const int qpos = qw + lrow;
 
-    const T* qp = static_cast<const T*>(a.q) + (int64_t)bh * a.Sq * D;
-    const T* kp = static_cast<const T*>(a.k) + (int64_t)bh * a.Skv * D;
-    const T* vp = static_cast<const T*>(a.v) + (int64_t)bh * a.Skv * D;
-    T* op = static_cast<T*>(a.o) + (int64_t)bh * a.Sq * D;
-    const __amdgpu_buffer_rsrc_t rq = fa_rsrc(qp, (uint32_t)((int64_t)a.Sq * D * 2));
-    const __amdgpu_buffer_rsrc_t rk = fa_rsrc(kp, (uint32_t)((int64_t)a.Skv * D * 2));
-    const __amdgpu_buffer_rsrc_t rv = fa_rsrc(vp, (uint32_t)((int64_t)a.Skv * D * 2));
+    const int b_i = bh / a.H, h_i = bh % a.H;
+    const T* qp = static_cast<const T*>(a.q) + b_i * a.qs[0] + h_i * a.qs[1];
+    const T* kp = static_cast<const T*>(a.k) + b_i * a.ks[0] + h_i * a.ks[1];
+    const T* vp = static_cast<const T*>(a.v) + b_i * a.vs[0] + h_i * a.vs[1];
+    T* op = static_cast<T*>(a.o) + b_i * a.os[0] + h_i * a.os[1];
+    const int q_rs = (int)a.qs[2], k_rs = (int)a.ks[2], v_rs = (int)a.vs[2];      // row pitches in elements
+    const __amdgpu_buffer_rsrc_t rq = fa_rsrc(qp, (uint32_t)((((int64_t)a.Sq - 1) * q_rs + D) * 2));
+    const __amdgpu_buffer_rsrc_t rk = fa_rsrc(kp, (uint32_t)((((int64_t)a.Skv - 1) * k_rs + D) * 2));
+    const __amdgpu_buffer_rsrc_t rv = fa_rsrc(vp, (uint32_t)((((int64_t)a.Skv - 1) * v_rs + D) * 2));
 
     // ---- Q^T operand: lane = query column, 8 consecutive d per k-step ------
     u32x4 qf[NS];
 #pragma unroll
     for (int s = 0; s < NS; s++) {
-        const uint32_t off = qpos < a.Sq ? (uint32_t)((qpos * D + 16 * s + 8 * lhalf) * 2) : kOobA;
+        const uint32_t off = qpos < a.Sq ? (uint32_t)((qpos * q_rs + 16 * s + 8 * lhalf) * 2) : kOobA;
         qf[s] = __builtin_amdgcn_raw_buffer_load_b128(rq, off, 0, 0);
         if (a.negate_q) {
             qf[s].x ^= 0x80008000u; qf[s].y ^= 0x80008000u;
@@ -82,8 +84,8 @@ __global__ __launch_bounds__(256, 2) void fa_fwd_kernel(FaArgs a) {
             const int blk = i * 4 + wave;                 // which KB of the tile
             const int row = blk * kRowsPerInst + ld_row;
             const int key = kv0 + row;
-            const uint32_t koff = key < a.Skv ? (uint32_t)((key * D + ((ld_pos ^ k_swz<D>(row)) << 3)) * 2) : kOobA;
-            const uint32_t voff = key < a.Skv ? (uint32_t)((key * D + ((ld_pos ^ v_swz<D>(row)) << 3)) * 2) : kOobA;
+            const uint32_t koff = key < a.Skv ? (uint32_t)((key * k_rs + ((ld_pos ^ k_swz<D>(row)) << 3)) * 2) : kOobA;
+            const uint32_t voff = key < a.Skv ? (uint32_t)((key * v_rs + ((ld_pos ^ v_swz<D>(row)) << 3)) * 2) : kOobA;
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, (fa_lds_void*)(smem + buf * kTile + blk * 1024), 16, koff, 0, 0, 0);
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, (fa_lds_void*)(smem + (2 + buf) * kTile + blk * 1024), 16, voff, 0, 0, 0);
         }
@@ -235,7 +237,7 @@ __global__ __launch_bounds__(256, 2) void fa_fwd_kernel(FaArgs a) {
     const float l_tot = half_sum(l_run);
     const float inv = l_tot > 1e-10f ? 1.f / l_tot : 0.f;
     if (qpos < a.Sq) {
-        T* orow = op + (int64_t)qpos * D;
+        T* orow = op + (int64_t)qpos * a.os[2];
 #pragma unroll
         for (int dt = 0; dt < ND; dt++)
 #pragma unroll
@@ -353,18 +355,18 @@ int launch_fa_pipe(hipStream_t s, const FaArgs& a, int dtype, bool causal);
 
 using namespace mhip;
 
-extern "C" int mhip_flash_attention(void* stream, const void* q, const void* k, const void* v,
-                                    const void* mask, void* o, int64_t B, int64_t H, int64_t Sq,
-                                    int64_t Skv, int64_t D, float scale, int is_causal,
-                                    int64_t mask_stride_b, int64_t mask_stride_h, int dtype) {
+// `strides`: NULL (packed [B,H,S,D]) or twelve element strides {batch, head, row} x {q, k, v, o}.
+static int fa_entry(const char* name, void* stream, const void* q, const void* k, const void* v, const void* mask, void* o,
+                    int64_t B, int64_t H, int64_t Sq, int64_t Skv, int64_t D, float scale, int is_causal,
+                    int64_t mask_stride_b, int64_t mask_stride_h, int dtype, const int64_t* strides) {
     if (B < 0 || H < 0 || Sq < 0 || Skv < 0 || D <= 0)
-        return fail(MHIP_ERR_INVALID_ARGUMENT, "mhip_flash_attention: bad size");
-    if (D > 256) return fail(MHIP_ERR_UNSUPPORTED, "mhip_flash_attention: head_dim %lld > 256", (long long)D);
+        return fail(MHIP_ERR_INVALID_ARGUMENT, "%s: bad size", name);
+    if (D > 256) return fail(MHIP_ERR_UNSUPPORTED, "%s: head_dim %lld > 256", name, (long long)D);
     if (B == 0 || H == 0 || Sq == 0) return MHIP_OK;
     if (!q || !o || (Skv > 0 && (!k || !v)))
-        return fail(MHIP_ERR_INVALID_ARGUMENT, "mhip_flash_attention: NULL tensor pointer");
+        return fail(MHIP_ERR_INVALID_ARGUMENT, "%s: NULL tensor pointer", name);
     if (Sq > 0x7FFFFFFF || Skv > 0x7FFFFFFF || B * H > 0x7FFFFFFF)
-        return fail(MHIP_ERR_UNSUPPORTED, "mhip_flash_attention: dimension exceeds 2^31-1");
+        return fail(MHIP_ERR_UNSUPPORTED, "%s: dimension exceeds 2^31-1", name);
     hipStream_t s = as_stream(stream);
     FaArgs a;
     a.q = q; a.k = k; a.v = v; a.mask = mask; a.o = o;
@@ -373,24 +375,63 @@ extern "C" int mhip_flash_attention(void* stream, const void* q, const void* k, 
     a.negate_q = scale < 0.f;
     a.is_causal = is_causal ? 1 : 0;
     a.mask_sb = mask_stride_b; a.mask_sh = mask_stride_h;
-    a.nqb = 0; a.xcd_map = 0;
+    a.nqb = 0; a.xcd_map = 0; a.pair_tiles = 0;
+    const int64_t packed[12] = {H * Sq * D, Sq * D, D, H * Skv * D, Skv * D, D, H * Skv * D, Skv * D, D, H * Sq * D, Sq * D, D};
+    bool is_packed = true;
+    int64_t max_row = D, max_span = 0;
+    for (int i = 0; i < 12; i++) {
+        const int64_t st = strides ? strides[i] : packed[i];
+        if (st < 0) return fail(MHIP_ERR_INVALID_ARGUMENT, "%s: negative stride", name);
+        (i < 3 ? a.qs : i < 6 ? a.ks : i < 9 ? a.vs : a.os)[i % 3] = st;
+        is_packed = is_packed && st == packed[i];
+    }
+    const int64_t* rows[4] = {a.qs, a.ks, a.vs, a.os};
+    bool strides_aligned = true;
+    for (int t = 0; t < 4; t++) {
+        if (rows[t][2] < D) return fail(MHIP_ERR_INVALID_ARGUMENT, "%s: row stride smaller than head_dim", name);
+        strides_aligned = strides_aligned && rows[t][0] % 8 == 0 && rows[t][1] % 8 == 0 && rows[t][2] % 8 == 0;
+        max_row = rows[t][2] > max_row ? rows[t][2] : max_row;
+        const int64_t n = (t == 0 || t == 3) ? Sq : Skv;
+        const int64_t span = (n > 0 ? (n - 1) * rows[t][2] : 0) + D;
+        max_span = span > max_span ? span : max_span;
+    }
     const bool is16 = dtype == MHIP_BF16 || dtype == MHIP_F16;
     const bool aligned = ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) |
                            reinterpret_cast<uintptr_t>(v) | reinterpret_cast<uintptr_t>(o)) & 15) == 0;
-    const bool fits = Sq * D * 2 < 0x7FFFFFFFLL && Skv * D * 2 < 0x7FFFFFFFLL;
-    if (is16 && aligned && fits && Skv > 0 && (D == 64 || D == 128)) {
+    const bool fits = max_span * 2 < 0x7FFFFFFFLL;
+    if (is16 && aligned && strides_aligned && fits && Skv > 0 && (D == 64 || D == 128)) {
         const bool hm = mask != nullptr;
-        if (fa_pipe_eligible(a, D, dtype, hm)) return launch_fa_pipe(s, a, dtype, is_causal != 0);
+        if (is_packed && fa_pipe_eligible(a, D, dtype, hm)) return launch_fa_pipe(s, a, dtype, is_causal != 0);
         if (dtype == MHIP_BF16)
             return D == 128 ? launch_fa<bf16_t, 128>(s, a, is_causal, hm)
                             : launch_fa<bf16_t, 64>(s, a, is_causal, hm);
         return D == 128 ? launch_fa<f16_t, 128>(s, a, is_causal, hm)
                         : launch_fa<f16_t, 64>(s, a, is_causal, hm);
     }
+    if (!is_packed)
+        return fail(MHIP_ERR_UNSUPPORTED, "%s: strided layouts need bf16 / f16, head_dim 64 or 128, 16-byte aligned pointers and "
+                                          "strides that are multiples of 8 elements", name);
     switch (dtype) {
         case MHIP_F32: return launch_fa_scalar<float>(s, a, (int)D, scale);
         case MHIP_BF16: return launch_fa_scalar<bf16_t>(s, a, (int)D, scale);
         case MHIP_F16: return launch_fa_scalar<f16_t>(s, a, (int)D, scale);
-        default: return fail(MHIP_ERR_UNSUPPORTED, "mhip_flash_attention: dtype %d", dtype);
+        default: return fail(MHIP_ERR_UNSUPPORTED, "%s: dtype %d", name, dtype);
     }
+}
+
+extern "C" int mhip_flash_attention(void* stream, const void* q, const void* k, const void* v,
+                                    const void* mask, void* o, int64_t B, int64_t H, int64_t Sq,
+                                    int64_t Skv, int64_t D, float scale, int is_causal,
+                                    int64_t mask_stride_b, int64_t mask_stride_h, int dtype) {
+    return fa_entry("mhip_flash_attention", stream, q, k, v, mask, o, B, H, Sq, Skv, D, scale, is_causal, mask_stride_b,
+                    mask_stride_h, dtype, nullptr);
+}
+
+extern "C" int mhip_flash_attention_strided(void* stream, const void* q, const void* k, const void* v,
+                                            const void* mask, void* o, int64_t B, int64_t H, int64_t Sq,
+                                            int64_t Skv, int64_t D, float scale, int is_causal,
+                                            int64_t mask_stride_b, int64_t mask_stride_h, int dtype,
+                                            const int64_t* strides) {
+    return fa_entry("mhip_flash_attention_strided", stream, q, k, v, mask, o, B, H, Sq, Skv, D, scale, is_causal,
+                    mask_stride_b, mask_stride_h, dtype, strides);
 }

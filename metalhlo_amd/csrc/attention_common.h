@@ -25,6 +25,9 @@ struct FaArgs {
     int nqb;          // query blocks per (batch, head)
     int xcd_map;      // 1: (batch*head) % 8 == 0, use the XCD-aware block order
     int pair_tiles;   // pipelined kernel, causal: a workgroup takes two query tiles (first + last, ...)
+    // Element strides {batch, head, row} of q, k, v, o (the last axis is contiguous).  Only
+    // fa_fwd_kernel reads them; every other kernel is given the packed [B,H,S,D] layout.
+    int64_t qs[3], ks[3], vs[3], os[3];
 };
 
 template <typename T> struct Mfma32A;

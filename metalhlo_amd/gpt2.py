@@ -94,12 +94,22 @@ class GPT2:
         # the graph's `convert` ops: fp32 parameters -> compute type, every step
         p = self.p32 if self.dtype == torch.float32 else self._views(kernels.convert(self.flat32, self.dtype))
         x = kernels.embed_tokens(ids, self.p32["wte"], self.p32["wpe"], self.dtype).reshape(B * S, d)
+        # the strided attention entry covers 16-bit types and head sizes 64 / 128
+        in_place = self.dtype in (torch.bfloat16, torch.float16) and d // H in (64, 128)
         for l in p["layers"]:
             h = kernels.layer_norm(x, l["ln1_g"], l["ln1_b"], eps=1e-5)
             qkv = kernels.matmul(h, l["w_qkv"], bias=l["b_qkv"])
-            q, k, v = kernels.split_qkv_heads(qkv.reshape(B, S, 3 * d), H)
-            a = kernels.flash_attention(q, k, v, is_causal=True)
-            a = kernels.transpose_0213(a).reshape(B * S, d)
+            if in_place:
+                # attention reads Q, K, V in place ([B,S,3,H,D] views of the projection) and
+                # writes [B,S,H,D]: no head split / merge passes over memory
+                q, k, v = qkv.view(B, S, 3, H, d // H).permute(2, 0, 3, 1, 4).unbind(0)
+                a = torch.empty(B, S, H, d // H, dtype=qkv.dtype, device=qkv.device)
+                kernels.flash_attention(q, k, v, is_causal=True, out=a.permute(0, 2, 1, 3))
+                a = a.view(B * S, d)
+            else:
+                q, k, v = kernels.split_qkv_heads(qkv.reshape(B, S, 3 * d), H)
+                a = kernels.flash_attention(q, k, v, is_causal=True)
+                a = kernels.transpose_0213(a).reshape(B * S, d)
             x = kernels.add(x, kernels.matmul(a, l["w_o"], bias=l["b_o"]))
             h = kernels.layer_norm(x, l["ln2_g"], l["ln2_b"], eps=1e-5)
             u = kernels.matmul(h, l["w_fc"], bias=l["b_fc"], activation="gelu")

@@ -147,12 +147,17 @@ def matmul(a, b, bias=None, activation: str = "none", trans_a: bool = False,
 
 
 def flash_attention(q, k, v, scale: Optional[float] = None, is_causal: bool = False,
-                    mask: Optional[torch.Tensor] = None):
+                    mask: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None):
     """softmax(scale * q k^T + mask, causal) v for [B,H,S,D] tensors.
-    Default scale 1/sqrt(D) (FlashAttentionKernel.swift:55)."""
-    _dev(q, k, v, mask)
+    Default scale 1/sqrt(D) (FlashAttentionKernel.swift:55).  q, k, v (and `out`, when given)
+    may be views with arbitrary batch / head / row strides as long as the last axis is
+    contiguous, e.g. slices of a fused QKV projection; packed tensors take the plain entry."""
+    for t in (q, k, v, out):
+        if t is not None and (not t.is_cuda or t.dim() != 4 or t.stride(3) != 1):
+            raise ValueError("attention operands must be 4-D device tensors with a contiguous last axis")
+    _dev(mask)
     lib = _lib.load()
-    if q.dim() != 4 or k.shape != v.shape or q.shape[:2] != k.shape[:2] or q.shape[3] != k.shape[3]:
+    if k.shape != v.shape or q.shape[:2] != k.shape[:2] or q.shape[3] != k.shape[3]:
         raise ValueError("expected q [B,H,Sq,D] and k,v [B,H,Skv,D]")
     if not (q.dtype == k.dtype == v.dtype):
         raise TypeError("q, k, v dtypes differ")
@@ -170,11 +175,20 @@ def flash_attention(q, k, v, scale: Optional[float] = None, is_causal: bool = Fa
             raise ValueError("mask must broadcast to [B,H,Sq,Skv] with full last two dims")
         msh = Sq * Skv if mask.shape[1] == H else 0
         msb = mask.shape[1] * Sq * Skv if mask.shape[0] == B else 0
-    o = torch.empty_like(q)
-    _lib.check(lib.mhip_flash_attention(_stream(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
-                                        _ptr(mask), o.data_ptr(), B, H, Sq, Skv, D, float(scale),
-                                        int(is_causal), msb, msh, _code(q)))
-    return o
+    if out is None:
+        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    elif out.shape != q.shape or out.dtype != q.dtype:
+        raise ValueError("out must have q's shape and dtype")
+    if all(t.is_contiguous() for t in (q, k, v, out)):
+        _lib.check(lib.mhip_flash_attention(_stream(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                                            _ptr(mask), out.data_ptr(), B, H, Sq, Skv, D, float(scale),
+                                            int(is_causal), msb, msh, _code(q)))
+    else:
+        strides = (C.c_int64 * 12)(*[t.stride(i) for t in (q, k, v, out) for i in range(3)])
+        _lib.check(lib.mhip_flash_attention_strided(_stream(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                                                    _ptr(mask), out.data_ptr(), B, H, Sq, Skv, D, float(scale),
+                                                    int(is_causal), msb, msh, _code(q), C.addressof(strides)))
+    return out
 
 
 # ---- glue -------------------------------------------------------------------

@@ -3,6 +3,8 @@ materialised-scores oracle.  fp32: 1e-5 relative; bf16/fp16: 2e-2 relative
 (floor max(tol, tol*|e|))."""
 import math
 
+import ctypes as C
+
 import numpy as np
 import pytest
 import torch
@@ -134,6 +136,38 @@ def test_attention_pipelined_scale_and_extremes(force_pipelined):
     b = kernels.flash_attention(q, k, v, is_causal=True)
     assert_close(a, as_f64(b), 2e-2, "pipelined == 128-row kernel")
     assert not torch.equal(a, b)         # two different kernels ran (their roundings differ)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=lambda d: NAME[d])
+@pytest.mark.parametrize("D", [64, 128])
+def test_attention_strided_views(D, dtype, lib):
+    """Q, K, V read in place from a fused projection [B,S,3,H,D] and O written as [B,S,H,D]:
+    the same numbers as packed tensors give, and the oracle's."""
+    from metalhlo_amd import kernels
+    B, H, S = 2, 3, 200
+    rng = np.random.default_rng(47)
+    qkv = to_dev(rng.standard_normal((B, S, 3, H, D)), dtype)
+    q, k, v = qkv.permute(2, 0, 3, 1, 4).unbind(0)                 # [B,H,S,D] views, row pitch 3*H*D
+    assert not q.is_contiguous()
+    out = torch.full((B, S, H, D), float("nan"), dtype=dtype, device="cuda")
+    for causal in (True, False):
+        kernels.flash_attention(q, k, v, is_causal=causal, out=out.permute(0, 2, 1, 3))
+        packed = kernels.flash_attention(q.contiguous(), k.contiguous(), v.contiguous(), is_causal=causal)
+        assert torch.equal(out.permute(0, 2, 1, 3), packed), "strided and packed results differ"
+        exp = oracle.attention(as_f64(q), as_f64(k), as_f64(v), is_causal=causal)
+        assert_close(out.permute(0, 2, 1, 3), exp, TOL[dtype], f"strided attention D={D} causal={causal}")
+    # layouts the strided entry refuses: fp32, odd strides
+    x = torch.zeros(4096, dtype=torch.float32, device="cuda")
+    p = x.data_ptr()
+    st = (C.c_int64 * 12)(*([2048, 1024, 128] * 4))
+    assert lib.mhip_flash_attention_strided(None, p, p, p, None, p, 1, 1, 8, 8, 64, 1.0, 0, 0, 0, 1, C.addressof(st)) == 2
+    st = (C.c_int64 * 12)(*([2048, 1024, 100] * 4))
+    assert lib.mhip_flash_attention_strided(None, p, p, p, None, p, 1, 1, 8, 8, 64, 1.0, 0, 0, 0, 3, C.addressof(st)) == 2
+    st = (C.c_int64 * 12)(*([2048, 1024, 32] * 4))                 # rows would overlap
+    assert lib.mhip_flash_attention_strided(None, p, p, p, None, p, 1, 1, 8, 8, 64, 1.0, 0, 0, 0, 3, C.addressof(st)) == 1
+    # NULL strides = the packed entry
+    assert lib.mhip_flash_attention_strided(None, p, p, p, None, p, 1, 1, 8, 8, 64, 1.0, 0, 0, 0, 1, None) == 0
+    torch.cuda.synchronize()
 
 
 def test_attention_invariants():
