@@ -123,6 +123,17 @@ int mhip_gemm(void* stream, const void* a, const void* b, const void* bias, void
               int64_t N, int64_t K, int64_t batch, int64_t stride_a, int64_t stride_b,
               int64_t stride_c, int trans_a, int trans_b, int activation, int dtype);
 
+/* The same with a residual: C[b] = act(op(A[b]) . op(B[b]) + bias[col]) + R[b], R laid out
+ * like C (same batch stride; R may be C itself).  The stored value is rounded to the element
+ * type before R is added and the sum is rounded again, i.e. bit for bit what mhip_gemm
+ * followed by mhip_add produces, without the extra pass over C.  Serves the
+ * `x + proj(...)` pairs of a transformer block, which the reference runs as dot_general
+ * followed by a separate add kernel (Compiler/CodeGenerator.swift:921-1100 binary ops). */
+int mhip_gemm_residual(void* stream, const void* a, const void* b, const void* bias,
+                       const void* residual, void* c, int64_t M, int64_t N, int64_t K,
+                       int64_t batch, int64_t stride_a, int64_t stride_b, int64_t stride_c,
+                       int trans_a, int trans_b, int activation, int dtype);
+
 /* Attention -------------------------------------------------------------- */
 
 /* O = softmax(scale * Q K^T + mask, causal) V.

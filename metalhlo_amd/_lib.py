@@ -26,6 +26,8 @@ SIGNATURES = {
     "mhip_bias_gelu": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i32]),
     "mhip_gemm": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
                          _i32, _i32, _i32, _i32]),
+    "mhip_gemm_residual": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
+                                  _i32, _i32, _i32, _i32]),
     "mhip_flash_attention": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64,
                                     _f32, _i32, _i64, _i64, _i32]),
     "mhip_flash_attention_strided": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64,

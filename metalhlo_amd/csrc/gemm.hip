@@ -140,6 +140,7 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_mfma_kernel(GemmArgs g) {
     const T* a = static_cast<const T*>(g.a) + batch * g.sa;
     const T* b = static_cast<const T*>(g.b) + batch * g.sb;
     T* c = static_cast<T*>(g.c) + batch * g.sc;
+    const T* res = g.residual ? static_cast<const T*>(g.residual) + batch * g.sc : nullptr;
 
     // A is stored [M][K] (k contiguous) unless TA ([K][M]); B is stored [K][N]
     // (k slow) unless TB ([N][K]).
@@ -265,7 +266,8 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_mfma_kernel(GemmArgs g) {
             const int m = m0 + wm * WTM + ml;
             const int n = n0 + wn * WTN + cc * 8;
             if (m < g.M && n < g.N) {
-                const u32x4 w = *reinterpret_cast<const u32x4*>(stage + ml * kRowPad + cc * 16);
+                u32x4 w = *reinterpret_cast<const u32x4*>(stage + ml * kRowPad + cc * 16);
+                if (res) w = add_chunk<T>(w, *reinterpret_cast<const u32x4*>(res + (int64_t)m * g.N + n));
                 *reinterpret_cast<u32x4*>(c + (int64_t)m * g.N + n) = w;
             }
         }
@@ -282,7 +284,11 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_mfma_kernel(GemmArgs g) {
             for (int cb = 0; cb < WTN / 64; cb++) {
                 const int nl = cb * 64 + lane;
                 const int n = n0 + wn * WTN + nl;
-                if (n < g.N) c16[(int64_t)m * g.N + n] = st16[ml * (kRowPad / 2) + nl];
+                if (n < g.N) {
+                    T val = __builtin_bit_cast(T, st16[ml * (kRowPad / 2) + nl]);
+                    if (res) val = Elem<T>::from_f32(Elem<T>::to_f32(val) + Elem<T>::to_f32(res[(int64_t)m * g.N + n]));
+                    c16[(int64_t)m * g.N + n] = __builtin_bit_cast(uint16_t, val);
+                }
             }
         }
     }
@@ -319,7 +325,11 @@ __global__ __launch_bounds__(256) void gemm_simple_kernel(GemmArgs g, int trans_
     if (m < g.M && n < g.N) {
         if (g.bias) acc += Elem<T>::to_f32(static_cast<const T*>(g.bias)[n]);
         if (g.act != MHIP_ACT_NONE) acc = apply_act(acc, g.act);
-        c[(int64_t)m * g.N + n] = Elem<T>::from_f32(acc);
+        T val = Elem<T>::from_f32(acc);
+        if (g.residual)    // second rounding on purpose: the same result as a separate add over the stored C
+            val = Elem<T>::from_f32(Elem<T>::to_f32(val) +
+                                    Elem<T>::to_f32((static_cast<const T*>(g.residual) + batch * g.sc)[(int64_t)m * g.N + n]));
+        c[(int64_t)m * g.N + n] = val;
     }
 }
 
@@ -401,10 +411,10 @@ static int launch_simple(hipStream_t s, const GemmArgs& g, int64_t batch, int ta
 
 using namespace mhip;
 
-extern "C" int mhip_gemm(void* stream, const void* a, const void* b, const void* bias, void* c,
-                         int64_t M, int64_t N, int64_t K, int64_t batch, int64_t stride_a,
-                         int64_t stride_b, int64_t stride_c, int trans_a, int trans_b,
-                         int activation, int dtype) {
+static int gemm_entry(void* stream, const void* a, const void* b, const void* bias, const void* residual, void* c,
+                      int64_t M, int64_t N, int64_t K, int64_t batch, int64_t stride_a,
+                      int64_t stride_b, int64_t stride_c, int trans_a, int trans_b,
+                      int activation, int dtype) {
     if (M < 0 || N < 0 || K < 0 || batch < 0)
         return fail(MHIP_ERR_INVALID_ARGUMENT, "mhip_gemm: negative size");
     if (activation < MHIP_ACT_NONE || activation > MHIP_ACT_SIGMOID)
@@ -421,6 +431,7 @@ extern "C" int mhip_gemm(void* stream, const void* a, const void* b, const void*
     g.ldb = trans_b ? (int)K : (int)N;
     g.sa = stride_a; g.sb = stride_b; g.sc = stride_c;
     g.act = activation;
+    g.residual = residual;
     g.tiles_m = g.tiles_n = 0;
 
     const bool is16 = dtype == MHIP_BF16 || dtype == MHIP_F16;
@@ -440,4 +451,20 @@ extern "C" int mhip_gemm(void* stream, const void* a, const void* b, const void*
         case MHIP_F16: return launch_simple<f16_t>(s, g, batch, trans_a, trans_b);
         default: return fail(MHIP_ERR_UNSUPPORTED, "mhip_gemm: dtype %d (need f32, f16 or bf16)", dtype);
     }
+}
+
+extern "C" int mhip_gemm(void* stream, const void* a, const void* b, const void* bias, void* c,
+                         int64_t M, int64_t N, int64_t K, int64_t batch, int64_t stride_a,
+                         int64_t stride_b, int64_t stride_c, int trans_a, int trans_b,
+                         int activation, int dtype) {
+    return gemm_entry(stream, a, b, bias, nullptr, c, M, N, K, batch, stride_a, stride_b, stride_c, trans_a, trans_b,
+                      activation, dtype);
+}
+
+extern "C" int mhip_gemm_residual(void* stream, const void* a, const void* b, const void* bias,
+                                  const void* residual, void* c, int64_t M, int64_t N, int64_t K,
+                                  int64_t batch, int64_t stride_a, int64_t stride_b, int64_t stride_c,
+                                  int trans_a, int trans_b, int activation, int dtype) {
+    return gemm_entry(stream, a, b, bias, residual, c, M, N, K, batch, stride_a, stride_b, stride_c, trans_a, trans_b,
+                      activation, dtype);
 }

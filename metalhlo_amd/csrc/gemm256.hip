@@ -118,6 +118,7 @@ __global__ __launch_bounds__(256) void gemm256_kernel(GemmArgs g) {
     const char* a = reinterpret_cast<const char*>(static_cast<const T*>(g.a) + batch * g.sa);
     const char* b = reinterpret_cast<const char*>(static_cast<const T*>(g.b) + batch * g.sb);
     T* c = static_cast<T*>(g.c) + batch * g.sc;
+    const T* res = g.residual ? static_cast<const T*>(g.residual) + batch * g.sc : nullptr;
     const uint32_t a_bytes = (uint32_t)((int64_t)(TA ? g.K : g.M) * g.lda * 2);
     const uint32_t b_bytes = (uint32_t)((int64_t)(TB ? g.N : g.K) * g.ldb * 2);
 
@@ -188,7 +189,8 @@ __global__ __launch_bounds__(256) void gemm256_kernel(GemmArgs g) {
         const int m = m0 + wm * 128 + ml;
         const int n = n0 + wn * 128 + cc * 8;
         if (m < g.M && n < g.N) {
-            const u32x4 w = *reinterpret_cast<const u32x4*>(stage + ml * kRowPad + cc * 16);
+            u32x4 w = *reinterpret_cast<const u32x4*>(stage + ml * kRowPad + cc * 16);
+            if (res) w = add_chunk<T>(w, *reinterpret_cast<const u32x4*>(res + (int64_t)m * g.N + n));
             *reinterpret_cast<u32x4*>(c + (int64_t)m * g.N + n) = w;
         }
     }

@@ -22,6 +22,7 @@ struct GemmArgs {
     int64_t sa, sb, sc;     // batch strides in elements
     int act;
     int tiles_m, tiles_n;
+    const void* residual = nullptr;   // C's layout and batch stride; added after the activation (may alias c)
 };
 
 template <typename T> struct Mfma32;
@@ -78,6 +79,21 @@ __device__ inline float apply_act_c(float v) {
     if (ACT == MHIP_ACT_TANH) return 1.f - 2.f * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(2.f * kLog2e * v));
     return v;
 }
+// eight stored elements (one 16-byte chunk of a C row) plus eight residual elements: each sum
+// is rounded once more, exactly what a separate add kernel over the stored C would produce
+template <typename T>
+__device__ inline u32x4 add_chunk(u32x4 w, u32x4 r) {
+    Pack4<T> a0 = __builtin_bit_cast(Pack4<T>, u32x2{w.x, w.y}), a1 = __builtin_bit_cast(Pack4<T>, u32x2{w.z, w.w});
+    const Pack4<T> r0 = __builtin_bit_cast(Pack4<T>, u32x2{r.x, r.y}), r1 = __builtin_bit_cast(Pack4<T>, u32x2{r.z, r.w});
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        a0.v[e] = Elem<T>::from_f32(Elem<T>::to_f32(a0.v[e]) + Elem<T>::to_f32(r0.v[e]));
+        a1.v[e] = Elem<T>::from_f32(Elem<T>::to_f32(a1.v[e]) + Elem<T>::to_f32(r1.v[e]));
+    }
+    const u32x2 lo = __builtin_bit_cast(u32x2, a0), hi = __builtin_bit_cast(u32x2, a1);
+    return u32x4{lo.x, lo.y, hi.x, hi.y};
+}
+
 template <typename F>
 __device__ inline void dispatch_act(int act, F&& f) {
     switch (act) {

@@ -110,10 +110,10 @@ class GPT2:
                 q, k, v = kernels.split_qkv_heads(qkv.reshape(B, S, 3 * d), H)
                 a = kernels.flash_attention(q, k, v, is_causal=True)
                 a = kernels.transpose_0213(a).reshape(B * S, d)
-            x = kernels.add(x, kernels.matmul(a, l["w_o"], bias=l["b_o"]))
+            x = kernels.matmul(a, l["w_o"], bias=l["b_o"], residual=x)          # x + proj(a), one kernel
             h = kernels.layer_norm(x, l["ln2_g"], l["ln2_b"], eps=1e-5)
             u = kernels.matmul(h, l["w_fc"], bias=l["b_fc"], activation="gelu")
-            x = kernels.add(x, kernels.matmul(u, l["w_proj"], bias=l["b_proj"]))
+            x = kernels.matmul(u, l["w_proj"], bias=l["b_proj"], residual=x)
         x = kernels.layer_norm(x, p["lnf_g"], p["lnf_b"], eps=1e-5)
         logits = kernels.matmul(x, p["wte_pad"], trans_b=True)   # tied head: x . wte^T (padded columns are 0)
         return logits.reshape(B, S, self.vocab_pad)[..., :cfg.vocab]

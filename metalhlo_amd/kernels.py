@@ -112,10 +112,11 @@ def gelu(x):
 
 
 def matmul(a, b, bias=None, activation: str = "none", trans_a: bool = False,
-           trans_b: bool = False, out: Optional[torch.Tensor] = None):
-    """act(op(a) @ op(b) + bias); leading dims of `a` are batch dims when `b` is
-    batched too, otherwise they fold into M."""
-    _dev(a, b, bias, out)
+           trans_b: bool = False, out: Optional[torch.Tensor] = None,
+           residual: Optional[torch.Tensor] = None):
+    """act(op(a) @ op(b) + bias) (+ residual, which has the result's shape and may be `out`);
+    leading dims of `a` are batch dims when `b` is batched too, otherwise they fold into M."""
+    _dev(a, b, bias, out, residual)
     lib = _lib.load()
     if a.dtype != b.dtype:
         raise TypeError("operand dtypes differ")
@@ -140,9 +141,16 @@ def matmul(a, b, bias=None, activation: str = "none", trans_a: bool = False,
         raise ValueError("bias must be [N] of the operand dtype")
     if out is None:
         out = torch.empty(out_lead + (N,), dtype=a.dtype, device=a.device)
-    _lib.check(lib.mhip_gemm(_stream(), a2.data_ptr(), b.data_ptr(), _ptr(bias), out.data_ptr(),
-                             M, N, K, batch, sa, sb, M * N, int(trans_a), int(trans_b),
-                             ACTIVATION_CODE[activation], _code(a)))
+    if residual is None:
+        _lib.check(lib.mhip_gemm(_stream(), a2.data_ptr(), b.data_ptr(), _ptr(bias), out.data_ptr(),
+                                 M, N, K, batch, sa, sb, M * N, int(trans_a), int(trans_b),
+                                 ACTIVATION_CODE[activation], _code(a)))
+    else:
+        if residual.numel() != out.numel() or residual.dtype != out.dtype:
+            raise ValueError("residual must have the result's size and dtype")
+        _lib.check(lib.mhip_gemm_residual(_stream(), a2.data_ptr(), b.data_ptr(), _ptr(bias), residual.data_ptr(),
+                                          out.data_ptr(), M, N, K, batch, sa, sb, M * N, int(trans_a), int(trans_b),
+                                          ACTIVATION_CODE[activation], _code(a)))
     return out
 
 

@@ -194,6 +194,34 @@ def test_gemm_large_exact_small_integers():
     assert torch.equal(kernels.matmul(a, b.t().contiguous(), trans_b=True), c)
 
 
+@pytest.mark.parametrize("tile", ["128", "256", "2560", "simple"])
+def test_gemm_residual_equals_gemm_then_add(tile, monkeypatch):
+    """act(A.B + bias) + R in one kernel is bit for bit mhip_gemm followed by mhip_add, on every
+    GEMM kernel (tile choice forced), batched and in place (R == C)."""
+    from metalhlo_amd import kernels
+    rng = np.random.default_rng(48)
+    for (batch, M, N, K, act) in [(1, 512, 768, 320, "none"), (3, 300, 264, 96, "gelu"), (1, 8192, 768, 768, "none")]:
+        if tile == "simple":
+            N += 1                                   # odd N: 16-byte paths off
+        else:
+            monkeypatch.setenv("MHIP_GEMM_TILE", tile)
+        shape_a, shape_b = ((batch, M, K), (batch, K, N)) if batch > 1 else ((M, K), (K, N))
+        a = to_dev(rng.standard_normal(shape_a), torch.bfloat16)
+        b = to_dev(rng.standard_normal(shape_b) * 0.1, torch.bfloat16)
+        bias = to_dev(rng.standard_normal(N), torch.bfloat16)
+        r = to_dev(rng.standard_normal(shape_a[:-1] + (N,)), torch.bfloat16)
+        two = kernels.add(kernels.matmul(a, b, bias=bias, activation=act), r)
+        one = kernels.matmul(a, b, bias=bias, activation=act, residual=r)
+        assert torch.equal(one, two), f"{tile} {(batch, M, N, K, act)}"
+        inplace = r.clone()
+        kernels.matmul(a, b, bias=bias, activation=act, residual=inplace, out=inplace)
+        assert torch.equal(inplace, two), f"in place, {tile} {(batch, M, N, K, act)}"
+    f = to_dev(rng.standard_normal((33, 17)), torch.float32)
+    g = to_dev(rng.standard_normal((17, 9)), torch.float32)
+    r = to_dev(rng.standard_normal((33, 9)), torch.float32)
+    assert torch.equal(kernels.matmul(f, g, residual=r), kernels.add(kernels.matmul(f, g), r))
+
+
 def test_gemm_errors(lib):
     assert lib.mhip_gemm(None, None, None, None, None, 4, 4, 4, 1, 0, 0, 0, 0, 0, 0, 3) == 1
     x = torch.zeros(4, 4, dtype=torch.int32, device="cuda")
