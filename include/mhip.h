@@ -115,7 +115,8 @@ int mhip_bias_gelu(void* stream, const void* x, const void* bias, void* y, int64
  * op(A) is [M,K] (stored [K,M] when trans_a), op(B) is [K,N] (stored [N,K]
  * when trans_b); strides are in elements between consecutive batch matrices
  * (0 broadcasts an operand).  bias (length N, same dtype) may be NULL.
- * fp32 accumulate, one rounding at the store.  dtype: BF16, F16, F32.
+ * fp32 accumulate, one rounding at the store.  dtype: BF16, F16, F32; also F64 (f64
+ * accumulate) and I32 / I64 (wrap-around), those three without activation.
  * Replaces the kernel_matmul family and kernel_matmul_bias_act
  * (Compiler/CodeGenerator.swift:3155-4068, 4797-4850); M/K/N/batch are what
  * dotGeneralDims (:5939-5970) derives. */
@@ -175,6 +176,21 @@ int mhip_gather_rows(void* stream, const void* table, const void* indices, void*
                      int64_t n_idx, int64_t n_rows, int64_t row_elems, int table_dtype,
                      int idx_dtype);
 
+/* General stablehlo.gather from a descriptor the caller derives from the dimension
+ * numbers: for the result element with indices i_0 .. i_{rank-1},
+ *   out[i] = operand[sum_d i_d * out_operand_strides[d]
+ *                    + sum_c clamp(indices[sum_d i_d * out_index_strides[d] + c * component_stride],
+ *                                  0, component_max[c]) * component_operand_strides[c]]
+ * (offset and batching dims carry an operand stride, batch dims an index stride; component c is
+ * the start index along operand dim start_index_map[c], clamped to dim - slice_size).  rank and
+ * n_components <= 8; elem_size in {1,2,4,8}; idx_dtype I32 or I64.
+ * Replaces the gather kernels of Compiler/CodeGenerator.swift:1133-1397 in their general form. */
+int mhip_gather(void* stream, const void* operand, const void* indices, void* out, int rank,
+                const int64_t* out_shape, const int64_t* out_operand_strides,
+                const int64_t* out_index_strides, int n_components, int64_t component_stride,
+                const int64_t* component_operand_strides, const int64_t* component_max, int elem_size,
+                int idx_dtype);
+
 /* dst = src, `bytes` bytes, device to device, as one streaming kernel (reshape /
  * copy; also the calibration kernel for the HBM traffic counters).
  * Replaces the copy kernels of Compiler/CodeGenerator.swift:851-921. */
@@ -193,7 +209,8 @@ int mhip_embed_tokens(void* stream, const void* ids, const void* wte, const void
 int mhip_add(void* stream, const void* a, const void* b, void* y, int64_t n, int dtype);
 
 /* y = convert(x), n elements (Compiler/CodeGenerator.swift:1012-1078).
- * Float narrowing is round-to-nearest-even; float -> int truncates toward zero. */
+ * Any pair of the element types; float narrowing is round-to-nearest-even, float -> int
+ * truncates toward zero, int -> int keeps the low bits, anything -> I1 is x != 0. */
 int mhip_convert(void* stream, const void* x, void* y, int64_t n, int src_dtype, int dst_dtype);
 
 /* [d0,d1,d2,d3] -> [d0,d2,d1,d3] (head split / merge;
@@ -227,11 +244,14 @@ typedef enum { MHIP_CMP_EQ = 0, MHIP_CMP_NE, MHIP_CMP_LT, MHIP_CMP_LE, MHIP_CMP_
 typedef enum { MHIP_RED_SUM = 0, MHIP_RED_MAX, MHIP_RED_MIN, MHIP_RED_PROD } mhip_reduce_op;
 
 /* y = op(x) elementwise (unary kernels, Compiler/CodeGenerator.swift:851-920).
- * F32/F16/BF16 (fp32 math, one rounding); NEG and ABS also on I32/I64. */
+ * F32/F16/BF16 (fp32 math, one rounding) and F64; NEG and ABS also on every integer
+ * type (negate wraps, also for the unsigned types). */
 int mhip_unary(void* stream, int op, const void* x, void* y, int64_t n, int dtype);
 
 /* y = a op b elementwise, equal shapes (binary kernels, CodeGenerator.swift:921-1010).
- * Floats: fp32 math, one rounding, max/min propagate NaN; integers wrap. */
+ * Floats: fp32 math (F64: f64), one rounding, max/min propagate NaN; integers wrap, POW
+ * with a negative exponent gives 1 / x^|e| truncated (1, +-1 or 0); I1: ADD and MAX are
+ * OR, MUL and MIN are AND, no DIV / POW. */
 int mhip_binary(void* stream, int op, const void* a, const void* b, void* y, int64_t n, int dtype);
 
 /* y[i] = (a[i] <dir> b[i]) as one byte 0/1 (stablehlo.compare, CodeGenerator.swift:1101). */

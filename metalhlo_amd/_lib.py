@@ -45,6 +45,8 @@ SIGNATURES = {
     "mhip_compare": (_i32, [_vp, _i32, _vp, _vp, _vp, _i64, _i32]),
     "mhip_select": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32]),
     "mhip_strided_copy": (_i32, [_vp, _vp, _vp, _i32, C.POINTER(_i64), C.POINTER(_i64), _i64, _i32]),
+    "mhip_gather": (_i32, [_vp, _vp, _vp, _vp, _i32, C.POINTER(_i64), C.POINTER(_i64), C.POINTER(_i64), _i32, _i64,
+                           C.POINTER(_i64), C.POINTER(_i64), _i32, _i32]),
     "mhip_reduce": (_i32, [_vp, _i32, _vp, _vp, _i64, _i64, _i64, C.c_double, _i32]),
     "mhip_fill": (_i32, [_vp, _vp, _i64, C.c_uint64, _i32]),
     "mhip_argmax": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32]),

@@ -19,40 +19,72 @@ static int ew_grid(int64_t n, unsigned* out) {
     return MHIP_OK;
 }
 
+// Compute type of a floating element type: fp32 for the 16- and 32-bit types (one rounding at
+// the store), double for f64.
 template <typename T> struct Num {
+    typedef float F;
     __device__ static float ld(const T* p, int64_t i) { return (float)p[i]; }
     __device__ static void st(T* p, int64_t i, float v) { p[i] = (T)v; }
+};
+template <> struct Num<double> {
+    typedef double F;
+    __device__ static double ld(const double* p, int64_t i) { return p[i]; }
+    __device__ static void st(double* p, int64_t i, double v) { p[i] = v; }
 };
 
 template <typename T>
 __global__ __launch_bounds__(256) void unary_kernel(const T* __restrict__ x, T* __restrict__ y,
                                                     int64_t n, int op) {
+    typedef typename Num<T>::F F;
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= n) return;
-    const float v = Num<T>::ld(x, i);
-    float r;
+    const F v = Num<T>::ld(x, i);
+    F r;
     switch (op) {
-        case MHIP_UN_EXP: r = expf(v); break;
-        case MHIP_UN_TANH: r = tanhf(v); break;
-        case MHIP_UN_RSQRT: r = 1.f / sqrtf(v); break;
-        case MHIP_UN_SQRT: r = sqrtf(v); break;
+        case MHIP_UN_EXP: r = exp(v); break;
+        case MHIP_UN_TANH: r = tanh(v); break;
+        case MHIP_UN_RSQRT: r = (F)1 / sqrt(v); break;
+        case MHIP_UN_SQRT: r = sqrt(v); break;
         case MHIP_UN_NEG: r = -v; break;
-        case MHIP_UN_LOGISTIC: r = 1.f / (1.f + expf(-v)); break;
-        case MHIP_UN_ABS: r = fabsf(v); break;
-        case MHIP_UN_LOG: r = logf(v); break;
-        case MHIP_UN_ERF: r = erff(v); break;
+        case MHIP_UN_LOGISTIC: r = (F)1 / ((F)1 + exp(-v)); break;
+        case MHIP_UN_ABS: r = fabs(v); break;
+        case MHIP_UN_LOG: r = log(v); break;
+        case MHIP_UN_ERF: r = erf(v); break;
         default: r = v; break;
     }
     Num<T>::st(y, i, r);
 }
 
+// negate wraps around (also for unsigned types); abs of an unsigned value is the value
 template <typename T>
 __global__ __launch_bounds__(256) void unary_int_kernel(const T* __restrict__ x, T* __restrict__ y,
                                                         int64_t n, int op) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= n) return;
+    typedef typename std::make_unsigned<T>::type U;
     const T v = x[i];
-    y[i] = op == MHIP_UN_NEG ? (T)(0 - v) : (op == MHIP_UN_ABS ? (v < 0 ? (T)(0 - v) : v) : v);
+    const T neg = (T)((U)0 - (U)v);
+    y[i] = op == MHIP_UN_NEG ? neg : (op == MHIP_UN_ABS ? ((std::is_signed<T>::value && v < 0) ? neg : v) : v);
+}
+
+// Integer power as StableHLO defines it: repeated wrap-around multiplication for a
+// non-negative exponent; for a negative one 1 / x^|e| truncated, i.e. 1 for x = 1,
+// (-1)^|e| for x = -1 and 0 otherwise.
+template <typename T>
+__device__ inline T int_pow(T base, T e) {
+    typedef typename std::make_unsigned<T>::type U;
+    if (std::is_signed<T>::value && e < 0) {
+        if (base == (T)1) return (T)1;
+        if (base == (T)-1) return ((U)e & 1) ? (T)-1 : (T)1;
+        return (T)0;
+    }
+    U r = 1, b = (U)base, k = (U)e;
+    while (k) {
+        if (k & 1) r *= b;
+        b *= b;
+        k >>= 1;
+    }
+    return (T)r;
 }
 
 // fp32 math for float types (one rounding at the store); exact wrap-around
@@ -73,24 +105,36 @@ __global__ __launch_bounds__(256) void binary_kernel(const T* __restrict__ a, co
             case MHIP_BIN_DIV: r = v == 0 ? (T)-1 : (T)(u / v); break;
             case MHIP_BIN_MAX: r = u > v ? u : v; break;
             case MHIP_BIN_MIN: r = u < v ? u : v; break;
+            case MHIP_BIN_POW: r = int_pow<T>(u, v); break;
             default: r = u; break;
         }
         y[i] = r;
     } else {
-        const float u = Num<T>::ld(a, i), v = Num<T>::ld(b, i);
-        float r;
+        typedef typename Num<T>::F F;
+        const F u = Num<T>::ld(a, i), v = Num<T>::ld(b, i);
+        F r;
         switch (op) {
             case MHIP_BIN_ADD: r = u + v; break;
             case MHIP_BIN_SUB: r = u - v; break;
             case MHIP_BIN_MUL: r = u * v; break;
             case MHIP_BIN_DIV: r = u / v; break;
-            case MHIP_BIN_MAX: r = (u != u || v != v) ? NAN : fmaxf(u, v); break;
-            case MHIP_BIN_MIN: r = (u != u || v != v) ? NAN : fminf(u, v); break;
-            case MHIP_BIN_POW: r = powf(u, v); break;
+            case MHIP_BIN_MAX: r = (u != u || v != v) ? (F)NAN : fmax(u, v); break;
+            case MHIP_BIN_MIN: r = (u != u || v != v) ? (F)NAN : fmin(u, v); break;
+            case MHIP_BIN_POW: r = pow(u, v); break;
             default: r = u; break;
         }
         Num<T>::st(y, i, r);
     }
+}
+
+// booleans (one byte each, 0 / 1): add and maximum are OR, multiply and minimum are AND
+__global__ __launch_bounds__(256) void binary_bool_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
+                                                          uint8_t* __restrict__ y, int64_t n, int op) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const bool u = a[i] != 0, v = b[i] != 0;
+    y[i] = (op == MHIP_BIN_ADD || op == MHIP_BIN_MAX) ? (u || v) : (op == MHIP_BIN_MUL || op == MHIP_BIN_MIN) ? (u && v)
+         : op == MHIP_BIN_SUB ? (u != v) : u;
 }
 
 template <typename T>
@@ -104,7 +148,7 @@ __global__ __launch_bounds__(256) void compare_kernel(const T* __restrict__ a, c
         r = dir == MHIP_CMP_EQ ? u == v : dir == MHIP_CMP_NE ? u != v : dir == MHIP_CMP_LT ? u < v
           : dir == MHIP_CMP_LE ? u <= v : dir == MHIP_CMP_GT ? u > v : u >= v;
     } else {
-        const float u = Num<T>::ld(a, i), v = Num<T>::ld(b, i);
+        const typename Num<T>::F u = Num<T>::ld(a, i), v = Num<T>::ld(b, i);
         r = dir == MHIP_CMP_EQ ? u == v : dir == MHIP_CMP_NE ? u != v : dir == MHIP_CMP_LT ? u < v
           : dir == MHIP_CMP_LE ? u <= v : dir == MHIP_CMP_GT ? u > v : u >= v;
     }
@@ -139,6 +183,39 @@ __global__ __launch_bounds__(256) void strided_copy_kernel(const W* __restrict__
             rem /= s.out_shape[d];
             src += idx * s.in_stride[d];
         }
+    }
+    y[o] = x[src];
+}
+
+// General gather: every output element reads operand[base(o) + sum_c clamp(index_c(o)) * stride_c].
+struct GatherArgs {
+    int rank, n_comp;
+    int64_t out_shape[8];
+    int64_t op_stride[8];    // operand elements per step of each result dim (offset and batching dims)
+    int64_t idx_stride[8];   // index elements per step of each result dim (batch dims)
+    int64_t comp_stride;     // between the components of one index vector
+    int64_t comp_op_stride[8], comp_max[8];
+};
+
+template <typename W, typename I>
+__global__ __launch_bounds__(256) void gather_kernel(const W* __restrict__ x, const I* __restrict__ idx,
+                                                     W* __restrict__ y, int64_t n, GatherArgs g) {
+    const int64_t o = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (o >= n) return;
+    int64_t rem = o, src = 0, ib = 0;
+#pragma unroll
+    for (int d = 7; d >= 0; d--) {
+        if (d < g.rank) {
+            const int64_t i = rem % g.out_shape[d];
+            rem /= g.out_shape[d];
+            src += i * g.op_stride[d];
+            ib += i * g.idx_stride[d];
+        }
+    }
+    for (int c = 0; c < g.n_comp; c++) {
+        int64_t v = (int64_t)idx[ib + c * g.comp_stride];
+        v = v < 0 ? 0 : (v > g.comp_max[c] ? g.comp_max[c] : v);
+        src += v * g.comp_op_stride[c];
     }
     y[o] = x[src];
 }
@@ -199,13 +276,25 @@ extern "C" int mhip_unary(void* stream, int op, const void* x, void* y, int64_t 
     unsigned grid;
     if (ew_grid(n, &grid)) return MHIP_ERR_UNSUPPORTED;
     hipStream_t s = as_stream(stream);
-    if (dtype == MHIP_I32 || dtype == MHIP_I64) {
+#define MHIP_UN_INT(T) hipLaunchKernelGGL((unary_int_kernel<T>), dim3(grid), dim3(256), 0, s, (const T*)x, (T*)y, n, op)
+    if (dtype >= MHIP_I8 && dtype <= MHIP_UI64) {
         if (op != MHIP_UN_NEG && op != MHIP_UN_ABS)
             return fail(MHIP_ERR_UNSUPPORTED, "%s: op %d on an integer type", what, op);
-        if (dtype == MHIP_I32)
-            hipLaunchKernelGGL((unary_int_kernel<int32_t>), dim3(grid), dim3(256), 0, s, (const int32_t*)x, (int32_t*)y, n, op);
-        else
-            hipLaunchKernelGGL((unary_int_kernel<int64_t>), dim3(grid), dim3(256), 0, s, (const int64_t*)x, (int64_t*)y, n, op);
+        switch (dtype) {
+            case MHIP_I8: MHIP_UN_INT(int8_t); break;
+            case MHIP_I16: MHIP_UN_INT(int16_t); break;
+            case MHIP_I32: MHIP_UN_INT(int32_t); break;
+            case MHIP_I64: MHIP_UN_INT(int64_t); break;
+            case MHIP_UI8: MHIP_UN_INT(uint8_t); break;
+            case MHIP_UI16: MHIP_UN_INT(uint16_t); break;
+            case MHIP_UI32: MHIP_UN_INT(uint32_t); break;
+            default: MHIP_UN_INT(uint64_t); break;
+        }
+        return check_launch(what);
+    }
+#undef MHIP_UN_INT
+    if (dtype == MHIP_F64) {
+        hipLaunchKernelGGL((unary_kernel<double>), dim3(grid), dim3(256), 0, s, (const double*)x, (double*)y, n, op);
         return check_launch(what);
     }
     MHIP_FLOAT_DISPATCH(dtype, hipLaunchKernelGGL((unary_kernel<T>), dim3(grid), dim3(256), 0, s, (const T*)x, (T*)y, n, op))
@@ -233,6 +322,13 @@ extern "C" int mhip_binary(void* stream, int op, const void* a, const void* b, v
         case MHIP_UI64: MHIP_BIN(uint64_t); break;
         case MHIP_I8: MHIP_BIN(int8_t); break;
         case MHIP_UI8: MHIP_BIN(uint8_t); break;
+        case MHIP_I16: MHIP_BIN(int16_t); break;
+        case MHIP_UI16: MHIP_BIN(uint16_t); break;
+        case MHIP_F64: MHIP_BIN(double); break;
+        case MHIP_I1:
+            if (op == MHIP_BIN_DIV || op == MHIP_BIN_POW) return fail(MHIP_ERR_UNSUPPORTED, "%s: op %d on booleans", what, op);
+            hipLaunchKernelGGL(binary_bool_kernel, dim3(grid), dim3(256), 0, s, (const uint8_t*)a, (const uint8_t*)b, (uint8_t*)y, n, op);
+            break;
         default: return fail(MHIP_ERR_UNSUPPORTED, "%s: dtype %d", what, dtype);
     }
 #undef MHIP_BIN
@@ -261,6 +357,9 @@ extern "C" int mhip_compare(void* stream, int direction, const void* a, const vo
         case MHIP_UI64: MHIP_CMP(uint64_t); break;
         case MHIP_I8: MHIP_CMP(int8_t); break;
         case MHIP_UI8: case MHIP_I1: MHIP_CMP(uint8_t); break;
+        case MHIP_I16: MHIP_CMP(int16_t); break;
+        case MHIP_UI16: MHIP_CMP(uint16_t); break;
+        case MHIP_F64: MHIP_CMP(double); break;
         default: return fail(MHIP_ERR_UNSUPPORTED, "%s: dtype %d", what, dtype);
     }
 #undef MHIP_CMP
@@ -320,6 +419,62 @@ extern "C" int mhip_strided_copy(void* stream, const void* x, void* y, int rank,
         default: return fail(MHIP_ERR_UNSUPPORTED, "%s: element size %d", what, elem_size);
     }
 #undef MHIP_SC
+    return check_launch(what);
+}
+
+extern "C" int mhip_gather(void* stream, const void* operand, const void* indices, void* out, int rank,
+                           const int64_t* out_shape, const int64_t* out_operand_strides,
+                           const int64_t* out_index_strides, int n_components, int64_t component_stride,
+                           const int64_t* component_operand_strides, const int64_t* component_max,
+                           int elem_size, int idx_dtype) {
+    const char* what = "mhip_gather";
+    if (rank < 0 || rank > 8 || n_components < 0 || n_components > 8)
+        return fail(MHIP_ERR_UNSUPPORTED, "%s: rank %d / %d index components (max 8)", what, rank, n_components);
+    if ((rank > 0 && (!out_shape || !out_operand_strides || !out_index_strides)) ||
+        (n_components > 0 && (!component_operand_strides || !component_max)))
+        return fail(MHIP_ERR_INVALID_ARGUMENT, "%s: NULL descriptor", what);
+    GatherArgs g;
+    g.rank = rank;
+    g.n_comp = n_components;
+    g.comp_stride = component_stride;
+    int64_t n = 1;
+    for (int d = 0; d < 8; d++) {
+        g.out_shape[d] = d < rank ? out_shape[d] : 1;
+        g.op_stride[d] = d < rank ? out_operand_strides[d] : 0;
+        g.idx_stride[d] = d < rank ? out_index_strides[d] : 0;
+        g.comp_op_stride[d] = d < n_components ? component_operand_strides[d] : 0;
+        g.comp_max[d] = d < n_components ? component_max[d] : 0;
+        if (d < rank) {
+            if (out_shape[d] < 0) return fail(MHIP_ERR_INVALID_ARGUMENT, "%s: negative dimension", what);
+            n *= out_shape[d];
+        }
+        if (d < n_components && component_max[d] < 0)
+            return fail(MHIP_ERR_INVALID_ARGUMENT, "%s: a slice is larger than the operand", what);
+    }
+    if (n == 0) return MHIP_OK;
+    if (!operand || !out || (n_components > 0 && !indices)) return fail(MHIP_ERR_INVALID_ARGUMENT, "%s: NULL pointer", what);
+    if (idx_dtype != MHIP_I32 && idx_dtype != MHIP_I64)
+        return fail(MHIP_ERR_UNSUPPORTED, "%s: index dtype %d (need i32 or i64)", what, idx_dtype);
+    unsigned grid;
+    if (ew_grid(n, &grid)) return MHIP_ERR_UNSUPPORTED;
+    hipStream_t s = as_stream(stream);
+#define MHIP_GA(W)                                                                                                      \
+    do {                                                                                                                \
+        if (idx_dtype == MHIP_I32)                                                                                      \
+            hipLaunchKernelGGL((gather_kernel<W, int32_t>), dim3(grid), dim3(256), 0, s, (const W*)operand,             \
+                               (const int32_t*)indices, (W*)out, n, g);                                                 \
+        else                                                                                                            \
+            hipLaunchKernelGGL((gather_kernel<W, int64_t>), dim3(grid), dim3(256), 0, s, (const W*)operand,             \
+                               (const int64_t*)indices, (W*)out, n, g);                                                 \
+    } while (0)
+    switch (elem_size) {
+        case 1: MHIP_GA(uint8_t); break;
+        case 2: MHIP_GA(uint16_t); break;
+        case 4: MHIP_GA(uint32_t); break;
+        case 8: MHIP_GA(uint64_t); break;
+        default: return fail(MHIP_ERR_UNSUPPORTED, "%s: element size %d", what, elem_size);
+    }
+#undef MHIP_GA
     return check_launch(what);
 }
 

@@ -334,6 +334,42 @@ __global__ __launch_bounds__(256) void gemm_simple_kernel(GemmArgs g, int trans_
 }
 
 // ---------------------------------------------------------------------------
+// Exact kernel for i32 / i64 (wrap-around arithmetic) and f64: accumulates in the element
+// type itself, k ascending.  Bias and residual are plain adds; no activation.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void gemm_exact_kernel(GemmArgs g, int trans_a, int trans_b) {
+    typedef typename std::conditional<std::is_integral<T>::value, typename std::make_unsigned<
+        typename std::conditional<std::is_integral<T>::value, T, int>::type>::type, T>::type A;   // wraps without UB
+    __shared__ A As[16][17];
+    __shared__ A Bs[16][17];
+    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+    const int64_t batch = blockIdx.z;
+    const T* a = static_cast<const T*>(g.a) + batch * g.sa;
+    const T* b = static_cast<const T*>(g.b) + batch * g.sb;
+    T* c = static_cast<T*>(g.c) + batch * g.sc;
+    const int m = blockIdx.y * 16 + ty, n = blockIdx.x * 16 + tx;
+    A acc = 0;
+    for (int k0 = 0; k0 < g.K; k0 += 16) {
+        const int ka = k0 + tx, kb = k0 + ty;
+        A av = 0, bv = 0;
+        if (m < g.M && ka < g.K) av = (A)(trans_a ? a[(int64_t)ka * g.lda + m] : a[(int64_t)m * g.lda + ka]);
+        if (n < g.N && kb < g.K) bv = (A)(trans_b ? b[(int64_t)n * g.ldb + kb] : b[(int64_t)kb * g.ldb + n]);
+        As[ty][tx] = av;
+        Bs[ty][tx] = bv;
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < 16; k++) acc += As[ty][k] * Bs[k][tx];
+        __syncthreads();
+    }
+    if (m < g.M && n < g.N) {
+        if (g.bias) acc += (A) static_cast<const T*>(g.bias)[n];
+        if (g.residual) acc += (A)(static_cast<const T*>(g.residual) + batch * g.sc)[(int64_t)m * g.N + n];
+        c[(int64_t)m * g.N + n] = (T)acc;
+    }
+}
+
+// ---------------------------------------------------------------------------
 // Host dispatch
 // ---------------------------------------------------------------------------
 template <typename T, int BM, int BN, int WGM, int WGN, bool TA, bool TB>
@@ -407,6 +443,16 @@ static int launch_simple(hipStream_t s, const GemmArgs& g, int64_t batch, int ta
     return check_launch("gemm_simple");
 }
 
+template <typename T>
+static int launch_exact(hipStream_t s, const GemmArgs& g, int64_t batch, int ta, int tb) {
+    if (g.act != MHIP_ACT_NONE) return fail(MHIP_ERR_UNSUPPORTED, "gemm: no activation on i32 / i64 / f64");
+    const int64_t gx = (g.N + 15) / 16, gy = (g.M + 15) / 16;
+    if (gy > 65535 || batch > 65535) return fail(MHIP_ERR_UNSUPPORTED, "gemm: grid too large");
+    hipLaunchKernelGGL((gemm_exact_kernel<T>), dim3((unsigned)gx, (unsigned)gy, (unsigned)batch),
+                       dim3(256), 0, s, g, ta, tb);
+    return check_launch("gemm_exact");
+}
+
 }  // namespace mhip
 
 using namespace mhip;
@@ -449,7 +495,10 @@ static int gemm_entry(void* stream, const void* a, const void* b, const void* bi
         case MHIP_F32: return launch_simple<float>(s, g, batch, trans_a, trans_b);
         case MHIP_BF16: return launch_simple<bf16_t>(s, g, batch, trans_a, trans_b);
         case MHIP_F16: return launch_simple<f16_t>(s, g, batch, trans_a, trans_b);
-        default: return fail(MHIP_ERR_UNSUPPORTED, "mhip_gemm: dtype %d (need f32, f16 or bf16)", dtype);
+        case MHIP_I32: return launch_exact<int32_t>(s, g, batch, trans_a, trans_b);
+        case MHIP_I64: return launch_exact<int64_t>(s, g, batch, trans_a, trans_b);
+        case MHIP_F64: return launch_exact<double>(s, g, batch, trans_a, trans_b);
+        default: return fail(MHIP_ERR_UNSUPPORTED, "mhip_gemm: dtype %d (need f32, f16, bf16, f64, i32 or i64)", dtype);
     }
 }
 

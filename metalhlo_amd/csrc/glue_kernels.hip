@@ -126,9 +126,22 @@ __global__ __launch_bounds__(256) void convert_kernel(const S* __restrict__ x, D
     if (i >= n) return;
     if constexpr (std::is_integral<S>::value && std::is_integral<D>::value) {
         y[i] = (D)x[i];  // integer -> integer keeps all 64 bits
+    } else if constexpr (std::is_integral<S>::value && sizeof(S) == 8 && std::is_same<D, double>::value) {
+        y[i] = (double)x[i];                        // 64-bit integer -> f64: one rounding
+    } else if constexpr (std::is_same<S, double>::value && std::is_integral<D>::value && sizeof(D) == 8) {
+        y[i] = (D)x[i];
     } else {
         Cvt<D>::st(y, i, Cvt<S>::ld(x, i));
     }
+}
+
+// anything -> boolean: x != 0 (one byte per element)
+template <typename S>
+__global__ __launch_bounds__(256) void to_bool_kernel(const S* __restrict__ x, uint8_t* __restrict__ y, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    if constexpr (std::is_integral<S>::value) y[i] = x[i] != 0;
+    else y[i] = Cvt<S>::ld(x, i) != 0.0;
 }
 
 // fp32 -> 16-bit float, eight elements per lane (two 16-byte loads, one 16-byte store)
@@ -367,6 +380,10 @@ static int convert_from(hipStream_t s, const void* x, void* y, int64_t n, int ds
         case MHIP_UI32: MHIP_CV(uint32_t); break;
         case MHIP_UI8: MHIP_CV(uint8_t); break;
         case MHIP_I8: MHIP_CV(int8_t); break;
+        case MHIP_I16: MHIP_CV(int16_t); break;
+        case MHIP_UI16: MHIP_CV(uint16_t); break;
+        case MHIP_UI64: MHIP_CV(uint64_t); break;
+        case MHIP_I1: hipLaunchKernelGGL((to_bool_kernel<S>), dim3(grid), dim3(256), 0, s, (const S*)x, (uint8_t*)y, n); break;
         default: return fail(MHIP_ERR_UNSUPPORTED, "mhip_convert: destination dtype %d", dst);
     }
 #undef MHIP_CV
@@ -404,6 +421,9 @@ extern "C" int mhip_convert(void* stream, const void* x, void* y, int64_t n, int
         case MHIP_UI32: return convert_from<uint32_t>(s, x, y, n, dst_dtype);
         case MHIP_UI8: case MHIP_I1: return convert_from<uint8_t>(s, x, y, n, dst_dtype);
         case MHIP_I8: return convert_from<int8_t>(s, x, y, n, dst_dtype);
+        case MHIP_I16: return convert_from<int16_t>(s, x, y, n, dst_dtype);
+        case MHIP_UI16: return convert_from<uint16_t>(s, x, y, n, dst_dtype);
+        case MHIP_UI64: return convert_from<uint64_t>(s, x, y, n, dst_dtype);
         default: return fail(MHIP_ERR_UNSUPPORTED, "mhip_convert: source dtype %d", src_dtype);
     }
 }

@@ -148,6 +148,78 @@ static DotPlan plan_dot(const Op& op, const TensorType& lt, const TensorType& rt
     return p;
 }
 
+static std::vector<int64_t> dense_strides(const std::vector<int64_t>& shape) {
+    std::vector<int64_t> s(shape.size(), 1);
+    for (int i = (int)shape.size() - 2; i >= 0; i--) s[i] = s[i + 1] * shape[i + 1];
+    return s;
+}
+
+// stablehlo.gather as the descriptor mhip_gather takes.  Attribute slots of Op: limits =
+// slice_sizes, dims = collapsed_slice_dims, starts = start_index_map, strides = offset_dims,
+// iota_dim = index_vector_dim, lhs_batch / rhs_batch = operand / start_indices batching dims.
+struct GatherPlan {
+    bool whole_rows = false;          // operand [rows, d], indices pick rows: the embedding-lookup kernel
+    std::vector<int64_t> out_op_stride, out_idx_stride, comp_op_stride, comp_max;
+    int64_t comp_stride = 0;
+};
+
+static GatherPlan plan_gather(const Op& op, const TensorType& xt, const TensorType& it) {
+    GatherPlan p;
+    const int64_t xr = (int64_t)xt.shape.size(), ir = (int64_t)it.shape.size(), rr = (int64_t)op.out.shape.size();
+    if (it.dtype != I32 && it.dtype != I64) throw UnsupportedOp(where(op) + "gather indices must be i32 or i64");
+    if (op.out.dtype != xt.dtype) throw ParseError(where(op) + "gather changes the element type");
+    const int64_t ivd = op.iota_dim < 0 ? ir : op.iota_dim;
+    auto has = [](const std::vector<int64_t>& v, int64_t d) { return std::find(v.begin(), v.end(), d) != v.end(); };
+    if ((int64_t)op.limits.size() != xr || ivd > ir || rr > 8 || op.starts.size() > 8 || op.lhs_batch.size() != op.rhs_batch.size())
+        throw ParseError(where(op) + "bad gather dimension numbers");
+    const int64_t n_comp = ivd < ir ? it.shape[ivd] : 1;
+    if ((int64_t)op.starts.size() != n_comp) throw ParseError(where(op) + "start_index_map does not match the index vector");
+    const auto xs = dense_strides(xt.shape), is = dense_strides(it.shape);
+    for (int64_t d = 0; d < xr; d++) {
+        if (op.limits[d] < 0 || op.limits[d] > xt.shape[d]) throw ParseError(where(op) + "slice size outside the operand");
+        if ((has(op.dims, d) || has(op.lhs_batch, d)) && op.limits[d] > 1) throw ParseError(where(op) + "collapsed / batching dims need slice size 1");
+    }
+    // operand dims that stay in the result, in order: one per offset dim
+    std::vector<int64_t> kept;
+    for (int64_t d = 0; d < xr; d++) if (!has(op.dims, d) && !has(op.lhs_batch, d)) kept.push_back(d);
+    if (kept.size() != op.strides.size() || (int64_t)(op.strides.size() + (size_t)(ir - (ivd < ir ? 1 : 0))) != rr)
+        throw ParseError(where(op) + "offset_dims do not match the result rank");
+    // batch dims of the result walk the dims of start_indices other than index_vector_dim
+    std::vector<int64_t> idx_dims;
+    for (int64_t d = 0; d < ir; d++) if (d != ivd) idx_dims.push_back(d);
+    p.out_op_stride.assign(rr, 0);
+    p.out_idx_stride.assign(rr, 0);
+    size_t nb = 0, no = 0;
+    for (int64_t r = 0; r < rr; r++) {
+        if (has(op.strides, r)) {
+            const int64_t d = kept.at(no++);
+            if (op.out.shape[r] != op.limits[d]) throw ParseError(where(op) + "result shape does not match slice_sizes");
+            p.out_op_stride[r] = xs[d];
+        } else {
+            const int64_t d = idx_dims.at(nb++);
+            if (op.out.shape[r] != it.shape[d]) throw ParseError(where(op) + "result shape does not match start_indices");
+            p.out_idx_stride[r] = is[d];
+            for (size_t b = 0; b < op.rhs_batch.size(); b++)
+                if (op.rhs_batch[b] == d) {
+                    const int64_t od = op.lhs_batch[b];
+                    if (od < 0 || od >= xr || xt.shape[od] != it.shape[d]) throw ParseError(where(op) + "batching dims differ in size");
+                    p.out_op_stride[r] = xs[od];
+                }
+        }
+    }
+    p.comp_stride = ivd < ir ? is[ivd] : 0;
+    for (int64_t c = 0; c < n_comp; c++) {
+        const int64_t d = op.starts[c];
+        if (d < 0 || d >= xr) throw ParseError(where(op) + "start_index_map out of range");
+        p.comp_op_stride.push_back(xs[d]);
+        p.comp_max.push_back(xt.shape[d] - op.limits[d]);
+    }
+    p.whole_rows = xr == 2 && op.dims == std::vector<int64_t>{0} && op.starts == std::vector<int64_t>{0} &&
+                   op.limits == std::vector<int64_t>{1, xt.shape[1]} && op.lhs_batch.empty() &&
+                   (ivd == ir || (ivd == ir - 1 && it.shape[ivd] == 1)) && op.strides == std::vector<int64_t>{rr - 1};
+    return p;
+}
+
 // Reduced dims must form one contiguous block [a, b]; gives outer/len/inner.
 static bool reduce_block(const std::vector<int64_t>& shape, std::vector<int64_t> dims, int64_t& outer, int64_t& len,
                          int64_t& inner) {
@@ -209,15 +281,16 @@ void compile(Executable& exe) {
             }
         } else if (kUnary.count(n)) {
             if (!(in(0) == op.out)) throw ParseError(where(op) + "operand and result types differ");
-            const bool int_ok = (n == "negate" || n == "abs") && (op.out.dtype == I32 || op.out.dtype == I64);
-            if (!is_kernel_float(op.out.dtype) && !int_ok) throw UnsupportedOp(where(op) + "element type not supported");
+            const bool is_int = op.out.dtype >= I8 && op.out.dtype <= UI64;
+            const bool int_ok = (n == "negate" || n == "abs") && is_int;
+            if (!is_kernel_float(op.out.dtype) && op.out.dtype != F64 && !int_ok) throw UnsupportedOp(where(op) + "element type not supported");
         } else if (kBinary.count(n)) {
             if (!(in(0) == op.out) || !(in(1) == op.out)) throw ParseError(where(op) + "operand and result types differ");
-            if (op.out.dtype == F64 || op.out.dtype == I1 || op.out.dtype == I16 || op.out.dtype == UI16)
-                throw UnsupportedOp(where(op) + "element type not supported");
-            if (n == "power" && !is_kernel_float(op.out.dtype)) throw UnsupportedOp(where(op) + "integer power is not supported");
+            if (op.out.dtype == I1 && (n == "divide" || n == "power")) throw UnsupportedOp(where(op) + "not defined on booleans");
         } else if (n == "convert") {
             if (in(0).shape != op.out.shape) throw ParseError(where(op) + "convert changes the shape");
+            auto cv = [](int d) { return d >= F16 && d <= UI64; };   // every element type the parser knows
+            if (!cv(in(0).dtype) || !cv(op.out.dtype)) throw UnsupportedOp(where(op) + "element type not supported");
         } else if (n == "reshape") {
             if (in(0).numel() != op.out.numel() || in(0).dtype != op.out.dtype) throw ParseError(where(op) + "reshape changes the element count or type");
         } else if (n == "transpose") {
@@ -248,22 +321,24 @@ void compile(Executable& exe) {
             if (!is_kernel_float(in(0).dtype) && in(0).dtype != I32 && in(0).dtype != I64) throw UnsupportedOp(where(op) + "element type not supported");
             for (auto d : op.dims) if (d < 0 || d >= (int64_t)in(0).shape.size()) throw ParseError(where(op) + "dimension out of range");
         } else if (n == "dot" || n == "dot_general") {
-            if (!is_kernel_float(in(0).dtype) || in(0).dtype != in(1).dtype || op.out.dtype != in(0).dtype)
-                throw UnsupportedOp(where(op) + "dot needs f32 / f16 / bf16 operands and a result of the same type");
+            // operands of one type; the result has that type, or a wider floating one (the
+            // operands are then converted first and the product is taken in the result type)
+            auto dot_type = [](int d) { return is_kernel_float(d) || d == F64 || d == I32 || d == I64; };
+            const bool widen = is_kernel_float(in(0).dtype) && (op.out.dtype == F32 || op.out.dtype == F64) &&
+                               dtype_bytes(op.out.dtype) > dtype_bytes(in(0).dtype);
+            if (!dot_type(in(0).dtype) || in(0).dtype != in(1).dtype || (op.out.dtype != in(0).dtype && !widen))
+                throw UnsupportedOp(where(op) + "dot needs f32 / f16 / bf16 / f64 / i32 / i64 operands of one type");
             (void)plan_dot(op, in(0), in(1));
         } else if (n == "iota") {
             if (op.iota_dim < 0 || op.iota_dim >= (int64_t)op.out.shape.size()) throw ParseError(where(op) + "iota dim out of range");
         } else if (n == "compare") {
             if (!(in(0) == in(1)) || op.out.dtype != I1 || op.out.shape != in(0).shape) throw ParseError(where(op) + "bad compare types");
-            if (in(0).dtype == F64 || in(0).dtype == I16 || in(0).dtype == UI16) throw UnsupportedOp(where(op) + "element type not supported");
+
         } else if (n == "select") {
             if (!(in(1) == op.out) || !(in(2) == op.out) || in(0).dtype != I1) throw ParseError(where(op) + "bad select types");
             if (in(0).numel() != 1 && in(0).shape != op.out.shape) throw ParseError(where(op) + "predicate shape mismatch");
         } else if (n == "gather") {
-            // whole-row gather only: operand [rows, d], one collapsed / mapped dim 0
-            if (in(0).shape.size() != 2 || op.dims != std::vector<int64_t>{0} || op.starts != std::vector<int64_t>{0} ||
-                op.limits != std::vector<int64_t>{1, in(0).shape[1]} || (in(1).dtype != I32 && in(1).dtype != I64))
-                throw UnsupportedOp(where(op) + "only whole-row gathers (embedding lookups) are supported");
+            (void)plan_gather(op, in(0), in(1));
         } else if (n == "custom_call") {
             bool ok = false;
             for (auto t : kTargets) ok |= op.target == t;
@@ -287,12 +362,6 @@ void compile(Executable& exe) {
 // ---------------------------------------------------------------- execution
 static void check(int st, const Op& op) {
     if (st != MHIP_OK) throw ExecError(where(op) + mhip_last_error());
-}
-
-static std::vector<int64_t> dense_strides(const std::vector<int64_t>& shape) {
-    std::vector<int64_t> s(shape.size(), 1);
-    for (int i = (int)shape.size() - 2; i >= 0; i--) s[i] = s[i + 1] * shape[i + 1];
-    return s;
 }
 
 static DeviceTensor permuted_copy(Client& c, const DeviceTensor& x, const std::vector<int64_t>& perm, const Op& op) {
@@ -390,6 +459,12 @@ std::vector<DeviceTensor> execute(Executable& exe, const std::vector<DeviceTenso
             } else if (n == "dot" || n == "dot_general") {
                 DotPlan p = plan_dot(op, in(0).type, in(1).type);
                 DeviceTensor a = in(0), b = in(1);
+                if (a.type.dtype != dt) {    // result wider than the operands: convert, then multiply in the result type
+                    DeviceTensor a2 = c.allocate(TensorType{a.type.shape, dt}), b2 = c.allocate(TensorType{b.type.shape, dt});
+                    check(mhip_convert(s, a.data(), a2.data(), a.type.numel(), a.type.dtype, dt), op);
+                    check(mhip_convert(s, b.data(), b2.data(), b.type.numel(), b.type.dtype, dt), op);
+                    a = a2; b = b2;
+                }
                 if (p.lhs_copy) a = permuted_copy(c, a, p.lhs_perm, op);
                 if (p.rhs_copy) b = permuted_copy(c, b, p.rhs_perm, op);
                 check(mhip_gemm(s, a.data(), b.data(), nullptr, out.data(), p.M, p.N, p.K, p.B, p.M * p.K, p.K * p.N,
@@ -407,8 +482,14 @@ std::vector<DeviceTensor> execute(Executable& exe, const std::vector<DeviceTenso
                 check(mhip_select(s, in(0).data(), in(1).data(), in(2).data(), out.data(), cnt, dtype_bytes(dt),
                                   in(0).type.numel() == 1 && cnt != 1), op);
             } else if (n == "gather") {
-                check(mhip_gather_rows(s, in(0).data(), in(1).data(), out.data(), in(1).type.numel(), in(0).type.shape[0],
-                                       in(0).type.shape[1], in(0).type.dtype, in(1).type.dtype), op);
+                const GatherPlan p = plan_gather(op, in(0).type, in(1).type);
+                if (p.whole_rows)
+                    check(mhip_gather_rows(s, in(0).data(), in(1).data(), out.data(), in(1).type.numel(), in(0).type.shape[0],
+                                           in(0).type.shape[1], in(0).type.dtype, in(1).type.dtype), op);
+                else
+                    check(mhip_gather(s, in(0).data(), in(1).data(), out.data(), (int)op.out.shape.size(), op.out.shape.data(),
+                                      p.out_op_stride.data(), p.out_idx_stride.data(), (int)p.comp_max.size(), p.comp_stride,
+                                      p.comp_op_stride.data(), p.comp_max.data(), dtype_bytes(dt), in(1).type.dtype), op);
             } else if (n == "custom_call") {
                 const Config cfg = parse_config(op.backend_config);
                 const TensorType& xt = in(0).type;

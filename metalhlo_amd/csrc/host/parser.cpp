@@ -227,9 +227,8 @@ static void parse_dense(const std::string& body, Op& op) {
             if (j == i) throw ParseError("line " + std::to_string(op.line) + ": bad dense literal near '" + b.substr(i, 16) + "'");
             const std::string tok = b.substr(i, j - i);
             l.is_int = is_int;
-            if (is_int) l.i = strtoll(tok.c_str(), nullptr, 10);
+            if (is_int) l.i = tok[0] == '-' ? strtoll(tok.c_str(), nullptr, 10) : (int64_t)strtoull(tok.c_str(), nullptr, 10);   // ui64 keeps all 64 bits
             else l.f = strtod(tok.c_str(), nullptr);
-            if (is_int && tok.size() > 1 && tok[0] != '-' && l.i < 0) l.i = (int64_t)strtoull(tok.c_str(), nullptr, 10);
             i = j;
         }
         lits.push_back(l);
@@ -489,6 +488,8 @@ struct Parser {
             ints_after_key(h, "start_index_map", op.starts);
             ints_after_key(h, "offset_dims", op.strides);
             if (!int_after_key(h, "index_vector_dim", op.iota_dim)) op.iota_dim = -1;
+            ints_after_key(h, "operand_batching_dims", op.lhs_batch);
+            ints_after_key(h, "start_indices_batching_dims", op.rhs_batch);
         } else if (n == "constant") {
             const size_t d = h.find("dense<");
             if (d == std::string::npos) fail("constant without dense<...>");

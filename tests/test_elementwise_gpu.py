@@ -101,6 +101,92 @@ def test_binary_int_wraps(lib):
         assert torch.equal(m.bool(), a < b)
 
 
+def test_narrow_unsigned_bool_and_f64_types(lib):
+    """The element types beside f32 / 16-bit floats / i32 / i64: i8, i16 and the unsigned types wrap
+    like numpy's; booleans are OR / AND; f64 computes in f64; integer power follows StableHLO."""
+    rng = np.random.default_rng(74)
+    codes = {np.int8: 5, np.int16: 6, np.uint8: 9, np.uint16: 10, np.uint32: 11, np.uint64: 12}
+    n = 777
+    for np_dt, code in codes.items():
+        info = np.iinfo(np_dt)
+        an = rng.integers(info.min, info.max, n, dtype=np_dt, endpoint=True)
+        bn = rng.integers(info.min, info.max, n, dtype=np_dt, endpoint=True)
+        # torch has no arithmetic on the wider unsigned types: move bytes, compute in numpy
+        a = torch.from_numpy(an.view(np.uint8)).cuda()
+        b = torch.from_numpy(bn.view(np.uint8)).cuda()
+        y = torch.empty_like(a)
+        with np.errstate(over="ignore"):
+            for name, e in (("add", an + bn), ("sub", an - bn), ("mul", an * bn), ("max", np.maximum(an, bn)),
+                            ("min", np.minimum(an, bn))):
+                ok(lib, lib.mhip_binary(None, BIN[name], p(a), p(b), p(y), n, code))
+                assert np.array_equal(y.cpu().numpy().view(np_dt), e.astype(np_dt)), (np_dt, name)
+            ok(lib, lib.mhip_unary(None, UN["neg"], p(a), p(y), n, code))
+            assert np.array_equal(y.cpu().numpy().view(np_dt), (0 - an).astype(np_dt)), np_dt
+            ok(lib, lib.mhip_unary(None, UN["abs"], p(a), p(y), n, code))
+            assert np.array_equal(y.cpu().numpy().view(np_dt), np.abs(an).astype(np_dt)), np_dt
+        m = torch.empty(n, dtype=torch.uint8, device="cuda")
+        ok(lib, lib.mhip_compare(None, CMP["GE"], p(a), p(b), p(m), n, code))
+        assert np.array_equal(m.cpu().numpy().astype(bool), an >= bn), np_dt
+    # booleans
+    a = torch.from_numpy(rng.integers(0, 2, n).astype(np.uint8)).cuda()
+    b = torch.from_numpy(rng.integers(0, 2, n).astype(np.uint8)).cuda()
+    y = torch.empty_like(a)
+    for name, e in (("add", a | b), ("max", a | b), ("mul", a & b), ("min", a & b)):
+        ok(lib, lib.mhip_binary(None, BIN[name], p(a), p(b), p(y), n, 4))
+        assert torch.equal(y, e), name
+    assert lib.mhip_binary(None, BIN["div"], p(a), p(b), p(y), n, 4) == 2
+    # f64
+    x = torch.from_numpy(rng.uniform(0.1, 3.0, n)).cuda()
+    z = torch.from_numpy(rng.uniform(-2.0, 2.0, n)).cuda()
+    y = torch.empty_like(x)
+    for name, e in (("exp", x.exp()), ("log", x.log()), ("sqrt", x.sqrt()), ("rsqrt", x.rsqrt()), ("tanh", x.tanh()),
+                    ("erf", x.erf()), ("logistic", x.sigmoid()), ("neg", -x)):
+        ok(lib, lib.mhip_unary(None, UN[name], p(x), p(y), n, 2))
+        assert torch.allclose(y, e, rtol=1e-13, atol=1e-13), name
+    for name, e in (("add", x + z), ("div", x / z), ("pow", x ** z), ("max", torch.maximum(x, z))):
+        ok(lib, lib.mhip_binary(None, BIN[name], p(x), p(z), p(y), n, 2))
+        assert torch.allclose(y, e, rtol=1e-13, atol=1e-13), name
+    # integer power: wrap-around products; a negative exponent gives 1 / x^|e| truncated
+    base = torch.from_numpy(rng.integers(-9, 10, n)).cuda()
+    e = torch.from_numpy(rng.integers(-3, 25, n)).cuda()
+    y = torch.empty_like(base)
+    ok(lib, lib.mhip_binary(None, BIN["pow"], p(base), p(e), p(y), n, DT[torch.int64]))
+    want = []
+    for bb, ee in zip(base.tolist(), e.tolist()):
+        if ee < 0:
+            want.append(1 if bb == 1 else ((-1) ** (-ee) if bb == -1 else 0))
+        else:
+            v = (bb ** ee) % (1 << 64)
+            want.append(v - (1 << 64) if v >= 1 << 63 else v)
+    assert y.tolist() == want
+
+
+def test_convert_all_pairs(lib):
+    """Every pair of the thirteen element types against numpy's conversion of values every type holds exactly."""
+    np_of = {0: np.float16, 1: np.float32, 2: np.float64, 4: np.bool_, 5: np.int8, 6: np.int16, 7: np.int32, 8: np.int64,
+             9: np.uint8, 10: np.uint16, 11: np.uint32, 12: np.uint64}
+    vals = np.array([0, 1, 2, 0, 7, 100, 127, 0, 3, 64])
+    for sc, sdt in np_of.items():
+        src = vals.astype(sdt)
+        x = torch.from_numpy(src.view(np.uint8).copy()).cuda()
+        for dc, ddt in np_of.items():
+            y = torch.zeros(len(vals) * np.dtype(ddt).itemsize, dtype=torch.uint8, device="cuda")
+            ok(lib, lib.mhip_convert(None, p(x), p(y), len(vals), sc, dc))
+            got = y.cpu().numpy().view(np.uint8 if ddt is np.bool_ else ddt)
+            assert np.array_equal(got, src.astype(ddt).astype(got.dtype)), (sdt, ddt)
+    # 64-bit integers keep every bit; negative -> unsigned wraps; f64 -> integer truncates toward zero
+    big = torch.tensor([2 ** 63 - 1, -1, -2 ** 63, 2 ** 53 + 1], dtype=torch.int64, device="cuda")
+    y = torch.empty_like(big)
+    ok(lib, lib.mhip_convert(None, p(big), p(y), 4, 8, 12))
+    assert torch.equal(y, big)
+    f = torch.tensor([-2.9, 2.9, -0.5, 1e15 + 1], dtype=torch.float64, device="cuda")
+    ok(lib, lib.mhip_convert(None, p(f), p(y), 4, 2, 8))
+    assert y.tolist() == [-2, 2, 0, 10 ** 15 + 1]
+    d = torch.empty(4, dtype=torch.float64, device="cuda")
+    ok(lib, lib.mhip_convert(None, p(big), p(d), 4, 8, 2))
+    assert d.tolist() == [float(2 ** 63 - 1), -1.0, float(-2 ** 63), float(2 ** 53 + 1)]
+
+
 def strided(lib, x, out_shape, strides, offset=0):
     y = torch.empty(out_shape, dtype=x.dtype, device="cuda")
     sh = (C.c_int64 * len(out_shape))(*out_shape)

@@ -222,10 +222,38 @@ def test_gemm_residual_equals_gemm_then_add(tile, monkeypatch):
     assert torch.equal(kernels.matmul(f, g, residual=r), kernels.add(kernels.matmul(f, g), r))
 
 
+@pytest.mark.parametrize("dtype", [torch.int32, torch.int64, torch.float64], ids=["i32", "i64", "f64"])
+def test_gemm_exact_types(dtype):
+    """i32 / i64 products wrap around like the CPU's; f64 accumulates in f64 (checked to 1e-12)."""
+    from metalhlo_amd import kernels
+    rng = np.random.default_rng(31)
+    for (batch, M, N, K, ta, tb) in [((), 33, 17, 45, False, False), ((3,), 20, 31, 16, True, False), ((2,), 7, 5, 130, False, True)]:
+        sa = batch + ((K, M) if ta else (M, K))
+        sb = batch + ((N, K) if tb else (K, N))
+        if dtype == torch.float64:
+            a, b = torch.from_numpy(rng.standard_normal(sa)), torch.from_numpy(rng.standard_normal(sb))
+        else:
+            hi = 2 ** 20 if dtype == torch.int32 else 2 ** 40                    # products overflow: wrap-around is exercised
+            a = torch.from_numpy(rng.integers(-hi, hi, sa)).to(dtype)
+            b = torch.from_numpy(rng.integers(-hi, hi, sb)).to(dtype)
+        ea = a.transpose(-1, -2) if ta else a
+        eb = b.transpose(-1, -2) if tb else b
+        if dtype == torch.float64:
+            e = ea @ eb
+        else:                                                                    # numpy integer matmul wraps
+            e = torch.from_numpy(np.matmul(ea.numpy(), eb.numpy()))
+        got = kernels.matmul(a.cuda(), b.cuda(), trans_a=ta, trans_b=tb).cpu()
+        if dtype == torch.float64:
+            assert torch.allclose(got, e, rtol=1e-12, atol=1e-12)
+        else:
+            assert torch.equal(got, e)
+
+
 def test_gemm_errors(lib):
     assert lib.mhip_gemm(None, None, None, None, None, 4, 4, 4, 1, 0, 0, 0, 0, 0, 0, 3) == 1
     x = torch.zeros(4, 4, dtype=torch.int32, device="cuda")
     p = x.data_ptr()
-    assert lib.mhip_gemm(None, p, p, None, p, 4, 4, 4, 1, 0, 0, 0, 0, 0, 0, 7) == 2   # int32 unsupported
+    assert lib.mhip_gemm(None, p, p, None, p, 4, 4, 4, 1, 0, 0, 0, 0, 0, 0, 5) == 2   # int8 unsupported
+    assert lib.mhip_gemm(None, p, p, None, p, 4, 4, 4, 1, 0, 0, 0, 0, 0, 1, 7) == 2   # no activation on int32
     assert lib.mhip_gemm(None, p, p, None, p, 4, 4, 4, 1, 0, 0, 0, 0, 0, 99, 1) == 1  # bad activation
     assert lib.mhip_gemm(None, p, p, None, p, 0, 4, 4, 1, 0, 0, 0, 0, 0, 0, 1) == 0   # empty is a no-op
