@@ -67,6 +67,7 @@ SIGNATURES = {
                                             C.POINTER(ExecutionProfile)]),
     "mhlo_free_string": (None, [_vp]),
     "mhlo_ext_executable_ops": (_vp, [_vp]),     # extension: op list after pattern recognition
+    "mhlo_ext_executable_plan": (_vp, [_vp]),    # extension: memory plan and launch statistics
 }
 
 _lib = None
@@ -126,6 +127,14 @@ class Session:
         p = self.lib.mhlo_ext_executable_ops(exe)
         try:
             return C.string_at(p).decode().split(",") if p else []
+        finally:
+            self.lib.mhlo_free_string(p)
+
+    def plan(self, exe) -> dict:
+        """Memory plan and launch statistics of an executable (integers by name)."""
+        p = self.lib.mhlo_ext_executable_plan(exe)
+        try:
+            return {k: int(v) for k, v in (kv.split("=") for kv in C.string_at(p).decode().split(","))} if p else {}
         finally:
             self.lib.mhlo_free_string(p)
 

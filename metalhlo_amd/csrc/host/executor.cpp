@@ -1,6 +1,7 @@
 #include "executor.h"
 
 #include <math.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <algorithm>
@@ -65,6 +66,77 @@ DeviceTensor Client::allocate(const TensorType& t) {
     d.mem->bytes = t.bytes();
     d.mem->ptr = pool.alloc(d.mem->bytes);
     return d;
+}
+
+Executable::~Executable() {
+    for (auto& g : graphs) if (g.exec) (void)hipGraphExecDestroy(g.exec);
+    if (arena) (void)hipFree(arena);
+}
+
+// Where the allocations of one walk over the program come from.
+struct Allocator {
+    enum Mode { POOL, RECORD, ARENA } mode = POOL;
+    Client* client = nullptr;
+    ArenaPlan* plan = nullptr;
+    char* base = nullptr;
+    bool escaping_in_arena = false;
+    size_t next = 0;
+
+    DeviceTensor allocate(const TensorType& t) {
+        if (mode == POOL) return client->allocate(t);
+        DeviceTensor d;
+        d.type = t;
+        d.mem = std::make_shared<DeviceMem>();
+        d.mem->bytes = t.bytes();
+        const size_t rounded = (t.bytes() + 255) & ~(size_t)255;
+        if (mode == RECORD) {
+            ArenaPlan::Slot sl;
+            sl.bytes = rounded;
+            sl.begin = plan->clock++;
+            plan->slots.push_back(sl);
+            d.mem->recorder = plan;
+            d.mem->slot = (int)plan->slots.size() - 1;
+            return d;
+        }
+        if (next >= plan->slots.size() || plan->slots[next].bytes != rounded)
+            throw ExecError("the execution does not follow the memory plan made at compile time");
+        const ArenaPlan::Slot& sl = plan->slots[next++];
+        if (sl.escapes && !escaping_in_arena) {
+            d.mem->pool = &client->pool;
+            d.mem->ptr = client->pool.alloc(d.mem->bytes);
+        } else {
+            d.mem->ptr = base + sl.offset;     // not owned: the arena outlives the execution
+        }
+        return d;
+    }
+};
+
+// Offsets for the recorded slots: largest first, each at the lowest 256-byte boundary where it
+// meets no already placed slot that is alive at the same time.
+static size_t place_slots(ArenaPlan& plan, bool escaping, size_t floor) {
+    std::vector<int> order;
+    for (int i = 0; i < (int)plan.slots.size(); i++) if (plan.slots[i].escapes == escaping) order.push_back(i);
+    std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return plan.slots[a].bytes > plan.slots[b].bytes; });
+    std::vector<int> placed;
+    size_t top = floor;
+    for (int i : order) {
+        ArenaPlan::Slot& s = plan.slots[i];
+        std::vector<std::pair<size_t, size_t>> busy;     // [offset, end) of the slots alive together with s
+        for (int j : placed) {
+            const ArenaPlan::Slot& o = plan.slots[j];
+            if (o.begin <= s.end && s.begin <= o.end) busy.emplace_back(o.offset, o.offset + o.bytes);
+        }
+        std::sort(busy.begin(), busy.end());
+        size_t at = floor;
+        for (auto& b : busy) {
+            if (at + s.bytes <= b.first) break;
+            at = std::max(at, b.second);
+        }
+        s.offset = at;
+        top = std::max(top, at + s.bytes);
+        placed.push_back(i);
+    }
+    return top;
 }
 
 // ---------------------------------------------------------------- op tables
@@ -253,6 +325,8 @@ static double scalar_constant(const Op& c) {
     }
 }
 
+static void plan_memory(Executable& exe);
+
 // ---------------------------------------------------------------- validation
 void compile(Executable& exe) {
     Function& fn = exe.fn;
@@ -355,8 +429,8 @@ void compile(Executable& exe) {
             throw UnsupportedOp(where(op) + "operation is outside the supported subset");
         }
     }
-    for (int r : fn.returns) (void)r;
     if (exe.client && exe.client->device >= 0) (void)hipStreamSynchronize(exe.client->stream);
+    plan_memory(exe);
 }
 
 // ---------------------------------------------------------------- execution
@@ -364,29 +438,27 @@ static void check(int st, const Op& op) {
     if (st != MHIP_OK) throw ExecError(where(op) + mhip_last_error());
 }
 
-static DeviceTensor permuted_copy(Client& c, const DeviceTensor& x, const std::vector<int64_t>& perm, const Op& op) {
+static DeviceTensor permuted_copy(Allocator& al, bool dry, void* stream, const DeviceTensor& x,
+                                  const std::vector<int64_t>& perm, const Op& op) {
     TensorType t;
     t.dtype = x.type.dtype;
     const auto st = dense_strides(x.type.shape);
     std::vector<int64_t> in_str;
     for (auto d : perm) { t.shape.push_back(x.type.shape[d]); in_str.push_back(st[d]); }
-    DeviceTensor y = c.allocate(t);
-    check(mhip_strided_copy(c.stream, x.data(), y.data(), (int)perm.size(), t.shape.data(), in_str.data(), 0,
-                            dtype_bytes(t.dtype)), op);
+    DeviceTensor y = al.allocate(t);
+    if (!dry)
+        check(mhip_strided_copy(stream, x.data(), y.data(), (int)perm.size(), t.shape.data(), in_str.data(), 0,
+                                dtype_bytes(t.dtype)), op);
     return y;
 }
 
-std::vector<DeviceTensor> execute(Executable& exe, const std::vector<DeviceTensor>& inputs, double* encode_s,
-                                  double* gpu_s) {
-    Client& c = *exe.client;
-    if (c.device < 0) throw NoDevice("no HIP device: cannot execute");
+// One walk over the program in order: every allocation comes from `al`, every launch goes to
+// the client's stream; with `dry` nothing is launched (the walk only shows `al` which
+// allocations an execution makes and when each is released).  Returns the value of each result.
+#define RUN(call) do { if (!dry) check((call), op); } while (0)
+static std::vector<DeviceTensor> run_ops(Executable& exe, const std::vector<DeviceTensor>& inputs, Allocator& al, bool dry) {
     const Function& fn = exe.fn;
-    if (inputs.size() != fn.arg_types.size())
-        throw InputMismatch("Expected " + std::to_string(fn.arg_types.size()) + " inputs, got " + std::to_string(inputs.size()));
-    for (size_t i = 0; i < inputs.size(); i++)
-        if (!(inputs[i].type == fn.arg_types[i]))
-            throw InputMismatch("Input " + std::to_string(i) + " has the wrong shape or element type");
-    const auto t0 = std::chrono::steady_clock::now();
+    void* s = exe.client ? exe.client->stream : nullptr;
     std::vector<DeviceTensor> val(fn.num_values);
     for (size_t i = 0; i < inputs.size(); i++) val[fn.arg_ids[i]] = inputs[i];
     // last use of every value, so that intermediates return to the pool early
@@ -395,7 +467,6 @@ std::vector<DeviceTensor> execute(Executable& exe, const std::vector<DeviceTenso
     for (int r : fn.returns) last[r] = (int)fn.ops.size();
     std::map<int, const Op*> producer;
     for (auto& op : fn.ops) producer[op.result] = &op;
-    void* s = c.stream;
 
     for (size_t oi = 0; oi < fn.ops.size(); oi++) {
         const Op& op = fn.ops[oi];
@@ -404,40 +475,41 @@ std::vector<DeviceTensor> execute(Executable& exe, const std::vector<DeviceTenso
         DeviceTensor out;
         if (n == "constant") {
             out = exe.constants[oi];
+            out.type = op.out;
         } else if (n == "reshape") {
             out = in(0);
             out.type = op.out;
         } else {
-            out = c.allocate(op.out);
+            out = al.allocate(op.out);
             const int dt = op.out.dtype;
             const int64_t cnt = op.out.numel();
             if (kUnary.count(n)) {
-                check(mhip_unary(s, kUnary.at(n), in(0).data(), out.data(), cnt, dt), op);
+                RUN(mhip_unary(s, kUnary.at(n), in(0).data(), out.data(), cnt, dt));
             } else if (kBinary.count(n)) {
-                check(mhip_binary(s, kBinary.at(n), in(0).data(), in(1).data(), out.data(), cnt, dt), op);
+                RUN(mhip_binary(s, kBinary.at(n), in(0).data(), in(1).data(), out.data(), cnt, dt));
             } else if (n == "convert") {
-                if (in(0).type.dtype == dt) check(mhip_copy(s, in(0).data(), out.data(), (int64_t)op.out.bytes()), op);
-                else check(mhip_convert(s, in(0).data(), out.data(), cnt, in(0).type.dtype, dt), op);
+                if (in(0).type.dtype == dt) RUN(mhip_copy(s, in(0).data(), out.data(), (int64_t)op.out.bytes()));
+                else RUN(mhip_convert(s, in(0).data(), out.data(), cnt, in(0).type.dtype, dt));
             } else if (n == "transpose") {
                 const auto st = dense_strides(in(0).type.shape);
                 std::vector<int64_t> is;
                 for (auto d : op.dims) is.push_back(st[d]);
-                check(mhip_strided_copy(s, in(0).data(), out.data(), (int)op.dims.size(), op.out.shape.data(), is.data(), 0,
-                                        dtype_bytes(dt)), op);
+                RUN(mhip_strided_copy(s, in(0).data(), out.data(), (int)op.dims.size(), op.out.shape.data(), is.data(), 0,
+                                        dtype_bytes(dt)));
             } else if (n == "broadcast_in_dim") {
                 const auto st = dense_strides(in(0).type.shape);
                 std::vector<int64_t> is(op.out.shape.size(), 0);
                 for (size_t d = 0; d < op.dims.size(); d++)
                     is[op.dims[d]] = in(0).type.shape[d] == 1 ? 0 : st[d];
-                check(mhip_strided_copy(s, in(0).data(), out.data(), (int)op.out.shape.size(), op.out.shape.data(), is.data(),
-                                        0, dtype_bytes(dt)), op);
+                RUN(mhip_strided_copy(s, in(0).data(), out.data(), (int)op.out.shape.size(), op.out.shape.data(), is.data(),
+                                        0, dtype_bytes(dt)));
             } else if (n == "slice") {
                 const auto st = dense_strides(in(0).type.shape);
                 std::vector<int64_t> is;
                 int64_t off = 0;
                 for (size_t d = 0; d < st.size(); d++) { is.push_back(st[d] * op.strides[d]); off += st[d] * op.starts[d]; }
-                check(mhip_strided_copy(s, in(0).data(), out.data(), (int)st.size(), op.out.shape.data(), is.data(), off,
-                                        dtype_bytes(dt)), op);
+                RUN(mhip_strided_copy(s, in(0).data(), out.data(), (int)st.size(), op.out.shape.data(), is.data(), off,
+                                        dtype_bytes(dt)));
             } else if (n == "reduce") {
                 const double init = scalar_constant(*producer.at(op.operands.at(1)));
                 int64_t outer, len, inner;
@@ -450,46 +522,46 @@ std::vector<DeviceTensor> execute(Executable& exe, const std::vector<DeviceTenso
                         if (std::find(red.begin(), red.end(), d) == red.end()) perm.push_back(d);
                     const size_t kept = perm.size();
                     perm.insert(perm.end(), red.begin(), red.end());
-                    x = permuted_copy(c, x, perm, op);
+                    x = permuted_copy(al, dry, s, x, perm, op);
                     outer = len = 1;
                     inner = 1;
                     for (size_t d = 0; d < perm.size(); d++) (d < kept ? outer : len) *= x.type.shape[d];
                 }
-                check(mhip_reduce(s, kReduce.at(op.reducer), x.data(), out.data(), outer, len, inner, init, dt), op);
+                RUN(mhip_reduce(s, kReduce.at(op.reducer), x.data(), out.data(), outer, len, inner, init, dt));
             } else if (n == "dot" || n == "dot_general") {
                 DotPlan p = plan_dot(op, in(0).type, in(1).type);
                 DeviceTensor a = in(0), b = in(1);
                 if (a.type.dtype != dt) {    // result wider than the operands: convert, then multiply in the result type
-                    DeviceTensor a2 = c.allocate(TensorType{a.type.shape, dt}), b2 = c.allocate(TensorType{b.type.shape, dt});
-                    check(mhip_convert(s, a.data(), a2.data(), a.type.numel(), a.type.dtype, dt), op);
-                    check(mhip_convert(s, b.data(), b2.data(), b.type.numel(), b.type.dtype, dt), op);
+                    DeviceTensor a2 = al.allocate(TensorType{a.type.shape, dt}), b2 = al.allocate(TensorType{b.type.shape, dt});
+                    RUN(mhip_convert(s, a.data(), a2.data(), a.type.numel(), a.type.dtype, dt));
+                    RUN(mhip_convert(s, b.data(), b2.data(), b.type.numel(), b.type.dtype, dt));
                     a = a2; b = b2;
                 }
-                if (p.lhs_copy) a = permuted_copy(c, a, p.lhs_perm, op);
-                if (p.rhs_copy) b = permuted_copy(c, b, p.rhs_perm, op);
-                check(mhip_gemm(s, a.data(), b.data(), nullptr, out.data(), p.M, p.N, p.K, p.B, p.M * p.K, p.K * p.N,
-                                p.M * p.N, p.trans_a, p.trans_b, MHIP_ACT_NONE, dt), op);
+                if (p.lhs_copy) a = permuted_copy(al, dry, s, a, p.lhs_perm, op);
+                if (p.rhs_copy) b = permuted_copy(al, dry, s, b, p.rhs_perm, op);
+                RUN(mhip_gemm(s, a.data(), b.data(), nullptr, out.data(), p.M, p.N, p.K, p.B, p.M * p.K, p.K * p.N,
+                                p.M * p.N, p.trans_a, p.trans_b, MHIP_ACT_NONE, dt));
             } else if (n == "iota") {
                 int64_t outer = 1, inner = 1;
                 for (int64_t d = 0; d < (int64_t)op.out.shape.size(); d++) {
                     if (d < op.iota_dim) outer *= op.out.shape[d];
                     else if (d > op.iota_dim) inner *= op.out.shape[d];
                 }
-                check(mhip_iota(s, out.data(), outer, op.out.shape[op.iota_dim], inner, dt), op);
+                RUN(mhip_iota(s, out.data(), outer, op.out.shape[op.iota_dim], inner, dt));
             } else if (n == "compare") {
-                check(mhip_compare(s, kCompare.at(op.direction), in(0).data(), in(1).data(), out.data(), cnt, in(0).type.dtype), op);
+                RUN(mhip_compare(s, kCompare.at(op.direction), in(0).data(), in(1).data(), out.data(), cnt, in(0).type.dtype));
             } else if (n == "select") {
-                check(mhip_select(s, in(0).data(), in(1).data(), in(2).data(), out.data(), cnt, dtype_bytes(dt),
-                                  in(0).type.numel() == 1 && cnt != 1), op);
+                RUN(mhip_select(s, in(0).data(), in(1).data(), in(2).data(), out.data(), cnt, dtype_bytes(dt),
+                                  in(0).type.numel() == 1 && cnt != 1));
             } else if (n == "gather") {
                 const GatherPlan p = plan_gather(op, in(0).type, in(1).type);
                 if (p.whole_rows)
-                    check(mhip_gather_rows(s, in(0).data(), in(1).data(), out.data(), in(1).type.numel(), in(0).type.shape[0],
-                                           in(0).type.shape[1], in(0).type.dtype, in(1).type.dtype), op);
+                    RUN(mhip_gather_rows(s, in(0).data(), in(1).data(), out.data(), in(1).type.numel(), in(0).type.shape[0],
+                                           in(0).type.shape[1], in(0).type.dtype, in(1).type.dtype));
                 else
-                    check(mhip_gather(s, in(0).data(), in(1).data(), out.data(), (int)op.out.shape.size(), op.out.shape.data(),
+                    RUN(mhip_gather(s, in(0).data(), in(1).data(), out.data(), (int)op.out.shape.size(), op.out.shape.data(),
                                       p.out_op_stride.data(), p.out_idx_stride.data(), (int)p.comp_max.size(), p.comp_stride,
-                                      p.comp_op_stride.data(), p.comp_max.data(), dtype_bytes(dt), in(1).type.dtype), op);
+                                      p.comp_op_stride.data(), p.comp_max.data(), dtype_bytes(dt), in(1).type.dtype));
             } else if (n == "custom_call") {
                 const Config cfg = parse_config(op.backend_config);
                 const TensorType& xt = in(0).type;
@@ -503,9 +575,9 @@ std::vector<DeviceTensor> execute(Executable& exe, const std::vector<DeviceTenso
                     outer = inner = 1;
                     for (int64_t d = 0; d < axis; d++) outer *= xt.shape[d];
                     for (int64_t d = axis + 1; d < (int64_t)xt.shape.size(); d++) inner *= xt.shape[d];
-                    check(mhip_softmax_strided(s, in(0).data(), out.data(), outer, xt.shape[axis], inner, dt), op);
+                    RUN(mhip_softmax_strided(s, in(0).data(), out.data(), outer, xt.shape[axis], inner, dt));
                 } else if (op.target == "fused_gelu") {
-                    check(mhip_bias_gelu(s, in(0).data(), nullptr, out.data(), rows, cols, dt), op);
+                    RUN(mhip_bias_gelu(s, in(0).data(), nullptr, out.data(), rows, cols, dt));
                 } else if (op.target == "fused_layer_norm" || op.target == "fused_rms_norm") {
                     const auto axes = cfg.get_int_array("axes", {-1});
                     if (axes.size() != 1 || (axes[0] != -1 && axes[0] != (int64_t)xt.shape.size() - 1))
@@ -514,9 +586,9 @@ std::vector<DeviceTensor> execute(Executable& exe, const std::vector<DeviceTenso
                     if (in(1).type.numel() != cols || in(1).type.dtype != dt) throw ExecError(where(op) + "gamma must be [cols] of the input type");
                     if (op.target == "fused_layer_norm") {
                         if (in(2).type.numel() != cols || in(2).type.dtype != dt) throw ExecError(where(op) + "beta must be [cols] of the input type");
-                        check(mhip_layer_norm(s, in(0).data(), in(1).data(), in(2).data(), out.data(), rows, cols, eps, dt), op);
+                        RUN(mhip_layer_norm(s, in(0).data(), in(1).data(), in(2).data(), out.data(), rows, cols, eps, dt));
                     } else {
-                        check(mhip_rms_norm(s, in(0).data(), in(1).data(), out.data(), rows, cols, eps, dt), op);
+                        RUN(mhip_rms_norm(s, in(0).data(), in(1).data(), out.data(), rows, cols, eps, dt));
                     }
                 } else if (op.target == "fused_matmul_bias_activation") {
                     const bool ta = cfg.get_bool("trans_a", false), tb = cfg.get_bool("trans_b", false);
@@ -528,8 +600,8 @@ std::vector<DeviceTensor> execute(Executable& exe, const std::vector<DeviceTenso
                     if (K != Kb || op.out.numel() != M * N) throw ExecError(where(op) + "operand shapes do not contract");
                     const void* bias = op.operands.size() > 2 ? in(2).data() : nullptr;
                     if (bias && (in(2).type.numel() != N || in(2).type.dtype != dt)) throw ExecError(where(op) + "bias must be [N] of the input type");
-                    check(mhip_gemm(s, in(0).data(), in(1).data(), bias, out.data(), M, N, K, 1, 0, 0, 0, ta, tb,
-                                    kActivation.at(cfg.get_string("activation", "none")), dt), op);
+                    RUN(mhip_gemm(s, in(0).data(), in(1).data(), bias, out.data(), M, N, K, 1, 0, 0, 0, ta, tb,
+                                    kActivation.at(cfg.get_string("activation", "none")), dt));
                 } else {   // fused_scaled_dot_product_attention
                     const TensorType& kt = in(1).type;
                     if (xt.shape.size() < 2 || kt.shape.size() != xt.shape.size() || !(in(2).type == kt) || kt.dtype != dt)
@@ -556,14 +628,176 @@ std::vector<DeviceTensor> execute(Executable& exe, const std::vector<DeviceTenso
                         msb = mb == B && B != 1 ? mh * Sq * Skv : 0;
                         mask = in(3).data();
                     }
-                    check(mhip_flash_attention(s, in(0).data(), in(1).data(), in(2).data(), mask, out.data(), B, H, Sq, Skv, D,
-                                               scale, cfg.get_bool("is_causal", false), msb, msh, dt), op);
+                    RUN(mhip_flash_attention(s, in(0).data(), in(1).data(), in(2).data(), mask, out.data(), B, H, Sq, Skv, D,
+                                               scale, cfg.get_bool("is_causal", false), msb, msh, dt));
                 }
             }
         }
         val[op.result] = out;
         for (int v : op.operands)
             if (last[v] == (int)oi) val[v] = DeviceTensor();
+    }
+    std::vector<DeviceTensor> rets;
+    for (int r : fn.returns) rets.push_back(val[r]);
+    return rets;
+}
+#undef RUN
+
+static bool env_flag(const char* name, bool dflt) {
+    const char* v = getenv(name);
+    return v && *v ? atoi(v) != 0 : dflt;
+}
+
+static void plan_memory(Executable& exe) {
+    exe.plan = ArenaPlan();
+    try {
+        Allocator al;
+        al.mode = Allocator::RECORD;
+        al.plan = &exe.plan;
+        std::vector<DeviceTensor> ins;
+        for (auto& t : exe.fn.arg_types) { DeviceTensor d; d.type = t; ins.push_back(d); }
+        {
+            const std::vector<DeviceTensor> rets = run_ops(exe, ins, al, true);
+            for (auto& r : rets) if (r.mem && r.mem->recorder) exe.plan.slots[r.mem->slot].escapes = true;
+        }
+        for (auto& sl : exe.plan.slots) {
+            if (sl.escapes) sl.end = 0x7FFFFFFF;
+            else exe.plan.sum_bytes += sl.bytes;
+        }
+        exe.plan.core_bytes = place_slots(exe.plan, false, 0);
+        exe.plan.full_bytes = place_slots(exe.plan, true, exe.plan.core_bytes);
+        exe.plan.valid = true;
+    } catch (const std::exception&) {
+        exe.plan = ArenaPlan();     // the execution reports the problem; it allocates per value
+    }
+}
+
+static void ensure_arena(Executable& exe, size_t bytes) {
+    bytes = std::max<size_t>(bytes, 256);
+    if (exe.arena && exe.arena_size >= bytes) return;
+    Client& c = *exe.client;
+    (void)hipStreamSynchronize(c.stream);
+    for (auto& g : exe.graphs) if (g.exec) (void)hipGraphExecDestroy(g.exec);     // they hold addresses of the old arena
+    exe.graphs.clear();
+    if (exe.arena) (void)hipFree(exe.arena);
+    exe.arena = nullptr;
+    exe.arena_size = 0;
+    if (hipMalloc(&exe.arena, bytes) != hipSuccess) {
+        (void)hipGetLastError();
+        exe.arena = nullptr;
+        throw BufferError("hipMalloc of the " + std::to_string(bytes) + "-byte arena failed");
+    }
+    exe.arena_size = bytes;
+}
+
+// Captures one walk over the program (every value, results included, at its arena address) into
+// a graph.  False when the capture or the instantiation fails; the stream is usable again then.
+static bool capture_graph(Executable& exe, const std::vector<DeviceTensor>& inputs, Executable::CapturedGraph& out) {
+    Client& c = *exe.client;
+    if (hipStreamBeginCapture(c.stream, hipStreamCaptureModeThreadLocal) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    Allocator al;
+    al.mode = Allocator::ARENA;
+    al.client = &c;
+    al.plan = &exe.plan;
+    al.base = static_cast<char*>(exe.arena);
+    al.escaping_in_arena = true;
+    std::vector<DeviceTensor> rets;
+    bool ok = true;
+    try { rets = run_ops(exe, inputs, al, false); } catch (const std::exception&) { ok = false; }
+    hipGraph_t g = nullptr;
+    const hipError_t e = hipStreamEndCapture(c.stream, &g);
+    hipGraphExec_t ex = nullptr;
+    if (ok && e == hipSuccess && g && hipGraphInstantiate(&ex, g, nullptr, nullptr, 0) != hipSuccess) ex = nullptr;
+    if (g) (void)hipGraphDestroy(g);
+    if (!ex) {
+        (void)hipGetLastError();
+        return false;
+    }
+    out.exec = ex;
+    out.inputs.clear();
+    for (auto& t : inputs) out.inputs.push_back(t.data());
+    out.returns.clear();
+    for (auto& r : rets) out.returns.emplace_back(r.data(), r.type);
+    return true;
+}
+
+std::vector<DeviceTensor> execute(Executable& exe, const std::vector<DeviceTensor>& inputs, double* encode_s,
+                                  double* gpu_s) {
+    Client& c = *exe.client;
+    if (c.device < 0) throw NoDevice("no HIP device: cannot execute");
+    const Function& fn = exe.fn;
+    if (inputs.size() != fn.arg_types.size())
+        throw InputMismatch("Expected " + std::to_string(fn.arg_types.size()) + " inputs, got " + std::to_string(inputs.size()));
+    for (size_t i = 0; i < inputs.size(); i++)
+        if (!(inputs[i].type == fn.arg_types[i]))
+            throw InputMismatch("Input " + std::to_string(i) + " has the wrong shape or element type");
+    const bool use_arena = exe.plan.valid && env_flag("METALHLO_ARENA", true);
+    // a replay costs one graph launch plus the copies of the results out of the arena: it pays
+    // from roughly twenty launches per execution on, so short programs stay eager by default
+    size_t launches = 0;
+    for (auto& op : fn.ops) launches += op.name != "constant" && op.name != "reshape";
+    const bool want_graph = use_arena && env_flag("METALHLO_HIP_GRAPH", exe.opt_level >= 3 && launches >= 16);
+    std::unique_lock<std::mutex> run_lock(exe.run_mu, std::defer_lock);
+    if (use_arena) run_lock.lock();          // the arena belongs to one execution at a time
+    const auto t0 = std::chrono::steady_clock::now();
+    std::vector<DeviceTensor> rets;
+    bool replayed = false;
+    if (use_arena) ensure_arena(exe, want_graph ? exe.plan.full_bytes : exe.plan.core_bytes);
+    // the first execution runs eagerly (kernels set their attributes, tuning tables load); from the
+    // second on the op list is one graph per set of input addresses
+    if (want_graph && !exe.graph_failed && exe.eager_runs > 0) {
+        Executable::CapturedGraph* hit = nullptr;
+        for (auto& g : exe.graphs) {
+            bool same = g.inputs.size() == inputs.size();
+            for (size_t i = 0; same && i < inputs.size(); i++) same = g.inputs[i] == inputs[i].data();
+            if (same) { hit = &g; break; }
+        }
+        if (!hit) {
+            Executable::CapturedGraph g;
+            if (capture_graph(exe, inputs, g)) {
+                if (exe.graphs.size() >= 8) {
+                    (void)hipStreamSynchronize(c.stream);
+                    (void)hipGraphExecDestroy(exe.graphs.front().exec);
+                    exe.graphs.erase(exe.graphs.begin());
+                }
+                exe.graphs.push_back(std::move(g));
+                hit = &exe.graphs.back();
+                exe.graph_captures++;
+            } else {
+                exe.graph_failed = true;     // this program stays on eager launches
+            }
+        }
+        if (hit) {
+            if (hipGraphLaunch(hit->exec, c.stream) != hipSuccess) {
+                const hipError_t e = hipGetLastError();
+                throw ExecError(std::string("graph launch failed: ") + hipGetErrorString(e));
+            }
+            exe.graph_replays++;
+            for (auto& r : hit->returns) {
+                DeviceTensor t;
+                t.type = r.second;
+                t.mem = std::make_shared<DeviceMem>();
+                t.mem->ptr = const_cast<void*>(r.first);      // not owned: copied out below
+                t.mem->bytes = r.second.bytes();
+                rets.push_back(t);
+            }
+            replayed = true;
+        }
+    }
+    if (!replayed) {
+        Allocator al;
+        al.client = &c;
+        if (use_arena) {
+            al.mode = Allocator::ARENA;
+            al.plan = &exe.plan;
+            al.base = static_cast<char*>(exe.arena);
+            al.escaping_in_arena = false;
+        }
+        rets = run_ops(exe, inputs, al, false);
+        exe.eager_runs++;
     }
     const auto t1 = std::chrono::steady_clock::now();
     if (hipStreamSynchronize(c.stream) != hipSuccess) {
@@ -574,15 +808,13 @@ std::vector<DeviceTensor> execute(Executable& exe, const std::vector<DeviceTenso
     if (encode_s) *encode_s = std::chrono::duration<double>(t1 - t0).count();
     if (gpu_s) *gpu_s = std::chrono::duration<double>(t2 - t0).count();
     std::vector<DeviceTensor> outs;
-    std::map<int, size_t> first_out;
-    for (size_t i = 0; i < fn.returns.size(); i++) {
-        const int r = fn.returns[i];
-        DeviceTensor o = first_out.count(r) ? outs[first_out[r]] : std::move(val[r]);
-        if (!first_out.count(r)) { val[r] = DeviceTensor(); first_out[r] = i; }
+    for (size_t i = 0; i < rets.size(); i++) {
+        DeviceTensor o = std::move(rets[i]);
+        rets[i] = DeviceTensor();
         if (!o.mem) throw ExecError("a returned value was never produced");
-        // an output must own its storage: inputs, constants, aliases and repeated
-        // results are copied out
-        const bool shared = o.mem.use_count() > 1;
+        // an output must own its storage: inputs, constants, aliases, repeated results and
+        // values that lie in the arena are copied out
+        const bool shared = o.mem.use_count() > 1 || !o.mem->pool;
         if (shared) {
             DeviceTensor cpy = c.allocate(o.type);
             if (mhip_copy(c.stream, o.data(), cpy.data(), (int64_t)o.type.bytes()) != MHIP_OK) throw ExecError(mhip_last_error());

@@ -6,6 +6,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
+#include <map>
 #include <memory>
 #include <mutex>
 #include <string>
@@ -32,11 +33,36 @@ private:
     std::multimap<size_t, void*> free_;
 };
 
+// Placement of every device allocation one execution makes (results of operations and the
+// temporaries inside them) in one arena, from the lifetimes a dry run of the program records
+// at compile time: slots whose lifetimes overlap never share bytes, offsets are multiples of
+// 256.  The role of the reference's StaticMemoryPlanner
+// (Sources/MetalHLOCore/Memory/StaticMemoryPlanner.swift:144-250).
+struct ArenaPlan {
+    struct Slot {
+        size_t bytes = 0;        // rounded up to 256
+        int begin = 0, end = 0;  // allocation / release time of the dry run
+        size_t offset = 0;
+        bool escapes = false;    // returned to the caller
+    };
+    std::vector<Slot> slots;     // in allocation order
+    size_t core_bytes = 0;       // arena for the slots that do not escape
+    size_t full_bytes = 0;       // ... plus the escaping ones behind them (graph replay needs fixed addresses)
+    size_t sum_bytes = 0;        // what one allocation per non-escaping slot takes
+    bool valid = false;
+    int clock = 0;
+};
+
 struct DeviceMem {
     DevicePool* pool = nullptr;
     void* ptr = nullptr;
     size_t bytes = 0;
-    ~DeviceMem() { if (pool && ptr) pool->release(ptr, bytes); }
+    ArenaPlan* recorder = nullptr;   // dry run: note the release time of slot `slot`
+    int slot = -1;
+    ~DeviceMem() {
+        if (recorder) recorder->slots[slot].end = recorder->clock++;
+        else if (pool && ptr) pool->release(ptr, bytes);
+    }
 };
 
 struct DeviceTensor {
@@ -62,14 +88,34 @@ struct Executable {
     int64_t exec_count = 0;
     double total_ms = 0, last_ms = 0;
     std::mutex mu;
+    // arena and captured graphs (one execution at a time per executable while they are in use)
+    ArenaPlan plan;
+    void* arena = nullptr;
+    size_t arena_size = 0;
+    std::mutex run_mu;
+    struct CapturedGraph {
+        std::vector<const void*> inputs;                     // device addresses the graph was captured with
+        hipGraphExec_t exec = nullptr;
+        std::vector<std::pair<const void*, TensorType>> returns;   // where each result lies after a replay
+    };
+    std::vector<CapturedGraph> graphs;
+    int64_t graph_captures = 0, graph_replays = 0, eager_runs = 0;
+    bool graph_failed = false;
+    ~Executable();
 };
 
-// Validates every op against what the kernels cover (throws UnsupportedOp) and
-// uploads constants when the client has a device.
+// Validates every op against what the kernels cover (throws UnsupportedOp), uploads constants
+// when the client has a device, and plans the arena.
 void compile(Executable& exe);
 
 // Runs the function.  `encode_s` = host time to issue all launches, `gpu_s` =
 // time from first launch to stream completion.
+// Memory: intermediates live in the executable's arena (METALHLO_ARENA=0: one pool block per
+// value instead); results are always fresh buffers the caller owns.
+// Launches: METALHLO_HIP_GRAPH=1 (default at optimisation level 3 for programs of sixteen or
+// more launches; =0 switches it off) captures the op list into a
+// HIP graph on the second execution and replays it while the input addresses stay the same
+// (up to eight address sets are kept); results are then copied out of the arena.
 std::vector<DeviceTensor> execute(Executable& exe, const std::vector<DeviceTensor>& inputs,
                                   double* encode_s, double* gpu_s);
 

@@ -555,7 +555,22 @@ struct Parser {
         if (c == std::string::npos) fail("op '" + name + "' has no type signature");
         op.attrs = rest.substr(0, c);
         parse_signature(rest.substr(c + 1), op);
-        for (auto& v : value_refs(op.attrs)) op.operands.push_back(value_id(v, false));
+        // generic form with a region, `"stablehlo.reduce"(%x, %init) ({ ^bb0(...): ... }) {attrs}`:
+        // the values named inside the region are the body's own, not operands
+        std::string outer = op.attrs;
+        const size_t r0 = outer.find("({");
+        if (r0 != std::string::npos) {
+            int depth = 0;
+            size_t r1 = r0 + 1;
+            for (; r1 < outer.size(); r1++) {
+                if (outer[r1] == '{') depth++;
+                else if (outer[r1] == '}' && --depth == 0) break;
+            }
+            const size_t close = outer.find(')', r1);
+            if (depth != 0 || close == std::string::npos) fail("unterminated region of '" + name + "'");
+            outer = outer.substr(0, r0) + outer.substr(close + 1);
+        }
+        for (auto& v : value_refs(outer)) op.operands.push_back(value_id(v, false));
         decode_attrs(op);
         if (result.empty()) fail("op '" + name + "' has no result");
         op.result = value_id(result, true);

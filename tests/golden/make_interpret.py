@@ -20,21 +20,31 @@ REL = "Tests/MetalHLOTests/Conformance/StableHLO/interpret"
 
 
 def statements(body_lines):
-    """Joins continuation lines: a statement starts with `%x =`, `check.` or a return."""
-    out, cur = [], None
+    """Joins continuation lines: a statement runs until its (), [] and {} are balanced again
+    (so a region, as in the generic form of reduce, stays inside its operation)."""
+    out, cur, depth = [], None, 0
     for no, ln in body_lines:
         s = ln.strip()
         if not s or s.startswith("//"):
             continue
-        if re.match(r"(%[\w#:]+\s*=|check\.|func\.return|return\b)", s):
-            if cur:
-                out.append(cur)
+        if cur is None:
             cur = [no, s]
-        elif cur:
+        else:
             cur[1] += " " + s
+        depth += sum(s.count(c) for c in "([{") - sum(s.count(c) for c in ")]}")
+        if depth <= 0 and not s.endswith(","):
+            out.append(cur)
+            cur, depth = None, 0
     if cur:
         out.append(cur)
-    return out
+    # a line that does not start a statement continues the previous one (wrapped signatures)
+    merged = []
+    for no, s in out:
+        if merged and not re.match(r"(%[\w#:]+\s*=|check\.|func\.return|return\b)", s):
+            merged[-1][1] += " " + s
+        else:
+            merged.append([no, s])
+    return merged
 
 
 def element_types(text):

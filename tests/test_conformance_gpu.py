@@ -92,7 +92,7 @@ def test_interpret_case(case, sess):
 
 def test_most_cases_are_executed(sess):
     """The skip above is for forms outside the operator subset, not a way to hide failures:
-    all 134 cases must compile."""
+    all 135 cases must compile."""
     from metalhlo_amd import capi
     ok = 0
     for case in CASES:
@@ -104,7 +104,7 @@ def test_most_cases_are_executed(sess):
             ok += 1
         except capi.MHLOError:
             pass
-    assert len(CASES) == 134 and ok == 134, (len(CASES), ok)
+    assert len(CASES) == 135 and ok == 135, (len(CASES), ok)
 
 
 def spec_gather(x, idx, offset_dims, collapsed, start_index_map, ivd, slice_sizes, op_batching=(), idx_batching=()):
