@@ -1,14 +1,19 @@
 // PJRT plugin (C API 0.90) over the C++ host: GetPjrtApi() returns the function table
 // declared in include/pjrt_abi.h.  Behaviour follows the reference plugin
 // (Sources/PJRTMetalHLO): platform "metalhlo" / version "0.1.0", one device (id 0), one
-// memory space "device" (PJRTTopology.swift:106-107, PJRTClient.swift:42-50); host buffers
-// are copied eagerly and the returned events are already complete (PJRTBuffer.swift:98-148);
+// memory space "device" (PJRTTopology.swift:106-107, PJRTClient.swift:42-50);
 // Compile takes StableHLO text (MLIR bytecode is converted by a jaxlib subprocess when one
 // is available, as PJRTExecutable.swift:23-239 does, else refused); Execute is synchronous
 // and single-device (PJRTExecutable.swift:2020-2098); a serialized executable is
 // `u32 1 | u64 length | MLIR text` and loading it recompiles (:342-359, :2148-2208).
-// Differences: H2D / D2H are explicit hipMemcpy on the client's stream instead of unified
-// memory; device attributes describe the GPU (architecture, CU count) instead of the ANE;
+// Differences: buffers are explicit device allocations and H2D / D2H are asynchronous
+// (the reference copies eagerly into unified memory and returns complete events,
+// PJRTBuffer.swift:98-148): a host buffer is staged into pinned memory during the call (so
+// done_with_host_buffer is complete at return) and DMA'd with hipMemcpyAsync on the client's
+// stream; a download DMAs into pinned memory and a completion thread, woken by the HIP event
+// recorded behind the copy, moves the bytes to the caller's destination and completes the
+// PJRT event (Await blocks, OnReady callbacks run on that thread).  Transfers above 256 MiB
+// take the synchronous path.  Device attributes describe the GPU (architecture, CU count) instead of the ANE;
 // the fingerprint is a stable FNV-1a hash of the program text.
 #include <stdio.h>
 #include <stdlib.h>
@@ -16,10 +21,15 @@
 #include <unistd.h>
 
 #include <atomic>
+#include <chrono>
+#include <condition_variable>
+#include <deque>
 #include <functional>
+#include <map>
 #include <memory>
 #include <mutex>
 #include <string>
+#include <thread>
 #include <vector>
 
 #include "../../../include/mhip.h"
@@ -34,11 +44,107 @@ struct PJRT_Error {
     std::string message;
 };
 
-struct PJRT_Event {
+// Completion state, shared between the PJRT_Event handles given out for it and the transfer
+// that completes it (a handle may be destroyed first).
+struct EventState {
     std::mutex mu;
-    bool ready = true;                         // everything here completes before it returns
+    std::condition_variable cv;
+    bool ready = true;
     PJRT_Error_Code code = PJRT_Error_Code_OK;
     std::string message;
+    std::vector<std::pair<PJRT_Event_OnReadyCallback, void*>> waiting;
+};
+
+struct PJRT_Event {
+    std::shared_ptr<EventState> state = std::make_shared<EventState>();
+};
+
+// Pinned staging memory and the thread that finishes transfers.  A transfer records a HIP event
+// behind its hipMemcpyAsync and queues {event, finish}; the thread waits for the events in queue
+// order (= stream order) and runs `finish` (copy out of the staging block, release it, complete
+// the PJRT event).
+struct TransferEngine {
+    static constexpr size_t kStageMax = (size_t)256 << 20;
+    struct Task { hipEvent_t done; std::function<void()> finish; };
+    std::mutex mu;
+    std::condition_variable cv;
+    std::deque<Task> queue;
+    std::multimap<size_t, void*> free_blocks;      // pinned, by capacity
+    std::vector<hipEvent_t> free_events;
+    std::thread worker;
+    bool running = false, stop = false;
+
+    static size_t capacity(size_t bytes) { size_t b = 4096; while (b < bytes) b <<= 1; return b; }
+    void* stage(size_t bytes) {
+        const size_t cap = capacity(bytes);
+        {
+            std::lock_guard<std::mutex> g(mu);
+            auto it = free_blocks.find(cap);
+            if (it != free_blocks.end()) { void* p = it->second; free_blocks.erase(it); return p; }
+        }
+        void* p = nullptr;
+        if (hipHostMalloc(&p, cap, hipHostMallocDefault) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+        return p;
+    }
+    void unstage(void* p, size_t bytes) {
+        std::lock_guard<std::mutex> g(mu);
+        free_blocks.emplace(capacity(bytes), p);
+    }
+    void start() {
+        running = true;
+        worker = std::thread([this] {
+            (void)hipSetDevice(0);
+            for (;;) {
+                Task t;
+                {
+                    std::unique_lock<std::mutex> g(mu);
+                    cv.wait(g, [this] { return stop || !queue.empty(); });
+                    if (queue.empty()) return;          // stop requested and nothing left
+                    t = std::move(queue.front());
+                    queue.pop_front();
+                }
+                (void)hipEventSynchronize(t.done);
+                t.finish();
+                std::lock_guard<std::mutex> g(mu);
+                free_events.push_back(t.done);
+            }
+        });
+    }
+    // `finish` runs on the completion thread once everything queued on `stream` so far is done.
+    // False (nothing queued, `finish` not run) when no event can be recorded.
+    bool after(hipStream_t stream, std::function<void()> finish) {
+        if (!running) return false;
+        hipEvent_t e = nullptr;
+        {
+            std::lock_guard<std::mutex> g(mu);
+            if (!free_events.empty()) { e = free_events.back(); free_events.pop_back(); }
+        }
+        if (!e && hipEventCreateWithFlags(&e, hipEventDisableTiming) != hipSuccess) { (void)hipGetLastError(); return false; }
+        if (hipEventRecord(e, stream) != hipSuccess) {
+            (void)hipGetLastError();
+            std::lock_guard<std::mutex> g(mu);
+            free_events.push_back(e);
+            return false;
+        }
+        {
+            std::lock_guard<std::mutex> g(mu);
+            queue.push_back(Task{e, std::move(finish)});
+        }
+        cv.notify_one();
+        return true;
+    }
+    void shutdown() {
+        if (running) {
+            { std::lock_guard<std::mutex> g(mu); stop = true; }
+            cv.notify_all();
+            worker.join();                               // drains the queue first
+            running = false;
+        }
+        for (auto& kv : free_blocks) (void)hipHostFree(kv.second);
+        free_blocks.clear();
+        for (auto e : free_events) (void)hipEventDestroy(e);
+        free_events.clear();
+    }
 };
 
 struct PJRT_DeviceDescription {
@@ -74,11 +180,13 @@ struct PJRT_Client {
     std::vector<PJRT_Device*> devices;
     std::vector<PJRT_Memory*> memories;
     PJRT_TopologyDescription topology;
+    TransferEngine transfers;
 };
 
 struct PJRT_Buffer {
     PJRT_Client* client = nullptr;
     DeviceTensor tensor;
+    std::shared_ptr<EventState> ready;         // the upload that fills it, while in flight (null: ready)
     std::vector<int64_t> dims;
     bool deleted = false;
     std::atomic<int> external_refs{0};
@@ -319,30 +427,69 @@ PJRT_Error* Event_Destroy(PJRT_Event_Destroy_Args* a) { REQUIRE_ARGS(a, "PJRT_Ev
 PJRT_Error* Event_IsReady(PJRT_Event_IsReady_Args* a) {
     REQUIRE_ARGS(a, "PJRT_Event_IsReady");
     REQUIRE(a->event, "event");
-    std::lock_guard<std::mutex> lock(a->event->mu);
-    a->is_ready = a->event->ready;
+    std::lock_guard<std::mutex> lock(a->event->state->mu);
+    a->is_ready = a->event->state->ready;
     return nullptr;
 }
-PJRT_Error* event_status(PJRT_Event* e) {
-    std::lock_guard<std::mutex> lock(e->mu);
-    return e->code == PJRT_Error_Code_OK ? nullptr : make_error(e->code, e->message);
+PJRT_Error* status_of(EventState& st) {      // st.mu held by the caller
+    return st.code == PJRT_Error_Code_OK ? nullptr : make_error(st.code, st.message);
 }
 PJRT_Error* Event_Error(PJRT_Event_Error_Args* a) {
     REQUIRE_ARGS(a, "PJRT_Event_Error");
     REQUIRE(a->event, "event");
-    return event_status(a->event);
+    std::lock_guard<std::mutex> lock(a->event->state->mu);
+    if (!a->event->state->ready) return make_error(PJRT_Error_Code_FAILED_PRECONDITION, "the event is not ready yet");
+    return status_of(*a->event->state);
 }
 PJRT_Error* Event_Await(PJRT_Event_Await_Args* a) {
     REQUIRE_ARGS(a, "PJRT_Event_Await");
     REQUIRE(a->event, "event");
-    return event_status(a->event);             // already complete: nothing to wait for
+    EventState& st = *a->event->state;
+    std::unique_lock<std::mutex> lock(st.mu);
+    if (!st.cv.wait_for(lock, std::chrono::seconds(300), [&] { return st.ready; }))
+        return make_error(PJRT_Error_Code_DEADLINE_EXCEEDED, "the transfer did not complete within 300 s");
+    return status_of(st);
 }
 PJRT_Error* Event_OnReady(PJRT_Event_OnReady_Args* a) {
     REQUIRE_ARGS(a, "PJRT_Event_OnReady");
     REQUIRE(a->event, "event");
     REQUIRE(a->callback, "callback");
-    a->callback(event_status(a->event), a->user_arg);   // inline on the calling thread; the callback owns the error
+    EventState& st = *a->event->state;
+    PJRT_Error* status = nullptr;
+    {
+        std::lock_guard<std::mutex> lock(st.mu);
+        if (!st.ready) {                        // runs on the completion thread when the transfer ends
+            st.waiting.emplace_back(a->callback, a->user_arg);
+            return nullptr;
+        }
+        status = status_of(st);
+    }
+    a->callback(status, a->user_arg);           // already complete: inline on the calling thread; the callback owns the error
     return nullptr;
+}
+
+// Marks a pending event complete, wakes the waiters and runs the callbacks registered so far.
+void complete(const std::shared_ptr<EventState>& st, PJRT_Error_Code code = PJRT_Error_Code_OK, const std::string& message = "") {
+    std::vector<std::pair<PJRT_Event_OnReadyCallback, void*>> run;
+    {
+        std::lock_guard<std::mutex> lock(st->mu);
+        st->ready = true;
+        st->code = code;
+        st->message = message;
+        run.swap(st->waiting);
+    }
+    st->cv.notify_all();
+    for (auto& cb : run) cb.first(code == PJRT_Error_Code_OK ? nullptr : make_error(code, message), cb.second);
+}
+std::shared_ptr<EventState> pending_state() {
+    auto st = std::make_shared<EventState>();
+    st->ready = false;
+    return st;
+}
+PJRT_Event* event_for(const std::shared_ptr<EventState>& st) {
+    PJRT_Event* e = new PJRT_Event();
+    if (st) e->state = st;
+    return e;
 }
 
 // ---- client ------------------------------------------------------------------------------
@@ -364,6 +511,8 @@ PJRT_Error* Client_Create(PJRT_Client_Create_Args* a) {
         int cus = 0;
         mhip_device_info(0, &cus, nullptr, arch, sizeof(arch));
         c->host.device_name += std::string(" (") + arch + ", " + std::to_string(cus) + " CUs)";
+        const char* sync = getenv("METALHLO_PJRT_SYNC_TRANSFERS");
+        if (!(sync && sync[0] == '1')) c->transfers.start();
     } else {
         c->host.device_name = "none (host-only client)";
     }
@@ -379,7 +528,9 @@ PJRT_Error* Client_Create(PJRT_Client_Create_Args* a) {
 PJRT_Error* Client_Destroy(PJRT_Client_Destroy_Args* a) {
     REQUIRE_ARGS(a, "PJRT_Client_Destroy");
     if (a->client) {
-        if (a->client->host.stream) { (void)hipStreamSynchronize(a->client->host.stream); (void)hipStreamDestroy(a->client->host.stream); }
+        if (a->client->host.stream) (void)hipStreamSynchronize(a->client->host.stream);
+        a->client->transfers.shutdown();          // finishes what is still queued, then frees the staging memory
+        if (a->client->host.stream) (void)hipStreamDestroy(a->client->host.stream);
         delete a->client;
     }
     return nullptr;
@@ -502,8 +653,26 @@ PJRT_Error* Client_BufferFromHostBuffer(PJRT_Client_BufferFromHostBuffer_Args* a
     PJRT_Buffer* b = nullptr;
     PJRT_Error* err = guarded([&] {
         DeviceTensor d = c->host.allocate(t);
-        if (t.bytes()) {
-            if (hipMemcpyAsync(d.data(), a->data, t.bytes(), hipMemcpyHostToDevice, c->host.stream) != hipSuccess ||
+        std::shared_ptr<EventState> ready;
+        const size_t n = t.bytes();
+        void* staged = n && n <= TransferEngine::kStageMax && c->transfers.running ? c->transfers.stage(n) : nullptr;
+        if (staged) {
+            // the caller's memory is read here and never again; the DMA runs behind this call
+            memcpy(staged, a->data, n);
+            if (hipMemcpyAsync(d.data(), staged, n, hipMemcpyHostToDevice, c->host.stream) != hipSuccess) {
+                (void)hipGetLastError();
+                c->transfers.unstage(staged, n);
+                throw BufferError("host to device copy failed");
+            }
+            ready = pending_state();
+            TransferEngine* eng = &c->transfers;
+            auto finish = [eng, staged, n, ready] { eng->unstage(staged, n); complete(ready); };
+            if (!c->transfers.after(c->host.stream, finish)) {
+                (void)hipStreamSynchronize(c->host.stream);
+                finish();
+            }
+        } else if (n) {
+            if (hipMemcpyAsync(d.data(), a->data, n, hipMemcpyHostToDevice, c->host.stream) != hipSuccess ||
                 hipStreamSynchronize(c->host.stream) != hipSuccess) {
                 (void)hipGetLastError();
                 throw BufferError("host to device copy failed");
@@ -513,10 +682,11 @@ PJRT_Error* Client_BufferFromHostBuffer(PJRT_Client_BufferFromHostBuffer_Args* a
         b->client = c;
         b->tensor = d;
         b->dims = t.shape;
+        b->ready = ready;
     });
     if (err) return err;
     a->buffer = b;
-    a->done_with_host_buffer = complete_event();          // the copy has finished: the host buffer is free
+    a->done_with_host_buffer = complete_event();          // staged or copied: the host buffer is free
     return nullptr;
 }
 
@@ -822,14 +992,41 @@ PJRT_Error* Buffer_Delete(PJRT_Buffer_Delete_Args* a) {
     return nullptr;
 }
 PJRT_Error* Buffer_IsDeleted(PJRT_Buffer_IsDeleted_Args* a) { BUF(a, "PJRT_Buffer_IsDeleted"); a->is_deleted = b.deleted; return nullptr; }
-PJRT_Error* copy_to_host(PJRT_Buffer& b, void* dst, size_t offset, size_t bytes) {
+// Device to host; *event completes when `dst` holds the bytes.
+PJRT_Error* copy_to_host(PJRT_Buffer& b, void* dst, size_t offset, size_t bytes, PJRT_Event** event) {
     if (b.deleted) return make_error(PJRT_Error_Code_FAILED_PRECONDITION, "the buffer was deleted");
-    if (bytes == 0) return nullptr;
-    if (hipMemcpyAsync(dst, static_cast<const char*>(b.tensor.data()) + offset, bytes, hipMemcpyDeviceToHost, b.client->host.stream) != hipSuccess ||
-        hipStreamSynchronize(b.client->host.stream) != hipSuccess) {
+    *event = nullptr;
+    if (bytes == 0) { *event = complete_event(); return nullptr; }
+    PJRT_Client* c = b.client;
+    const char* src = static_cast<const char*>(b.tensor.data()) + offset;
+    void* staged = bytes <= TransferEngine::kStageMax && c->transfers.running ? c->transfers.stage(bytes) : nullptr;
+    if (staged) {
+        if (hipMemcpyAsync(staged, src, bytes, hipMemcpyDeviceToHost, c->host.stream) != hipSuccess) {
+            (void)hipGetLastError();
+            c->transfers.unstage(staged, bytes);
+            return make_error(PJRT_Error_Code_INTERNAL, "device to host copy failed");
+        }
+        auto st = pending_state();
+        TransferEngine* eng = &c->transfers;
+        const DeviceTensor keep = b.tensor;      // the device memory outlives the buffer handle until the copy ends
+        auto finish = [eng, staged, dst, bytes, st, keep] {
+            memcpy(dst, staged, bytes);
+            eng->unstage(staged, bytes);
+            complete(st);
+        };
+        if (!c->transfers.after(c->host.stream, finish)) {
+            (void)hipStreamSynchronize(c->host.stream);
+            finish();
+        }
+        *event = event_for(st);
+        return nullptr;
+    }
+    if (hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, c->host.stream) != hipSuccess ||
+        hipStreamSynchronize(c->host.stream) != hipSuccess) {
         (void)hipGetLastError();
         return make_error(PJRT_Error_Code_INTERNAL, "device to host copy failed");
     }
+    *event = complete_event();
     return nullptr;
 }
 PJRT_Error* Buffer_ToHostBuffer(PJRT_Buffer_ToHostBuffer_Args* a) {
@@ -840,9 +1037,7 @@ PJRT_Error* Buffer_ToHostBuffer(PJRT_Buffer_ToHostBuffer_Args* a) {
     if (!a->dst) { a->dst_size = need; return nullptr; }    // size query
     if (a->dst_size < need)
         return invalid("dst_size (" + std::to_string(a->dst_size) + ") is smaller than the buffer (" + std::to_string(need) + " bytes)");
-    if (PJRT_Error* err = copy_to_host(b, a->dst, 0, need)) return err;
-    a->event = complete_event();
-    return nullptr;
+    return copy_to_host(b, a->dst, 0, need, &a->event);
 }
 PJRT_Error* Buffer_CopyRawToHost(PJRT_Buffer_CopyRawToHost_Args* a) {
     BUF(a, "PJRT_Buffer_CopyRawToHost");
@@ -850,9 +1045,7 @@ PJRT_Error* Buffer_CopyRawToHost(PJRT_Buffer_CopyRawToHost_Args* a) {
     const int64_t total = (int64_t)b.tensor.type.bytes();
     if (a->offset < 0 || a->transfer_size < 0 || a->offset + a->transfer_size > total)
         return make_error(PJRT_Error_Code_OUT_OF_RANGE, "offset + transfer_size exceeds the buffer (" + std::to_string(total) + " bytes)");
-    if (PJRT_Error* err = copy_to_host(b, a->dst, (size_t)a->offset, (size_t)a->transfer_size)) return err;
-    a->event = complete_event();
-    return nullptr;
+    return copy_to_host(b, a->dst, (size_t)a->offset, (size_t)a->transfer_size, &a->event);
 }
 PJRT_Error* clone_buffer(PJRT_Buffer& b, PJRT_Buffer** out) {
     if (b.deleted) return make_error(PJRT_Error_Code_FAILED_PRECONDITION, "the buffer was deleted");
@@ -885,7 +1078,11 @@ PJRT_Error* Buffer_CopyToMemory(PJRT_Buffer_CopyToMemory_Args* a) {
     return clone_buffer(b, &a->dst_buffer);
 }
 PJRT_Error* Buffer_IsOnCpu(PJRT_Buffer_IsOnCpu_Args* a) { BUF(a, "PJRT_Buffer_IsOnCpu"); (void)b; a->is_on_cpu = false; return nullptr; }
-PJRT_Error* Buffer_ReadyEvent(PJRT_Buffer_ReadyEvent_Args* a) { BUF(a, "PJRT_Buffer_ReadyEvent"); (void)b; a->event = complete_event(); return nullptr; }
+PJRT_Error* Buffer_ReadyEvent(PJRT_Buffer_ReadyEvent_Args* a) {
+    BUF(a, "PJRT_Buffer_ReadyEvent");
+    a->event = event_for(b.ready);              // pending while the upload that fills the buffer is in flight
+    return nullptr;
+}
 PJRT_Error* Buffer_UnsafePointer(PJRT_Buffer_UnsafePointer_Args* a) { REQUIRE_ARGS(a, "PJRT_Buffer_UnsafePointer"); return unimplemented("PJRT_Buffer_UnsafePointer"); }
 PJRT_Error* Buffer_IncreaseExternalReferenceCount(PJRT_Buffer_IncreaseExternalReferenceCount_Args* a) {
     BUF(a, "PJRT_Buffer_IncreaseExternalReferenceCount");

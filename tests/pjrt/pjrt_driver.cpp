@@ -3,13 +3,17 @@
 // Prints one "ok <case>" line per case; the first failed check prints "FAIL ..." and exits 1.
 // The cases restate Tests/PJRTMetalHLOTests/PJRTPluginTests.swift (table version and slots
 // :160-180, error lifecycle :182-207, events :209-235, platform and device :237-261, host
-// round trip :263-285, compile + execute add :287-318, serialize / deserialize :406-467).
+// round trip :263-285, compile + execute add :287-318, serialize / deserialize :406-467);
+// case_async_transfers has no counterpart there (the reference's transfers complete inside
+// the call): it covers the asynchronous uploads and downloads of this plugin.
 #include <dlfcn.h>
 #include <math.h>
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
+#include <unistd.h>
 
+#include <atomic>
 #include <string>
 #include <vector>
 
@@ -389,6 +393,17 @@ static void download(PJRT_Buffer* b, void* dst, size_t bytes) {
     OK(api->PJRT_Event_Await(&aw));
     destroy_event(t.event);
 }
+static void await_and_destroy(PJRT_Event* e) {
+    CHECK(e != nullptr);
+    ARGS(PJRT_Event_Await_Args, aw);
+    aw.event = e;
+    OK(api->PJRT_Event_Await(&aw));
+    ARGS(PJRT_Event_IsReady_Args, r);
+    r.event = e;
+    OK(api->PJRT_Event_IsReady(&r));
+    CHECK(r.is_ready);
+    destroy_event(e);
+}
 static void case_round_trip(PJRT_Client* c) {
     const float x[6] = {1.5f, -2.f, 3.25f, 4.f, 5.f, -6.75f};
     PJRT_Buffer* b = upload(c, x, PJRT_Buffer_Type_F32, {2, 3});
@@ -424,7 +439,7 @@ static void case_round_trip(PJRT_Client* c) {
     raw.offset = 8;
     raw.transfer_size = 8;
     OK(api->PJRT_Buffer_CopyRawToHost(&raw));
-    destroy_event(raw.event);
+    await_and_destroy(raw.event);                          // the bytes are in `part` once the event completes
     CHECK(part[0] == 3.25f && part[1] == 4.f);
     raw.offset = 20;
     CHECK(code_of(api->PJRT_Buffer_CopyRawToHost(&raw)) == PJRT_Error_Code_OUT_OF_RANGE);
@@ -495,6 +510,108 @@ static void case_round_trip(PJRT_Client* c) {
     CHECK(ms.bytes_limit_is_set && ms.bytes_limit > (1ll << 30) && ms.bytes_in_use > 0 && ms.device == ds.devices[0]);
     printf("ok round_trip\n");
 }
+// Transfers in flight: uploads return once the host bytes are staged (the source may change
+// right away), downloads return a pending event; data is right after Await, also when the
+// source buffer handle is destroyed first; OnReady callbacks registered on pending events run
+// exactly once; an execution queued behind uploads that nobody awaited sees their data.
+static std::atomic<int> async_callbacks{0};
+static void on_async_ready(PJRT_Error* e, void* user) {
+    CHECK(e == nullptr && user == &async_callbacks);
+    async_callbacks++;
+}
+static void case_async_transfers(PJRT_Client* c) {
+    const int kBuffers = 48;
+    const size_t kElems = 256 * 1024;                      // 1 MiB of f32 each
+    std::vector<std::vector<float>> src(kBuffers, std::vector<float>(kElems)), dst(kBuffers, std::vector<float>(kElems, -1.f));
+    std::vector<PJRT_Buffer*> bufs;
+    for (int i = 0; i < kBuffers; i++) {
+        for (size_t j = 0; j < kElems; j++) src[i][j] = (float)(i * 1000003 % 977) + (float)(j % 4093) * 0.25f;
+        bufs.push_back(upload(c, src[i].data(), PJRT_Buffer_Type_F32, {(int64_t)kElems}));
+        src[i][0] = -12345.f;                               // done_with_host_buffer was complete: the upload no longer reads this
+        src[i][kElems - 1] = -54321.f;
+    }
+    std::vector<PJRT_Event*> events;
+    int pending = 0;
+    for (int i = 0; i < kBuffers; i++) {
+        ARGS(PJRT_Buffer_ToHostBuffer_Args, t);
+        t.src = bufs[i];
+        t.dst = dst[i].data();
+        t.dst_size = kElems * sizeof(float);
+        OK(api->PJRT_Buffer_ToHostBuffer(&t));
+        CHECK(t.event != nullptr);
+        ARGS(PJRT_Event_IsReady_Args, r);
+        r.event = t.event;
+        OK(api->PJRT_Event_IsReady(&r));
+        pending += !r.is_ready;
+        ARGS(PJRT_Event_OnReady_Args, cb);
+        cb.event = t.event;
+        cb.callback = on_async_ready;
+        cb.user_arg = &async_callbacks;
+        OK(api->PJRT_Event_OnReady(&cb));
+        events.push_back(t.event);
+        if (i % 2 == 0) { destroy_buffer(bufs[i]); bufs[i] = nullptr; }   // the copy in flight keeps the memory
+    }
+    for (auto e : events) await_and_destroy(e);
+    for (int spin = 0; spin < 5000 && async_callbacks.load() < kBuffers; spin++) usleep(1000);
+    CHECK(async_callbacks.load() == kBuffers);
+    for (int i = 0; i < kBuffers; i++) {
+        CHECK(dst[i][0] == (float)(i * 1000003 % 977) && dst[i][kElems - 1] == (float)(i * 1000003 % 977) + (float)((kElems - 1) % 4093) * 0.25f);
+        for (size_t j = 1; j + 1 < kElems; j++) CHECK(dst[i][j] == src[i][j]);
+    }
+    printf("  %d of %d downloads were still pending when ToHostBuffer returned\n", pending, kBuffers);
+    for (auto b : bufs) if (b) destroy_buffer(b);
+    // ReadyEvent of a large upload: awaitable, ready afterwards; raw slices of it
+    const size_t big = 16u << 20;                           // 64 MiB
+    std::vector<float> host(big);
+    for (size_t j = 0; j < big; j++) host[j] = (float)(j % 65521);
+    PJRT_Buffer* bb = upload(c, host.data(), PJRT_Buffer_Type_F32, {(int64_t)big});
+    ARGS(PJRT_Buffer_ReadyEvent_Args, re);
+    re.buffer = bb;
+    OK(api->PJRT_Buffer_ReadyEvent(&re));
+    await_and_destroy(re.event);
+    float tailv[4] = {0};
+    ARGS(PJRT_Buffer_CopyRawToHost_Args, raw);
+    raw.buffer = bb;
+    raw.dst = tailv;
+    raw.offset = (int64_t)((big - 4) * sizeof(float));
+    raw.transfer_size = sizeof(tailv);
+    OK(api->PJRT_Buffer_CopyRawToHost(&raw));
+    await_and_destroy(raw.event);
+    for (int j = 0; j < 4; j++) CHECK(tailv[j] == (float)((big - 4 + j) % 65521));
+    destroy_buffer(bb);
+    // an execution right behind two uploads nobody waited for
+    const char* add_big =
+        "module { func.func @main(%a: tensor<1048576xf32>, %b: tensor<1048576xf32>) -> (tensor<1048576xf32>) {\n"
+        "  %0 = stablehlo.add %a, %b : tensor<1048576xf32>\n  return %0 : tensor<1048576xf32>\n} }\n";
+    PJRT_LoadedExecutable* le = nullptr;
+    OK(compile(c, add_big, "mlir", &le));
+    std::vector<float> x(1048576), y(1048576), z(1048576, 0.f);
+    for (size_t j = 0; j < x.size(); j++) { x[j] = (float)(j % 1021); y[j] = (float)(j % 509) * 0.5f; }
+    PJRT_Buffer* in[2] = {upload(c, x.data(), PJRT_Buffer_Type_F32, {1048576}), upload(c, y.data(), PJRT_Buffer_Type_F32, {1048576})};
+    PJRT_Buffer* const* lists[1] = {in};
+    PJRT_Buffer* out[1] = {nullptr};
+    PJRT_Buffer** out_lists[1] = {out};
+    PJRT_Event* done[1] = {nullptr};
+    ARGS(PJRT_ExecuteOptions, opts);
+    ARGS(PJRT_LoadedExecutable_Execute_Args, ex);
+    ex.executable = le;
+    ex.options = &opts;
+    ex.argument_lists = lists;
+    ex.num_devices = 1;
+    ex.num_args = 2;
+    ex.output_lists = out_lists;
+    ex.device_complete_events = done;
+    OK(api->PJRT_LoadedExecutable_Execute(&ex));
+    await_and_destroy(done[0]);
+    download(out[0], z.data(), z.size() * sizeof(float));
+    for (size_t j = 0; j < z.size(); j++) CHECK(z[j] == x[j] + y[j]);
+    destroy_buffer(out[0]);
+    destroy_buffer(in[0]);
+    destroy_buffer(in[1]);
+    destroy_loaded(le);
+    printf("ok async_transfers\n");
+}
+
 static std::vector<float> run1(PJRT_LoadedExecutable* le, std::vector<PJRT_Buffer*> in, size_t n_out) {
     PJRT_Buffer* const* lists[1] = {in.data()};
     PJRT_Buffer* outs[1] = {nullptr};
@@ -598,6 +715,7 @@ int main(int argc, char** argv) {
     if (gpu) {
         case_round_trip(c);
         case_execute(c);
+        case_async_transfers(c);
     } else {
         case_no_device_buffers(c);
     }

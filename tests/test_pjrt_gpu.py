@@ -1,5 +1,7 @@
 """PJRT plugin on the GPU: host <-> device round trips, events, compile + execute, serialize ->
-deserialize -> execute, a fused kernel through the plugin (tests/pjrt/pjrt_driver.cpp, gpu mode)."""
+deserialize -> execute, a fused kernel through the plugin, asynchronous transfers in flight
+(tests/pjrt/pjrt_driver.cpp, gpu mode); once more with METALHLO_PJRT_SYNC_TRANSFERS=1, where
+every transfer completes inside its call."""
 import os
 import subprocess
 
@@ -12,9 +14,12 @@ DRIVER = os.path.join(ROOT, "tests", "pjrt", "pjrt_driver")
 pytestmark = pytest.mark.gpu
 
 
-def test_driver_gpu_cases():
+@pytest.mark.parametrize("sync", ["0", "1"], ids=["async", "sync"])
+def test_driver_gpu_cases(sync):
     assert os.path.exists(PLUGIN) and os.path.exists(DRIVER), "plugin / driver not built"
-    r = subprocess.run([DRIVER, PLUGIN, "gpu"], capture_output=True, text=True, timeout=120)
+    env = dict(os.environ, METALHLO_PJRT_SYNC_TRANSFERS=sync)
+    r = subprocess.run([DRIVER, PLUGIN, "gpu"], capture_output=True, text=True, timeout=120, env=env)
     assert r.returncode == 0, r.stdout[-3000:] + r.stderr[-3000:]
-    for case in ("table", "errors", "platform", "compile", "round_trip", "execute", "all"):
+    for case in ("table", "errors", "platform", "compile", "round_trip", "execute", "async_transfers", "all"):
         assert f"ok {case}\n" in r.stdout, r.stdout
+    print(r.stdout)
