@@ -118,6 +118,54 @@ struct Rewriter {
         return true;
     }
 
+    // Statistics (one value per row) are often carried in keepdims style: reshaped or broadcast
+    // to a shape with extra unit dims, computed on there, and spread over the row at the end.
+    // relabel_src skips the ops that only rename the dims of `v` (reshape; broadcast_in_dim that
+    // keeps the element count and the order); both keep the linear order of the elements.
+    int relabel_src(int v, std::set<size_t>& nodes) const {
+        for (int hop = 0; hop < 4; hop++) {
+            const Op* o = op_of(v);
+            if (!o || o->operands.empty()) return v;
+            const bool same_count = type.at(o->operands[0]).numel() == o->out.numel();
+            bool rename = o->name == "reshape" && same_count;
+            if (o->name == "broadcast_in_dim" && same_count) {
+                rename = true;
+                for (size_t i = 1; i < o->dims.size(); i++) rename &= o->dims[i] > o->dims[i - 1];
+            }
+            if (!rename) return v;
+            nodes.insert(index_of(o));
+            v = o->operands[0];
+        }
+        return v;
+    }
+    // v = a per-row statistic spread over exactly one axis of the result shape: broadcast_in_dim
+    // with increasing dims whose operand has, for every result dim but `axis`, either that dim
+    // in full or nothing where the dim is 1.  Returns the statistic (renames skipped), -1 if not.
+    int spread_src(int v, int64_t& axis, std::set<size_t>& nodes) const {
+        const Op* b = op_named(v, "broadcast_in_dim");
+        if (!b) return -1;
+        const auto& S = b->out.shape;
+        const auto& T = type.at(b->operands[0]).shape;
+        if (b->dims.size() != T.size()) return -1;
+        std::vector<int64_t> got(S.size(), 1);
+        for (size_t i = 0; i < T.size(); i++) {
+            const int64_t d = b->dims[i];
+            if (d < 0 || d >= (int64_t)S.size() || (i > 0 && d <= b->dims[i - 1])) return -1;
+            if (T[i] != S[d] && T[i] != 1) return -1;
+            got[d] = T[i];
+        }
+        int64_t a = -1;
+        for (size_t d = 0; d < S.size(); d++)
+            if (got[d] != S[d]) {
+                if (a >= 0) return -1;
+                a = (int64_t)d;
+            }
+        if (a < 0) return -1;
+        axis = a;
+        nodes.insert(index_of(b));
+        return relabel_src(b->operands[0], nodes);
+    }
+
     // reduce of `x` over the single axis `axis` with `reducer`; the neutral element is checked
     const Op* reduce_over(int v, const char* reducer, int64_t& axis, int& x) const {
         const Op* r = op_named(v, "reduce");
@@ -152,22 +200,24 @@ struct Rewriter {
         const Op& root = fn.ops[ri];
         if (root.name != "divide" || !dtype_is_float(root.out.dtype)) return false;
         const Op* e = op_named(root.operands[0], "exponential");
-        const Op* sb = op_named(root.operands[1], "broadcast_in_dim");
-        if (!e || !sb) return false;
-        int64_t ax_s, ax_m;
+        if (!e) return false;
+        std::set<size_t> in = {ri, index_of(e)};
+        int64_t ax_s, ax_m, ax_b;
         int e_in, x;
-        const Op* s = reduce_over(sb->operands[0], "add", ax_s, e_in);
-        if (!s || e_in != e->result) return false;
-        const size_t rank = root.out.shape.size();
-        if (!dims_skip_axis(sb->dims, rank, ax_s)) return false;
+        const int sum = spread_src(root.operands[1], ax_b, in);
+        if (sum < 0) return false;
+        const Op* s = reduce_over(sum, "add", ax_s, e_in);
+        if (!s || e_in != e->result || ax_s != ax_b) return false;
         const Op* sh = op_named(e->operands[0], "subtract");
         if (!sh) return false;
-        const Op* mb = op_named(sh->operands[1], "broadcast_in_dim");
-        if (!mb) return false;
-        const Op* m = reduce_over(mb->operands[0], "maximum", ax_m, x);
-        if (!m || ax_m != ax_s || x != sh->operands[0] || !dims_skip_axis(mb->dims, rank, ax_m)) return false;
+        const int mx = spread_src(sh->operands[1], ax_b, in);
+        if (mx < 0) return false;
+        const Op* m = reduce_over(mx, "maximum", ax_m, x);
+        if (!m || ax_m != ax_s || ax_b != ax_s || x != sh->operands[0]) return false;
         if (!(type.at(x) == root.out)) return false;
-        std::set<size_t> in = {ri, index_of(e), index_of(sb), index_of(s), index_of(sh), index_of(mb), index_of(m)};
+        in.insert(index_of(s));
+        in.insert(index_of(sh));
+        in.insert(index_of(m));
         if (!closed(in, ri)) return false;
         char cfg[64];
         snprintf(cfg, sizeof cfg, "{\"axis\": %lld}", (long long)ax_s);
@@ -263,6 +313,7 @@ struct Rewriter {
     // ------------------------------------------------------------------ LayerNorm / RMSNorm
     // mean over the last axis: reduce_add(u) / N  or  reduce_add(u) * (1/N)
     bool mean_last(int v, int& u, std::set<size_t>& nodes) const {
+        v = relabel_src(v, nodes);
         const Op* o = op_of(v);
         if (!o || (o->name != "divide" && o->name != "multiply")) return false;
         for (int k = 0; k < 2; k++) {
@@ -271,7 +322,7 @@ struct Rewriter {
             int64_t axis;
             int src;
             std::set<size_t> via;
-            const Op* r = reduce_over(o->operands[k], "add", axis, src);
+            const Op* r = reduce_over(relabel_src(o->operands[k], nodes), "add", axis, src);
             if (!r || !splat_value(o->operands[1 - k], c, &via)) continue;
             const auto& shp = type.at(src).shape;
             if (shp.empty() || axis != (int64_t)shp.size() - 1) continue;
@@ -284,10 +335,14 @@ struct Rewriter {
         }
         return false;
     }
-    // v = broadcast over the last axis of a [.., 1]-less statistic
-    const Op* bcast_stat(int v, size_t rank) const {
-        const Op* b = op_named(v, "broadcast_in_dim");
-        return (b && dims_skip_axis(b->dims, rank, (int64_t)rank - 1)) ? b : nullptr;
+    // v = a statistic spread over the last axis; returns the statistic, -1 if not
+    int spread_last(int v, size_t rank, std::set<size_t>& nodes) const {
+        int64_t axis;
+        std::set<size_t> t = nodes;
+        const int src = spread_src(v, axis, t);
+        if (src < 0 || axis != (int64_t)rank - 1) return -1;
+        nodes = t;
+        return src;
     }
     // v = c * bcast(rsqrt(mean(c*c) + eps)); centred: c = x - bcast(mean(x))
     bool norm_core(int v, int& x, double& eps, bool& centred, std::set<size_t>& nodes) const {
@@ -296,14 +351,16 @@ struct Rewriter {
         const size_t rank = m->out.shape.size();
         if (rank < 1) return false;
         for (int k = 0; k < 2; k++) {
-            const Op* rb = bcast_stat(m->operands[k], rank);
-            if (!rb) continue;
+            std::set<size_t> tmp = {index_of(m)};
+            const int stat = spread_last(m->operands[k], rank, tmp);
+            if (stat < 0) continue;
             const int c = m->operands[1 - k];
-            const Op* rs = op_named(rb->operands[0], "rsqrt");
+            const Op* rs = op_named(stat, "rsqrt");
             if (!rs) continue;
-            const Op* ve = op_named(rs->operands[0], "add");
+            const Op* ve = op_named(relabel_src(rs->operands[0], tmp), "add");
             if (!ve) continue;
-            std::set<size_t> tmp = {index_of(m), index_of(rb), index_of(rs), index_of(ve)};
+            tmp.insert(index_of(rs));
+            tmp.insert(index_of(ve));
             for (int j = 0; j < 2; j++) {
                 double e;
                 int sq;
@@ -314,12 +371,11 @@ struct Rewriter {
                 if (!sqo || sqo->operands[0] != c || sqo->operands[1] != c) continue;
                 t2.insert(index_of(sqo));
                 const Op* sub = op_named(c, "subtract");
-                const Op* mb = sub ? bcast_stat(sub->operands[1], rank) : nullptr;
                 int mx;
                 std::set<size_t> t3 = t2;
-                if (sub && mb && mean_last(mb->operands[0], mx, t3) && mx == sub->operands[0]) {
+                const int mean = sub ? spread_last(sub->operands[1], rank, t3) : -1;
+                if (sub && mean >= 0 && mean_last(mean, mx, t3) && mx == sub->operands[0]) {
                     t3.insert(index_of(sub));
-                    t3.insert(index_of(mb));
                     x = mx;
                     centred = true;
                     nodes.insert(t3.begin(), t3.end());

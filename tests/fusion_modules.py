@@ -151,3 +151,63 @@ MATMUL_BIAS_RELU = """func.func @main(%x: tensor<32x64xf32>, %w: tensor<64x128xf
   %zero = stablehlo.constant dense<0.0> : tensor<32x128xf32>
   %r = stablehlo.maximum %h, %zero : tensor<32x128xf32>
   return %r : tensor<32x128xf32> }"""
+
+# keepdims style, as array libraries write `x - max(x, axis, keepdims=True)`: the statistic is
+# renamed to a shape with a unit dim (broadcast_in_dim or reshape), possibly computed on there,
+# and spread over the row by a second broadcast
+SOFTMAX_KEEPDIMS = """module @jit_softmax attributes {mhlo.num_partitions = 1 : i32, mhlo.num_replicas = 1 : i32} {
+  func.func public @main(%arg0: tensor<8x32xf32> {mhlo.layout_mode = "default"}) -> (tensor<8x32xf32> {jax.result_info = "", mhlo.layout_mode = "default"}) {
+    %cst = stablehlo.constant dense<0xFF800000> : tensor<f32>
+    %0 = stablehlo.reduce(%arg0 init: %cst) applies stablehlo.maximum across dimensions = [1] : (tensor<8x32xf32>, tensor<f32>) -> tensor<8xf32>
+    %1 = stablehlo.broadcast_in_dim %0, dims = [0] : (tensor<8xf32>) -> tensor<8x1xf32>
+    %2 = stablehlo.broadcast_in_dim %1, dims = [0, 1] : (tensor<8x1xf32>) -> tensor<8x32xf32>
+    %3 = stablehlo.subtract %arg0, %2 : tensor<8x32xf32>
+    %4 = stablehlo.exponential %3 : tensor<8x32xf32>
+    %cst_0 = stablehlo.constant dense<0.000000e+00> : tensor<f32>
+    %5 = stablehlo.reduce(%4 init: %cst_0) applies stablehlo.add across dimensions = [1] : (tensor<8x32xf32>, tensor<f32>) -> tensor<8xf32>
+    %6 = stablehlo.reshape %5 : (tensor<8xf32>) -> tensor<8x1xf32>
+    %7 = stablehlo.broadcast_in_dim %6, dims = [0, 1] : (tensor<8x1xf32>) -> tensor<8x32xf32>
+    %8 = stablehlo.divide %4, %7 : tensor<8x32xf32>
+    return %8 : tensor<8x32xf32>
+  }
+}"""
+
+LAYER_NORM_KEEPDIMS = """func.func @main(%x: tensor<16x64xf32>, %g: tensor<64xf32>, %b: tensor<64xf32>) -> tensor<16x64xf32> {
+  %zero = stablehlo.constant dense<0.0> : tensor<f32>
+  %n = stablehlo.constant dense<64.0> : tensor<16xf32>
+  %n1 = stablehlo.constant dense<64.0> : tensor<16x1xf32>
+  %eps = stablehlo.constant dense<1.0e-5> : tensor<16x1xf32>
+  %s = stablehlo.reduce(%x init: %zero) applies stablehlo.add across dimensions = [1] : (tensor<16x64xf32>, tensor<f32>) -> tensor<16xf32>
+  %mean = stablehlo.divide %s, %n : tensor<16xf32>
+  %mk = stablehlo.broadcast_in_dim %mean, dims = [0] : (tensor<16xf32>) -> tensor<16x1xf32>
+  %mb = stablehlo.broadcast_in_dim %mk, dims = [0, 1] : (tensor<16x1xf32>) -> tensor<16x64xf32>
+  %c = stablehlo.subtract %x, %mb : tensor<16x64xf32>
+  %sq = stablehlo.multiply %c, %c : tensor<16x64xf32>
+  %s2 = stablehlo.reduce(%sq init: %zero) applies stablehlo.add across dimensions = [1] : (tensor<16x64xf32>, tensor<f32>) -> tensor<16xf32>
+  %s2k = stablehlo.reshape %s2 : (tensor<16xf32>) -> tensor<16x1xf32>
+  %var = stablehlo.divide %s2k, %n1 : tensor<16x1xf32>
+  %ve = stablehlo.add %var, %eps : tensor<16x1xf32>
+  %r = stablehlo.rsqrt %ve : tensor<16x1xf32>
+  %rb = stablehlo.broadcast_in_dim %r, dims = [0, 1] : (tensor<16x1xf32>) -> tensor<16x64xf32>
+  %xn = stablehlo.multiply %c, %rb : tensor<16x64xf32>
+  %gb = stablehlo.broadcast_in_dim %g, dims = [1] : (tensor<64xf32>) -> tensor<16x64xf32>
+  %bb = stablehlo.broadcast_in_dim %b, dims = [1] : (tensor<64xf32>) -> tensor<16x64xf32>
+  %y = stablehlo.multiply %xn, %gb : tensor<16x64xf32>
+  %z = stablehlo.add %y, %bb : tensor<16x64xf32>
+  return %z : tensor<16x64xf32> }"""
+
+# the unit dim is put in front and the values are spread over axis 0: a column statistic, not a
+# row statistic -- must not be taken for the softmax over axis 1
+NOT_SOFTMAX_WRONG_SPREAD = """func.func @main(%x: tensor<8x8xf32>) -> tensor<8x8xf32> {
+  %ninf = stablehlo.constant dense<0xFF800000> : tensor<f32>
+  %zero = stablehlo.constant dense<0.0> : tensor<f32>
+  %m = stablehlo.reduce(%x init: %ninf) applies stablehlo.maximum across dimensions = [1] : (tensor<8x8xf32>, tensor<f32>) -> tensor<8xf32>
+  %mk = stablehlo.reshape %m : (tensor<8xf32>) -> tensor<1x8xf32>
+  %mb = stablehlo.broadcast_in_dim %mk, dims = [0, 1] : (tensor<1x8xf32>) -> tensor<8x8xf32>
+  %sh = stablehlo.subtract %x, %mb : tensor<8x8xf32>
+  %e = stablehlo.exponential %sh : tensor<8x8xf32>
+  %s = stablehlo.reduce(%e init: %zero) applies stablehlo.add across dimensions = [1] : (tensor<8x8xf32>, tensor<f32>) -> tensor<8xf32>
+  %sk = stablehlo.reshape %s : (tensor<8xf32>) -> tensor<1x8xf32>
+  %sb = stablehlo.broadcast_in_dim %sk, dims = [0, 1] : (tensor<1x8xf32>) -> tensor<8x8xf32>
+  %y = stablehlo.divide %e, %sb : tensor<8x8xf32>
+  return %y : tensor<8x8xf32> }"""

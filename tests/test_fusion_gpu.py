@@ -60,6 +60,29 @@ def test_softmax_gelu_norms(sess):
     close(b, exp, 1e-5)
 
 
+def test_keepdims_forms(sess):
+    rng = np.random.default_rng(82)
+    x = rng.standard_normal((8, 32)).astype(np.float32)
+    a, b = both(sess, M.SOFTMAX_KEEPDIMS, [(x, "f32")], "fused_softmax")
+    close(a, oracle.softmax(x.astype(np.float64)), 1e-5)
+    close(b, oracle.softmax(x.astype(np.float64)), 1e-5)
+    x = (3 + 2 * rng.standard_normal((16, 64))).astype(np.float32)
+    g = (1 + 0.1 * rng.standard_normal(64)).astype(np.float32)
+    bt = (0.1 * rng.standard_normal(64)).astype(np.float32)
+    a, b = both(sess, M.LAYER_NORM_KEEPDIMS, [(x, "f32"), (g, "f32"), (bt, "f32")], "fused_layer_norm")
+    exp = oracle.layer_norm(x.astype(np.float64), g.astype(np.float64), bt.astype(np.float64), 1e-5)
+    close(a, exp, 1e-5)
+    close(b, exp, 2e-5)
+    # the look-alike that spreads the row statistic over axis 0 runs as written: out[i, j] = e[i, j] / sum_k e[j, k]
+    x = rng.standard_normal((8, 8)).astype(np.float32)
+    exe = sess.compile(M.NOT_SOFTMAX_WRONG_SPREAD)
+    (got,) = sess.run(exe, [(x, "f32")])
+    sess.lib.mhlo_executable_destroy(exe)
+    x64 = x.astype(np.float64)
+    e = np.exp(x64 - x64.max(axis=1)[None, :])
+    close(got, e / e.sum(axis=1)[None, :], 1e-5)
+
+
 @pytest.mark.parametrize("with_mask,transpose_k,divide", [(False, True, False), (True, False, True), (True, True, False)])
 def test_attention_chain(sess, with_mask, transpose_k, divide):
     B, H, S, D = 2, 3, 64, 32

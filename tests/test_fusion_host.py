@@ -34,6 +34,15 @@ def test_softmax_chain_becomes_one_call(sess):
     assert "fused_softmax" not in ops(sess, M.SOFTMAX_ESCAPING)
 
 
+def test_keepdims_statistics_are_followed(sess):
+    """Statistics carried with a unit dim (broadcast_in_dim or reshape to [rows, 1], arithmetic on
+    that shape, one spreading broadcast at the end) are the same patterns; a statistic spread
+    over the other axis is not."""
+    assert ops(sess, M.SOFTMAX_KEEPDIMS) == ["fused_softmax"]
+    assert ops(sess, M.LAYER_NORM_KEEPDIMS) == ["fused_layer_norm"]
+    assert "fused_softmax" not in ops(sess, M.NOT_SOFTMAX_WRONG_SPREAD)
+
+
 def test_gelu_only_with_the_right_constants(sess):
     assert ops(sess, M.GELU) == ["fused_gelu"]
     assert "fused_gelu" not in ops(sess, M.NOT_GELU) and "tanh" in ops(sess, M.NOT_GELU)
