@@ -285,7 +285,7 @@ int mhip_fill(void* stream, void* y, int64_t n, uint64_t pattern, int elem_size)
  * 4 waves, 256x256 / 8 waves, 256x256 / 4 waves with the five-stage LDS ring) with
  * `iters` launches each on `stream`, stores the fastest in the process-wide tuning
  * table that mhip_gemm consults before its heuristic, and reports it (variant code
- * 128 | 256 | 2560, microseconds per launch).  Overwrites c; synchronises with the
+ * 128 | 256 | 2560 | 2561, microseconds per launch).  Overwrites c; synchronises with the
  * stream.  (Tuning/AutoTuner.swift:301-458.) */
 int mhip_gemm_autotune(void* stream, const void* a, const void* b, const void* bias, void* c,
                        int64_t M, int64_t N, int64_t K, int64_t batch, int64_t stride_a,

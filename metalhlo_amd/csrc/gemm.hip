@@ -398,28 +398,45 @@ static int launch_mfma(hipStream_t s, GemmArgs g, int64_t batch) {
 }
 
 // gemm256.hip: 4-wave 256x256 kernel with a hand-scheduled main loop.
-bool gemm256_eligible(const GemmArgs& g, int64_t batch, int dtype);
-int launch_gemm256(hipStream_t s, const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype);
+bool gemm256_eligible(const GemmArgs& g, int64_t batch, int dtype, int bw = 256);
+int launch_gemm256(hipStream_t s, const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype, int bw = 256);
 // tuning.hip: variant prescribed by the tuning table for this problem, 0 = none.
 int tuned_gemm_variant(const GemmArgs& g, int64_t batch, int ta, int tb, int dtype);
 
-// Which kernel serves a 16-bit problem (MHIP_GEMM_TILE = 128 | 256 | 2560 forces one):
-//   * the four-wave 256x256 kernel (gemm256.hip) when it is eligible and K is long
-//     enough (>= 1024) to amortise its one-workgroup-per-CU prologue and epilogue;
-//   * the eight-wave 256x256 kernel for large problems it cannot take whose rows of C
-//     are not 16-byte aligned (odd N): its eight waves hide the narrow stores;
+// Which kernel serves a 16-bit problem (MHIP_GEMM_TILE = 128 | 256 | 2560 | 2561 forces one):
+//   * the four-wave ring kernel (gemm256.hip) on 256x256 tiles (2560) or 256x128 tiles
+//     (2561) when K >= 512 and the problem is eligible: one workgroup per CU, so its time is
+//     rounds x (stages x per-stage time + prologue and epilogue), rounds = ceil(tiles / 256 CUs);
+//     the cheaper of the two by that count is taken.  In units of one MFMA issue slot per wave
+//     a K stage costs 32 on the wide tile and 18 on the narrow one (16 MFMAs, but three
+//     fragment reads for every four MFMAs instead of two), prologue + epilogue about 700 and
+//     500 -- figures fitted to seven measured shapes (4096^3: wide; [8192,768] x K 3072
+//     or 768, [8192,2304..3072] x K 768: narrow);
+//   * the eight-wave 256x256 kernel for large problems the ring kernel cannot take whose
+//     rows of C are not 16-byte aligned (odd N): its eight waves hide the narrow stores;
 //   * otherwise 128x128 tiles, two workgroups per CU (short K, few tiles).
 // An entry of the tuning table (mhip_gemm_autotune) for the problem overrides the heuristic.
 template <typename T, bool TA, bool TB>
 static int pick_tile(hipStream_t s, const GemmArgs& g, int64_t batch) {
-    const int64_t big = (int64_t)((g.M + 255) / 256) * ((g.N + 255) / 256) * batch;
+    const int64_t tiles_m = (g.M + 255) / 256;
+    const int64_t big = tiles_m * ((g.N + 255) / 256) * batch;
     constexpr int dt = std::is_same<T, bf16_t>::value ? MHIP_BF16 : MHIP_F16;
     int force = tune_int("MHIP_GEMM_TILE", 0);
     if (force == 0) force = tuned_gemm_variant(g, batch, TA, TB, dt);   // tuning table / running tuner
-    // the four-wave ring kernel: long K always; short K (its five-stage prologue weighs more)
-    // when there are clearly more 256x256 tiles than CUs
-    if (force == 2560 || (force == 0 && (g.K >= 1024 || (g.K >= 512 && big >= 320)))) {
+    if (force == 2561) {
+        if (gemm256_eligible(g, batch, dt, 128)) return launch_gemm256(s, g, batch, TA, TB, dt, 128);
+    }
+    if (force == 2560) {
         if (gemm256_eligible(g, batch, dt)) return launch_gemm256(s, g, batch, TA, TB, dt);
+    }
+    if (force == 0 && g.K >= 512) {
+        constexpr int cus = 256;                       // compute units of the device this is written for
+        const int64_t narrow = tiles_m * ((g.N + 127) / 128) * batch, stages = g.K / 32;
+        const bool wide_ok = gemm256_eligible(g, batch, dt), narrow_ok = gemm256_eligible(g, batch, dt, 128);
+        const int64_t wide_cost = ((big + cus - 1) / cus) * (stages * 32 + 700);
+        const int64_t narrow_cost = ((narrow + cus - 1) / cus) * (stages * 18 + 500);
+        if (narrow_ok && (!wide_ok || narrow_cost < wide_cost)) return launch_gemm256(s, g, batch, TA, TB, dt, 128);
+        if (wide_ok) return launch_gemm256(s, g, batch, TA, TB, dt);
     }
     const bool want256 = force == 256 || (force != 128 && big >= 192 && (g.K >= 1024 || g.N % 8 != 0));
     if (want256) return launch_mfma<T, 256, 256, 2, 4, TA, TB>(s, g, batch);

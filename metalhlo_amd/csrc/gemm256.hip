@@ -1,6 +1,6 @@
 // Large-problem GEMM for gfx950: 256x256 C tile, four waves (one per SIMD), each
 // wave a 128x128 sub-tile = 4x4 v_mfma_f32_32x32x16 accumulators that fill the
-// AGPR file.  The main loop is generated, hand-scheduled inline assembly
+// AGPR file; and the same kernel on a 256x128 tile (each wave 128x64, B tile 128 wide).  The main loop is generated, hand-scheduled inline assembly
 // (gen_gemm256_loop.py -> gemm256_loop.inc: schedule and register map are
 // documented there); this file computes the per-thread addresses it consumes and
 // holds the epilogue.
@@ -64,56 +64,72 @@ struct KMajor {
 };
 
 // ---- operand with k as the slow memory axis -------------------------------------
-// One load instruction of wave w in pass p fills k rows 8p + 2w, 8p + 2w + 1
-// (512 bytes each): lane -> k row (lane >> 5), position (lane & 31).
+// Tile of W mn-columns: k-rows of 2W bytes.  One load instruction of a wave fills 1 KB =
+// 1024 / 2W consecutive k-rows (W = 256: k rows 8p + 2w, 8p + 2w + 1 of pass p, lane -> k row
+// lane >> 5, position lane & 31; W = 128: k rows 16p + 4w .. + 3, lane -> lane >> 4, lane & 15).
+template <int W>
 struct MnMajor {
+    static constexpr int kLanesPerRow = W / 8;           // 16-byte chunks per k-row
+    static constexpr int kRowsPerSlot = 64 / kLanesPerRow;
     __device__ static uint32_t goff(int lane, int wave, int col0, int ld, int cols_total) {
-        const int k = 2 * wave + (lane >> 5);
-        const int c = (lane & 31) ^ ((k & 3) << 2);
+        const int k = kRowsPerSlot * wave + lane / kLanesPerRow;
+        const int c = (lane % kLanesPerRow) ^ ((k & 3) << 2);
         const int col = col0 + c * 8;
         return col < cols_total ? (uint32_t)(((int64_t)k * ld + col) * 2) : kOob;
     }
-    __device__ static uint32_t pass_stride(int ld) { return (uint32_t)(8 * ld * 2); }
+    __device__ static uint32_t pass_stride(int ld) { return (uint32_t)(4 * kRowsPerSlot * ld * 2); }
     __device__ static uint32_t stage_stride(int ld) { return (uint32_t)(32 * ld * 2); }
-    // read addresses of ring buffers 0 and 1: element j = mn block j at k-step 0
-    // (+ 8192 per k-step, + 2048 for the upper four k of a fragment, + 32768 for
-    // buffer 1); the loop derives the other buffers' addresses
+    // read addresses of ring buffers 0 and 1: element j = this wave's mn block j (32 columns)
+    // at k-step 0 (+ 16 k-rows per k-step, + 4 k-rows for the upper four k of a fragment,
+    // + one stage buffer for buffer 1); the loop derives the other buffers' addresses.
+    // The 64-byte position of a block in its k-row is (block ^ (k & 3)): the chunk swizzle above.
     __device__ static u32x4 raddr(int lane, int mn_block0, uint32_t base) {
         const int i = lane & 15, gq = lane >> 4;
         const int xr = (i >> 2) & 3;
-        const int mn = mn_block0 + 16 * (gq & 1) + 4 * (i & 3);
-        const uint32_t b = base + (uint32_t)((8 * (gq >> 1) + (i >> 2)) * 512 + ((mn >> 3) << 4) + (mn & 7) * 2);
+        const int blk0 = mn_block0 >> 5;
+        const uint32_t b = base + (uint32_t)((8 * (gq >> 1) + (i >> 2)) * (2 * W) + (16 * (gq & 1) + 4 * (i & 3)) * 2);
         u32x4 r;
-        r.x = b + (uint32_t)((0 ^ xr) << 6); r.y = b + (uint32_t)((1 ^ xr) << 6);
-        r.z = b + (uint32_t)((2 ^ xr) << 6); r.w = b + (uint32_t)((3 ^ xr) << 6);
+        r.x = b + (uint32_t)(((blk0 + 0) ^ xr) << 6); r.y = b + (uint32_t)(((blk0 + 1) ^ xr) << 6);
+        r.z = b + (uint32_t)(((blk0 + 2) ^ xr) << 6); r.w = b + (uint32_t)(((blk0 + 3) ^ xr) << 6);
         return r;
     }
 };
 
-template <typename T, bool TA, bool TB>
-__device__ inline void main_loop(f32x16 (&acc)[16], u32x4 ra, u32x4 rb, u32x2& misc,
+template <typename T, bool TA, bool TB, int BW>
+__device__ inline void main_loop(f32x16 (&acc)[BW / 16], u32x4 ra, u32x4 rb, u32x2& misc,
                                  __amdgpu_buffer_rsrc_t rsa, __amdgpu_buffer_rsrc_t rsb, uint32_t pa,
                                  uint32_t pb, uint32_t ta, uint32_t tb, uint32_t m0b, uint32_t kt) {
     constexpr bool bf = std::is_same<T, bf16_t>::value;
-    if constexpr (bf && !TA && !TB) gemm256_loop_nn_bf16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt);
-    if constexpr (bf && !TA && TB) gemm256_loop_nt_bf16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt);
-    if constexpr (bf && TA && !TB) gemm256_loop_tn_bf16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt);
-    if constexpr (bf && TA && TB) gemm256_loop_tt_bf16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt);
-    if constexpr (!bf && !TA && !TB) gemm256_loop_nn_f16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt);
-    if constexpr (!bf && !TA && TB) gemm256_loop_nt_f16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt);
-    if constexpr (!bf && TA && !TB) gemm256_loop_tn_f16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt);
-    if constexpr (!bf && TA && TB) gemm256_loop_tt_f16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt);
+#define MHIP_LOOP(cond, name)                                                                        \
+    if constexpr (cond) {                                                                            \
+        if constexpr (BW == 256) gemm256_loop_##name(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt); \
+        else gemm256x128_loop_##name(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt);           \
+    }
+    MHIP_LOOP(bf && !TA && !TB, nn_bf16)
+    MHIP_LOOP(bf && !TA && TB, nt_bf16)
+    MHIP_LOOP(bf && TA && !TB, tn_bf16)
+    MHIP_LOOP(bf && TA && TB, tt_bf16)
+    MHIP_LOOP(!bf && !TA && !TB, nn_f16)
+    MHIP_LOOP(!bf && !TA && TB, nt_f16)
+    MHIP_LOOP(!bf && TA && !TB, tn_f16)
+    MHIP_LOOP(!bf && TA && TB, tt_f16)
+#undef MHIP_LOOP
 }
 
-template <typename T, bool TA, bool TB>
+// BW = 256: the 256x256 tile (each wave 128x128).  BW = 128: a 256x128 tile (each wave
+// 128x64, half the accumulators, a 24 KB stage) for problems whose 256x256 tiling would
+// leave compute units idle or a last round nearly empty.
+template <typename T, bool TA, bool TB, int BW>
 __global__ __launch_bounds__(256) void gemm256_kernel(GemmArgs g) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    using LA = typename std::conditional<TA, MnMajor, KMajor>::type;
-    using LB = typename std::conditional<TB, KMajor, MnMajor>::type;
+    using LA = typename std::conditional<TA, MnMajor<256>, KMajor>::type;
+    using LB = typename std::conditional<TB, KMajor, MnMajor<BW>>::type;
+    constexpr int WN = BW / 2;            // columns per wave
+    constexpr int NBF = BW / 64;          // 32-column accumulator blocks per wave
 
     int tm, tn;
     tile_of(blockIdx.x, gridDim.x, g.tiles_m, g.tiles_n, tm, tn);
-    const int m0 = tm * 256, n0 = tn * 256;
+    const int m0 = tm * 256, n0 = tn * BW;
     const int64_t batch = blockIdx.y;
     const char* a = reinterpret_cast<const char*>(static_cast<const T*>(g.a) + batch * g.sa);
     const char* b = reinterpret_cast<const char*>(static_cast<const T*>(g.b) + batch * g.sb);
@@ -129,7 +145,7 @@ __global__ __launch_bounds__(256) void gemm256_kernel(GemmArgs g) {
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
 
     const u32x4 ra = LA::raddr(lane, wm * 128, lds0);
-    const u32x4 rb = LB::raddr(lane, wn * 128, lds0 + kOperBytes);
+    const u32x4 rb = LB::raddr(lane, wn * WN, lds0 + kOperBytes);
     u32x2 misc;
     misc.x = LA::goff(lane, wave, m0, g.lda, g.M);
     misc.y = LB::goff(lane, wave, n0, g.ldb, g.N);
@@ -140,9 +156,9 @@ __global__ __launch_bounds__(256) void gemm256_kernel(GemmArgs g) {
     const __amdgpu_buffer_rsrc_t rsb =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(b), 0, b_bytes, 0x00020000);
 
-    f32x16 acc[16];
-    main_loop<T, TA, TB>(acc, ra, rb, misc, rsa, rsb, LA::pass_stride(g.lda), LB::pass_stride(g.ldb),
-                         LA::stage_stride(g.lda), LB::stage_stride(g.ldb), m0b, (uint32_t)(g.K / 32));
+    f32x16 acc[4 * NBF];
+    main_loop<T, TA, TB, BW>(acc, ra, rb, misc, rsa, rsb, LA::pass_stride(g.lda), LB::pass_stride(g.ldb),
+                             LA::stage_stride(g.lda), LB::stage_stride(g.ldb), m0b, (uint32_t)(g.K / 32));
 
     // The loop ends with every wave's outstanding loads landed and a barrier, so the
     // ring may be reused as the staging area below.  Waves may still have (unused)
@@ -151,14 +167,14 @@ __global__ __launch_bounds__(256) void gemm256_kernel(GemmArgs g) {
     // Accumulator tiles are transposed: lane = row m (lrow), register group
     // q = r / 4 holds columns 8q + 4*lhalf + r % 4 of the 32-column block.
     const T* bias = static_cast<const T*>(g.bias);
-    constexpr int kRowPad = 128 * 2 + 16;
+    constexpr int kRowPad = WN * 2 + 16;
     char* stage = smem + wave * (128 * kRowPad);
     dispatch_act(g.act, [&](auto act_tag) {
     constexpr int ACT = decltype(act_tag)::value;
-    static_for<16>([&](auto jq_tag) {
+    static_for<4 * NBF>([&](auto jq_tag) {
         constexpr int j = decltype(jq_tag)::value >> 2, q = decltype(jq_tag)::value & 3;
         const int nl = j * 32 + 8 * q + 4 * lhalf;
-        const int n = n0 + wn * 128 + nl;
+        const int n = n0 + wn * WN + nl;
         float bv[4] = {0.f, 0.f, 0.f, 0.f};
         if (bias && n < g.N) {
             const Pack4<T> t = __builtin_bit_cast(Pack4<T>, *reinterpret_cast<const u32x2*>(bias + n));
@@ -170,24 +186,26 @@ __global__ __launch_bounds__(256) void gemm256_kernel(GemmArgs g) {
             Pack4<T> o;
             static_for<4>([&](auto e_tag) {
                 constexpr int e = decltype(e_tag)::value;
-                float v = acc[i * 4 + j][4 * q + e] + bv[e];
+                float v = acc[i * NBF + j][4 * q + e] + bv[e];
                 v = apply_act_c<ACT>(v);
                 o.v[e] = Elem<T>::from_f32(v);
             });
             *reinterpret_cast<u32x2*>(stage + (i * 32 + lrow) * kRowPad + nl * 2) =
                 __builtin_bit_cast(u32x2, o);
         });
-        // one register group at a time: do not let 256 accumulator reads pile up
+        // one register group at a time: do not let all the accumulator reads pile up
         __builtin_amdgcn_sched_barrier(0);
     });
     });
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // a wave re-reads only its own rows
-    const int cc = lane & 15, rr = lane >> 4;
+    constexpr int kChunks = WN / 8;                      // 16-byte chunks per row of the wave's sub-tile
+    constexpr int kRowsPerPass = 64 / kChunks;
+    const int cc = lane % kChunks, rr = lane / kChunks;
 #pragma unroll 4
-    for (int p = 0; p < 32; p++) {
-        const int ml = p * 4 + rr;
+    for (int p = 0; p < 128 / kRowsPerPass; p++) {
+        const int ml = p * kRowsPerPass + rr;
         const int m = m0 + wm * 128 + ml;
-        const int n = n0 + wn * 128 + cc * 8;
+        const int n = n0 + wn * WN + cc * 8;
         if (m < g.M && n < g.N) {
             u32x4 w = *reinterpret_cast<const u32x4*>(stage + ml * kRowPad + cc * 16);
             if (res) w = add_chunk<T>(w, *reinterpret_cast<const u32x4*>(res + (int64_t)m * g.N + n));
@@ -196,10 +214,10 @@ __global__ __launch_bounds__(256) void gemm256_kernel(GemmArgs g) {
     }
 }
 
-template <typename T, bool TA, bool TB>
+template <typename T, bool TA, bool TB, int BW>
 int launch256(hipStream_t s, GemmArgs g, int64_t batch) {
-    constexpr int kSmem = 5 * 32 * 1024;   // ring of five stage buffers; the epilogue staging (136 KB) reuses it
-    auto kern = gemm256_kernel<T, TA, TB>;
+    constexpr int kSmem = 5 * (16 + BW / 16) * 1024;   // ring of five stage buffers; the epilogue staging reuses it
+    auto kern = gemm256_kernel<T, TA, TB, BW>;
     static std::once_flag once;
     static hipError_t attr_err = hipSuccess;
     std::call_once(once, [&] {
@@ -210,41 +228,45 @@ int launch256(hipStream_t s, GemmArgs g, int64_t batch) {
         return fail(MHIP_ERR_LAUNCH, "gemm256: cannot reserve %d bytes of LDS: %s", kSmem,
                     hipGetErrorString(attr_err));
     g.tiles_m = (g.M + 255) / 256;
-    g.tiles_n = (g.N + 255) / 256;
+    g.tiles_n = (g.N + BW - 1) / BW;
     hipLaunchKernelGGL(kern, dim3((unsigned)(g.tiles_m * g.tiles_n), (unsigned)batch), dim3(256),
                        kSmem, s, g);
     return check_launch("gemm256");
 }
 
-template <typename T>
+template <typename T, int BW>
 int layout256(hipStream_t s, const GemmArgs& g, int64_t batch, int ta, int tb) {
-    if (!ta && !tb) return launch256<T, false, false>(s, g, batch);
-    if (!ta && tb) return launch256<T, false, true>(s, g, batch);
-    if (ta && !tb) return launch256<T, true, false>(s, g, batch);
-    return launch256<T, true, true>(s, g, batch);
+    if (!ta && !tb) return launch256<T, false, false, BW>(s, g, batch);
+    if (!ta && tb) return launch256<T, false, true, BW>(s, g, batch);
+    if (ta && !tb) return launch256<T, true, false, BW>(s, g, batch);
+    return launch256<T, true, true, BW>(s, g, batch);
 }
 
 }  // namespace
 
-// The kernel needs whole K stages, 16-byte-aligned operand rows (checked by the
-// caller), an output it can store 16 bytes at a time, operands small enough for
+// The kernels need whole K stages, 16-byte-aligned operand rows (checked by the
+// caller), an output they can store 16 bytes at a time, operands small enough for
 // 32-bit byte offsets including the prefetch overrun of five K stages, and enough
-// 256x256 tiles to occupy the device.
-bool gemm256_eligible(const GemmArgs& g, int64_t batch, int dtype) {
+// tiles (256 x `bw`) to occupy the device.
+bool gemm256_eligible(const GemmArgs& g, int64_t batch, int dtype, int bw) {
     if (dtype != MHIP_BF16 && dtype != MHIP_F16) return false;
     if (g.K % 32 != 0 || g.K < 32) return false;
     if (g.N % 8 != 0 || (reinterpret_cast<uintptr_t>(g.c) & 15) != 0 || g.sc % 8 != 0) return false;
     if (g.bias && (reinterpret_cast<uintptr_t>(g.bias) & 7) != 0) return false;
     const int64_t a_bytes = (int64_t)g.M * g.K * 2, b_bytes = (int64_t)g.N * g.K * 2;
     if (a_bytes >= 0x70000000LL || b_bytes >= 0x70000000LL) return false;
-    const int64_t tiles = (int64_t)((g.M + 255) / 256) * ((g.N + 255) / 256) * batch;
+    const int64_t tiles = (int64_t)((g.M + 255) / 256) * ((g.N + bw - 1) / bw) * batch;
     return tiles >= 192 && tiles <= 0x7FFFFFFF && batch <= 65535;
 }
 
 int launch_gemm256(hipStream_t s, const GemmArgs& g, int64_t batch, int trans_a, int trans_b,
-                   int dtype) {
-    if (dtype == MHIP_BF16) return layout256<bf16_t>(s, g, batch, trans_a, trans_b);
-    return layout256<f16_t>(s, g, batch, trans_a, trans_b);
+                   int dtype, int bw) {
+    if (bw == 128) {
+        if (dtype == MHIP_BF16) return layout256<bf16_t, 128>(s, g, batch, trans_a, trans_b);
+        return layout256<f16_t, 128>(s, g, batch, trans_a, trans_b);
+    }
+    if (dtype == MHIP_BF16) return layout256<bf16_t, 256>(s, g, batch, trans_a, trans_b);
+    return layout256<f16_t, 256>(s, g, batch, trans_a, trans_b);
 }
 
 }  // namespace mhip

@@ -52,8 +52,19 @@ EXP = os.environ.get("GEMM256_EXP", "")   # timing experiments only: noload, nom
 
 NST = 5               # ring stages
 UNROLL = 10           # stages per loop body: lcm(ring, pair issue, fragment set rotation)
-STAGE = 32768         # bytes per stage buffer
-OPER = 16384          # bytes per operand tile
+OPER = 16384          # bytes of the A tile (256 rows x 32 k); the B tile follows it in a stage buffer
+# Set per emitted function: the B tile is 256 or 128 columns wide.  The narrow form gives a
+# 256x128 workgroup tile (each wave 128x64 = 4x2 accumulators, 128 AGPRs) for problems
+# whose 256x256 tiling leaves compute units idle.
+BW = 256              # B tile width
+NBF = 4               # B fragments (32 columns each) per wave = BW / 64
+STAGE = 32768         # bytes per stage buffer = OPER + BW * 64
+
+
+def configure(bw):
+    global BW, NBF, STAGE
+    BW, NBF, STAGE = bw, bw // 64, OPER + bw * 64
+
 SET = {n: (32 * n, 32 * n + 16) for n in range(4)}   # fragment set -> (A base vgpr, B base vgpr)
 RA, RB = 192, 204
 GOFF = {"A": 216, "B": 217}
@@ -72,14 +83,15 @@ def frag_reads(kind, which, g, s, fset):
     addr = RA if which == "A" else RB
     h, lo = g >> 1, (g & 1) * STAGE
     out = []
-    for j in range(4):
+    rowb = 512 if which == "A" else 2 * BW      # bytes per k-row of an MN tile
+    for j in range(4 if which == "A" else NBF):
         dst = base + 4 * j
         if kind == "K":
             out.append(f"ds_read_b128 {vr(dst, 4)}, v{addr + 2 * h + s} offset:{lo + j * 2048}")
         else:
-            off = lo + s * 8192
+            off = lo + s * 16 * rowb
             out.append(f"ds_read_b64_tr_b16 {vr(dst, 2)}, v{addr + 4 * h + j} offset:{off}")
-            out.append(f"ds_read_b64_tr_b16 {vr(dst + 2, 2)}, v{addr + 4 * h + j} offset:{off + 2048}")
+            out.append(f"ds_read_b64_tr_b16 {vr(dst + 2, 2)}, v{addr + 4 * h + j} offset:{off + 4 * rowb}")
     return out
 
 
@@ -107,15 +119,16 @@ def trigger_group(kinds, t):
     """Loads triggered by the barrier of stage t (buffer t % 5 has just become free)."""
     grp = []
     for which in ("A", "B"):
+        passes = 4 if which == "A" else NBF     # 4 KB (one 1 KB slot per wave) per pass
         if kinds[which] == "K":
             if t % 2 == 0:
-                for p in range(4):
+                for p in range(passes):
                     grp.append(load_instr(which, t + 4, p))
                     grp.append(load_instr(which, t + 5, p, second_half=True))
                 grp.append(dict(stage=None, lines=[f"v_add_u32 v{GOFF[which]}, 128, v{GOFF[which]}",
                                                    f"v_add_u32 v{GOFF2[which]}, 128, v{GOFF2[which]}"]))
         else:
-            for p in range(4):
+            for p in range(passes):
                 grp.append(load_instr(which, t + 5, p))
             step = "%[ta]" if which == "A" else "%[tb]"
             grp.append(dict(stage=None, lines=[f"v_add_u32 v{GOFF[which]}, {step}, v{GOFF[which]}"]))
@@ -131,8 +144,8 @@ def mfmas(mnem, fset):
     a, b = SET[fset]
     out = []
     for i in range(4):
-        for j in range(4):
-            acc = 16 * (4 * i + j)
+        for j in range(NBF):
+            acc = 16 * (NBF * i + j)
             # (B, A): the accumulator tile comes out transposed (lane = row m)
             out.append(f"{mnem} a[{acc}:{acc + 15}], {vr(b + 4 * j, 4)}, {vr(a + 4 * i, 4)}, a[{acc}:{acc + 15}]")
     return out
@@ -228,7 +241,7 @@ def stage_iteration(mnem, kinds, t, vmcnt):
 def body(mnem, kinds):
     pro_vmcnt, vmcnts = simulate(kinds)
     out = []
-    for r in range(256):
+    for r in range(64 * NBF):
         out.append(f"v_accvgpr_write_b32 a{r}, 0")
     for which, pin in (("A", "%[pa]"), ("B", "%[pb]")):
         for i in range(1, 4):
@@ -277,13 +290,13 @@ def body(mnem, kinds):
 def emit(name, mnem, ka, kb):
     lines = body(mnem, {"A": ka, "B": kb})
     print(f"// {name}: A operand {ka}-major, B operand {kb}-major, {mnem}")
-    print(f"__device__ __forceinline__ void {name}(f32x16 (&acc)[16], u32x4 ra, u32x4 rb, u32x2& goff,")
+    print(f"__device__ __forceinline__ void {name}(f32x16 (&acc)[{4 * NBF}], u32x4 ra, u32x4 rb, u32x2& goff,")
     print("        __amdgpu_buffer_rsrc_t rsa, __amdgpu_buffer_rsrc_t rsb, uint32_t pa, uint32_t pb,")
     print("        uint32_t ta, uint32_t tb, uint32_t m0b, uint32_t kt) {")
     print("    asm volatile(")
     for ln in lines:
         print(f'        "{ln}\\n"')
-    outs = ", ".join(f'"={{a[{16 * i}:{16 * i + 15}]}}"(acc[{i}])' for i in range(16))
+    outs = ", ".join(f'"={{a[{16 * i}:{16 * i + 15}]}}"(acc[{i}])' for i in range(4 * NBF))
     print(f"        : {outs},")
     print(f'          "+{{v[{GOFF["A"]}:{GOFF["B"]}]}}"(goff)')
     print(f'        : "{{v[{RA}:{RA + 3}]}}"(ra), "{{v[{RB}:{RB + 3}]}}"(rb),')
@@ -297,11 +310,13 @@ def emit(name, mnem, ka, kb):
 
 def main():
     print("// Generated by gen_gemm256_loop.py -- do not edit by hand.")
-    print("// Main loops of the 256x256 GEMM kernel (the generator documents the schedule")
+    print("// Main loops of the 256x256 and 256x128 GEMM kernels (the generator documents the schedule")
     print("// and the register map).\n")
-    for tname, mnem in (("bf16", "v_mfma_f32_32x32x16_bf16"), ("f16", "v_mfma_f32_32x32x16_f16")):
-        for lname, ka, kb in (("nn", "K", "MN"), ("nt", "K", "K"), ("tn", "MN", "MN"), ("tt", "MN", "K")):
-            emit(f"gemm256_loop_{lname}_{tname}", mnem, ka, kb)
+    for bw, stem in ((256, "gemm256_loop"), (128, "gemm256x128_loop")):
+        configure(bw)
+        for tname, mnem in (("bf16", "v_mfma_f32_32x32x16_bf16"), ("f16", "v_mfma_f32_32x32x16_f16")):
+            for lname, ka, kb in (("nn", "K", "MN"), ("nt", "K", "K"), ("tn", "MN", "MN"), ("tt", "MN", "K")):
+                emit(f"{stem}_{lname}_{tname}", mnem, ka, kb)
 
 
 if __name__ == "__main__":

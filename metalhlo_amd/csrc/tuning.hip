@@ -17,7 +17,7 @@
 
 namespace mhip {
 
-bool gemm256_eligible(const GemmArgs& g, int64_t batch, int dtype);
+bool gemm256_eligible(const GemmArgs& g, int64_t batch, int dtype, int bw = 256);
 
 namespace {
 using Key = std::tuple<int64_t, int64_t, int64_t, int64_t, int, int, int>;
@@ -38,7 +38,7 @@ int load_file(const char* path, bool quiet) {
         int ta, tb, dt, variant;
         float us;
         if (sscanf(line, "gemm %lld %lld %lld %lld %d %d %d %d %f", &M, &N, &K, &B, &ta, &tb, &dt, &variant, &us) != 9 ||
-            (variant != 128 && variant != 256 && variant != 2560)) {
+            (variant != 128 && variant != 256 && variant != 2560 && variant != 2561)) {
             st = quiet ? MHIP_OK : fail(MHIP_ERR_INVALID_ARGUMENT, "tuning: malformed line in %s: %s", path, line);
             break;
         }
@@ -83,11 +83,12 @@ extern "C" int mhip_gemm_autotune(void* stream, const void* a, const void* b, co
     g.a = a; g.b = b; g.bias = bias; g.c = c;
     g.M = (int)M; g.N = (int)N; g.K = (int)K;
     g.sa = stride_a; g.sb = stride_b; g.sc = stride_c;
-    const int candidates[3] = {128, 256, 2560};
+    const int candidates[4] = {128, 256, 2560, 2561};
     int best = 0, st = MHIP_OK;
     float best_us = 0.f;
     for (int v : candidates) {
         if (v == 2560 && !gemm256_eligible(g, batch, dtype)) continue;    // validity filter
+        if (v == 2561 && !gemm256_eligible(g, batch, dtype, 128)) continue;
         g_forced = v;
         for (int i = 0; i < 2 && st == MHIP_OK; i++)
             st = mhip_gemm(stream, a, b, bias, c, M, N, K, batch, stride_a, stride_b, stride_c, trans_a, trans_b, activation, dtype);

@@ -290,7 +290,7 @@ def autotune_matmul(a, b, bias=None, activation: str = "none", trans_a: bool = F
                     trans_b: bool = False, iters: int = 10):
     """Times the GEMM kernel variants for this 2-D problem and stores the fastest in the
     library's tuning table (used by every later matmul of the same shape, layout and
-    type).  Returns (variant code 128 | 256 | 2560, microseconds per launch)."""
+    type).  Returns (variant code 128 | 256 | 2560 | 2561, microseconds per launch)."""
     _dev(a, b, bias)
     lib = _lib.load()
     if a.dim() != 2 or b.dim() != 2 or a.dtype != b.dtype:

@@ -155,14 +155,17 @@ BIG = [(4096, 3072, 32), (3585, 3848, 96), (4000, 3608, 160), (3600, 4104, 448),
 @pytest.mark.parametrize("layout", [(False, False), (False, True), (True, False), (True, True)],
                          ids=["nn", "nt", "tn", "tt"])
 @pytest.mark.parametrize("shape", BIG, ids=lambda s: "x".join(map(str, s)))
-def test_gemm_large_tiles(shape, layout, dtype):
+@pytest.mark.parametrize("tile", ["2560", "2561"], ids=["256x256", "256x128"])
+def test_gemm_large_tiles(shape, layout, dtype, tile):
+    """The four-wave ring kernel on both of its tile widths (forced: also where the default picks
+    another kernel), ragged M and N included."""
     from metalhlo_amd import kernels
     M, N, K = shape
     ta, tb = layout
     a, b = _ab(M, N, K, dtype, 27, ta, tb)
     rng = np.random.default_rng(28)
     bias = to_dev(rng.standard_normal(N) * 0.5, dtype)
-    os.environ["MHIP_GEMM_TILE"] = "2560"      # this kernel also where the default picks another (short K)
+    os.environ["MHIP_GEMM_TILE"] = tile
     try:
         c = kernels.matmul(a, b, bias, "relu", trans_a=ta, trans_b=tb)
     finally:
@@ -194,7 +197,7 @@ def test_gemm_large_exact_small_integers():
     assert torch.equal(kernels.matmul(a, b.t().contiguous(), trans_b=True), c)
 
 
-@pytest.mark.parametrize("tile", ["128", "256", "2560", "simple"])
+@pytest.mark.parametrize("tile", ["128", "256", "2560", "2561", "simple"])
 def test_gemm_residual_equals_gemm_then_add(tile, monkeypatch):
     """act(A.B + bias) + R in one kernel is bit for bit mhip_gemm followed by mhip_add, on every
     GEMM kernel (tile choice forced), batched and in place (R == C)."""
