@@ -35,13 +35,13 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by what the same
 # counter reads for the 'copy' workload (256 MiB in, 256 MiB out); see profiles/<workload>.txt.
 MEASURED_TRAFFIC = {
-    "gemm": 238902106,
-    "attention": 775878327,
-    "attention_full": 268950097,
-    "softmax": 536720377,
-    "layer_norm": 536913493,
-    "rms_norm": 536798961,
-    "bias_gelu": 536775641,
+    "gemm": 238901384,
+    "attention": 773135522,
+    "attention_full": 268909839,
+    "softmax": 536709952,
+    "layer_norm": 536897658,
+    "rms_norm": 536783693,
+    "bias_gelu": 536757341,
     "copy": 536870912,
 }
 
