@@ -4,8 +4,8 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--only]
 
 One "step" is one launch of the workload's kernel over one batch of synthetic
-input that already sits in HBM.  The headline workload is BASELINE.json
-configs[1] (bf16 GEMM 4096^3, fp32 accumulate); the other BASELINE kernels
+input that already sits in HBM.  The headline workload is the bf16 GEMM 4096^3
+(fp32 accumulate, the second benchmark configuration); the other kernels of the path
 (flash attention, softmax, LayerNorm, RMSNorm, bias+GELU) are timed the same way
 and reported under "kernels" of the same JSON line unless --only is given.
 

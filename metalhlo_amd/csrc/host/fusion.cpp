@@ -107,17 +107,6 @@ struct Rewriter {
 
     static bool near(double a, double b, double tol) { return fabs(a - b) <= tol; }
 
-    // dims of a broadcast_in_dim that puts an operand of rank r-1 back over every axis but `axis`
-    static bool dims_skip_axis(const std::vector<int64_t>& dims, size_t rank, int64_t axis) {
-        if (dims.size() + 1 != rank) return false;
-        int64_t d = 0;
-        for (int64_t got : dims) {
-            if (d == axis) d++;
-            if (got != d++) return false;
-        }
-        return true;
-    }
-
     // Statistics (one value per row) are often carried in keepdims style: reshaped or broadcast
     // to a shape with extra unit dims, computed on there, and spread over the row at the end.
     // relabel_src skips the ops that only rename the dims of `v` (reshape; broadcast_in_dim that
@@ -406,10 +395,9 @@ struct Rewriter {
         if (!dtype_is_float(root.out.dtype) || root.out.dtype == F64 || root.out.shape.empty()) return false;
         const size_t rank = root.out.shape.size();
         const int64_t cols = root.out.shape.back();
-        int x, gamma = -1, beta = -1;
+        int x;
         double eps;
         bool centred;
-        std::set<size_t> in = {ri};
         if (root.name == "add") {            // (core * gamma) + beta
             for (int k = 0; k < 2; k++) {
                 std::set<size_t> t = {ri};
@@ -445,7 +433,6 @@ struct Rewriter {
             replace(ri, t2, "fused_rms_norm", {x, g}, cfg);
             return true;
         }
-        (void)gamma; (void)beta; (void)in;
         return false;
     }
 

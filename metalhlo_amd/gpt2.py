@@ -1,4 +1,4 @@
-"""GPT-2 forward through the fused kernels (BASELINE config 5).
+"""GPT-2 forward through the fused kernels (the GPT-2-small benchmark configuration: B8 S1024).
 
 The op sequence is the one the reference's fusion passes produce for a pre-LN
 GPT-2 block — fused_layer_norm, fused_matmul_bias_activation (bias only, and

@@ -24,7 +24,7 @@ def _qkv(B, H, Sq, Skv, D, dtype, seed):
 
 
 def test_c1_fp32_causal_sdpa():
-    """BASELINE config 0: fp32, B1 H4 S128 D64, causal, scale 1/8, seed 1234 —
+    """The first benchmark configuration: fp32, B1 H4 S128 D64, causal, scale 1/8, seed 1234 —
     causal flag and additive -inf mask variants must both match the oracle."""
     from metalhlo_amd import kernels
     q, k, v = _qkv(1, 4, 128, 128, 64, torch.float32, 1234)
@@ -190,7 +190,7 @@ def test_attention_invariants():
 
 @pytest.mark.parametrize("causal,S", [(True, 4096), (False, 2048)], ids=["causal4096", "full2048"])
 def test_attention_baseline_shape_sampled(causal, S):
-    """BASELINE config 3: bf16 B4 H32 D128 (seed 4). Oracle on sampled (b,h) slices and rows."""
+    """The attention benchmark configuration: bf16 B4 H32 D128 (seed 4). Oracle on sampled (b,h) slices and rows."""
     from metalhlo_amd import kernels
     B, H, D = 4, 32, 128
     g = torch.Generator(device="cuda").manual_seed(4)

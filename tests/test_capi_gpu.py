@@ -104,7 +104,7 @@ def test_decomposed_softmax_and_gelu(sess):
 
 
 def test_config0_fused_sdpa_module(sess):
-    """BASELINE config 0: single StableHLO module for fused SDPA, fp32 B1 H4 S128 D64,
+    """The first benchmark configuration: single StableHLO module for fused SDPA, fp32 B1 H4 S128 D64,
     causal, scale 1/8, N(0,1) inputs (seed 1234): causal flag and additive-mask forms."""
     rng = np.random.default_rng(1234)
     q, k, v = (rng.standard_normal((1, 4, 128, 64)).astype(np.float32) for _ in range(3))

@@ -131,7 +131,7 @@ def test_reference_dot_known_answers():
 
 
 def test_gemm_4096_sampled_rows():
-    """BASELINE GEMM config: 4096^3 bf16, uniform[-1,1] (seed 2). Oracle on 64 sampled rows."""
+    """The benchmark GEMM: 4096^3 bf16, uniform[-1,1] (seed 2). Oracle on 64 sampled rows."""
     from metalhlo_amd import kernels
     rng = np.random.default_rng(2)
     a = to_dev(rng.uniform(-1, 1, (4096, 4096)), torch.bfloat16)

@@ -44,7 +44,7 @@ def test_gpt2_reduced_depth_full_width():
 
 
 def test_gpt2_small_baseline_shape():
-    """BASELINE config 4: 12 layers, B8 S1024.  The oracle runs on batch element 0
+    """The benchmark configuration: 12 layers, B8 S1024.  The oracle runs on batch element 0
     alone (sequences are independent); properties cover the rest."""
     from metalhlo_amd.gpt2 import GPT2, GPT2Config, init_params
     cfg = GPT2Config()

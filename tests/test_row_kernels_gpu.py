@@ -124,7 +124,7 @@ def test_empty_and_errors(lib):
 
 
 def test_invariants_full_size():
-    """BASELINE row-kernel shape [32768, 4096] bf16: size-independent properties."""
+    """The benchmark row-kernel shape [32768, 4096] bf16: size-independent properties."""
     from metalhlo_amd import kernels
     g = torch.Generator(device="cuda").manual_seed(3)
     x = torch.randn(32768, 4096, generator=g, device="cuda", dtype=torch.float32).to(torch.bfloat16)
