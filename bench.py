@@ -163,7 +163,7 @@ def measure(wl, steps, warmup, torch, key=None):
 
 
 # ---------------------------------------------------------------- CPU baseline (oracle port)
-def cpu_baseline_gemm(sample_rows=512, N=4096, K=4096):
+def cpu_baseline_gemm(sample_rows=4096, N=4096, K=4096):
     import numpy as np
     from oracle import oracle
     lib = C.CDLL(os.path.join(ROOT, "oracle", "liboracle.so"))
@@ -183,7 +183,8 @@ def cpu_baseline_gemm(sample_rows=512, N=4096, K=4096):
     return dict(value=round(2.0 * sample_rows * N * K / best / 1e12, 5), unit="TFLOP/s",
                 cores=int(lib.orc_num_threads()), kind="port",
                 sample=f"oracle/oracle_kernels.c orc_gemm on {sample_rows} of 4096 rows of A "
-                       f"(x full B), bf16 in / fp32 accumulate, best of 3; host has {os.cpu_count()} logical CPUs")
+                       f"(x full B), bf16 in / fp32 accumulate, one warm-up + best of 3 "
+                       f"({best:.2f} s each); host has {os.cpu_count()} logical CPUs")
 
 
 def main():

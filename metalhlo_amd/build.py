@@ -120,18 +120,10 @@ def build_host(verbose: bool = True) -> list:
     return outs
 
 
-def build_oracle(verbose: bool = True) -> str:
-    d = os.path.join(ROOT, "oracle")
-    _run(["make", "-C", d, "-B", "liboracle.so"])
-    if verbose:
-        print("  make  oracle/liboracle.so", flush=True)
-    return os.path.join(d, "liboracle.so")
-
-
 def build_all(verbose: bool = True):
+    """The product: the HIP kernel library and the host libraries over it."""
     build_kernels(verbose)
     build_host(verbose)
-    build_oracle(verbose)
 
 
 if __name__ == "__main__":
