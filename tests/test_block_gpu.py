@@ -1,0 +1,93 @@
+"""GPU: one whole pre-LayerNorm transformer block written in plain StableHLO (93 operations, no
+custom calls; tests/fusion_modules.py transformer_block) through mhlo_compile: the pattern
+recogniser turns it into LayerNorm / GEMM+bias(+GELU) / attention kernels plus the head
+split and merge glue (26 operations), and both that and the program run as written agree with
+the float64 oracle of the block.  f32: |got - e| <= max(tol, tol |e|) with tol 5e-5 for the
+whole block (about ten chained operators, each held to 1e-5 on its own); bf16: the
+end-to-end rule used for the GPT-2 logits (99.5 % within 2e-2, worst 6e-2)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from oracle import oracle
+from tests import fusion_modules as fm
+from tests.test_arena_gpu import run_with
+
+pytestmark = pytest.mark.gpu
+
+B, S, H, D, F = 2, 64, 4, 32, 256
+d = H * D
+FUSED = ["fused_layer_norm", "fused_matmul_bias_activation", "slice", "reshape", "transpose", "slice", "reshape", "transpose",
+         "slice", "reshape", "transpose", "iota", "iota", "compare", "constant", "constant", "select",
+         "fused_scaled_dot_product_attention", "transpose", "reshape", "fused_matmul_bias_activation", "add",
+         "fused_layer_norm", "fused_matmul_bias_activation", "fused_matmul_bias_activation", "add"]
+
+
+@pytest.fixture(scope="module")
+def sess():
+    from metalhlo_amd import capi
+    s = capi.Session()
+    yield s
+    s.close()
+
+
+def block_inputs(seed):
+    rng = np.random.default_rng(seed)
+    n = lambda *shape, s=1.0: (s * rng.standard_normal(shape)).astype(np.float32)
+    return [n(B, S, d), 1 + n(d, s=0.1), n(d, s=0.1), n(d, 3 * d, s=d ** -0.5), n(3 * d, s=0.1), n(d, d, s=d ** -0.5), n(d, s=0.1),
+            1 + n(d, s=0.1), n(d, s=0.1), n(d, F, s=d ** -0.5), n(F, s=0.1), n(F, d, s=F ** -0.5), n(d, s=0.1)]
+
+
+def block_oracle(x, g1, b1, wqkv, bqkv, wo, bo, g2, b2, w1, c1, w2, c2):
+    f = lambda a: np.asarray(a, dtype=np.float64)
+    x, g1, b1, wqkv, bqkv, wo, bo, g2, b2, w1, c1, w2, c2 = map(f, (x, g1, b1, wqkv, bqkv, wo, bo, g2, b2, w1, c1, w2, c2))
+    h = oracle.layer_norm(x, g1, b1, 1e-5)
+    qkv = oracle.matmul_bias_act(h.reshape(B * S, d), wqkv, bqkv).reshape(B, S, 3, H, D)
+    q, k, v = (qkv[:, :, i].transpose(0, 2, 1, 3) for i in range(3))
+    o = oracle.attention(q, k, v, scale=D ** -0.5, is_causal=True)
+    o = o.transpose(0, 2, 1, 3).reshape(B * S, d)
+    r1 = x + oracle.matmul_bias_act(o, wo, bo).reshape(B, S, d)
+    h2 = oracle.layer_norm(r1, g2, b2, 1e-5)
+    up = oracle.matmul_bias_act(h2.reshape(B * S, d), w1, c1, "gelu")
+    return r1 + oracle.matmul_bias_act(up, w2, c2).reshape(B, S, d)
+
+
+def test_block_f32_fused_and_as_written(sess, monkeypatch):
+    text = fm.transformer_block(B, S, H, D, F, "f32")
+    ins = block_inputs(11)
+    exp = block_oracle(*ins)
+    fused, plain = sess.compile(text), sess.compile(text, 0)
+    assert sess.ops(fused) == FUSED
+    assert len(sess.ops(plain)) == 93 and not any(o.startswith("fused_") for o in sess.ops(plain))
+    args = [(a, "f32") for a in ins]
+    for exe in (fused, plain):
+        (got,) = sess.run(exe, args)
+        err = np.abs(got.astype(np.float64) - exp)
+        assert np.all(err <= np.maximum(5e-5, 5e-5 * np.abs(exp))), err.max()
+    # the program as written is long enough for graph replay: replays equal the eager run bit for bit
+    monkeypatch.setenv("METALHLO_HIP_GRAPH", "1")
+    graphed = sess.compile(text, 0)
+    bufs = [sess.buffer(a, t) for a, t in args]
+    (want,) = sess.run(plain, args)
+    for i in range(4):
+        assert np.array_equal(run_with(sess, graphed, bufs)[0], want), f"replay {i}"
+    p = sess.plan(graphed)
+    assert p["graph_captures"] == 1 and p["graph_replays"] == 3 and p["arena_bytes"] < p["unshared_bytes"] // 4
+    for b in bufs:
+        sess.lib.mhlo_buffer_destroy(b)
+    for exe in (fused, plain, graphed):
+        sess.lib.mhlo_executable_destroy(exe)
+
+
+def test_block_bf16_fused(sess):
+    text = fm.transformer_block(B, S, H, D, F, "bf16")
+    ins = [oracle.bf16_bits_to_f32(oracle.bf16_round_bits(a)) for a in block_inputs(12)]     # what the kernels see
+    exp = block_oracle(*ins)
+    exe = sess.compile(text)
+    assert sess.ops(exe) == FUSED
+    (got,) = sess.run(exe, [(oracle.bf16_round_bits(a), "bf16") for a in ins])
+    sess.lib.mhlo_executable_destroy(exe)
+    err = np.abs(oracle.bf16_bits_to_f32(got).astype(np.float64) - exp)
+    ok = err <= np.maximum(2e-2, 2e-2 * np.abs(exp))
+    assert ok.mean() >= 0.995 and np.all(err <= np.maximum(6e-2, 6e-2 * np.abs(exp))), (ok.mean(), err.max())

@@ -43,6 +43,17 @@ def test_keepdims_statistics_are_followed(sess):
     assert "fused_softmax" not in ops(sess, M.NOT_SOFTMAX_WRONG_SPREAD)
 
 
+def test_whole_transformer_block_fuses(sess):
+    """A pre-LayerNorm transformer block in plain StableHLO: 93 operations become 26, every
+    LayerNorm, GEMM+bias(+GELU) and the attention core one kernel each."""
+    got = ops(sess, M.transformer_block())
+    assert len(ops(sess, M.transformer_block(), 0)) == 93
+    assert [o for o in got if o.startswith("fused_")] == [
+        "fused_layer_norm", "fused_matmul_bias_activation", "fused_scaled_dot_product_attention", "fused_matmul_bias_activation",
+        "fused_layer_norm", "fused_matmul_bias_activation", "fused_matmul_bias_activation"]
+    assert len(got) == 26 and not {"reduce", "exponential", "tanh", "rsqrt", "dot_general", "divide"} & set(got)
+
+
 def test_gelu_only_with_the_right_constants(sess):
     assert ops(sess, M.GELU) == ["fused_gelu"]
     assert "fused_gelu" not in ops(sess, M.NOT_GELU) and "tanh" in ops(sess, M.NOT_GELU)
