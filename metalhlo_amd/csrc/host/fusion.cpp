@@ -443,6 +443,28 @@ struct Rewriter {
             if (v[i] != (int64_t)i) return false;
         return true;
     }
+    // mask [S, S] = select(compare(key index, query index), ...) over two iotas that keeps (adds 0)
+    // where key <= query and adds -inf (or anything <= -1e30) elsewhere: the kernel's causal flag
+    bool causal_mask(int mask) const {
+        const Op* sel = op_named(mask, "select");
+        if (!sel || sel->operands.size() != 3 || sel->out.shape.size() != 2 || sel->out.shape[0] != sel->out.shape[1]) return false;
+        const Op* cmp = op_named(sel->operands[0], "compare");
+        if (!cmp || cmp->operands.size() != 2 || cmp->out.shape != sel->out.shape) return false;
+        const Op* l = op_named(cmp->operands[0], "iota");
+        const Op* r = op_named(cmp->operands[1], "iota");
+        if (!l || !r || l->out.shape != sel->out.shape || r->out.shape != sel->out.shape || dtype_is_float(l->out.dtype) ||
+            l->out.dtype != r->out.dtype || l->iota_dim + r->iota_dim != 1)
+            return false;
+        // written as <key> DIR <query>: swap the direction when the query index (dim 0) is on the left
+        std::string dir = cmp->direction;
+        if (l->iota_dim == 0) dir = dir == "LE" ? "GE" : dir == "GE" ? "LE" : dir == "LT" ? "GT" : dir == "GT" ? "LT" : dir;
+        const bool pred_keeps = dir == "LE", pred_masks = dir == "GT";
+        if (!pred_keeps && !pred_masks) return false;
+        double keep, drop;
+        if (!splat_value(sel->operands[pred_keeps ? 1 : 2], keep) || !splat_value(sel->operands[pred_keeps ? 2 : 1], drop)) return false;
+        return keep == 0.0 && drop <= -1e30;
+    }
+
     bool attention(size_t ri) {
         const Op& pv = fn.ops[ri];
         if (pv.name != "dot_general" || !dtype_is_float(pv.out.dtype) || pv.out.dtype == F64) return false;
@@ -515,6 +537,12 @@ struct Rewriter {
                 }
             }
         }
+        bool causal = false;
+        if (mask >= 0 && qt.shape[r - 2] == kt.shape[r - 2] && type.at(mask).shape == std::vector<int64_t>{qt.shape[r - 2], kt.shape[r - 2]} &&
+            causal_mask(mask)) {
+            causal = true;      // the mask's producers stay behind for other users and are swept when there are none
+            mask = -1;
+        }
         if (mask >= 0) {                                    // must end in [Sq, Skv] and broadcast over batch / heads
             const TensorType& mt = type.at(mask);
             const size_t mr = mt.shape.size();
@@ -529,7 +557,8 @@ struct Rewriter {
         }
         if (!closed(in, ri)) return false;
         char cfg[128];
-        snprintf(cfg, sizeof cfg, "{\"scale\": %.9g, \"has_mask\": %s, \"is_causal\": false}", scale, mask >= 0 ? "true" : "false");
+        snprintf(cfg, sizeof cfg, "{\"scale\": %.9g, \"has_mask\": %s, \"is_causal\": %s}", scale, mask >= 0 ? "true" : "false",
+                 causal ? "true" : "false");
         std::vector<int> ops = {q, k, v};
         if (mask >= 0) ops.push_back(mask);
         replace(ri, in, "fused_scaled_dot_product_attention", ops, cfg);

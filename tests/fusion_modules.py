@@ -310,3 +310,43 @@ def transformer_block(B=2, S=64, H=4, D=32, F=256, dtype="f32"):
     emit(f"  %res2 = stablehlo.add %res1, {down} : {x3}")
     emit(f"  return %res2 : {x3} }}")
     return "\n".join(L)
+
+
+def masked_attention(form, B=2, H=2, S=64, D=32, dtype="f32"):
+    """Attention whose additive [S, S] mask is built in the program from two iotas.  `form`:
+    "le" keep where key <= query (compare LE key, query); "ge_swapped" the same written GE query, key;
+    "gt_drop" select(key > query, -inf, 0); "big_negative" -1e30 in place of -inf;
+    "anti" keep where key >= query (NOT causal); "keep_one" adds 1 where kept (NOT a pure mask)."""
+    t, st, rt = f"tensor<{B}x{H}x{S}x{D}x{dtype}>", f"tensor<{B}x{H}x{S}x{S}x{dtype}>", f"tensor<{B}x{H}x{S}x{dtype}>"
+    it, mt = f"tensor<{S}x{S}xi32>", f"tensor<{S}x{S}x{dtype}>"
+    neg = {"f32": "0xFF800000", "bf16": "0xFF80", "f16": "0xFC00"}[dtype]
+    cmp_line, sel = {
+        "le": ("LE, %ki, %qi", "%mz, %mn"), "ge_swapped": ("GE, %qi, %ki", "%mz, %mn"), "gt_drop": ("GT, %ki, %qi", "%mn, %mz"),
+        "big_negative": ("LE, %ki, %qi", "%mz, %mn"), "anti": ("GE, %ki, %qi", "%mz, %mn"), "keep_one": ("LE, %ki, %qi", "%mz, %mn"),
+    }[form]
+    drop = "-1.0e30" if form == "big_negative" else neg
+    keep = "1.0" if form == "keep_one" else "0.0"
+    return "\n".join([
+        f"func.func @main(%q: {t}, %k: {t}, %v: {t}) -> {t} {{",
+        f"  %s0 = stablehlo.dot_general %q, %k, batching_dims = [0, 1] x [0, 1], contracting_dims = [3] x [3] : ({t}, {t}) -> {st}",
+        f"  %sc = stablehlo.constant dense<{D ** -0.5!r}> : {st}",
+        f"  %s1 = stablehlo.multiply %s0, %sc : {st}",
+        f"  %qi = stablehlo.iota dim = 0 : {it}",
+        f"  %ki = stablehlo.iota dim = 1 : {it}",
+        f"  %pred = stablehlo.compare {cmp_line}, SIGNED : ({it}, {it}) -> tensor<{S}x{S}xi1>",
+        f"  %mz = stablehlo.constant dense<{keep}> : {mt}",
+        f"  %mn = stablehlo.constant dense<{drop}> : {mt}",
+        f"  %mask = stablehlo.select %pred, {sel} : tensor<{S}x{S}xi1>, {mt}",
+        f"  %mbc = stablehlo.broadcast_in_dim %mask, dims = [2, 3] : ({mt}) -> {st}",
+        f"  %s2 = stablehlo.add %s1, %mbc : {st}",
+        f"  %ninf = stablehlo.constant dense<{neg}> : tensor<{dtype}>",
+        f"  %zero = stablehlo.constant dense<0.0> : tensor<{dtype}>",
+        f"  %m = stablehlo.reduce(%s2 init: %ninf) applies stablehlo.maximum across dimensions = [3] : ({st}, tensor<{dtype}>) -> {rt}",
+        f"  %mb = stablehlo.broadcast_in_dim %m, dims = [0, 1, 2] : ({rt}) -> {st}",
+        f"  %sh = stablehlo.subtract %s2, %mb : {st}",
+        f"  %e = stablehlo.exponential %sh : {st}",
+        f"  %s = stablehlo.reduce(%e init: %zero) applies stablehlo.add across dimensions = [3] : ({st}, tensor<{dtype}>) -> {rt}",
+        f"  %sb = stablehlo.broadcast_in_dim %s, dims = [0, 1, 2] : ({rt}) -> {st}",
+        f"  %p = stablehlo.divide %e, %sb : {st}",
+        f"  %o = stablehlo.dot_general %p, %v, batching_dims = [0, 1] x [0, 1], contracting_dims = [3] x [2] : ({st}, {t}) -> {t}",
+        f"  return %o : {t} }}"])

@@ -1,7 +1,7 @@
 """GPU: one whole pre-LayerNorm transformer block written in plain StableHLO (93 operations, no
 custom calls; tests/fusion_modules.py transformer_block) through mhlo_compile: the pattern
 recogniser turns it into LayerNorm / GEMM+bias(+GELU) / attention kernels plus the head
-split and merge glue (26 operations), and both that and the program run as written agree with
+split and merge glue (20 operations; the causal mask built from iotas becomes the causal flag), and both that and the program run as written agree with
 the float64 oracle of the block.  f32: |got - e| <= max(tol, tol |e|) with tol 5e-5 for the
 whole block (about ten chained operators, each held to 1e-5 on its own); bf16: the
 end-to-end rule used for the GPT-2 logits (99.5 % within 2e-2, worst 6e-2)."""
@@ -19,8 +19,7 @@ pytestmark = pytest.mark.gpu
 B, S, H, D, F = 2, 64, 4, 32, 256
 d = H * D
 FUSED = ["fused_layer_norm", "fused_matmul_bias_activation", "slice", "reshape", "transpose", "slice", "reshape", "transpose",
-         "slice", "reshape", "transpose", "iota", "iota", "compare", "constant", "constant", "select",
-         "fused_scaled_dot_product_attention", "transpose", "reshape", "fused_matmul_bias_activation", "add",
+         "slice", "reshape", "transpose", "fused_scaled_dot_product_attention", "transpose", "reshape", "fused_matmul_bias_activation", "add",
          "fused_layer_norm", "fused_matmul_bias_activation", "fused_matmul_bias_activation", "add"]
 
 

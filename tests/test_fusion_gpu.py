@@ -60,6 +60,22 @@ def test_softmax_gelu_norms(sess):
     close(b, exp, 1e-5)
 
 
+@pytest.mark.parametrize("form", ["le", "ge_swapped", "gt_drop", "big_negative", "anti", "keep_one"])
+def test_masks_built_from_iotas(sess, form):
+    """Causal spellings run with the causal flag, the others with their mask: both must equal the
+    oracle with the mask the program describes, and the program run as written."""
+    B, H, S, D = 2, 2, 64, 32
+    rng = np.random.default_rng(83)
+    q, k, v = (rng.standard_normal((B, H, S, D)).astype(np.float32) for _ in range(3))
+    qi, ki = np.arange(S)[:, None], np.arange(S)[None, :]
+    keep = (ki >= qi) if form == "anti" else (ki <= qi)
+    mask = np.where(keep, 1.0 if form == "keep_one" else 0.0, -1e30 if form == "big_negative" else -np.inf)
+    exp = oracle.attention(q.astype(np.float64), k.astype(np.float64), v.astype(np.float64), scale=D ** -0.5, mask=mask)
+    a, b = both(sess, M.masked_attention(form), [(q, "f32"), (k, "f32"), (v, "f32")], "fused_scaled_dot_product_attention")
+    close(a, exp, 1e-5)
+    close(b, exp, 1e-5)
+
+
 def test_keepdims_forms(sess):
     rng = np.random.default_rng(82)
     x = rng.standard_normal((8, 32)).astype(np.float32)

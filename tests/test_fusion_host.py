@@ -44,14 +44,30 @@ def test_keepdims_statistics_are_followed(sess):
 
 
 def test_whole_transformer_block_fuses(sess):
-    """A pre-LayerNorm transformer block in plain StableHLO: 93 operations become 26, every
-    LayerNorm, GEMM+bias(+GELU) and the attention core one kernel each."""
+    """A pre-LayerNorm transformer block in plain StableHLO: 93 operations become 20, every
+    LayerNorm, GEMM+bias(+GELU) and the attention core one kernel each; the causal mask the
+    program builds from iotas becomes the kernel's causal flag and its operations disappear."""
     got = ops(sess, M.transformer_block())
     assert len(ops(sess, M.transformer_block(), 0)) == 93
     assert [o for o in got if o.startswith("fused_")] == [
         "fused_layer_norm", "fused_matmul_bias_activation", "fused_scaled_dot_product_attention", "fused_matmul_bias_activation",
         "fused_layer_norm", "fused_matmul_bias_activation", "fused_matmul_bias_activation"]
-    assert len(got) == 26 and not {"reduce", "exponential", "tanh", "rsqrt", "dot_general", "divide"} & set(got)
+    assert len(got) == 20 and not {"reduce", "exponential", "tanh", "rsqrt", "dot_general", "divide", "iota", "select"} & set(got)
+
+
+@pytest.mark.parametrize("form,causal", [("le", True), ("ge_swapped", True), ("gt_drop", True), ("big_negative", True),
+                                         ("anti", False), ("keep_one", False)])
+def test_causal_mask_from_iotas_becomes_the_causal_flag(sess, form, causal):
+    """select(compare(iota, iota), 0, -inf) in any of its spellings is the causal flag (no mask
+    operand, no mask operations left); the mirrored comparison or a mask that adds something
+    where it keeps stays an additive mask."""
+    exe = sess.compile(M.masked_attention(form))
+    got = sess.ops(exe)
+    sess.lib.mhlo_executable_destroy(exe)
+    if causal:
+        assert got == ["fused_scaled_dot_product_attention"]
+    else:
+        assert got.count("fused_scaled_dot_product_attention") == 1 and "select" in got and "iota" in got
 
 
 def test_gelu_only_with_the_right_constants(sess):
