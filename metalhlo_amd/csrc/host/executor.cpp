@@ -602,6 +602,46 @@ static std::vector<DeviceTensor> run_ops(Executable& exe, const std::vector<Devi
                     if (bias && (in(2).type.numel() != N || in(2).type.dtype != dt)) throw ExecError(where(op) + "bias must be [N] of the input type");
                     RUN(mhip_gemm(s, in(0).data(), in(1).data(), bias, out.data(), M, N, K, 1, 0, 0, 0, ta, tb,
                                     kActivation.at(cfg.get_string("activation", "none")), dt));
+                } else if (!cfg.get_int_array("views", {}).empty()) {   // attention reading / writing views in place
+                    const auto dims = cfg.get_int_array("dims", {});
+                    const auto vw = cfg.get_int_array("views", {});
+                    if (dims.size() != 5 || vw.size() != 16) throw ExecError(where(op) + "views need dims [B,H,Sq,Skv,D] and 16 view entries");
+                    const int64_t B = dims[0], H = dims[1], Sq = dims[2], Skv = dims[3], D = dims[4];
+                    const int64_t es = dtype_bytes(dt);
+                    // every view must stay inside the tensor it is a window of
+                    const int64_t rows[4] = {Sq, Skv, Skv, Sq};
+                    const int64_t have[4] = {in(0).type.numel(), in(1).type.numel(), in(2).type.numel(), op.out.numel()};
+                    int64_t strides[12];
+                    for (int t = 0; t < 4; t++) {
+                        const int64_t off = vw[4 * t], sb = vw[4 * t + 1], sh = vw[4 * t + 2], sr = vw[4 * t + 3];
+                        if (off < 0 || sb < 0 || sh < 0 || sr < D ||
+                            off + (B - 1) * sb + (H - 1) * sh + (rows[t] - 1) * sr + D > have[t])
+                            throw ExecError(where(op) + "a view reaches outside its tensor");
+                        strides[3 * t] = sb; strides[3 * t + 1] = sh; strides[3 * t + 2] = sr;
+                    }
+                    if (in(0).type.dtype != dt || in(1).type.dtype != dt || in(2).type.dtype != dt)
+                        throw ExecError(where(op) + "q, k, v and the result must have one element type");
+                    const bool has_mask = cfg.get_bool("has_mask", false) && op.operands.size() > 3;
+                    const void* mask = nullptr;
+                    int64_t msb = 0, msh = 0;
+                    if (has_mask) {
+                        const TensorType& mt = in(3).type;
+                        const size_t mr = mt.shape.size();
+                        if (mr < 2 || mt.shape[mr - 1] != Skv || mt.shape[mr - 2] != Sq || mt.dtype != dt)
+                            throw ExecError(where(op) + "mask must end in [Sq, Skv] and have the input type");
+                        const int64_t mh = mr >= 3 ? mt.shape[mr - 3] : 1;
+                        int64_t mb = 1;
+                        for (size_t d = 0; d + 3 < mr; d++) mb *= mt.shape[d];
+                        if ((mh != 1 && mh != H) || (mb != 1 && mb != B)) throw ExecError(where(op) + "mask does not broadcast to [B, H, Sq, Skv]");
+                        msh = mh == H && H != 1 ? Sq * Skv : 0;
+                        msb = mb == B && B != 1 ? mh * Sq * Skv : 0;
+                        mask = in(3).data();
+                    }
+                    auto at = [&](const void* p, int64_t off) { return static_cast<const char*>(p) + off * es; };
+                    RUN(mhip_flash_attention_strided(s, at(in(0).data(), vw[0]), at(in(1).data(), vw[4]), at(in(2).data(), vw[8]), mask,
+                                                     const_cast<char*>(at(out.data(), vw[12])), B, H, Sq, Skv, D,
+                                                     (float)cfg.get_float("scale", 1.0), cfg.get_bool("is_causal", false), msb, msh, dt,
+                                                     strides));
                 } else {   // fused_scaled_dot_product_attention
                     const TensorType& kt = in(1).type;
                     if (xt.shape.size() < 2 || kt.shape.size() != xt.shape.size() || !(in(2).type == kt) || kt.dtype != dt)

@@ -565,6 +565,89 @@ struct Rewriter {
         return true;
     }
 
+    // ------------------------------------------------------------------ attention on views
+    // A [B,H,S,D] operand that is only a re-arranged window of a [B,S,W] tensor --
+    // transpose{0,2,1,3}(reshape [B,S,H*D] -> [B,S,H,D] (slice [:, :, off : off + H*D] (t))), the
+    // slice optional -- is read in place: element (b,h,s,d) lies at off + b*S*W + s*W + h*D + d.
+    struct View { int src; int64_t off, sb, sh, sr; };
+    bool head_view(int v, View& out) const {
+        const Op* t = op_named(v, "transpose");
+        if (!t || t->dims != std::vector<int64_t>{0, 2, 1, 3}) return false;
+        const Op* r = op_named(t->operands[0], "reshape");
+        if (!r || r->out.shape.size() != 4) return false;
+        const int64_t B = r->out.shape[0], S = r->out.shape[1], H = r->out.shape[2], D = r->out.shape[3];
+        const TensorType& rt = type.at(r->operands[0]);
+        if (rt.shape != std::vector<int64_t>{B, S, H * D}) return false;
+        out = View{r->operands[0], 0, S * H * D, D, H * D};
+        if (const Op* sl = op_named(r->operands[0], "slice")) {
+            const TensorType& bt = type.at(sl->operands[0]);
+            if (bt.shape.size() == 3 && sl->strides == std::vector<int64_t>{1, 1, 1} && sl->starts[0] == 0 && sl->starts[1] == 0 &&
+                sl->limits[0] == B && sl->limits[1] == S && bt.shape[0] == B && bt.shape[1] == S) {
+                const int64_t W = bt.shape[2];
+                out = View{sl->operands[0], sl->starts[2], S * W, D, W};
+            }
+        }
+        return out.off % 8 == 0 && out.sr % 8 == 0 && out.sb % 8 == 0;
+    }
+    // Rewrites a fused attention whose operands (or whose only consumer) are such views to read
+    // (write) them in place: the config gains "dims" [B,H,Sq,Skv,D] and "views" = {offset, batch,
+    // head, row strides} x {q, k, v, o}; the glue operations lose their users and are swept.
+    bool attention_views(size_t ri) {
+        Op& at = fn.ops[ri];
+        if (at.name != "custom_call" || at.target != "fused_scaled_dot_product_attention" || at.out.shape.size() != 4) return false;
+        if (at.out.dtype != BF16 && at.out.dtype != F16) return false;
+        const Config cfg = parse_config(at.backend_config);
+        if (!cfg.get_int_array("views", {}).empty()) return false;
+        const TensorType qt = type.at(at.operands[0]), kt = type.at(at.operands[1]);
+        const int64_t B = qt.shape[0], H = qt.shape[1], Sq = qt.shape[2], D = qt.shape[3], Skv = kt.shape[2];
+        if (D != 64 && D != 128) return false;
+        View views[4];
+        bool any = false;
+        for (int i = 0; i < 3; i++) {
+            const int64_t S = i == 0 ? Sq : Skv;
+            views[i] = View{at.operands[i], 0, H * S * D, S * D, D};          // packed [B,H,S,D]
+            View w;
+            if (head_view(at.operands[i], w)) { views[i] = w; any = true; }
+        }
+        // the result: written as [B,S,H,D] when its only use is the head merge
+        views[3] = View{-1, 0, H * Sq * D, Sq * D, D};
+        size_t root = ri;
+        const Op* tr = nullptr;
+        const Op* rs = nullptr;
+        if (uses(at.result) == 1) {
+            for (size_t i = 0; i < fn.ops.size() && !tr; i++)
+                if (!dead[i] && fn.ops[i].name == "transpose" && fn.ops[i].operands[0] == at.result &&
+                    fn.ops[i].dims == std::vector<int64_t>{0, 2, 1, 3})
+                    tr = &fn.ops[i];
+            if (tr && uses(tr->result) == 1)
+                for (size_t i = 0; i < fn.ops.size() && !rs; i++)
+                    if (!dead[i] && fn.ops[i].name == "reshape" && fn.ops[i].operands[0] == tr->result &&
+                        fn.ops[i].out.shape == std::vector<int64_t>{B, Sq, H * D})
+                        rs = &fn.ops[i];
+        }
+        if (rs) {
+            views[3] = View{-1, 0, Sq * H * D, D, H * D};
+            root = index_of(rs);
+            any = true;
+        }
+        if (!any) return false;
+        std::string c;
+        char num[64];
+        snprintf(num, sizeof num, "%.9g", cfg.get_float("scale", 1.0));
+        c = std::string("{\"scale\": ") + num + ", \"has_mask\": " + (cfg.get_bool("has_mask", false) ? "true" : "false") +
+            ", \"is_causal\": " + (cfg.get_bool("is_causal", false) ? "true" : "false") + ", \"dims\": [" + std::to_string(B) + ", " +
+            std::to_string(H) + ", " + std::to_string(Sq) + ", " + std::to_string(Skv) + ", " + std::to_string(D) + "], \"views\": [";
+        for (int i = 0; i < 4; i++)
+            c += std::to_string(views[i].off) + ", " + std::to_string(views[i].sb) + ", " + std::to_string(views[i].sh) + ", " +
+                 std::to_string(views[i].sr) + (i < 3 ? ", " : "]}");
+        std::vector<int> operands = {views[0].src, views[1].src, views[2].src};
+        for (size_t i = 3; i < at.operands.size(); i++) operands.push_back(at.operands[i]);
+        std::set<size_t> interior = {root};
+        if (root != ri) { interior.insert(ri); interior.insert(index_of(tr)); }
+        replace(root, interior, "fused_scaled_dot_product_attention", operands, c);
+        return true;
+    }
+
     // ------------------------------------------------------------------ matmul + bias (+ activation)
     bool plain_matmul(const Op* d) const {
         if (!d || (d->name != "dot" && d->name != "dot_general") || d->operands.size() != 2) return false;
@@ -658,6 +741,7 @@ int fuse_patterns(Function& fn) {
     Rewriter rw(fn);
     rw.pass([&](size_t i) { rw.softmax(i) || rw.gelu(i) || rw.norm(i); });
     rw.pass([&](size_t i) { rw.attention(i) || rw.matmul_bias_act(i); });
+    rw.pass([&](size_t i) { rw.attention_views(i); });
     return rw.fused;
 }
 

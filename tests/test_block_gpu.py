@@ -38,18 +38,22 @@ def block_inputs(seed):
             1 + n(d, s=0.1), n(d, s=0.1), n(d, F, s=d ** -0.5), n(F, s=0.1), n(F, d, s=F ** -0.5), n(d, s=0.1)]
 
 
-def block_oracle(x, g1, b1, wqkv, bqkv, wo, bo, g2, b2, w1, c1, w2, c2):
-    f = lambda a: np.asarray(a, dtype=np.float64)
-    x, g1, b1, wqkv, bqkv, wo, bo, g2, b2, w1, c1, w2, c2 = map(f, (x, g1, b1, wqkv, bqkv, wo, bo, g2, b2, w1, c1, w2, c2))
+def block_oracle_d(ins, Dh):
+    x, g1, b1, wqkv, bqkv, wo, bo, g2, b2, w1, c1, w2, c2 = (np.asarray(a, dtype=np.float64) for a in ins)
+    dd = H * Dh
     h = oracle.layer_norm(x, g1, b1, 1e-5)
-    qkv = oracle.matmul_bias_act(h.reshape(B * S, d), wqkv, bqkv).reshape(B, S, 3, H, D)
+    qkv = oracle.matmul_bias_act(h.reshape(B * S, dd), wqkv, bqkv).reshape(B, S, 3, H, Dh)
     q, k, v = (qkv[:, :, i].transpose(0, 2, 1, 3) for i in range(3))
-    o = oracle.attention(q, k, v, scale=D ** -0.5, is_causal=True)
-    o = o.transpose(0, 2, 1, 3).reshape(B * S, d)
-    r1 = x + oracle.matmul_bias_act(o, wo, bo).reshape(B, S, d)
+    o = oracle.attention(q, k, v, scale=Dh ** -0.5, is_causal=True)
+    o = o.transpose(0, 2, 1, 3).reshape(B * S, dd)
+    r1 = x + oracle.matmul_bias_act(o, wo, bo).reshape(B, S, dd)
     h2 = oracle.layer_norm(r1, g2, b2, 1e-5)
-    up = oracle.matmul_bias_act(h2.reshape(B * S, d), w1, c1, "gelu")
-    return r1 + oracle.matmul_bias_act(up, w2, c2).reshape(B, S, d)
+    up = oracle.matmul_bias_act(h2.reshape(B * S, dd), w1, c1, "gelu")
+    return r1 + oracle.matmul_bias_act(up, w2, c2).reshape(B, S, dd)
+
+
+def block_oracle(*ins):
+    return block_oracle_d(ins, D)
 
 
 def test_block_f32_fused_and_as_written(sess, monkeypatch):
@@ -88,5 +92,40 @@ def test_block_bf16_fused(sess):
     (got,) = sess.run(exe, [(oracle.bf16_round_bits(a), "bf16") for a in ins])
     sess.lib.mhlo_executable_destroy(exe)
     err = np.abs(oracle.bf16_bits_to_f32(got).astype(np.float64) - exp)
+    ok = err <= np.maximum(2e-2, 2e-2 * np.abs(exp))
+    assert ok.mean() >= 0.995 and np.all(err <= np.maximum(6e-2, 6e-2 * np.abs(exp))), (ok.mean(), err.max())
+
+
+def test_block_bf16_attention_reads_the_projection_in_place(sess):
+    """With a 16-bit type and D = 64 the head split (slice / reshape / transpose of the fused QKV
+    projection) and the head merge are not run at all: attention reads its operands as strided
+    views of the projection and writes [B,S,H,D] directly.  Nine operations remain, and the
+    result equals the one with the glue materialised (same kernels, same order of arithmetic)."""
+    Dh = 64
+    text = fm.transformer_block(B, S, H, Dh, F, "bf16")
+    rng = np.random.default_rng(13)
+    dd = H * Dh
+    n = lambda *shape, s=1.0: oracle.bf16_round_bits((s * rng.standard_normal(shape)).astype(np.float32))
+    ins = [n(B, S, dd), n(dd, s=0.1), n(dd, s=0.1), n(dd, 3 * dd, s=dd ** -0.5), n(3 * dd, s=0.1), n(dd, dd, s=dd ** -0.5), n(dd, s=0.1),
+           n(dd, s=0.1), n(dd, s=0.1), n(dd, F, s=dd ** -0.5), n(F, s=0.1), n(F, dd, s=F ** -0.5), n(dd, s=0.1)]
+    ins[1] = oracle.bf16_round_bits(1 + oracle.bf16_bits_to_f32(ins[1]))
+    ins[7] = oracle.bf16_round_bits(1 + oracle.bf16_bits_to_f32(ins[7]))
+    args = [(a, "bf16") for a in ins]
+    fused, plain = sess.compile(text), sess.compile(text, 0)
+    assert sess.ops(fused) == ["fused_layer_norm", "fused_matmul_bias_activation", "fused_scaled_dot_product_attention",
+                               "fused_matmul_bias_activation", "add", "fused_layer_norm", "fused_matmul_bias_activation",
+                               "fused_matmul_bias_activation", "add"]
+    (a,), (b,) = sess.run(fused, args), sess.run(plain, args)
+    sess.lib.mhlo_executable_destroy(fused)
+    sess.lib.mhlo_executable_destroy(plain)
+    fa, fb = oracle.bf16_bits_to_f32(a).astype(np.float64), oracle.bf16_bits_to_f32(b).astype(np.float64)
+    # against the program run operation by operation (bf16 after every one of its 93 operations)
+    err = np.abs(fa - fb)
+    ok = err <= np.maximum(2e-2, 2e-2 * np.abs(fb))
+    assert ok.mean() >= 0.995 and np.all(err <= np.maximum(6e-2, 6e-2 * np.abs(fb))), (ok.mean(), err.max())
+    # against the float64 oracle of the block
+    f = [oracle.bf16_bits_to_f32(x) for x in ins]
+    exp = block_oracle_d(f, Dh)
+    err = np.abs(fa - exp)
     ok = err <= np.maximum(2e-2, 2e-2 * np.abs(exp))
     assert ok.mean() >= 0.995 and np.all(err <= np.maximum(6e-2, 6e-2 * np.abs(exp))), (ok.mean(), err.max())

@@ -55,6 +55,29 @@ def test_whole_transformer_block_fuses(sess):
     assert len(got) == 20 and not {"reduce", "exponential", "tanh", "rsqrt", "dot_general", "divide", "iota", "select"} & set(got)
 
 
+def test_attention_reads_views_of_the_projection(sess):
+    """16-bit types with D = 64 / 128: the head split and merge around attention are folded into
+    strides (nine operations left); f32 or D = 32 keep the glue (the strided entry is 16-bit MFMA only)."""
+    got = ops(sess, M.transformer_block(2, 64, 4, 64, 256, "bf16"))
+    assert got == ["fused_layer_norm", "fused_matmul_bias_activation", "fused_scaled_dot_product_attention",
+                   "fused_matmul_bias_activation", "add", "fused_layer_norm", "fused_matmul_bias_activation",
+                   "fused_matmul_bias_activation", "add"]
+    assert len(ops(sess, M.transformer_block(2, 64, 4, 64, 256, "f32"))) == 20
+    assert len(ops(sess, M.transformer_block(2, 64, 4, 32, 256, "bf16"))) == 20
+
+
+def test_views_leave_glue_that_has_other_users(sess):
+    """The split tensors are also results of the function here: they must still be produced, while
+    attention reads the projection in place all the same."""
+    text = M.transformer_block(2, 64, 4, 64, 256, "bf16")
+    hs = "tensor<2x4x64x64xbf16>"
+    text = text.replace(") -> tensor<2x64x256xbf16> {", f") -> (tensor<2x64x256xbf16>, {hs}) {{")
+    text = text.replace("return %res2 : tensor<2x64x256xbf16>", f"return %res2, %kh : tensor<2x64x256xbf16>, {hs}")
+    got = ops(sess, text)
+    assert got.count("transpose") == 1 and got.count("slice") == 1 and got.count("fused_scaled_dot_product_attention") == 1
+    assert len(got) == 12
+
+
 @pytest.mark.parametrize("form,causal", [("le", True), ("ge_swapped", True), ("gt_drop", True), ("big_negative", True),
                                          ("anti", False), ("keep_one", False)])
 def test_causal_mask_from_iotas_becomes_the_causal_flag(sess, form, causal):
