@@ -598,10 +598,16 @@ static std::vector<DeviceTensor> run_ops(Executable& exe, const std::vector<Devi
                     const int64_t K = ta ? xt.shape[0] : cols, M = ta ? xt.shape[1] : rows;
                     const int64_t Kb = tb ? wt.shape[1] : wt.shape[0], N = tb ? wt.shape[0] : wt.shape[1];
                     if (K != Kb || op.out.numel() != M * N) throw ExecError(where(op) + "operand shapes do not contract");
-                    const void* bias = op.operands.size() > 2 ? in(2).data() : nullptr;
+                    // operands: x, w, [bias], [residual, when the config says "has_residual"]
+                    const bool has_res = cfg.get_bool("has_residual", false);
+                    const size_t n_plain = op.operands.size() - (has_res ? 1 : 0);
+                    if (has_res && op.operands.size() < 3) throw ExecError(where(op) + "has_residual without a residual operand");
+                    const void* bias = n_plain > 2 ? in(2).data() : nullptr;
                     if (bias && (in(2).type.numel() != N || in(2).type.dtype != dt)) throw ExecError(where(op) + "bias must be [N] of the input type");
-                    RUN(mhip_gemm(s, in(0).data(), in(1).data(), bias, out.data(), M, N, K, 1, 0, 0, 0, ta, tb,
-                                    kActivation.at(cfg.get_string("activation", "none")), dt));
+                    const DeviceTensor* res = has_res ? &in(op.operands.size() - 1) : nullptr;
+                    if (res && !(res->type == op.out)) throw ExecError(where(op) + "the residual must have the result's type");
+                    RUN(mhip_gemm_residual(s, in(0).data(), in(1).data(), bias, res ? res->data() : nullptr, out.data(), M, N, K, 1, 0, 0, 0,
+                                           ta, tb, kActivation.at(cfg.get_string("activation", "none")), dt));
                 } else if (!cfg.get_int_array("views", {}).empty()) {   // attention reading / writing views in place
                     const auto dims = cfg.get_int_array("dims", {});
                     const auto vw = cfg.get_int_array("views", {});

@@ -699,6 +699,29 @@ struct Rewriter {
         return false;
     }
 
+    // add(r, fused_matmul_bias_activation(x, w, bias)) with the product used nowhere else: the
+    // residual goes into the GEMM epilogue (last operand, "has_residual"); the kernel adds it after
+    // rounding the product, so the bits are those of the separate add
+    bool matmul_residual(size_t ri) {
+        const Op& root = fn.ops[ri];
+        if (root.name != "add" || !dtype_is_float(root.out.dtype) || root.out.dtype == F64) return false;
+        for (int k = 0; k < 2; k++) {
+            const Op* mm = op_named(root.operands[k], "custom_call");
+            if (!mm || mm->target != "fused_matmul_bias_activation" || mm->operands.size() != 3 || uses(mm->result) != 1) continue;
+            if (parse_config(mm->backend_config).get_bool("has_residual", false)) continue;
+            const int r = root.operands[1 - k];
+            if (!(type.at(r) == root.out) || !(mm->out == root.out)) continue;
+            std::string cfg = mm->backend_config;
+            const size_t close = cfg.rfind('}');
+            if (close == std::string::npos) continue;
+            cfg = cfg.substr(0, close) + ", \"has_residual\": true}";
+            const std::vector<int> ops = {mm->operands[0], mm->operands[1], mm->operands[2], r};
+            replace(ri, {ri, index_of(mm)}, "fused_matmul_bias_activation", ops, cfg);
+            return true;
+        }
+        return false;
+    }
+
     // drop rewritten ops and everything that has become unused
     void sweep() {
         bool changed = true;
@@ -741,7 +764,7 @@ int fuse_patterns(Function& fn) {
     Rewriter rw(fn);
     rw.pass([&](size_t i) { rw.softmax(i) || rw.gelu(i) || rw.norm(i); });
     rw.pass([&](size_t i) { rw.attention(i) || rw.matmul_bias_act(i); });
-    rw.pass([&](size_t i) { rw.attention_views(i); });
+    rw.pass([&](size_t i) { rw.attention_views(i) || rw.matmul_residual(i); });
     return rw.fused;
 }
 

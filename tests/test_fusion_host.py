@@ -44,26 +44,38 @@ def test_keepdims_statistics_are_followed(sess):
 
 
 def test_whole_transformer_block_fuses(sess):
-    """A pre-LayerNorm transformer block in plain StableHLO: 93 operations become 20, every
+    """A pre-LayerNorm transformer block in plain StableHLO: 93 operations become 18, every
     LayerNorm, GEMM+bias(+GELU) and the attention core one kernel each; the causal mask the
-    program builds from iotas becomes the kernel's causal flag and its operations disappear."""
+    program builds from iotas becomes the kernel's causal flag and its operations disappear; the
+    two residual adds go into the epilogues of the GEMMs in front of them."""
     got = ops(sess, M.transformer_block())
     assert len(ops(sess, M.transformer_block(), 0)) == 93
     assert [o for o in got if o.startswith("fused_")] == [
         "fused_layer_norm", "fused_matmul_bias_activation", "fused_scaled_dot_product_attention", "fused_matmul_bias_activation",
         "fused_layer_norm", "fused_matmul_bias_activation", "fused_matmul_bias_activation"]
-    assert len(got) == 20 and not {"reduce", "exponential", "tanh", "rsqrt", "dot_general", "divide", "iota", "select"} & set(got)
+    assert len(got) == 18 and not {"reduce", "exponential", "tanh", "rsqrt", "dot_general", "divide", "iota", "select", "add"} & set(got)
 
 
 def test_attention_reads_views_of_the_projection(sess):
     """16-bit types with D = 64 / 128: the head split and merge around attention are folded into
-    strides (nine operations left); f32 or D = 32 keep the glue (the strided entry is 16-bit MFMA only)."""
+    strides (seven operations left, one kernel each); f32 or D = 32 keep the glue (the strided entry is 16-bit MFMA only)."""
     got = ops(sess, M.transformer_block(2, 64, 4, 64, 256, "bf16"))
     assert got == ["fused_layer_norm", "fused_matmul_bias_activation", "fused_scaled_dot_product_attention",
-                   "fused_matmul_bias_activation", "add", "fused_layer_norm", "fused_matmul_bias_activation",
-                   "fused_matmul_bias_activation", "add"]
-    assert len(ops(sess, M.transformer_block(2, 64, 4, 64, 256, "f32"))) == 20
-    assert len(ops(sess, M.transformer_block(2, 64, 4, 32, 256, "bf16"))) == 20
+                   "fused_matmul_bias_activation", "fused_layer_norm", "fused_matmul_bias_activation",
+                   "fused_matmul_bias_activation"]
+    assert len(ops(sess, M.transformer_block(2, 64, 4, 64, 256, "f32"))) == 18
+    assert len(ops(sess, M.transformer_block(2, 64, 4, 32, 256, "bf16"))) == 18
+
+
+def test_residual_goes_into_the_gemm_epilogue_only_when_the_product_has_no_other_user(sess):
+    t = "tensor<32x128xf32>"
+    head = (f"func.func @main(%x: tensor<32x64xf32>, %w: tensor<64x128xf32>, %b: tensor<128xf32>, %r: {t}) -> RESULT {{\n"
+            f"  %d = stablehlo.dot_general %x, %w, contracting_dims = [1] x [0] : (tensor<32x64xf32>, tensor<64x128xf32>) -> {t}\n"
+            f"  %bb = stablehlo.broadcast_in_dim %b, dims = [1] : (tensor<128xf32>) -> {t}\n"
+            f"  %h = stablehlo.add %d, %bb : {t}\n  %y = stablehlo.add %r, %h : {t}\n")
+    assert ops(sess, head.replace("RESULT", t) + f"  return %y : {t} }}") == ["fused_matmul_bias_activation"]
+    both = head.replace("RESULT", f"({t}, {t})") + f"  return %y, %h : {t}, {t} }}"
+    assert ops(sess, both) == ["fused_matmul_bias_activation", "add"]
 
 
 def test_views_leave_glue_that_has_other_users(sess):
@@ -75,7 +87,7 @@ def test_views_leave_glue_that_has_other_users(sess):
     text = text.replace("return %res2 : tensor<2x64x256xbf16>", f"return %res2, %kh : tensor<2x64x256xbf16>, {hs}")
     got = ops(sess, text)
     assert got.count("transpose") == 1 and got.count("slice") == 1 and got.count("fused_scaled_dot_product_attention") == 1
-    assert len(got) == 12
+    assert len(got) == 10
 
 
 @pytest.mark.parametrize("form,causal", [("le", True), ("ge_swapped", True), ("gt_drop", True), ("big_negative", True),
