@@ -350,3 +350,61 @@ def masked_attention(form, B=2, H=2, S=64, D=32, dtype="f32"):
         f"  %p = stablehlo.divide %e, %sb : {st}",
         f"  %o = stablehlo.dot_general %p, %v, batching_dims = [0, 1] x [0, 1], contracting_dims = [3] x [2] : ({st}, {t}) -> {t}",
         f"  return %o : {t} }}"])
+
+
+GPT2_LAYER_PARAMS = ["ln1_g", "ln1_b", "w_qkv", "b_qkv", "w_o", "b_o", "ln2_g", "ln2_b", "w_fc", "b_fc", "w_proj", "b_proj"]
+
+
+def gpt2_program(B, S, n_layer, H, D, F, vocab, n_pos, dtype="bf16"):
+    """A whole pre-LayerNorm GPT-2 forward in plain StableHLO with fp32 parameters converted to the
+    compute type where they are used: token gather + learned positions, `n_layer` blocks as
+    transformer_block writes them, final LayerNorm, logits against the tied embedding.
+    Arguments: ids [B,S] i32, wte [vocab,d], wpe [n_pos,d], then per layer the twelve tensors of
+    GPT2_LAYER_PARAMS, then lnf_g, lnf_b (all f32).  Result: logits [B,S,vocab] in `dtype`."""
+    import re
+    d, e = H * D, dtype
+    x3, x3f = f"tensor<{B}x{S}x{d}x{e}>", f"tensor<{B}x{S}x{d}xf32>"
+    shapes = {"ln1_g": [d], "ln1_b": [d], "w_qkv": [d, 3 * d], "b_qkv": [3 * d], "w_o": [d, d], "b_o": [d], "ln2_g": [d], "ln2_b": [d],
+              "w_fc": [d, F], "b_fc": [F], "w_proj": [F, d], "b_proj": [d]}
+    tt = lambda shape, et: "tensor<" + "".join(f"{n}x" for n in shape) + et + ">"
+    args = [f"%ids: tensor<{B}x{S}xi32>", f"%wte: {tt([vocab, d], 'f32')}", f"%wpe: {tt([n_pos, d], 'f32')}"]
+    for i in range(n_layer):
+        args += [f"%p{i}_{n}: {tt(shapes[n], 'f32')}" for n in GPT2_LAYER_PARAMS]
+    args += [f"%lnf_g: {tt([d], 'f32')}", f"%lnf_b: {tt([d], 'f32')}"]
+    out_t = tt([B, S, vocab], e)
+    L = [f"func.func @main({', '.join(args)}) -> {out_t} {{", f"  %zero = stablehlo.constant dense<0.0> : tensor<{e}>"]
+    L.append(f'  %tok = "stablehlo.gather"(%wte, %ids) {{ dimension_numbers = #stablehlo.gather<offset_dims = [2], collapsed_slice_dims = [0], '
+             f'start_index_map = [0], index_vector_dim = 2>, slice_sizes = array<i64: 1, {d}>, indices_are_sorted = false }} '
+             f': ({tt([vocab, d], "f32")}, tensor<{B}x{S}xi32>) -> {x3f}')
+    L.append(f"  %pos = stablehlo.slice %wpe [0:{S}, 0:{d}] : ({tt([n_pos, d], 'f32')}) -> {tt([S, d], 'f32')}")
+    L.append(f"  %posb = stablehlo.broadcast_in_dim %pos, dims = [1, 2] : ({tt([S, d], 'f32')}) -> {x3f}")
+    L.append(f"  %emb = stablehlo.add %tok, %posb : {x3f}")
+    L.append(f"  %h0 = stablehlo.convert %emb : ({x3f}) -> {x3}")
+    block = transformer_block(B, S, H, D, F, e).split("\n")[2:-1]          # without the signature, %zero and the return
+    arg_of = dict(zip(["g1", "b1", "wqkv", "bqkv", "wo", "bo", "g2", "b2", "w1", "c1", "w2", "c2"], GPT2_LAYER_PARAMS))
+    cur = "%h0"
+    for i in range(n_layer):
+        for n in GPT2_LAYER_PARAMS:
+            L.append(f"  %c{i}_{n} = stablehlo.convert %p{i}_{n} : ({tt(shapes[n], 'f32')}) -> {tt(shapes[n], e)}")
+
+        def rename(m, i=i, cur=cur):
+            name = m.group(1)
+            if name == "zero":
+                return "%zero"
+            if name == "x":
+                return cur
+            if name in arg_of:
+                return f"%c{i}_{arg_of[name]}"
+            return f"%L{i}_{name}"
+        L += [re.sub(r"%([A-Za-z0-9_]+)", rename, ln) for ln in block]
+        cur = f"%L{i}_res2"
+    # final LayerNorm: the block's own spelling, on the last residual stream
+    ln = transformer_block(B, S, H, D, F, e).split("\n")[2:19]
+    L.append(f"  %cf_g = stablehlo.convert %lnf_g : ({tt([d], 'f32')}) -> {tt([d], e)}")
+    L.append(f"  %cf_b = stablehlo.convert %lnf_b : ({tt([d], 'f32')}) -> {tt([d], e)}")
+    final = {"x": cur, "g1": "%cf_g", "b1": "%cf_b", "zero": "%zero"}
+    L += [re.sub(r"%([A-Za-z0-9_]+)", lambda m: final.get(m.group(1), f"%F_{m.group(1)}"), l2) for l2 in ln]
+    L.append(f"  %cwte = stablehlo.convert %wte : ({tt([vocab, d], 'f32')}) -> {tt([vocab, d], e)}")
+    L.append(f"  %logits = stablehlo.dot_general %F_ln1o, %cwte, contracting_dims = [2] x [1] : ({x3}, {tt([vocab, d], e)}) -> {out_t}")
+    L.append(f"  return %logits : {out_t} }}")
+    return "\n".join(L)

@@ -9,6 +9,7 @@ import ctypes as C
 
 import numpy as np
 import pytest
+import torch  # noqa: F401  (before the C API library: torch brings its own HIP runtime, and the first one loaded serves the process)
 
 from oracle import oracle
 from tests import fusion_modules as fm
@@ -129,3 +130,39 @@ def test_block_bf16_attention_reads_the_projection_in_place(sess):
     err = np.abs(fa - exp)
     ok = err <= np.maximum(2e-2, 2e-2 * np.abs(exp))
     assert ok.mean() >= 0.995 and np.all(err <= np.maximum(6e-2, 6e-2 * np.abs(exp))), (ok.mean(), err.max())
+
+
+def test_gpt2_program_through_the_c_api(sess):
+    """A whole GPT-2 forward (reduced: 2 layers, d 256, vocab 1000) as one plain StableHLO module with
+    fp32 parameters: compiled by mhlo_compile it runs as gather + per layer twelve parameter
+    converts and the seven fused kernels, and its logits follow the float64 oracle of the model
+    (the end-to-end rule of the bf16 GPT-2 tests) and the hand-written forward of metalhlo_amd.gpt2."""
+    from metalhlo_amd.gpt2 import GPT2, GPT2Config, init_params
+    cfg = GPT2Config(vocab=1000, n_pos=128, d_model=256, n_head=4, n_layer=2, d_ff=1024)
+    Bq, Sq = 2, 64
+    params = init_params(cfg, seed=21)
+    rng = np.random.default_rng(22)
+    for lyr in params["layers"]:                      # non-trivial biases and LayerNorm parameters
+        for name, a in lyr.items():
+            if a.ndim == 1:
+                lyr[name] = (a + 0.05 * rng.standard_normal(a.shape)).astype(np.float32)
+    ids = rng.integers(0, cfg.vocab, (Bq, Sq)).astype(np.int32)
+    text = fm.gpt2_program(Bq, Sq, cfg.n_layer, cfg.n_head, cfg.d_model // cfg.n_head, cfg.d_ff, cfg.vocab, cfg.n_pos)
+    exe = sess.compile(text)
+    ops = sess.ops(exe)
+    assert ops.count("fused_scaled_dot_product_attention") == 2 and ops.count("fused_matmul_bias_activation") == 8
+    assert ops.count("fused_layer_norm") == 5 and not {"reduce", "exponential", "tanh", "transpose", "select"} & set(ops)
+    args = [(ids, "i32"), (params["wte"], "f32"), (params["wpe"], "f32")]
+    for lyr in params["layers"]:
+        args += [(lyr[n], "f32") for n in fm.GPT2_LAYER_PARAMS]
+    args += [(params["lnf_g"], "f32"), (params["lnf_b"], "f32")]
+    (got,) = sess.run(exe, args)
+    sess.lib.mhlo_executable_destroy(exe)
+    got = oracle.bf16_bits_to_f32(got).astype(np.float64)
+    exp = oracle.gpt2_forward(ids, params, cfg.n_head, "bf16")
+    err = np.abs(got - exp)
+    ok = err <= np.maximum(2e-2, 2e-2 * np.abs(exp))
+    assert got.shape == (Bq, Sq, cfg.vocab) and ok.mean() >= 0.995 and np.all(err <= np.maximum(6e-2, 6e-2 * np.abs(exp))), (ok.mean(), err.max())
+    hand = GPT2(cfg, params).forward(torch.from_numpy(ids).cuda()).float().cpu().numpy().astype(np.float64)
+    err = np.abs(got - hand)
+    assert (err <= np.maximum(2e-2, 2e-2 * np.abs(hand))).mean() >= 0.995
