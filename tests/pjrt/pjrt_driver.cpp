@@ -11,6 +11,7 @@
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
+#include <sys/stat.h>
 #include <unistd.h>
 
 #include <atomic>
@@ -242,6 +243,47 @@ static void case_compile(PJRT_Client* c) {
     setenv("METALHLO_PYTHON", "/nonexistent/python", 1);     // no converter: bytecode is refused with a clear message
     CHECK(code_of(compile(c, std::string("ML\xEFR\x01garbage", 12), "mlir", &le), &msg) == PJRT_Error_Code_UNIMPLEMENTED);
     CHECK(msg.find("jaxlib") != std::string::npos);
+    // a converter that answers: the plugin hands it the bytecode in a file (last argument) and
+    // compiles the text it prints.  This stand-in checks the magic of that file and prints a
+    // three-input module, so the executable below can only come from its output.
+    {
+        char path[] = "/tmp/pjrt_fake_converter_XXXXXX";
+        const int fd = mkstemp(path);
+        CHECK(fd >= 0);
+        const char* script =
+            "#!/bin/sh\nfor last; do :; done\n"
+            "[ \"$(head -c 2 \"$last\")\" = ML ] || exit 3\n"
+            "cat <<'EOT'\nmodule @from_bytecode {\n  func.func @main(%a: tensor<4xf32>, %b: tensor<4xf32>, %c: tensor<4xf32>) -> tensor<4xf32> {\n"
+            "    %0 = stablehlo.add %a, %b : tensor<4xf32>\n    %1 = stablehlo.multiply %0, %c : tensor<4xf32>\n"
+            "    return %1 : tensor<4xf32>\n  }\n}\nEOT\n";
+        CHECK(write(fd, script, strlen(script)) == (ssize_t)strlen(script));
+        close(fd);
+        CHECK(chmod(path, 0700) == 0);
+        setenv("METALHLO_PYTHON", path, 1);
+        PJRT_LoadedExecutable* from_bc = nullptr;
+        OK(compile(c, std::string("ML\xEFR\x01garbage", 12), "mlir", &from_bc));
+        ARGS(PJRT_LoadedExecutable_GetExecutable_Args, g2);
+        g2.loaded_executable = from_bc;
+        OK(api->PJRT_LoadedExecutable_GetExecutable(&g2));
+        ARGS(PJRT_Executable_OutputElementTypes_Args, ot);
+        ot.executable = g2.executable;
+        OK(api->PJRT_Executable_OutputElementTypes(&ot));
+        CHECK(ot.num_output_types == 1 && ot.output_types[0] == PJRT_Buffer_Type_F32);
+        ARGS(PJRT_Executable_Serialize_Args, se);
+        se.executable = g2.executable;
+        OK(api->PJRT_Executable_Serialize(&se));
+        CHECK(std::string(se.serialized_bytes, se.serialized_bytes_size).find("@from_bytecode") != std::string::npos);
+        se.serialized_executable_deleter(se.serialized_executable);
+        ARGS(PJRT_Executable_Destroy_Args, de);
+        de.executable = g2.executable;
+        OK(api->PJRT_Executable_Destroy(&de));
+        destroy_loaded(from_bc);
+        // a converter that fails is reported like a missing one
+        unlink(path);
+        setenv("METALHLO_PYTHON", "/bin/false", 1);
+        CHECK(code_of(compile(c, std::string("ML\xEFR\x01garbage", 12), "mlir", &from_bc), &msg) == PJRT_Error_Code_UNIMPLEMENTED);
+        unsetenv("METALHLO_PYTHON");
+    }
     OK(compile(c, kAdd, "mlir", &le));
     CHECK(le != nullptr);
     ARGS(PJRT_LoadedExecutable_GetExecutable_Args, ge);
