@@ -29,6 +29,7 @@ namespace mhip {
 namespace {
 
 constexpr uint32_t kOperBytes = 16 * 1024;   // B tile offset inside a 32 KB stage buffer
+typedef u32x4 u32x4_unaligned __attribute__((aligned(2)));
 
 template <typename F, int... I>
 __device__ inline void static_for_impl(F& f, std::integer_sequence<int, I...>) {
@@ -176,10 +177,14 @@ __global__ __launch_bounds__(256) void gemm256_kernel(GemmArgs g) {
         const int nl = j * 32 + 8 * q + 4 * lhalf;
         const int n = n0 + wn * WN + nl;
         float bv[4] = {0.f, 0.f, 0.f, 0.f};
-        if (bias && n < g.N) {
+        if (bias && n + 4 <= g.N) {
             const Pack4<T> t = __builtin_bit_cast(Pack4<T>, *reinterpret_cast<const u32x2*>(bias + n));
 #pragma unroll
             for (int e = 0; e < 4; e++) bv[e] = Elem<T>::to_f32(t.v[e]);
+        } else if (bias) {                       // the last columns of an N that is no multiple of 4
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                if (n + e < g.N) bv[e] = Elem<T>::to_f32(bias[n + e]);
         }
         static_for<4>([&](auto i_tag) {
             constexpr int i = decltype(i_tag)::value;
@@ -201,15 +206,31 @@ __global__ __launch_bounds__(256) void gemm256_kernel(GemmArgs g) {
     constexpr int kChunks = WN / 8;                      // 16-byte chunks per row of the wave's sub-tile
     constexpr int kRowsPerPass = 64 / kChunks;
     const int cc = lane % kChunks, rr = lane / kChunks;
+    const bool rows_aligned = g.N % 8 == 0;
 #pragma unroll 4
     for (int p = 0; p < 128 / kRowsPerPass; p++) {
         const int ml = p * kRowsPerPass + rr;
         const int m = m0 + wm * 128 + ml;
         const int n = n0 + wn * WN + cc * 8;
-        if (m < g.M && n < g.N) {
+        if (m < g.M && n + 8 <= g.N) {
             u32x4 w = *reinterpret_cast<const u32x4*>(stage + ml * kRowPad + cc * 16);
-            if (res) w = add_chunk<T>(w, *reinterpret_cast<const u32x4*>(res + (int64_t)m * g.N + n));
-            *reinterpret_cast<u32x4*>(c + (int64_t)m * g.N + n) = w;
+            if (rows_aligned) {
+                if (res) w = add_chunk<T>(w, *reinterpret_cast<const u32x4*>(res + (int64_t)m * g.N + n));
+                *reinterpret_cast<u32x4*>(c + (int64_t)m * g.N + n) = w;
+            } else {
+                // N is no multiple of 8: rows of C start at any even byte.  The device takes 16-byte
+                // accesses at such addresses (alignment is not enforced for global memory); the type
+                // says so, so the compiler assumes nothing more.
+                if (res) w = add_chunk<T>(w, *reinterpret_cast<const u32x4_unaligned*>(res + (int64_t)m * g.N + n));
+                *reinterpret_cast<u32x4_unaligned*>(c + (int64_t)m * g.N + n) = w;
+            }
+        } else if (m < g.M && n < g.N) {         // the last, partial chunk of a row
+            const T* sv = reinterpret_cast<const T*>(stage + ml * kRowPad + cc * 16);
+            for (int e = 0; e < g.N - n; e++) {
+                T val = sv[e];
+                if (res) val = Elem<T>::from_f32(Elem<T>::to_f32(val) + Elem<T>::to_f32(res[(int64_t)m * g.N + n + e]));
+                c[(int64_t)m * g.N + n + e] = val;
+            }
         }
     }
 }
@@ -245,13 +266,15 @@ int layout256(hipStream_t s, const GemmArgs& g, int64_t batch, int ta, int tb) {
 }  // namespace
 
 // The kernels need whole K stages, 16-byte-aligned operand rows (checked by the
-// caller), an output they can store 16 bytes at a time, operands small enough for
+// caller), a 16-byte-aligned output (its rows may start anywhere when N is no multiple of 8:
+// they are then stored with unaligned 16-byte accesses), operands small enough for
 // 32-bit byte offsets including the prefetch overrun of five K stages, and enough
 // tiles (256 x `bw`) to occupy the device.
 bool gemm256_eligible(const GemmArgs& g, int64_t batch, int dtype, int bw) {
     if (dtype != MHIP_BF16 && dtype != MHIP_F16) return false;
     if (g.K % 32 != 0 || g.K < 32) return false;
-    if (g.N % 8 != 0 || (reinterpret_cast<uintptr_t>(g.c) & 15) != 0 || g.sc % 8 != 0) return false;
+    if ((reinterpret_cast<uintptr_t>(g.c) & 15) != 0 || (batch > 1 && g.sc % 8 != 0)) return false;
+    if (g.residual && (reinterpret_cast<uintptr_t>(g.residual) & 15) != 0) return false;
     if (g.bias && (reinterpret_cast<uintptr_t>(g.bias) & 7) != 0) return false;
     const int64_t a_bytes = (int64_t)g.M * g.K * 2, b_bytes = (int64_t)g.N * g.K * 2;
     if (a_bytes >= 0x70000000LL || b_bytes >= 0x70000000LL) return false;
