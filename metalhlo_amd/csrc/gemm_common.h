@@ -68,16 +68,21 @@ __device__ inline float apply_act_c(float v) {
     constexpr float kLog2e = 1.4426950408889634f;
     if (ACT == MHIP_ACT_NONE) return v;
     if (ACT == MHIP_ACT_RELU) return fmaxf(v, 0.f);
+    float r = v;
     if (ACT == MHIP_ACT_GELU) {
         constexpr float c0 = -2.f * kLog2e * 0.7978845608028654f;
         constexpr float c1 = c0 * 0.044715f;
         const float t = v * fmaf(v * v, c1, c0);
-        return v * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(t));
+        r = v * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(t));
     }
-    if (ACT == MHIP_ACT_SILU) return v * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-kLog2e * v));
-    if (ACT == MHIP_ACT_SIGMOID) return __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-kLog2e * v));
-    if (ACT == MHIP_ACT_TANH) return 1.f - 2.f * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(2.f * kLog2e * v));
-    return v;
+    if (ACT == MHIP_ACT_SILU) r = v * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-kLog2e * v));
+    if (ACT == MHIP_ACT_SIGMOID) r = __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-kLog2e * v));
+    if (ACT == MHIP_ACT_TANH) r = 1.f - 2.f * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(2.f * kLog2e * v));
+    // The fp32 result is final here.  Without this the compiler may merge the last multiply with
+    // the conversion to f16 that follows (one rounding instead of two) in some kernels and not in
+    // others, and the same problem would round differently depending on the tile choice.
+    asm("" : "+v"(r));
+    return r;
 }
 // eight stored elements (one 16-byte chunk of a C row) plus eight residual elements: each sum
 // is rounded once more, exactly what a separate add kernel over the stored C would produce

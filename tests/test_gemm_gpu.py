@@ -199,20 +199,19 @@ def test_gemm_ring_kernel_rows_of_c_at_any_alignment(tile, dtype, monkeypatch):
         bias = to_dev(rng.standard_normal(N) * 0.5, dtype)
         r = to_dev(rng.standard_normal((M, N)), dtype)
         monkeypatch.setenv("MHIP_GEMM_TILE", tile)
-        c = kernels.matmul(a, b, bias, "relu", trans_a=ta, trans_b=True, residual=r)
+        c = kernels.matmul(a, b, bias, "gelu", trans_a=ta, trans_b=True, residual=r)
         guard = torch.full((M * N + 64,), 7.0, dtype=dtype, device="cuda")
         kernels.matmul(a, b, bias, "gelu", trans_a=ta, trans_b=True, out=guard[:M * N].view(M, N))
         assert torch.all(guard[M * N:] == 7.0)
         monkeypatch.setenv("MHIP_GEMM_TILE", "128")
-        c128 = kernels.matmul(a, b, bias, "relu", trans_a=ta, trans_b=True, residual=r)
+        c128 = kernels.matmul(a, b, bias, "gelu", trans_a=ta, trans_b=True, residual=r)
         assert torch.equal(c, c128), (M, N, K, ta)
         rows = np.unique(np.r_[0, 1, 255, 256, M - 1, rng.integers(0, M, 20)])
         A = as_f64(a).T if ta else as_f64(a)
-        exp = oracle.matmul_bias_act(A[rows], as_f64(b).T, as_f64(bias), "relu")
+        exp = oracle.matmul_bias_act(A[rows], as_f64(b).T, as_f64(bias), "gelu")
+        assert_close(guard[:M * N].view(M, N)[rows], exp, TOL[dtype], f"odd N {(M, N, K)}")
         exp = as_f64(to_dev(exp, dtype).cpu()) + as_f64(r)[rows]                     # product rounded, then the residual added
-        assert_close(c[rows], exp, TOL[dtype], f"odd N {(M, N, K)}")
-        gelu = oracle.matmul_bias_act(A[rows], as_f64(b).T, as_f64(bias), "gelu")
-        assert_close(guard[:M * N].view(M, N)[rows], gelu, TOL[dtype], f"odd N gelu {(M, N, K)}")
+        assert_close(c[rows], exp, TOL[dtype], f"odd N + residual {(M, N, K)}")
 
 
 def test_gemm_large_exact_small_integers():
