@@ -213,6 +213,13 @@ int mhip_add(void* stream, const void* a, const void* b, void* y, int64_t n, int
  * truncates toward zero, int -> int keeps the low bits, anything -> I1 is x != 0. */
 int mhip_convert(void* stream, const void* x, void* y, int64_t n, int src_dtype, int dst_dtype);
 
+/* ys[i] = convert(xs[i]), ns[i] elements each, for `count` tensors in as few launches as the
+ * table allows (96 tensors per launch): the same conversion (CodeGenerator.swift:1012-1078,
+ * round to nearest even) as mhip_convert, for the many small tensors of a model's parameters.
+ * F32 -> BF16 / F16 only; anything else returns 2 and the caller converts one by one. */
+int mhip_convert_batch(void* stream, int count, const void* const* xs, void* const* ys,
+                       const int64_t* ns, int src_dtype, int dst_dtype);
+
 /* [d0,d1,d2,d3] -> [d0,d2,d1,d3] (head split / merge;
  * Compiler/CodeGenerator.swift:2840-3056). Any 2/4-byte type. */
 int mhip_transpose_0213(void* stream, const void* x, void* y, int64_t d0, int64_t d1, int64_t d2,

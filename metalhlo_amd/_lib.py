@@ -37,6 +37,7 @@ SIGNATURES = {
     "mhip_embed_tokens": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32, _i32]),
     "mhip_add": (_i32, [_vp, _vp, _vp, _vp, _i64, _i32]),
     "mhip_convert": (_i32, [_vp, _vp, _vp, _i64, _i32, _i32]),
+    "mhip_convert_batch": (_i32, [_vp, _i32, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_i64), _i32, _i32]),
     "mhip_transpose_0213": (_i32, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32]),
     "mhip_split_qkv_heads": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32]),
     "mhip_iota": (_i32, [_vp, _vp, _i64, _i64, _i64, _i32]),

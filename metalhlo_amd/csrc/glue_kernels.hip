@@ -161,6 +161,47 @@ __global__ __launch_bounds__(256) void narrow_vec_kernel(const float* __restrict
     store16(y + i * 8, o);
 }
 
+// fp32 -> 16-bit float for up to kBatchMax tensors in one launch (a model's parameters: many
+// of them small).  The table travels in the kernel arguments; a workgroup handles 2048
+// consecutive elements of one tensor, which it finds by bisecting the running block counts.
+constexpr int kBatchMax = 96;
+struct ConvertBatch {
+    const float* x[kBatchMax];
+    void* y[kBatchMax];
+    int64_t n[kBatchMax];
+    uint32_t first_block[kBatchMax + 1];
+    int count;
+};
+static_assert(sizeof(ConvertBatch) <= 4000, "the table must fit the kernel argument space");
+
+template <typename D>
+__global__ __launch_bounds__(256) void narrow_batch_kernel(ConvertBatch b) {
+    int lo = 0, hi = b.count - 1;                  // largest t with first_block[t] <= blockIdx.x
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (b.first_block[mid] <= blockIdx.x) lo = mid; else hi = mid - 1;
+    }
+    const float* x = b.x[lo];
+    D* y = static_cast<D*>(b.y[lo]);
+    const int64_t n = b.n[lo];
+    const int64_t i = ((int64_t)(blockIdx.x - b.first_block[lo]) * 256 + threadIdx.x) * 8;
+    if (i >= n) return;
+    const bool vec = i + 8 <= n && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15) == 0;
+    if (vec) {
+        const f32x4 p = *reinterpret_cast<const f32x4*>(x + i);
+        const f32x4 q = *reinterpret_cast<const f32x4*>(x + i + 4);
+        Vec16<D> o;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            o.v[e] = Elem<D>::from_f32(p[e]);
+            o.v[4 + e] = Elem<D>::from_f32(q[e]);
+        }
+        store16(y + i, o);
+    } else {
+        for (int64_t e = i; e < n && e < i + 8; e++) y[e] = Elem<D>::from_f32(x[e]);
+    }
+}
+
 // ---- [d0,d1,d2,d3] -> [d0,d2,d1,d3] ------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void transpose_0213_kernel(const T* __restrict__ x,
@@ -426,6 +467,43 @@ extern "C" int mhip_convert(void* stream, const void* x, void* y, int64_t n, int
         case MHIP_UI64: return convert_from<uint64_t>(s, x, y, n, dst_dtype);
         default: return fail(MHIP_ERR_UNSUPPORTED, "mhip_convert: source dtype %d", src_dtype);
     }
+}
+
+extern "C" int mhip_convert_batch(void* stream, int count, const void* const* xs, void* const* ys,
+                                  const int64_t* ns, int src_dtype, int dst_dtype) {
+    const char* what = "mhip_convert_batch";
+    if (count < 0 || (count > 0 && (!xs || !ys || !ns))) return fail(MHIP_ERR_INVALID_ARGUMENT, "%s: bad table", what);
+    if (src_dtype != MHIP_F32 || (dst_dtype != MHIP_BF16 && dst_dtype != MHIP_F16))
+        return fail(MHIP_ERR_UNSUPPORTED, "%s: f32 -> bf16 / f16 only (got %d -> %d)", what, src_dtype, dst_dtype);
+    hipStream_t s = as_stream(stream);
+    for (int done = 0; done < count;) {
+        ConvertBatch b;
+        b.count = 0;
+        uint64_t blocks = 0;
+        for (; done < count && b.count < kBatchMax; done++) {
+            if (ns[done] < 0) return fail(MHIP_ERR_INVALID_ARGUMENT, "%s: negative size", what);
+            if (ns[done] == 0) continue;
+            if (!xs[done] || !ys[done]) return fail(MHIP_ERR_INVALID_ARGUMENT, "%s: NULL pointer", what);
+            const uint64_t nb = (uint64_t)((ns[done] + 2047) / 2048);
+            if (blocks + nb > 0x7FFFFFFFull) break;           // the rest goes into another launch
+            b.x[b.count] = static_cast<const float*>(xs[done]);
+            b.y[b.count] = ys[done];
+            b.n[b.count] = ns[done];
+            b.first_block[b.count] = (uint32_t)blocks;
+            blocks += nb;
+            b.count++;
+        }
+        if (b.count == 0) {
+            if (done < count) return fail(MHIP_ERR_UNSUPPORTED, "%s: tensor too large for one launch", what);
+            break;
+        }
+        b.first_block[b.count] = (uint32_t)blocks;
+        if (dst_dtype == MHIP_BF16) hipLaunchKernelGGL((narrow_batch_kernel<bf16_t>), dim3((unsigned)blocks), dim3(256), 0, s, b);
+        else hipLaunchKernelGGL((narrow_batch_kernel<f16_t>), dim3((unsigned)blocks), dim3(256), 0, s, b);
+        const int st = check_launch(what);
+        if (st != MHIP_OK) return st;
+    }
+    return MHIP_OK;
 }
 
 extern "C" int mhip_transpose_0213(void* stream, const void* x, void* y, int64_t d0, int64_t d1,

@@ -328,7 +328,43 @@ static double scalar_constant(const Op& c) {
 static void plan_memory(Executable& exe);
 
 // ---------------------------------------------------------------- validation
+// Many programs convert every fp32 parameter to the 16-bit compute type where it is used: a
+// launch per tensor, most of them tiny.  Converts that depend on nothing but an argument are
+// moved to the front and run as one batched launch (mhip_convert_batch); the converted tensors
+// then live for the whole execution.  Only from eight such converts on, and not at level 0.
+static void hoist_parameter_converts(Executable& exe) {
+    Function& fn = exe.fn;
+    exe.batched_converts = 0;
+    if (exe.opt_level < 1) return;
+    std::vector<bool> is_arg(fn.num_values, false);
+    for (int a : fn.arg_ids) is_arg[a] = true;
+    std::vector<TensorType> arg_type(fn.num_values);
+    for (size_t i = 0; i < fn.arg_ids.size(); i++) arg_type[fn.arg_ids[i]] = fn.arg_types[i];
+    int dst = -1;
+    std::vector<size_t> picked;
+    for (size_t i = 0; i < fn.ops.size(); i++) {
+        const Op& op = fn.ops[i];
+        if (op.name != "convert" || op.operands.size() != 1 || !is_arg[op.operands[0]]) continue;
+        if (arg_type[op.operands[0]].dtype != F32 || (op.out.dtype != BF16 && op.out.dtype != F16)) continue;
+        if (arg_type[op.operands[0]].shape != op.out.shape) continue;
+        if (dst < 0) dst = op.out.dtype;
+        if (op.out.dtype != dst) continue;
+        picked.push_back(i);
+    }
+    if (picked.size() < 8) return;
+    std::vector<Op> front, rest;
+    size_t k = 0;
+    for (size_t i = 0; i < fn.ops.size(); i++) {
+        if (k < picked.size() && picked[k] == i) { front.push_back(std::move(fn.ops[i])); k++; }
+        else rest.push_back(std::move(fn.ops[i]));
+    }
+    exe.batched_converts = front.size();
+    front.insert(front.end(), std::make_move_iterator(rest.begin()), std::make_move_iterator(rest.end()));
+    fn.ops = std::move(front);
+}
+
 void compile(Executable& exe) {
+    hoist_parameter_converts(exe);
     Function& fn = exe.fn;
     std::vector<TensorType> vt = value_types(fn);
     std::map<int, const Op*> producer;
@@ -468,7 +504,22 @@ static std::vector<DeviceTensor> run_ops(Executable& exe, const std::vector<Devi
     std::map<int, const Op*> producer;
     for (auto& op : fn.ops) producer[op.result] = &op;
 
-    for (size_t oi = 0; oi < fn.ops.size(); oi++) {
+    if (exe.batched_converts) {            // the parameter converts at the head of the program, one launch
+        std::vector<const void*> xs;
+        std::vector<void*> ys;
+        std::vector<int64_t> ns;
+        for (size_t oi = 0; oi < exe.batched_converts; oi++) {
+            const Op& op = fn.ops[oi];
+            DeviceTensor out = al.allocate(op.out);
+            xs.push_back(val[op.operands[0]].data());
+            ys.push_back(out.data());
+            ns.push_back(op.out.numel());
+            val[op.result] = out;
+        }
+        const Op& op = fn.ops[0];
+        RUN(mhip_convert_batch(s, (int)xs.size(), xs.data(), ys.data(), ns.data(), F32, op.out.dtype));
+    }
+    for (size_t oi = exe.batched_converts; oi < fn.ops.size(); oi++) {
         const Op& op = fn.ops[oi];
         const std::string& n = op.name;
         auto in = [&](size_t i) -> const DeviceTensor& { return val[op.operands.at(i)]; };

@@ -84,6 +84,7 @@ struct Executable {
     Function fn;
     int opt_level = 2;
     std::vector<DeviceTensor> constants;   // per op index (empty when the op is not a constant)
+    size_t batched_converts = 0;           // leading ops: f32 -> 16-bit converts of arguments, run as one batch
     // statistics (milliseconds), CInterface.swift:63-96
     int64_t exec_count = 0;
     double total_ms = 0, last_ms = 0;

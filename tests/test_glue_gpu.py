@@ -104,3 +104,35 @@ def test_argmax_ties_and_nan():
     # vocab-sized row
     big = torch.from_numpy(rng.standard_normal((8, 50257)).astype(np.float32)).cuda()
     assert torch.equal(kernels.argmax(big).long(), big.argmax(-1))
+
+
+def test_convert_batch_matches_single_converts(lib):
+    """Many tensors in one launch: same bits as one mhip_convert each (and as torch's rounding), for
+    sizes around the 8-element vectors and the 2048-element blocks, unaligned bases, empty
+    tensors, and more tensors than one launch's table holds."""
+    import ctypes as C
+    rng = np.random.default_rng(91)
+    sizes = [1, 7, 8, 9, 2047, 2048, 2049, 0, 768, 3 * 768, 768 * 768, 5] + [int(v) for v in rng.integers(1, 5000, 120)]
+    for dst, code in ((torch.bfloat16, 3), (torch.float16, 0)):
+        big = torch.from_numpy(rng.standard_normal(sum(sizes) + 16 * len(sizes) + 64).astype(np.float32)).cuda()
+        outs_flat = torch.full((big.numel(),), 9.0, dtype=dst, device="cuda")
+        xs, ys, off = [], [], 0
+        for i, n in enumerate(sizes):
+            off += (i % 4)                                   # every alignment of the base modulo 4 elements
+            xs.append(big[off:off + n])
+            ys.append(outs_flat[off:off + n])
+            off += n + 8
+        px = (C.c_void_p * len(sizes))(*[x.data_ptr() for x in xs])
+        py = (C.c_void_p * len(sizes))(*[y.data_ptr() for y in ys])
+        pn = (C.c_int64 * len(sizes))(*sizes)
+        assert lib.mhip_convert_batch(None, len(sizes), px, py, pn, 1, code) == 0, lib.mhip_last_error()
+        torch.cuda.synchronize()
+        want = torch.full_like(outs_flat, 9.0)
+        off = 0
+        for i, n in enumerate(sizes):
+            off += (i % 4)
+            want[off:off + n] = big[off:off + n].to(dst)
+            off += n + 8
+        assert torch.equal(outs_flat, want)                  # converted where asked, untouched elsewhere
+    assert lib.mhip_convert_batch(None, 1, px, py, pn, 3, 1) == 2      # only f32 -> 16-bit
+    assert lib.mhip_convert_batch(None, 0, None, None, None, 1, 3) == 0
