@@ -190,8 +190,8 @@ def cpu_baseline_gemm(sample_rows=4096, N=4096, K=4096):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="gemm",
                     choices=["gemm", "attention", "attention_full", "softmax", "layer_norm", "rms_norm", "bias_gelu", "copy", "gpt2"])
     ap.add_argument("--only", action="store_true", help="time only --workload (for profiling runs)")
