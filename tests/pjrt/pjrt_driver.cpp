@@ -304,6 +304,13 @@ static void case_compile(PJRT_Client* c) {
     np.executable = ge.executable;
     OK(api->PJRT_Executable_NumPartitions(&np));
     CHECK(nr.num_replicas == 1 && np.num_partitions == 1);
+    // memory statistics come from the plan made at compile time: two 16-byte arguments, one
+    // 16-byte result, no intermediates for a single add
+    ARGS(PJRT_Executable_GetCompiledMemoryStats_Args, cm);
+    cm.executable = ge.executable;
+    OK(api->PJRT_Executable_GetCompiledMemoryStats(&cm));
+    CHECK(cm.argument_size_in_bytes == 32 && cm.output_size_in_bytes == 16 && cm.temp_size_in_bytes == 0);
+    CHECK(cm.peak_memory_in_bytes == 48 && cm.generated_code_size_in_bytes == 0 && cm.host_temp_size_in_bytes == 0);
     ARGS(PJRT_Executable_OutputElementTypes_Args, ot);
     ot.executable = ge.executable;
     OK(api->PJRT_Executable_OutputElementTypes(&ot));
