@@ -363,6 +363,62 @@ static void hoist_parameter_converts(Executable& exe) {
     fn.ops = std::move(front);
 }
 
+// [batch dims, lhs free dims, rhs free dims]: the shape dot / dot_general writes
+static std::vector<int64_t> dot_result_shape(const Op& op, const TensorType& lt, const TensorType& rt) {
+    std::vector<int64_t> lb = op.lhs_batch, rb = op.rhs_batch, lc = op.lhs_contract, rc = op.rhs_contract;
+    if (op.name == "dot") { lc = {(int64_t)lt.shape.size() - 1}; rc = {0}; }
+    auto in = [](const std::vector<int64_t>& v, int64_t d) { return std::find(v.begin(), v.end(), d) != v.end(); };
+    std::vector<int64_t> shape;
+    for (auto d : lb) shape.push_back(lt.shape.at(d));
+    for (int64_t d = 0; d < (int64_t)lt.shape.size(); d++) if (!in(lb, d) && !in(lc, d)) shape.push_back(lt.shape[d]);
+    for (int64_t d = 0; d < (int64_t)rt.shape.size(); d++) if (!in(rb, d) && !in(rc, d)) shape.push_back(rt.shape[d]);
+    return shape;
+}
+
+// The fused kernels derive every extent from their operands and write a result of the operands'
+// element type: a custom_call whose declared result (or an operand) says otherwise would be an
+// out-of-bounds write or a misread buffer, so it is refused here, before anything runs.
+static void check_custom_call_types(const Op& op, const std::vector<TensorType>& vt) {
+    auto in = [&](size_t i) -> const TensorType& { return vt[op.operands.at(i)]; };
+    const int dt = op.out.dtype;
+    for (size_t i = 0; i < op.operands.size(); i++)
+        if (in(i).dtype != dt) throw ParseError(where(op) + "every operand must have the result's element type");
+    const Config cfg = parse_config(op.backend_config);
+    const TensorType& xt = in(0);
+    const int64_t cols = xt.shape.empty() ? 1 : xt.shape.back();
+    if (op.target == "fused_softmax" || op.target == "fused_gelu" || op.target == "fused_layer_norm" || op.target == "fused_rms_norm") {
+        if (!(xt == op.out)) throw ParseError(where(op) + "the result type must be the input's");
+        if (op.target == "fused_layer_norm" || op.target == "fused_rms_norm") {
+            if (in(1).numel() != cols) throw ParseError(where(op) + "gamma must be [cols] of the input type");
+            if (op.target == "fused_layer_norm" && in(2).numel() != cols) throw ParseError(where(op) + "beta must be [cols] of the input type");
+        }
+    } else if (op.target == "fused_matmul_bias_activation") {
+        const bool ta = cfg.get_bool("trans_a", false), tb = cfg.get_bool("trans_b", false);
+        const TensorType& wt = in(1);
+        if (wt.shape.size() != 2 || xt.shape.size() < 2 || (ta && xt.shape.size() != 2))
+            throw ParseError(where(op) + "expected x [.., M, K] and w [K, N]");
+        const int64_t K = ta ? xt.shape[0] : cols;
+        const int64_t Kb = tb ? wt.shape[1] : wt.shape[0], N = tb ? wt.shape[0] : wt.shape[1];
+        std::vector<int64_t> want = ta ? std::vector<int64_t>{xt.shape[1]} : std::vector<int64_t>(xt.shape.begin(), xt.shape.end() - 1);
+        want.push_back(N);
+        if (K != Kb) throw ParseError(where(op) + "operand shapes do not contract");
+        if (op.out.shape != want) throw ParseError(where(op) + "the result shape is not [.., M, N]");
+        const bool has_res = cfg.get_bool("has_residual", false);
+        const size_t n_plain = op.operands.size() - (has_res ? 1 : 0);
+        if (has_res && op.operands.size() < 3) throw ParseError(where(op) + "has_residual without a residual operand");
+        if (n_plain > 2 && in(2).numel() != N) throw ParseError(where(op) + "bias must be [N] of the input type");
+        if (has_res && !(in(op.operands.size() - 1) == op.out)) throw ParseError(where(op) + "the residual must have the result's type");
+    } else if (op.target == "fused_scaled_dot_product_attention" && cfg.get_int_array("views", {}).empty()) {
+        const TensorType& kt = in(1);
+        const size_t r = xt.shape.size();
+        if (r < 2 || kt.shape.size() != r || !(in(2) == kt) || kt.shape[r - 1] != xt.shape[r - 1])
+            throw ParseError(where(op) + "expected q [.., Sq, D] and k, v [.., Skv, D]");
+        for (size_t d = 0; d + 2 < r; d++)
+            if (kt.shape[d] != xt.shape[d]) throw ParseError(where(op) + "q and k differ in a batch / head dimension");
+        if (!(xt == op.out)) throw ParseError(where(op) + "the result type must be q's");
+    }
+}
+
 void compile(Executable& exe) {
     hoist_parameter_converts(exe);
     Function& fn = exe.fn;
@@ -430,6 +486,12 @@ void compile(Executable& exe) {
             if (it == producer.end() || it->second->name != "constant") throw UnsupportedOp(where(op) + "init value must be a constant");
             if (!is_kernel_float(in(0).dtype) && in(0).dtype != I32 && in(0).dtype != I64) throw UnsupportedOp(where(op) + "element type not supported");
             for (auto d : op.dims) if (d < 0 || d >= (int64_t)in(0).shape.size()) throw ParseError(where(op) + "dimension out of range");
+            // the kernel writes one element per kept position: the declared result must be exactly that
+            std::vector<int64_t> kept;
+            for (int64_t d = 0; d < (int64_t)in(0).shape.size(); d++)
+                if (std::find(op.dims.begin(), op.dims.end(), d) == op.dims.end()) kept.push_back(in(0).shape[d]);
+            if (op.out.shape != kept || op.out.dtype != in(0).dtype)
+                throw ParseError(where(op) + "the result type is not the operand's without the reduced dimensions");
         } else if (n == "dot" || n == "dot_general") {
             // operands of one type; the result has that type, or a wider floating one (the
             // operands are then converted first and the product is taken in the result type)
@@ -439,6 +501,8 @@ void compile(Executable& exe) {
             if (!dot_type(in(0).dtype) || in(0).dtype != in(1).dtype || (op.out.dtype != in(0).dtype && !widen))
                 throw UnsupportedOp(where(op) + "dot needs f32 / f16 / bf16 / f64 / i32 / i64 operands of one type");
             (void)plan_dot(op, in(0), in(1));
+            if (op.out.shape != dot_result_shape(op, in(0), in(1)))
+                throw ParseError(where(op) + "the result shape is not [batch, lhs free, rhs free]");
         } else if (n == "iota") {
             if (op.iota_dim < 0 || op.iota_dim >= (int64_t)op.out.shape.size()) throw ParseError(where(op) + "iota dim out of range");
         } else if (n == "compare") {
@@ -461,6 +525,7 @@ void compile(Executable& exe) {
             if (op.target == "fused_matmul_bias_activation" &&
                 !kActivation.count(parse_config(op.backend_config).get_string("activation", "none")))
                 throw UnsupportedOp(where(op) + "unknown activation");
+            check_custom_call_types(op, vt);
         } else {
             throw UnsupportedOp(where(op) + "operation is outside the supported subset");
         }

@@ -106,6 +106,20 @@ struct Rewriter {
     }
 
     static bool near(double a, double b, double tol) { return fabs(a - b) <= tol; }
+    // the element types the fused kernels compute in
+    static bool fused_float(int dt) { return dt == F32 || dt == F16 || dt == BF16; }
+    // `c` is the constant `want` as a program of element type `dt` can spell it: `want` rounded to
+    // that type, give or take one unit in the last place (another value is another function)
+    static bool is_const(double c, double want, int dt) {
+        double r = (double)(float)want, rel = 2.4e-7;
+        if (dt == BF16) {
+            const uint32_t w = (uint32_t)f32_to_bf16_bits((float)want) << 16;
+            float f; memcpy(&f, &w, 4); r = f; rel = 1.0 / 128;
+        } else if (dt == F16) {
+            r = (double)(float)(_Float16)(float)want; rel = 1.0 / 1024;
+        }
+        return fabs(c - r) <= fabs(r) * rel;
+    }
 
     // Statistics (one value per row) are often carried in keepdims style: reshaped or broadcast
     // to a shape with extra unit dims, computed on there, and spread over the row at the end.
@@ -187,7 +201,7 @@ struct Rewriter {
     // divide(e, bcast(reduce_add(e))), e = exp(subtract(x, bcast(reduce_max(x))))
     bool softmax(size_t ri) {
         const Op& root = fn.ops[ri];
-        if (root.name != "divide" || !dtype_is_float(root.out.dtype)) return false;
+        if (root.name != "divide" || !fused_float(root.out.dtype)) return false;
         const Op* e = op_named(root.operands[0], "exponential");
         if (!e) return false;
         std::set<size_t> in = {ri, index_of(e)};
@@ -251,7 +265,8 @@ struct Rewriter {
 
     bool gelu(size_t ri) {
         const Op& root = fn.ops[ri];
-        if (root.name != "multiply" || !dtype_is_float(root.out.dtype)) return false;
+        if (root.name != "multiply" || !fused_float(root.out.dtype)) return false;
+        const int dt = root.out.dtype;
         std::vector<int> leaves;
         std::set<size_t> in;
         product_leaves(root.result, true, leaves, in);
@@ -275,7 +290,7 @@ struct Rewriter {
         int inner = -1, ks = 0;
         for (int v : l2) {
             double c;
-            if (splat_value(v, c) && near(c, 0.7978845608028654, 0.01)) ks++;
+            if (splat_value(v, c) && is_const(c, 0.7978845608028654, dt)) ks++;
             else inner = v;
         }
         if (ks != 1 || inner < 0) return false;
@@ -290,7 +305,7 @@ struct Rewriter {
         for (int v : l3) {
             double c;
             if (v == x) xs++;
-            else if (splat_value(v, c) && near(c, 0.044715, 0.005)) cs++;
+            else if (splat_value(v, c) && is_const(c, 0.044715, dt)) cs++;
             else return false;
         }
         if (xs != 3 || cs != 1 || !(type.at(x) == root.out)) return false;
@@ -652,8 +667,10 @@ struct Rewriter {
     bool plain_matmul(const Op* d) const {
         if (!d || (d->name != "dot" && d->name != "dot_general") || d->operands.size() != 2) return false;
         const TensorType &xt = type.at(d->operands[0]), &wt = type.at(d->operands[1]);
-        if (wt.shape.size() != 2 || xt.shape.size() < 2 || !dtype_is_float(xt.dtype) || xt.dtype == F64 || wt.dtype != xt.dtype)
+        if (wt.shape.size() != 2 || xt.shape.size() < 2 || !fused_float(xt.dtype) || wt.dtype != xt.dtype)
             return false;
+        // a widening product (16-bit operands, f32 result) is not what the fused kernel computes
+        if (d->out.dtype != xt.dtype) return false;
         if (d->name == "dot") return xt.shape.size() == 2;
         if (d->name != "dot_general") return false;
         return d->lhs_batch.empty() && d->rhs_batch.empty() &&

@@ -129,3 +129,83 @@ def test_attention_absorbs_scale_mask_and_transpose(sess, with_mask, transpose_k
 def test_matmul_bias_activation(sess):
     assert ops(sess, M.FFN_UP) == ["fused_matmul_bias_activation"]
     assert ops(sess, M.MATMUL_BIAS_RELU) == ["fused_matmul_bias_activation"]
+
+
+def test_widening_dot_stays_unfused(sess):
+    """bf16 x bf16 -> f32 (what preferred_element_type emits) followed by an f32 bias add is not
+    what the fused kernel computes (it reads x, w and writes the result in ONE type): the
+    module keeps its dot_general, which converts first."""
+    text = ("func.func @main(%x: tensor<32x64xbf16>, %w: tensor<64x128xbf16>, %b: tensor<128xf32>) -> tensor<32x128xf32> {\n"
+            "  %d = stablehlo.dot_general %x, %w, contracting_dims = [1] x [0] : (tensor<32x64xbf16>, tensor<64x128xbf16>) -> tensor<32x128xf32>\n"
+            "  %bb = stablehlo.broadcast_in_dim %b, dims = [1] : (tensor<128xf32>) -> tensor<32x128xf32>\n"
+            "  %h = stablehlo.add %d, %bb : tensor<32x128xf32>\n  return %h : tensor<32x128xf32> }")
+    assert ops(sess, text) == ["dot_general", "broadcast_in_dim", "add"]
+    assert ops(sess, text, 0) == ["dot_general", "broadcast_in_dim", "add"]
+
+
+def test_gelu_constants_at_the_precision_of_the_element_type(sess):
+    """Near misses (0.79 for sqrt(2/pi), 0.049 for 0.044715) are other functions and stay as
+    written; bf16 programs spell the constants as their bf16 roundings and still fuse; f64 has no
+    fused kernel and must keep compiling at every level."""
+    assert "fused_gelu" not in ops(sess, M.GELU.replace("0.7978845608", "0.79"))
+    assert "fused_gelu" not in ops(sess, M.GELU.replace("0.044715", "0.049"))
+    assert "fused_gelu" not in ops(sess, M.GELU.replace("0.044715", "0.0447"))
+    assert ops(sess, M.GELU.replace("0.7978845608", "0.79788456")) == ["fused_gelu"]
+    bf = M.GELU.replace("xf32", "xbf16")
+    assert ops(sess, bf) == ["fused_gelu"]
+    assert "fused_gelu" not in ops(sess, bf.replace("0.7978845608", "0.79"))        # two bf16 steps away
+    f64 = M.GELU.replace("xf32", "xf64")
+    assert "fused_gelu" not in ops(sess, f64) and "tanh" in ops(sess, f64)
+    assert ops(sess, f64) == ops(sess, f64, 0)
+
+
+BAD_RESULT_TYPES = {
+    "dot_general_small_result":
+        "func.func @main(%a: tensor<64x128xf32>, %b: tensor<128x256xf32>) -> tensor<8x8xf32> {\n"
+        "  %d = stablehlo.dot_general %a, %b, contracting_dims = [1] x [0] : (tensor<64x128xf32>, tensor<128x256xf32>) -> tensor<8x8xf32>\n"
+        "  return %d : tensor<8x8xf32> }",
+    "reduce_small_result":
+        "func.func @main(%a: tensor<64x128xf32>) -> tensor<4xf32> {\n"
+        "  %z = stablehlo.constant dense<0.0> : tensor<f32>\n"
+        "  %r = stablehlo.reduce(%a init: %z) applies stablehlo.add across dimensions = [1] : (tensor<64x128xf32>, tensor<f32>) -> tensor<4xf32>\n"
+        "  return %r : tensor<4xf32> }",
+    "gelu_half_result":
+        "func.func @main(%a: tensor<64x128xf32>) -> tensor<32x128xf32> {\n"
+        "  %r = stablehlo.custom_call @fused_gelu(%a) : (tensor<64x128xf32>) -> tensor<32x128xf32>\n"
+        "  return %r : tensor<32x128xf32> }",
+    "softmax_changes_type":
+        "func.func @main(%a: tensor<64x128xbf16>) -> tensor<64x128xf32> {\n"
+        "  %r = stablehlo.custom_call @fused_softmax(%a) {backend_config = \"{\\\"axis\\\": -1}\"} : (tensor<64x128xbf16>) -> tensor<64x128xf32>\n"
+        "  return %r : tensor<64x128xf32> }",
+    "matmul_changes_type":
+        "func.func @main(%a: tensor<64x128xbf16>, %w: tensor<128x32xbf16>) -> tensor<64x32xf32> {\n"
+        "  %r = stablehlo.custom_call @fused_matmul_bias_activation(%a, %w) : (tensor<64x128xbf16>, tensor<128x32xbf16>) -> tensor<64x32xf32>\n"
+        "  return %r : tensor<64x32xf32> }",
+    "matmul_wrong_shape":
+        "func.func @main(%a: tensor<64x128xf32>, %w: tensor<128x32xf32>) -> tensor<32x64xf32> {\n"
+        "  %r = stablehlo.custom_call @fused_matmul_bias_activation(%a, %w) : (tensor<64x128xf32>, tensor<128x32xf32>) -> tensor<32x64xf32>\n"
+        "  return %r : tensor<32x64xf32> }",
+    "attention_result_not_q":
+        "func.func @main(%q: tensor<2x64x32xf32>, %k: tensor<2x64x32xf32>, %v: tensor<2x64x32xf32>) -> tensor<2x32x32xf32> {\n"
+        "  %r = stablehlo.custom_call @fused_scaled_dot_product_attention(%q, %k, %v) : (tensor<2x64x32xf32>, tensor<2x64x32xf32>, tensor<2x64x32xf32>) -> tensor<2x32x32xf32>\n"
+        "  return %r : tensor<2x32x32xf32> }",
+    "attention_q_other_type":
+        "func.func @main(%q: tensor<2x64x32xbf16>, %k: tensor<2x64x32xf32>, %v: tensor<2x64x32xf32>) -> tensor<2x64x32xf32> {\n"
+        "  %r = stablehlo.custom_call @fused_scaled_dot_product_attention(%q, %k, %v) : (tensor<2x64x32xbf16>, tensor<2x64x32xf32>, tensor<2x64x32xf32>) -> tensor<2x64x32xf32>\n"
+        "  return %r : tensor<2x64x32xf32> }",
+    "layer_norm_short_gamma":
+        "func.func @main(%x: tensor<8x64xf32>, %g: tensor<32xf32>, %b: tensor<64xf32>) -> tensor<8x64xf32> {\n"
+        "  %r = stablehlo.custom_call @fused_layer_norm(%x, %g, %b) : (tensor<8x64xf32>, tensor<32xf32>, tensor<64xf32>) -> tensor<8x64xf32>\n"
+        "  return %r : tensor<8x64xf32> }",
+}
+
+
+@pytest.mark.parametrize("name", sorted(BAD_RESULT_TYPES))
+@pytest.mark.parametrize("level", [0, 2])
+def test_declared_result_types_are_checked_at_compile_time(sess, name, level):
+    """A result (or operand) type the kernel would not honour is refused with PARSE_FAILED before
+    anything can run: the kernels size their writes from the operands, not from the declaration.
+    Host-only: these modules are never executed."""
+    with pytest.raises(capi.MHLOError) as e:
+        ops(sess, BAD_RESULT_TYPES[name], level)
+    assert e.value.code == 3, (e.value.code, str(e.value))      # MHLO_ERROR_PARSE_FAILED

@@ -252,3 +252,87 @@ def test_gpt2_oracle_shapes_and_determinism():
     assert np.allclose(lo[:, :-1], lo2[:, :-1], atol=1e-12) and not np.allclose(lo[:, -1], lo2[:, -1])
     lb = oracle.gpt2_forward(ids, params, nh, "bf16")
     assert np.max(np.abs(lb - lo)) < 2e-2 * max(1.0, np.max(np.abs(lo)))
+
+
+def _gpt2_params(rng, d, L, V, P, trivial=False):
+    """Random GPT-2 parameters; non-trivial gamma / beta / biases unless asked otherwise, so
+    that a misplaced residual, a missing final LayerNorm or a post-LN ordering changes the logits."""
+    n = lambda *s: rng.normal(0, 0.3, s)
+    g = (lambda: np.ones(d)) if trivial else (lambda: 1 + 0.3 * rng.standard_normal(d))
+    b = (lambda k: np.zeros(k)) if trivial else (lambda k: 0.2 * rng.standard_normal(k))
+
+    def lyr():
+        return dict(ln1_g=g(), ln1_b=b(d), w_qkv=n(d, 3 * d), b_qkv=b(3 * d), w_o=n(d, d), b_o=b(d),
+                    ln2_g=g(), ln2_b=b(d), w_fc=n(d, 4 * d), b_fc=b(4 * d), w_proj=n(4 * d, d), b_proj=b(d))
+    return dict(wte=n(V, d), wpe=n(P, d), layers=[lyr() for _ in range(L)], lnf_g=g(), lnf_b=b(d))
+
+
+def _torch_gpt2(ids, params, n_head, order="pre", final_ln=True):
+    """GPT-2 built from torch fp64 library calls only (Sources/GPT2EndToEnd/main.swift:35-40 for the
+    architecture, Examples/FlaxExample/flax_metalhlo_bf16.py:68 for the pre-LN block): nothing of
+    the oracle is used.  `order` / `final_ln` build the wrong variants the pin must reject."""
+    import torch
+    import torch.nn.functional as F
+    t = lambda a: torch.from_numpy(np.asarray(a, np.float64))
+    ids_t = torch.from_numpy(np.asarray(ids)).long()
+    bsz, seq = ids_t.shape
+    wte = t(params["wte"])
+    d = wte.shape[1]
+    x = F.embedding(ids_t, wte) + F.embedding(torch.arange(seq), t(params["wpe"]))[None]
+    heads = lambda z: z.view(bsz, seq, n_head, d // n_head).transpose(1, 2)
+    for l in params["layers"]:
+        ln1 = lambda z: F.layer_norm(z, (d,), t(l["ln1_g"]), t(l["ln1_b"]), 1e-5)
+        ln2 = lambda z: F.layer_norm(z, (d,), t(l["ln2_g"]), t(l["ln2_b"]), 1e-5)
+
+        def attn(z):
+            q, k, v = F.linear(z, t(l["w_qkv"]).T, t(l["b_qkv"])).split(d, dim=-1)
+            a = F.scaled_dot_product_attention(heads(q), heads(k), heads(v), is_causal=True)
+            return F.linear(a.transpose(1, 2).reshape(bsz, seq, d), t(l["w_o"]).T, t(l["b_o"]))
+
+        def mlp(z):
+            u = F.gelu(F.linear(z, t(l["w_fc"]).T, t(l["b_fc"])), approximate="tanh")
+            return F.linear(u, t(l["w_proj"]).T, t(l["b_proj"]))
+        if order == "pre":
+            x = x + attn(ln1(x))
+            x = x + mlp(ln2(x))
+        elif order == "post":
+            x = ln1(x + attn(x))
+            x = ln2(x + mlp(x))
+        elif order == "no_residual":
+            x = attn(ln1(x))
+            x = x + mlp(ln2(x))
+    if final_ln:
+        x = F.layer_norm(x, (d,), t(params["lnf_g"]), t(params["lnf_b"]), 1e-5)
+    return F.linear(x, wte).numpy()
+
+
+@pytest.mark.parametrize("d,nh,L,V,S,B", [(32, 4, 1, 61, 10, 2), (48, 3, 2, 97, 17, 3), (64, 8, 3, 50, 33, 1)])
+def test_gpt2_oracle_equals_torch_fp64_library_composition(d, nh, L, V, S, B):
+    """Pins oracle.gpt2_forward: the same model from torch fp64 library calls (embedding,
+    layer_norm, linear, scaled_dot_product_attention(is_causal), gelu(tanh), tied head) must
+    agree to 1e-10, and the plausible mistakes (post-LN, a dropped residual, no final LN)
+    must not."""
+    rng = np.random.default_rng(100 + d)
+    params = _gpt2_params(rng, d, L, V, S + 3)
+    ids = rng.integers(0, V, (B, S))
+    got = oracle.gpt2_forward(ids, params, nh, "f64")
+    exp = _torch_gpt2(ids, params, nh)
+    assert got.shape == exp.shape == (B, S, V)
+    scale = np.max(np.abs(exp))
+    assert np.max(np.abs(got - exp)) <= 1e-10 * max(1.0, scale)
+    for wrong in (dict(order="post"), dict(order="no_residual"), dict(final_ln=False)):
+        bad = _torch_gpt2(ids, params, nh, **wrong)
+        assert np.max(np.abs(got - bad)) > 1e-3 * scale, wrong
+
+
+def test_gpt2_oracle_bf16_rounding_points_stay_near_f64():
+    """The bf16 variant only inserts roundings: it stays within the end-to-end bf16 bar of the
+    pinned f64 function on a model with non-trivial parameters."""
+    rng = np.random.default_rng(11)
+    params = _gpt2_params(rng, 32, 2, 61, 16)
+    for k in ("wte", "wpe"):
+        params[k] = params[k] * 0.1
+    ids = rng.integers(0, 61, (2, 12))
+    lo = oracle.gpt2_forward(ids, params, 4, "f64")
+    lb = oracle.gpt2_forward(ids, params, 4, "bf16")
+    assert np.sqrt(np.mean((lb - lo) ** 2)) < 2e-2 * np.sqrt(np.mean(lo ** 2))
