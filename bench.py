@@ -104,19 +104,19 @@ def wl_rows(torch, kernels, op, rows=32768, cols=4096):
     base = 2.0 * rows * cols * 2
     if op == "softmax":
         fn = lambda i: lib.mhip_softmax(st(), xs[i % n].data_ptr(), ys[i % n].data_ptr(), rows, cols, 3)
-        extra, kern = 0, "row_wave_kernel<bf16,softmax>"
+        extra, kern = 0, "row_split_kernel<bf16,softmax>"
     elif op == "layer_norm":
         fn = lambda i: lib.mhip_layer_norm(st(), xs[i % n].data_ptr(), gam.data_ptr(), bet.data_ptr(),
                                            ys[i % n].data_ptr(), rows, cols, 1e-5, 3)
-        extra, kern = 2 * cols * 2, "row_wave_kernel<bf16,layer_norm>"
+        extra, kern = 2 * cols * 2, "row_split_kernel<bf16,layer_norm>"
     elif op == "rms_norm":
         fn = lambda i: lib.mhip_rms_norm(st(), xs[i % n].data_ptr(), gam.data_ptr(), ys[i % n].data_ptr(),
                                          rows, cols, 1e-6, 3)
-        extra, kern = cols * 2, "row_wave_kernel<bf16,rms_norm>"
+        extra, kern = cols * 2, "row_split_kernel<bf16,rms_norm>"
     elif op == "bias_gelu":
         fn = lambda i: lib.mhip_bias_gelu(st(), xs[i % n].data_ptr(), bias.data_ptr(), ys[i % n].data_ptr(),
                                           rows, cols, 3)
-        extra, kern = cols * 2, "bias_gelu_vec_kernel<bf16>"
+        extra, kern = cols * 2, "bias_gelu_tile_kernel<bf16>"
     else:
         raise ValueError(op)
     return dict(name=f"bf16 {op} [{rows},{cols}]", fn=fn, flops=0.0, bytes=base + extra, bound="hbm",

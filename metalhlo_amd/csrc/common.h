@@ -37,6 +37,21 @@ int tune_int(const char* name, int fallback);
 
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 
+// How a vectorisable row-operator launch (softmax / LayerNorm / RMSNorm over 16-byte-aligned rows)
+// is carried out.  `kind`: 1 = one wave per row, parameters staged in LDS, persistent grid;
+// 2 = a row split over the waves of a workgroup.  `r` = rows per wave group (split only),
+// `ordered` = the grid covers the rows once in address order (split only; 0 = persistent grid),
+// `per_cu` = resident workgroups per CU of a persistent grid (0 = what the occupancy query says).
+// Zero / negative fields mean "choose".
+struct RowLaunch { int kind = 0, r = 0, ordered = -1, per_cu = 0; };
+
+// The launch a tuning pass recorded for this problem on this device, if any (tuning.hip).
+bool tuned_row_launch(int op, int dtype, int64_t rows, int64_t cols, bool has_gamma, bool has_beta, RowLaunch* out);
+
+// One launch of row operator `op` (0 softmax, 1 LayerNorm, 2 RMSNorm) carried out as `how` says.
+int row_launch_as(int op, const RowLaunch& how, void* stream, const void* x, const void* g, const void* b, void* y,
+                  int64_t rows, int64_t cols, float eps, int dtype);
+
 template <typename T> struct Elem;
 template <> struct Elem<float> {
     static constexpr int kPerVec = 4;  // elements per 16-byte vector

@@ -63,6 +63,8 @@ int tuned_gemm_variant(const GemmArgs& g, int64_t batch, int ta, int tb, int dty
     return it == g_table.end() ? 0 : it->second.variant;
 }
 
+bool tuned_row_launch(int, int, int64_t, int64_t, bool, bool, RowLaunch*) { return false; }
+
 }  // namespace mhip
 
 using namespace mhip;

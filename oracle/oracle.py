@@ -55,12 +55,17 @@ def bf16_round_bits(x) -> np.ndarray:
     Follows Runtime/BufferStorage.swift:328-344:
     ``rounded = bits + 0x7FFF + ((bits >> 16) & 1)``.
     """
-    f = np.asarray(x, dtype=np.float32)
-    bits = f.view(np.uint32).astype(np.uint64)
-    rounded = (bits + 0x7FFF + ((bits >> 16) & 1)) & 0xFFFFFFFF
-    out = (rounded >> 16).astype(np.uint16)
-    out = np.where(np.isnan(f), np.uint16(0x7FC0), out)
-    return out.astype(np.uint16)
+    f = np.ascontiguousarray(x, dtype=np.float32)
+    bits = f.view(np.uint32)
+    # 32-bit arithmetic: the sum only wraps for patterns above 0xFFFF8000, which are NaNs and
+    # are overwritten below
+    rounded = (bits >> 16) & np.uint32(1)
+    rounded += np.uint32(0x7FFF)
+    rounded += bits
+    rounded >>= 16
+    out = rounded.astype(np.uint16)
+    out[np.isnan(f)] = 0x7FC0
+    return out
 
 
 def bf16_bits_to_f32(bits) -> np.ndarray:
@@ -348,7 +353,8 @@ def gpt2_forward(ids, params, n_head: int, compute_dtype: str = "bf16") -> np.nd
     wte, wpe = params["wte"], params["wpe"]
     d = wte.shape[1]
     hd = d // n_head
-    x = r(np.asarray(wte, np.float64)[ids] + np.asarray(wpe, np.float64)[None, :seq])
+    wte = np.asarray(wte, np.float64)
+    x = r(wte[ids] + np.asarray(wpe, np.float64)[None, :seq])
     for lyr in params["layers"]:
         h = r(layer_norm(x, r(lyr["ln1_g"]), r(lyr["ln1_b"]), 1e-5))
         qkv = r(gemm(h, r(lyr["w_qkv"])) + r(lyr["b_qkv"]))
@@ -361,4 +367,4 @@ def gpt2_forward(ids, params, n_head: int, compute_dtype: str = "bf16") -> np.nd
         u = r(bias_gelu(gemm(h, r(lyr["w_fc"])), r(lyr["b_fc"])))
         x = r(x + r(gemm(u, r(lyr["w_proj"])) + r(lyr["b_proj"])))
     x = r(layer_norm(x, r(params["lnf_g"]), r(params["lnf_b"]), 1e-5))
-    return gemm(x, r(np.asarray(wte, np.float64)).T)
+    return gemm(x, r(wte).T)
