@@ -12,9 +12,14 @@ and reported under "kernels" of the same JSON line unless --only is given.
 Timing: HIP events recorded on the stream the kernels are launched on, around
 exactly K launches, after W warm-up launches, bracketed by device
 synchronisation.  `roofline.achieved` = algorithmic FLOPs (or bytes) per launch
-divided by the mean launch duration from those events.
-`cpu_baseline` times the C restatement under oracle/ on the host cores, on a
-bounded sample of the same workload (never part of the measured GPU path).
+divided by the mean launch duration from those events.  A device that has idled
+needs tens of milliseconds of work before it holds its clocks, far more than five
+warm-up launches of a 100 us kernel; `--ramp-ms` (default 150, reported as
+`clock_ramp_ms`, 0 switches it off) keeps the device busy with the same kernel for
+that long before the W warm-up launches of every workload.
+`cpu_baseline` (per kernel) times the same operator on the host cores with torch's
+CPU kernels, and for the GEMM also the C restatement under oracle/, each on a
+bounded sample of the workload (never part of the measured GPU path).
 """
 from __future__ import annotations
 
@@ -44,6 +49,22 @@ MEASURED_TRAFFIC = {
     "bias_gelu": 536757341,
     "copy": 536870912,
 }
+
+
+RAMP_MS = 0.0
+
+
+def _ramp(fn, torch):
+    """Keeps the device busy with fn for RAMP_MS milliseconds (untimed)."""
+    if RAMP_MS <= 0:
+        return
+    t0 = time.perf_counter()
+    i = 0
+    while (time.perf_counter() - t0) * 1e3 < RAMP_MS:
+        for _ in range(8):
+            fn(i)
+            i += 1
+        torch.cuda.synchronize()
 
 
 def _time_launches(fn, steps, warmup, torch):
@@ -143,11 +164,52 @@ def wl_gpt2(torch, kernels, B=8, S=1024):
     graphed = model.capture(ids)     # one HIP graph replay per step instead of ~135 host launches
     return dict(name=f"GPT-2-small forward B{B} S{S}, bf16 compute / fp32 params (converted every step), HIP graph replay",
                 fn=lambda i: graphed(ids), flops=GPT2.flops(cfg, B, S), bytes=0.0, bound="mfma",
-                kernel="fused pipeline (12 x [LN, GEMM+bias, attention, GEMM+bias, add, LN, GEMM+bias+GELU, GEMM+bias, add])")
+                kernel="fused pipeline (convert, embed, 12 x [LN, GEMM+bias, attention, GEMM+bias+residual, LN, "
+                       "GEMM+bias+GELU, GEMM+bias+residual], LN, logits GEMM)")
+
+
+def wl_gpt2_capi(torch, kernels, B=8, S=1024):
+    """The same forward pass written as ONE plain StableHLO module (no custom calls, fp32
+    parameters) and run through the C API: mhlo_compile recognises the fused operators,
+    mhlo_execute runs them.  Parameters stay resident as mhlo buffers; a step is one
+    mhlo_execute (synchronous: it returns when the logits are complete) plus the release of
+    its result.  Timed by the host clock around the calls."""
+    import ctypes
+    import numpy as np
+    from metalhlo_amd import capi, programs
+    from metalhlo_amd.gpt2 import GPT2, GPT2Config, init_params
+    cfg = GPT2Config()
+    text = programs.gpt2_program(B, S, cfg.n_layer, cfg.n_head, cfg.d_model // cfg.n_head, cfg.d_ff, cfg.vocab, cfg.n_pos)
+    sess = capi.Session()
+    exe = sess.compile(text)
+    p = init_params(cfg, seed=5)
+    rng = np.random.default_rng(5)
+    ids = rng.integers(0, cfg.vocab, (B, S)).astype(np.int32)
+    arrs = [(ids, "i32"), (p["wte"], "f32"), (p["wpe"], "f32")]
+    for l in p["layers"]:
+        arrs += [(l[n], "f32") for n in programs.GPT2_LAYER_PARAMS]
+    arrs += [(p["lnf_g"], "f32"), (p["lnf_b"], "f32")]
+    bufs = [sess.buffer(a, t) for a, t in arrs]
+    arr = (ctypes.c_void_p * len(bufs))(*bufs)
+    outs = (ctypes.c_void_p * 1)()
+    got = ctypes.c_int32()
+
+    def step(i):
+        rc = sess.lib.mhlo_execute(exe, arr, len(bufs), outs, ctypes.byref(got))
+        if rc != 0:
+            raise RuntimeError("mhlo_execute failed: %s" % sess.lib.mhlo_get_last_error())
+        sess.lib.mhlo_buffer_destroy(outs[0])
+    return dict(name=f"GPT-2-small forward B{B} S{S} from one plain StableHLO module through mhlo_compile / mhlo_execute "
+                     f"(fp32 parameters converted every step, {len(sess.ops(exe))} operations after pattern recognition)",
+                fn=step, flops=GPT2.flops(cfg, B, S), bytes=0.0, bound="mfma", host_timed=True, keep=(sess, bufs),
+                kernel="mhlo_execute: batched converts, gather, 12 x 7 fused kernels, LN, logits GEMM")
 
 
 def measure(wl, steps, warmup, torch, key=None):
+    _ramp(wl["fn"], torch)
     sec, wall = _time_launches(wl["fn"], steps, warmup, torch)
+    if wl.get("host_timed"):        # the calls are synchronous and run on the library's own stream
+        sec = wall
     if wl["bound"] == "mfma":
         ach = wl["flops"] / sec / 1e12
         roof = dict(bound="mfma", achieved=round(ach, 2), peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
@@ -162,8 +224,19 @@ def measure(wl, steps, warmup, torch, key=None):
                 us_per_launch=round(sec * 1e6, 2), wall_us_per_launch=round(wall * 1e6, 2), roofline=roof)
 
 
-# ---------------------------------------------------------------- CPU baseline (oracle port)
-def cpu_baseline_gemm(sample_rows=4096, N=4096, K=4096):
+# ---------------------------------------------------------------- CPU baselines
+def _best_of(fn, reps=3):
+    fn()                                    # warm-up
+    best = float("inf")
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        fn()
+        best = min(best, time.perf_counter() - t0)
+    return best
+
+
+def cpu_baseline_gemm_port(sample_rows=4096, N=4096, K=4096):
+    """The C restatement of the oracle (OpenMP) on the same GEMM."""
     import numpy as np
     from oracle import oracle
     lib = C.CDLL(os.path.join(ROOT, "oracle", "liboracle.so"))
@@ -174,17 +247,79 @@ def cpu_baseline_gemm(sample_rows=4096, N=4096, K=4096):
     c = np.empty((sample_rows, N), np.uint16)
     p = lambda x: x.ctypes.data_as(C.c_void_p)
     args = (p(a), p(b), p(c), C.c_int64(sample_rows), C.c_int64(N), C.c_int64(K), 1)
-    lib.orc_gemm(*args)                     # warm-up
-    best = float("inf")
-    for _ in range(3):
-        t0 = time.perf_counter()
-        lib.orc_gemm(*args)
-        best = min(best, time.perf_counter() - t0)
+    best = _best_of(lambda: lib.orc_gemm(*args))
     return dict(value=round(2.0 * sample_rows * N * K / best / 1e12, 5), unit="TFLOP/s",
                 cores=int(lib.orc_num_threads()), kind="port",
                 sample=f"oracle/oracle_kernels.c orc_gemm on {sample_rows} of 4096 rows of A "
                        f"(x full B), bf16 in / fp32 accumulate, one warm-up + best of 3 "
                        f"({best:.2f} s each); host has {os.cpu_count()} logical CPUs")
+
+
+def cpu_baseline_torch(name, torch):
+    """The operator of workload `name` with torch's CPU kernels (the library stand-in for the
+    CPU path the reference's own suites compare with; jax is not installed), on a bounded
+    sample, scaled to the workload's unit.  `cores` = torch's intra-op threads."""
+    import torch.nn.functional as F
+    th = torch.get_num_threads()
+    g = torch.Generator().manual_seed(7)
+    bf = torch.bfloat16
+    base = dict(cores=th, kind="port")
+    if name == "gemm":
+        a = (torch.rand(4096, 4096, generator=g) * 2 - 1).to(bf)
+        b = (torch.rand(4096, 4096, generator=g) * 2 - 1).to(bf)
+        t = _best_of(lambda: torch.matmul(a, b))
+        return dict(base, value=round(2.0 * 4096 ** 3 / t / 1e12, 4), unit="TFLOP/s",
+                    sample=f"torch.matmul on CPU, bf16 4096^3 (the whole workload), best of 3: {t:.3f} s")
+    if name in ("attention", "attention_full"):
+        S, causal = (4096, True) if name == "attention" else (2048, False)
+        q, k, v = (torch.randn(1, 1, S, 128, generator=g).to(bf) for _ in range(3))
+        t = _best_of(lambda: F.scaled_dot_product_attention(q, k, v, is_causal=causal))
+        flops = 4.0 * S * S * 128 * (0.5 if causal else 1.0)
+        return dict(base, value=round(flops / t / 1e12, 4), unit="TFLOP/s",
+                    sample=f"torch scaled_dot_product_attention on CPU, bf16, ONE of the 128 (batch, head) slices "
+                           f"(S {S}, D 128, {'causal' if causal else 'full'}), best of 3: {t:.3f} s; the rate carries over, "
+                           f"the whole workload is 128 such slices")
+    if name in ("softmax", "layer_norm", "rms_norm", "bias_gelu"):
+        rows, cols = 8192, 4096
+        x = torch.randn(rows, cols, generator=g).to(bf)
+        w = torch.ones(cols, dtype=bf)
+        z = torch.zeros(cols, dtype=bf)
+        fn = {"softmax": lambda: F.softmax(x, dim=-1),
+              "layer_norm": lambda: F.layer_norm(x, (cols,), w, z, 1e-5),
+              "rms_norm": lambda: (x.float() * torch.rsqrt(x.float().pow(2).mean(-1, keepdim=True) + 1e-6) * w.float()).to(bf),
+              "bias_gelu": lambda: F.gelu(x + z, approximate="tanh")}[name]
+        t = _best_of(fn)
+        return dict(base, value=round(2.0 * rows * cols * 2 / t / 1e9, 2), unit="GB/s",
+                    sample=f"torch on CPU, bf16, {rows} of the 32768 rows x {cols} (algorithmic bytes of the sample / time), "
+                           f"best of 3: {t * 1e3:.1f} ms")
+    if name in ("gpt2", "gpt2_capi"):
+        from metalhlo_amd.gpt2 import GPT2Config, init_params
+        cfg = GPT2Config()
+        p = init_params(cfg, seed=5)
+        tb = lambda a: torch.from_numpy(a).to(bf)
+        wte, wpe = tb(p["wte"]), tb(p["wpe"])
+        layers = [{k: tb(v) for k, v in l.items()} for l in p["layers"]]
+        lnf = tb(p["lnf_g"]), tb(p["lnf_b"])
+        ids = torch.randint(0, cfg.vocab, (1, 1024), generator=g)
+        d, H = cfg.d_model, cfg.n_head
+
+        def fwd():
+            x = F.embedding(ids, wte) + wpe[None, :1024]
+            for l in layers:
+                h = F.layer_norm(x, (d,), l["ln1_g"], l["ln1_b"], 1e-5)
+                q, k, v = F.linear(h, l["w_qkv"].T, l["b_qkv"]).split(d, dim=-1)
+                sh = lambda t_: t_.view(1, 1024, H, d // H).transpose(1, 2)
+                a = F.scaled_dot_product_attention(sh(q), sh(k), sh(v), is_causal=True).transpose(1, 2).reshape(1, 1024, d)
+                x = x + F.linear(a, l["w_o"].T, l["b_o"])
+                h = F.layer_norm(x, (d,), l["ln2_g"], l["ln2_b"], 1e-5)
+                x = x + F.linear(F.gelu(F.linear(h, l["w_fc"].T, l["b_fc"]), approximate="tanh"), l["w_proj"].T, l["b_proj"])
+            return F.linear(F.layer_norm(x, (d,), lnf[0], lnf[1], 1e-5), wte)
+        with torch.no_grad():
+            t = _best_of(fwd, reps=2)
+        return dict(base, value=round(t * 8 * 1e3, 1), unit="ms",
+                    sample=f"torch on CPU, bf16, ONE of the 8 sequences (12 layers, S 1024, full vocabulary): {t * 1e3:.0f} ms, "
+                           f"times 8 for the batch")
+    return None
 
 
 def main():
@@ -193,7 +328,10 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="gemm",
-                    choices=["gemm", "attention", "attention_full", "softmax", "layer_norm", "rms_norm", "bias_gelu", "copy", "gpt2"])
+                    choices=["gemm", "attention", "attention_full", "softmax", "layer_norm", "rms_norm", "bias_gelu", "copy", "gpt2",
+                             "gpt2_capi"])
+    ap.add_argument("--ramp-ms", type=float, default=150.0,
+                    help="milliseconds of untimed launches of the same kernel in front of the warm-up steps (0 = none)")
     ap.add_argument("--only", action="store_true", help="time only --workload (for profiling runs)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
@@ -204,6 +342,8 @@ def main():
     import torch
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible; the kernels have no CPU path")
+    global RAMP_MS
+    RAMP_MS = args.ramp_ms
     from metalhlo_amd import _lib, kernels
     _lib.load()
     torch.cuda.set_device(0)
@@ -219,24 +359,42 @@ def main():
             return wl_copy(torch, kernels)
         if name == "gpt2":
             return wl_gpt2(torch, kernels)
+        if name == "gpt2_capi":
+            return wl_gpt2_capi(torch, kernels)
         return wl_rows(torch, kernels, name)
 
-    head = measure(build(args.workload), args.steps, args.warmup, torch, args.workload)
+    slow = ("gpt2", "gpt2_capi")        # milliseconds per step: fewer steps
+
+    def run(name):
+        k = min(args.steps, 10) if name in slow else args.steps
+        w = min(args.warmup, 3) if name in slow else args.warmup
+        wl = build(name)
+        r = measure(wl, k, w, torch, name)
+        if name in slow:
+            r["fwd_ms"] = round(r["us_per_launch"] / 1e3, 3)
+        del wl
+        torch.cuda.empty_cache()
+        return r
+
+    head = run(args.workload)
     others = {}
     if not args.only:
-        for name in ["gemm", "attention", "attention_full", "softmax", "layer_norm", "rms_norm", "bias_gelu", "gpt2"]:
+        for name in ["gemm", "attention", "attention_full", "softmax", "layer_norm", "rms_norm", "bias_gelu", "gpt2", "gpt2_capi"]:
             if name == args.workload:
                 continue
-            torch.cuda.empty_cache()
-            k_steps = min(args.steps, 10) if name == "gpt2" else args.steps
-            others[name] = measure(build(name), k_steps, min(args.warmup, 3) if name == "gpt2" else args.warmup, torch, name)
-            if name == "gpt2":
-                others[name]["fwd_ms"] = round(others[name]["us_per_launch"] / 1e3, 3)
+            others[name] = run(name)
             print(f"[bench] {name}: {others[name]['value']} {others[name]['unit']} "
                   f"({others[name]['roofline']['frac'] * 100:.1f}% of peak)", file=sys.stderr, flush=True)
     cpu = None
-    if not args.no_cpu and args.workload == "gemm":
-        cpu = cpu_baseline_gemm()
+    if not args.no_cpu:
+        # the CPU leg: after every GPU measurement, on the host cores, bounded samples
+        cpu = cpu_baseline_torch(args.workload, torch)
+        if args.workload == "gemm" and cpu is not None:
+            cpu["c_port"] = cpu_baseline_gemm_port()
+        for name in others:
+            others[name]["cpu_baseline"] = cpu_baseline_torch(name, torch)
+            print(f"[bench] cpu {name}: {others[name]['cpu_baseline']['value']} {others[name]['cpu_baseline']['unit']}",
+                  file=sys.stderr, flush=True)
 
     line = {
         "metric": "bf16 attn/GEMM TFLOP/s + norm/softmax GB/s (% roofline); GPT-2 fwd ms",
@@ -245,6 +403,7 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": head["workload"], "kernel": head["kernel"]},
+        "clock_ramp_ms": args.ramp_ms,
         "roofline": head["roofline"],
         "cpu_baseline": cpu,
         "kernels": others,

@@ -286,26 +286,49 @@ int mhip_reduce(void* stream, int op, const void* x, void* y, int64_t outer, int
 /* y[i] = the low elem_size bytes of `pattern`, n elements (splat constants). */
 int mhip_fill(void* stream, void* y, int64_t n, uint64_t pattern, int elem_size);
 
-/* Autotuner ----------------------------------------------------------------- */
+/* Autotuner -----------------------------------------------------------------
+ * The role of the reference's AutoTuner (Tuning/AutoTuner.swift:12-103,301-458: a search space,
+ * a validity filter, timed candidates) and TuningDatabase (Tuning/TuningDatabase.swift:15-160:
+ * results persisted per device).  Each pass times every launch form the library has for the
+ * problem (forms the shape, the 160 KB of LDS or the register file rule out are skipped) with
+ * `iters` real launches on `stream`, stores the fastest in the process-wide table the entry
+ * point consults before its heuristic, and reports it.  Passes overwrite their output tensor
+ * and synchronise with the stream. */
 
-/* Times every GEMM kernel variant that can serve this 16-bit problem (128x128 tiles /
- * 4 waves, 256x256 / 8 waves, 256x256 / 4 waves with the five-stage LDS ring) with
- * `iters` launches each on `stream`, stores the fastest in the process-wide tuning
- * table that mhip_gemm consults before its heuristic, and reports it (variant code
- * 128 | 256 | 2560 | 2561, microseconds per launch).  Overwrites c; synchronises with the
- * stream.  (Tuning/AutoTuner.swift:301-458.) */
+/* GEMM kernel variants (128x128 tiles / 4 waves, 256x256 / 8 waves, the four-wave LDS-ring kernel
+ * on 256x256 and on 256x128 tiles): variant code 128 | 256 | 2560 | 2561, microseconds per launch. */
 int mhip_gemm_autotune(void* stream, const void* a, const void* b, const void* bias, void* c,
                        int64_t M, int64_t N, int64_t K, int64_t batch, int64_t stride_a,
                        int64_t stride_b, int64_t stride_c, int trans_a, int trans_b, int activation,
                        int dtype, int iters, int* out_variant, float* out_us);
 
-/* The tuning table as text, one "gemm M N K batch trans_a trans_b dtype variant us" line
- * per entry (Tuning/TuningDatabase.swift:109-150).  Loading merges into the table; the
- * file named by the environment variable MHIP_TUNING_DB is loaded at first use. */
+/* Row operators (op 0 softmax, 1 LayerNorm, 2 RMSNorm; arguments as for the operator itself).
+ * Searched: one wave per row with the parameters in LDS on a persistent grid (resident workgroups
+ * per CU 0 = occupancy query, 2, 4, 6, 8) or a row split over the waves of a workgroup (one or two
+ * rows per wave group; grid in address order, or persistent with 0 / 8 / 16 workgroups per CU).
+ * out_choice[4] = {kind 1 | 2, rows per wave group, ordered 0 | 1, workgroups per CU}. */
+int mhip_row_autotune(void* stream, int op, const void* x, const void* gamma, const void* beta, void* y,
+                      int64_t rows, int64_t cols, float eps, int dtype, int iters, int* out_choice,
+                      float* out_us);
+
+/* Attention kernels for packed [B,H,S,D] operands without a mask: 1 = 128 query rows per workgroup,
+ * 2 = the 256-row pipelined kernel (head size 128, Sq >= 256), 3 = the same with causal tiles
+ * paired (causal only).  (AutoTuner.swift:629-723 chooses an attention block size likewise.) */
+int mhip_attention_autotune(void* stream, const void* q, const void* k, const void* v, void* o, int64_t B,
+                            int64_t H, int64_t Sq, int64_t Skv, int64_t D, float scale, int is_causal,
+                            int dtype, int iters, int* out_variant, float* out_us);
+
+/* The tuning table as text, one "<operator> <device> <problem> = <choice> @ <microseconds>" line per
+ * entry (Tuning/TuningDatabase.swift:109-150); <device> is the architecture name and the number
+ * of compute units ("gfx950/256", TuningDatabase.swift:15-60 keys by device too), and only
+ * entries of the current device are used.  Loading merges into the table; the file named by the
+ * environment variable MHIP_TUNING_DB is loaded at first use. */
 int mhip_tuning_save(const char* path);
 int mhip_tuning_load(const char* path);
 void mhip_tuning_clear(void);
 int mhip_tuning_count(void);
+/* The current device's key as it appears in the table (library-owned string). */
+const char* mhip_tuning_device(void);
 
 #ifdef __cplusplus
 }

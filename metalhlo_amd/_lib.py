@@ -53,10 +53,15 @@ SIGNATURES = {
     "mhip_argmax": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32]),
     "mhip_gemm_autotune": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _i32,
                                   _i32, _i32, C.POINTER(C.c_int), C.POINTER(C.c_float)]),
+    "mhip_row_autotune": (_i32, [_vp, _i32, _vp, _vp, _vp, _vp, _i64, _i64, C.c_float, _i32, _i32, C.POINTER(C.c_int),
+                                 C.POINTER(C.c_float)]),
+    "mhip_attention_autotune": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, C.c_float, _i32, _i32, _i32,
+                                       C.POINTER(C.c_int), C.POINTER(C.c_float)]),
     "mhip_tuning_save": (_i32, [C.c_char_p]),
     "mhip_tuning_load": (_i32, [C.c_char_p]),
     "mhip_tuning_clear": (None, []),
     "mhip_tuning_count": (_i32, []),
+    "mhip_tuning_device": (C.c_char_p, []),
 }
 
 _lib = None

@@ -349,8 +349,8 @@ static int launch_fa_scalar(hipStream_t s, FaArgs a, int D, float scale) {
 
 namespace mhip {
 // attention_pipe.hip: head size 128, four waves x 64 query rows, matrix / softmax overlap in one wave.
-bool fa_pipe_eligible(const FaArgs& a, int64_t D, int dtype, bool has_mask);
-int launch_fa_pipe(hipStream_t s, const FaArgs& a, int dtype, bool causal);
+bool fa_pipe_eligible(const FaArgs& a, int64_t D, int dtype, bool has_mask, int variant);
+int launch_fa_pipe(hipStream_t s, const FaArgs& a, int dtype, bool causal, int pair);
 }  // namespace mhip
 
 using namespace mhip;
@@ -401,7 +401,10 @@ static int fa_entry(const char* name, void* stream, const void* q, const void* k
     const bool fits = max_span * 2 < 0x7FFFFFFFLL;
     if (is16 && aligned && strides_aligned && fits && Skv > 0 && (D == 64 || D == 128)) {
         const bool hm = mask != nullptr;
-        if (is_packed && fa_pipe_eligible(a, D, dtype, hm)) return launch_fa_pipe(s, a, dtype, is_causal != 0);
+        // 0 = no tuned choice; 1 = 128-row kernel; 2 / 3 = 256-row pipelined kernel, causal tiles unpaired / paired
+        const int variant = is_packed ? tuned_attention_variant(dtype, B * H, Sq, Skv, D, is_causal != 0) : 0;
+        if (is_packed && fa_pipe_eligible(a, D, dtype, hm, variant))
+            return launch_fa_pipe(s, a, dtype, is_causal != 0, variant == 2 ? 0 : variant == 3 ? 1 : -1);
         if (dtype == MHIP_BF16)
             return D == 128 ? launch_fa<bf16_t, 128>(s, a, is_causal, hm)
                             : launch_fa<bf16_t, 64>(s, a, is_causal, hm);

@@ -48,6 +48,10 @@ struct RowLaunch { int kind = 0, r = 0, ordered = -1, per_cu = 0; };
 // The launch a tuning pass recorded for this problem on this device, if any (tuning.hip).
 bool tuned_row_launch(int op, int dtype, int64_t rows, int64_t cols, bool has_gamma, bool has_beta, RowLaunch* out);
 
+// The attention kernel a tuning pass recorded (or is timing) for this problem: 0 = none, 1 = the
+// 128-row kernel, 2 / 3 = the 256-row pipelined kernel with causal tiles unpaired / paired (tuning.hip).
+int tuned_attention_variant(int dtype, int64_t batch_heads, int64_t Sq, int64_t Skv, int64_t D, bool causal);
+
 // One launch of row operator `op` (0 softmax, 1 LayerNorm, 2 RMSNorm) carried out as `how` says.
 int row_launch_as(int op, const RowLaunch& how, void* stream, const void* x, const void* g, const void* b, void* y,
                   int64_t rows, int64_t cols, float eps, int dtype);

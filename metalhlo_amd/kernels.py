@@ -305,6 +305,40 @@ def autotune_matmul(a, b, bias=None, activation: str = "none", trans_a: bool = F
     return variant.value, us.value
 
 
+def autotune_row(op: str, x, gamma=None, beta=None, eps: float = 1e-5, iters: int = 10):
+    """Times the launch forms of a row operator ("softmax", "layer_norm", "rms_norm") for x
+    [rows, cols] and stores the fastest in the tuning table.  Returns ((kind, rows per wave
+    group, ordered, workgroups per CU), microseconds per launch)."""
+    _dev(x, gamma, beta)
+    lib = _lib.load()
+    code = {"softmax": 0, "layer_norm": 1, "rms_norm": 2}[op]
+    cols = x.shape[-1]
+    out = torch.empty_like(x)
+    choice, us = (C.c_int * 4)(), C.c_float(0.0)
+    _lib.check(lib.mhip_row_autotune(_stream(), code, x.data_ptr(), _ptr(gamma), _ptr(beta), out.data_ptr(),
+                                     x.numel() // cols, cols, float(eps), _code(x), int(iters), choice, C.byref(us)))
+    return tuple(choice), us.value
+
+
+def autotune_attention(q, k, v, scale=None, is_causal: bool = False, iters: int = 5):
+    """Times the attention kernels that can serve packed q [B,H,Sq,D], k, v [B,H,Skv,D] and stores
+    the fastest in the tuning table.  Returns (variant 1 | 2 | 3, microseconds per launch)."""
+    _dev(q, k, v)
+    lib = _lib.load()
+    B, H, Sq, D = q.shape
+    out = torch.empty_like(q)
+    variant, us = C.c_int(0), C.c_float(0.0)
+    _lib.check(lib.mhip_attention_autotune(_stream(), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), B, H, Sq,
+                                           k.shape[2], D, float(D ** -0.5 if scale is None else scale), int(is_causal),
+                                           _code(q), int(iters), C.byref(variant), C.byref(us)))
+    return variant.value, us.value
+
+
+def tuning_device() -> str:
+    """The current device's key in the tuning table (architecture name / compute units)."""
+    return _lib.load().mhip_tuning_device().decode()
+
+
 def tuning_save(path: str) -> None:
     _lib.check(_lib.load().mhip_tuning_save(str(path).encode()))
 
