@@ -57,7 +57,9 @@ typedef enum {
     MHIP_ACT_GELU = 2, /* tanh approximation, CustomCallHandlers.swift:540-558 */
     MHIP_ACT_SILU = 3,
     MHIP_ACT_TANH = 4,
-    MHIP_ACT_SIGMOID = 5
+    MHIP_ACT_SIGMOID = 5,
+    MHIP_ACT_GELU_ERF = 6 /* 0.5 x (1 + erf(x / sqrt 2)): what "gelu_exact" names (CustomCallHandlers.swift:893-894;
+                            the reference falls back to the tanh form there, :540-558, this build does not) */
 } mhip_activation;
 
 /* Library / device ------------------------------------------------------- */
@@ -108,6 +110,11 @@ int mhip_rms_norm(void* stream, const void* x, const void* gamma, void* y, int64
  * of generateMatMulBiasActSource (Compiler/CodeGenerator.swift:4797-4850). */
 int mhip_bias_gelu(void* stream, const void* x, const void* bias, void* y, int64_t rows,
                    int64_t cols, int dtype);
+/* The same with the exact form 0.5 v (1 + erf(v / sqrt 2)), v = x + bias: what a decomposed
+ * erf GELU (jax.nn.gelu(approximate=False)) is rewritten to.  The reference has no kernel for it
+ * (Metal/Kernels/GELUKernel.swift:15-123 is the tanh form only). */
+int mhip_bias_gelu_erf(void* stream, const void* x, const void* bias, void* y, int64_t rows,
+                       int64_t cols, int dtype);
 
 /* dot_general ------------------------------------------------------------ */
 

@@ -24,6 +24,7 @@ SIGNATURES = {
     "mhip_layer_norm": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _f32, _i32]),
     "mhip_rms_norm": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _f32, _i32]),
     "mhip_bias_gelu": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i32]),
+    "mhip_bias_gelu_erf": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i32]),
     "mhip_gemm": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
                          _i32, _i32, _i32, _i32]),
     "mhip_gemm_residual": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64,

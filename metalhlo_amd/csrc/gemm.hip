@@ -480,7 +480,7 @@ static int gemm_entry(void* stream, const void* a, const void* b, const void* bi
                       int activation, int dtype) {
     if (M < 0 || N < 0 || K < 0 || batch < 0)
         return fail(MHIP_ERR_INVALID_ARGUMENT, "mhip_gemm: negative size");
-    if (activation < MHIP_ACT_NONE || activation > MHIP_ACT_SIGMOID)
+    if (activation < MHIP_ACT_NONE || activation > MHIP_ACT_GELU_ERF)
         return fail(MHIP_ERR_INVALID_ARGUMENT, "mhip_gemm: unknown activation %d", activation);
     if (M == 0 || N == 0 || batch == 0) return MHIP_OK;
     if (!a || !b || !c) return fail(MHIP_ERR_INVALID_ARGUMENT, "mhip_gemm: NULL matrix pointer");

@@ -51,6 +51,7 @@ __device__ inline float apply_act(float v, int act) {
         case MHIP_ACT_SILU: return v / (1.f + expf(-v));
         case MHIP_ACT_TANH: return tanhf(v);
         case MHIP_ACT_SIGMOID: return 1.f / (1.f + expf(-v));
+        case MHIP_ACT_GELU_ERF: return 0.5f * v * (1.f + erff(v * 0.7071067811865476f));
         default: return v;
     }
 }
@@ -78,6 +79,7 @@ __device__ inline float apply_act_c(float v) {
     if (ACT == MHIP_ACT_SILU) r = v * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-kLog2e * v));
     if (ACT == MHIP_ACT_SIGMOID) r = __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-kLog2e * v));
     if (ACT == MHIP_ACT_TANH) r = 1.f - 2.f * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(2.f * kLog2e * v));
+    if (ACT == MHIP_ACT_GELU_ERF) r = 0.5f * v * (1.f + erff(v * 0.7071067811865476f));
     // The fp32 result is final here.  Without this the compiler may merge the last multiply with
     // the conversion to f16 that follows (one rounding instead of two) in some kernels and not in
     // others, and the same problem would round differently depending on the tile choice.
@@ -107,6 +109,7 @@ __device__ inline void dispatch_act(int act, F&& f) {
         case MHIP_ACT_SILU: f(std::integral_constant<int, MHIP_ACT_SILU>{}); break;
         case MHIP_ACT_TANH: f(std::integral_constant<int, MHIP_ACT_TANH>{}); break;
         case MHIP_ACT_SIGMOID: f(std::integral_constant<int, MHIP_ACT_SIGMOID>{}); break;
+        case MHIP_ACT_GELU_ERF: f(std::integral_constant<int, MHIP_ACT_GELU_ERF>{}); break;
         default: f(std::integral_constant<int, MHIP_ACT_NONE>{}); break;
     }
 }

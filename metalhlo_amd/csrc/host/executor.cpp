@@ -153,10 +153,12 @@ static const std::map<std::string, int> kReduce = {{"add", MHIP_RED_SUM}, {"maxi
                                                    {"minimum", MHIP_RED_MIN}, {"multiply", MHIP_RED_PROD}};
 static const std::map<std::string, int> kActivation = {{"none", MHIP_ACT_NONE}, {"relu", MHIP_ACT_RELU},
                                                        {"gelu", MHIP_ACT_GELU}, {"silu", MHIP_ACT_SILU},
-                                                       {"tanh", MHIP_ACT_TANH}, {"sigmoid", MHIP_ACT_SIGMOID}};
+                                                       {"tanh", MHIP_ACT_TANH}, {"sigmoid", MHIP_ACT_SIGMOID},
+                                                       {"gelu_approximate", MHIP_ACT_GELU}, {"geluApproximate", MHIP_ACT_GELU},
+                                                       {"swish", MHIP_ACT_SILU}, {"gelu_exact", MHIP_ACT_GELU_ERF}};
 // custom_call targets served by a kernel (Compiler/CustomCallHandlers.swift:75-89)
 static const char* kTargets[] = {"fused_scaled_dot_product_attention", "fused_layer_norm", "fused_rms_norm",
-                                 "fused_softmax", "fused_gelu", "fused_matmul_bias_activation"};
+                                 "fused_softmax", "fused_gelu", "fused_matmul_bias_activation", "fused_ffn"};
 
 static std::string where(const Op& op) { return "line " + std::to_string(op.line) + " (stablehlo." + op.name + "): "; }
 
@@ -408,6 +410,15 @@ static void check_custom_call_types(const Op& op, const std::vector<TensorType>&
         if (has_res && op.operands.size() < 3) throw ParseError(where(op) + "has_residual without a residual operand");
         if (n_plain > 2 && in(2).numel() != N) throw ParseError(where(op) + "bias must be [N] of the input type");
         if (has_res && !(in(op.operands.size() - 1) == op.out)) throw ParseError(where(op) + "the residual must have the result's type");
+    } else if (op.target == "fused_ffn") {
+        // x [.., M, d], up [d, F], down [F, d2] -> [.., M, d2]  (CustomCallHandlers.swift:861-882)
+        const TensorType &up = in(1), &down = in(2);
+        if (xt.shape.size() < 2 || up.shape.size() != 2 || down.shape.size() != 2 || up.shape[0] != cols || down.shape[0] != up.shape[1])
+            throw ParseError(where(op) + "expected x [.., M, d], up [d, F] and down [F, d2]");
+        std::vector<int64_t> want(xt.shape.begin(), xt.shape.end() - 1);
+        want.push_back(down.shape[1]);
+        if (op.out.shape != want) throw ParseError(where(op) + "the result shape is not [.., M, d2]");
+        if (cfg.get_bool("is_gated", false)) throw UnsupportedOp(where(op) + "gated feed-forward blocks are not supported");
     } else if (op.target == "fused_scaled_dot_product_attention" && cfg.get_int_array("views", {}).empty()) {
         const TensorType& kt = in(1);
         const size_t r = xt.shape.size();
@@ -517,13 +528,15 @@ void compile(Executable& exe) {
             bool ok = false;
             for (auto t : kTargets) ok |= op.target == t;
             if (!ok) throw UnsupportedOp(where(op) + "Unsupported custom call target: " + op.target);
-            const size_t need = op.target == "fused_scaled_dot_product_attention" || op.target == "fused_layer_norm" ? 3
+            const size_t need = op.target == "fused_scaled_dot_product_attention" || op.target == "fused_layer_norm" || op.target == "fused_ffn" ? 3
                               : op.target == "fused_rms_norm" || op.target == "fused_matmul_bias_activation" ? 2 : 1;
             if (op.operands.size() < need)
                 throw ParseError(where(op) + "Invalid input count: expected " + std::to_string(need) + ", got " + std::to_string(op.operands.size()));
             if (!is_kernel_float(in(0).dtype)) throw UnsupportedOp(where(op) + "element type not supported");
             if (op.target == "fused_matmul_bias_activation" &&
                 !kActivation.count(parse_config(op.backend_config).get_string("activation", "none")))
+                throw UnsupportedOp(where(op) + "unknown activation");
+            if (op.target == "fused_ffn" && !kActivation.count(parse_config(op.backend_config).get_string("activation", "gelu")))
                 throw UnsupportedOp(where(op) + "unknown activation");
             check_custom_call_types(op, vt);
         } else {
@@ -693,7 +706,19 @@ static std::vector<DeviceTensor> run_ops(Executable& exe, const std::vector<Devi
                     for (int64_t d = axis + 1; d < (int64_t)xt.shape.size(); d++) inner *= xt.shape[d];
                     RUN(mhip_softmax_strided(s, in(0).data(), out.data(), outer, xt.shape[axis], inner, dt));
                 } else if (op.target == "fused_gelu") {
-                    RUN(mhip_bias_gelu(s, in(0).data(), nullptr, out.data(), rows, cols, dt));
+                    // "approximate": false alone means the tanh form too, as in the reference
+                    // (CustomCallHandlers.swift:694-707); the recogniser marks a decomposed erf GELU
+                    // with "erf": true, which runs the exact form
+                    if (cfg.get_bool("erf", false)) RUN(mhip_bias_gelu_erf(s, in(0).data(), nullptr, out.data(), rows, cols, dt));
+                    else RUN(mhip_bias_gelu(s, in(0).data(), nullptr, out.data(), rows, cols, dt));
+                } else if (op.target == "fused_ffn") {
+                    // act(x . up) . down: two GEMMs, the hidden activations in a temporary
+                    const TensorType &up = in(1).type, &down = in(2).type;
+                    const int64_t F = up.shape[1], d2 = down.shape[1];
+                    DeviceTensor hidden = al.allocate(TensorType{{rows, F}, dt});
+                    RUN(mhip_gemm(s, in(0).data(), in(1).data(), nullptr, hidden.data(), rows, F, cols, 1, 0, 0, 0, 0, 0,
+                                  kActivation.at(cfg.get_string("activation", "gelu")), dt));
+                    RUN(mhip_gemm(s, hidden.data(), in(2).data(), nullptr, out.data(), rows, d2, F, 1, 0, 0, 0, 0, 0, MHIP_ACT_NONE, dt));
                 } else if (op.target == "fused_layer_norm" || op.target == "fused_rms_norm") {
                     const auto axes = cfg.get_int_array("axes", {-1});
                     if (axes.size() != 1 || (axes[0] != -1 && axes[0] != (int64_t)xt.shape.size() - 1))

@@ -212,7 +212,18 @@ struct Rewriter {
         const Op* s = reduce_over(sum, "add", ax_s, e_in);
         if (!s || e_in != e->result || ax_s != ax_b) return false;
         const Op* sh = op_named(e->operands[0], "subtract");
-        if (!sh) return false;
+        if (!sh) {
+            // exp(x) / sum(exp(x)) without the shift by the row maximum: the same function wherever the
+            // spelled form does not overflow (the fused kernel always shifts, so it stays finite there too)
+            x = e->operands[0];
+            if (!(type.at(x) == root.out)) return false;
+            in.insert(index_of(s));
+            if (!closed(in, ri)) return false;
+            char cfg0[64];
+            snprintf(cfg0, sizeof cfg0, "{\"axis\": %lld}", (long long)ax_s);
+            replace(ri, in, "fused_softmax", {x}, cfg0);
+            return true;
+        }
         const int mx = spread_src(sh->operands[1], ax_b, in);
         if (mx < 0) return false;
         const Op* m = reduce_over(mx, "maximum", ax_m, x);
@@ -314,6 +325,56 @@ struct Rewriter {
         return true;
     }
 
+    // ------------------------------------------------------------------ GELU (erf form)
+    // x * (1 + erf(x / sqrt 2)) * 0.5 in any association and operand order, the last factor also as
+    // a division by 2, the erf argument as x * (1 / sqrt 2) or x / sqrt 2: what
+    // jax.nn.gelu(approximate=False) lowers to.  It becomes a fused_gelu marked "erf": true, which
+    // runs the exact function (not the tanh approximation the reference substitutes).
+    bool gelu_erf(size_t ri) {
+        const Op& root = fn.ops[ri];
+        if (!fused_float(root.out.dtype)) return false;
+        const int dt = root.out.dtype;
+        std::set<size_t> in = {ri};
+        std::vector<int> leaves;
+        int halves = 0;
+        if (root.name == "divide") {                     // (...) / 2
+            double c;
+            if (!splat_value(root.operands[1], c) || c != 2.0) return false;
+            halves = 1;
+            product_leaves(root.operands[0], uses(root.operands[0]) == 1, leaves, in);
+        } else if (root.name == "multiply") {
+            product_leaves(root.result, true, leaves, in);
+        } else {
+            return false;
+        }
+        int x = -1, er = -1;
+        for (int v : leaves) {
+            double c;
+            int inner;
+            std::set<size_t> tmp;
+            if (splat_value(v, c) && c == 0.5) halves++;
+            else if (add_const(v, 1.0, 0.0, inner, tmp) && op_named(inner, "erf")) { er = inner; in.insert(tmp.begin(), tmp.end()); }
+            else if (x < 0) x = v;
+            else return false;
+        }
+        if (halves != 1 || x < 0 || er < 0 || leaves.size() != (root.name == "divide" ? 2u : 3u)) return false;
+        const Op* e = op_named(er, "erf");
+        in.insert(index_of(e));
+        const Op* arg = op_of(e->operands[0]);
+        if (!arg || (arg->name != "multiply" && arg->name != "divide")) return false;
+        in.insert(index_of(arg));
+        bool ok = false;
+        for (int k = 0; k < 2 && !ok; k++) {
+            if (arg->name == "divide" && k == 0) continue;          // x / sqrt 2: the constant is the divisor
+            double c;
+            if (arg->operands[1 - k] != x || !splat_value(arg->operands[k], c)) continue;
+            ok = arg->name == "divide" ? is_const(c, 1.4142135623730951, dt) : is_const(c, 0.7071067811865476, dt);
+        }
+        if (!ok || !(type.at(x) == root.out) || !closed(in, ri)) return false;
+        replace(ri, in, "fused_gelu", {x}, "{\"approximate\": false, \"erf\": true}");
+        return true;
+    }
+
     // ------------------------------------------------------------------ LayerNorm / RMSNorm
     // mean over the last axis: reduce_add(u) / N  or  reduce_add(u) * (1/N)
     bool mean_last(int v, int& u, std::set<size_t>& nodes) const {
@@ -348,6 +409,36 @@ struct Rewriter {
         nodes = t;
         return src;
     }
+    // The variance spelled mean(x * x) - mean(x) * mean(x) (the one-pass form jax.numpy.var and
+    // flax's LayerNorm with use_fast_variance emit), with `c` = x - bcast(mean(x)) of the same
+    // mean.  The fused kernel computes the two-pass variance: the same quantity without the
+    // cancellation of the spelled form.
+    bool one_pass_variance(int var, int c, size_t rank, const std::set<size_t>& base, int& x, std::set<size_t>& nodes) const {
+        std::set<size_t> t = base;
+        const Op* vs = op_named(relabel_src(var, t), "subtract");
+        if (!vs) return false;
+        int sq;
+        if (!mean_last(vs->operands[0], sq, t)) return false;
+        const Op* sqo = op_named(sq, "multiply");
+        if (!sqo || sqo->operands[0] != sqo->operands[1]) return false;
+        const int xx = sqo->operands[0];
+        const Op* m2 = op_named(relabel_src(vs->operands[1], t), "multiply");
+        if (!m2 || m2->operands[0] != m2->operands[1]) return false;
+        int mx;
+        if (!mean_last(m2->operands[0], mx, t) || mx != xx) return false;
+        const Op* sub = op_named(c, "subtract");
+        if (!sub || sub->operands[0] != xx) return false;
+        const int spread = spread_last(sub->operands[1], rank, t);
+        std::set<size_t> scratch;
+        if (spread < 0 || relabel_src(spread, scratch) != relabel_src(m2->operands[0], scratch)) return false;
+        t.insert(index_of(vs));
+        t.insert(index_of(sqo));
+        t.insert(index_of(m2));
+        t.insert(index_of(sub));
+        x = xx;
+        nodes.insert(t.begin(), t.end());
+        return true;
+    }
     // v = c * bcast(rsqrt(mean(c*c) + eps)); centred: c = x - bcast(mean(x))
     bool norm_core(int v, int& x, double& eps, bool& centred, std::set<size_t>& nodes) const {
         const Op* m = op_named(v, "multiply");
@@ -370,6 +461,11 @@ struct Rewriter {
                 int sq;
                 std::set<size_t> t2 = tmp;
                 if (!splat_value(ve->operands[j], e) || !(e > 0 && e < 1e-1)) continue;
+                if (one_pass_variance(ve->operands[1 - j], c, rank, tmp, x, nodes)) {   // mean(x^2) - mean(x)^2
+                    centred = true;
+                    eps = e;
+                    return true;
+                }
                 if (!mean_last(ve->operands[1 - j], sq, t2)) continue;
                 const Op* sqo = op_named(sq, "multiply");
                 if (!sqo || sqo->operands[0] != c || sqo->operands[1] != c) continue;
@@ -688,11 +784,23 @@ struct Rewriter {
             int src = -1;
             if (root.name == "tanh") { act = "tanh"; src = root.operands[0]; }
             else if (root.name == "logistic") { act = "sigmoid"; src = root.operands[0]; }
-            else if (root.name == "custom_call" && root.target == "fused_gelu") { act = "gelu"; src = root.operands[0]; }
+            else if (root.name == "custom_call" && root.target == "fused_gelu") {
+                act = parse_config(root.backend_config).get_bool("erf", false) ? "gelu_exact" : "gelu";
+                src = root.operands[0];
+            }
             else if (root.name == "maximum") {
                 double c;
                 for (int k = 0; k < 2; k++)
                     if (splat_value(root.operands[k], c) && c == 0.0) { act = "relu"; src = root.operands[1 - k]; }
+            } else if (root.name == "multiply") {          // h * logistic(h): SiLU
+                for (int k = 0; k < 2; k++) {
+                    const Op* lg = op_named(root.operands[k], "logistic");
+                    if (lg && lg->operands[0] == root.operands[1 - k] && uses(lg->result) == 1) {
+                        act = "silu";
+                        src = root.operands[1 - k];
+                        in.insert(index_of(lg));
+                    }
+                }
             }
             if (src < 0) return false;
             add = op_named(src, "add");
@@ -770,7 +878,7 @@ int fuse_patterns(Function& fn) {
     // malformed operations are reported by the validation that follows; do not look inside them
     static const std::map<std::string, size_t> kArity = {
         {"add", 2}, {"subtract", 2}, {"multiply", 2}, {"divide", 2}, {"maximum", 2}, {"minimum", 2}, {"dot", 2},
-        {"dot_general", 2}, {"reduce", 2}, {"exponential", 1}, {"tanh", 1}, {"rsqrt", 1}, {"logistic", 1},
+        {"dot_general", 2}, {"reduce", 2}, {"exponential", 1}, {"tanh", 1}, {"rsqrt", 1}, {"logistic", 1}, {"erf", 1},
         {"broadcast_in_dim", 1}, {"reshape", 1}, {"convert", 1}, {"transpose", 1}};
     for (const Op& op : fn.ops) {
         auto it = kArity.find(op.name);
@@ -779,7 +887,7 @@ int fuse_patterns(Function& fn) {
             if (v < 0 || v >= fn.num_values) return 0;
     }
     Rewriter rw(fn);
-    rw.pass([&](size_t i) { rw.softmax(i) || rw.gelu(i) || rw.norm(i); });
+    rw.pass([&](size_t i) { rw.softmax(i) || rw.gelu(i) || rw.gelu_erf(i) || rw.norm(i); });
     rw.pass([&](size_t i) { rw.attention(i) || rw.matmul_bias_act(i); });
     rw.pass([&](size_t i) { rw.attention_views(i) || rw.matmul_residual(i); });
     return rw.fused;

@@ -53,6 +53,10 @@ struct Op {
     std::vector<int64_t> starts, limits, strides;   // slice
     int64_t iota_dim = 0;
     std::string target, backend_config, direction, reducer;
+    // `call` only, and only until parse_module has inlined it: the other results of a
+    // multi-result call (`%r:2 = call ...`, used as %r#0, %r#1) and all result types
+    std::vector<int> more_results;
+    std::vector<TensorType> out_types;
     std::vector<uint8_t> constant;    // dense bytes in `out` layout (splat already expanded)
     bool splat = false;
     uint64_t splat_bits = 0;
@@ -69,8 +73,10 @@ struct Function {
     int num_values = 0;
 };
 
-// Parses a module (or a bare func.func) and returns its entry function
-// (`main` when present, else the first).  Throws ParseError / UnsupportedOp.
+// Parses a module (or a bare func.func) and returns its entry function (`main` when present,
+// else the first) with every `call` / `func.call` of another function of the module inlined
+// (the reference resolves callees the same way, Parser/Parser.swift:31-226; tracing front ends
+// emit private helper functions such as @_where routinely).  Throws ParseError / UnsupportedOp.
 Function parse_module(const std::string& text);
 
 // Rewrites decomposed softmax / GELU(tanh) / LayerNorm / RMSNorm / attention /

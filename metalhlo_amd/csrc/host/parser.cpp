@@ -321,7 +321,10 @@ struct Parser {
             if (t[i] == '%') {
                 size_t j = i + 1;
                 while (j < t.size() && (isalnum((unsigned char)t[j]) || t[j] == '_' || t[j] == '.' || t[j] == '$' || t[j] == '-')) j++;
-                if (j < t.size() && t[j] == '#') fail("multi-result values (" + t.substr(i, j - i + 2) + ") are not supported");
+                if (j < t.size() && t[j] == '#') {        // %r#1: result 1 of a multi-result op
+                    j++;
+                    while (j < t.size() && isdigit((unsigned char)t[j])) j++;
+                }
                 r.push_back(t.substr(i, j - i));
                 i = j - 1;
             }
@@ -360,9 +363,11 @@ struct Parser {
             } else {
                 outs.push_back(parse_type(sig, q, line));
             }
-            if (outs.size() != 1) throw UnsupportedOp("line " + std::to_string(line) + ": ops with " + std::to_string(outs.size()) + " results are not supported");
+            if (outs.size() != 1 && op.name != "call")
+                throw UnsupportedOp("line " + std::to_string(line) + ": ops with " + std::to_string(outs.size()) + " results are not supported");
             op.in_types = ins;
-            op.out = outs[0];
+            if (!outs.empty()) op.out = outs[0];
+            op.out_types = outs;
         } else {
             while (q < sig.size()) {
                 ws();
@@ -534,7 +539,6 @@ struct Parser {
             const size_t eq = t.find('=');
             if (eq == std::string::npos) fail("expected '=' after the result name");
             result = trim(t.substr(0, eq));
-            if (result.find(':') != std::string::npos) throw UnsupportedOp("line " + std::to_string(line) + ": multi-result op " + result);
             t = trim(t.substr(eq + 1));
         }
         std::string name;
@@ -547,9 +551,27 @@ struct Parser {
             while (q < t.size() && !isspace((unsigned char)t[q]) && t[q] != '(') q++;
             name = t.substr(0, q);
         }
-        for (const char* pre : {"stablehlo.", "mhlo.", "chlo."})
+        for (const char* pre : {"stablehlo.", "mhlo.", "chlo.", "func."})
             if (starts_with(name, pre)) { name = name.substr(strlen(pre)); break; }
         op.name = name;
+        // `%r:2 = call ...` defines %r#0 and %r#1; `%a, %b = call ...` names them one by one
+        std::vector<std::string> result_names;
+        if (!result.empty()) {
+            const size_t colon = result.find(':');
+            if (colon != std::string::npos || result.find(',') != std::string::npos) {
+                if (name != "call") throw UnsupportedOp("line " + std::to_string(line) + ": multi-result op " + result);
+                if (colon != std::string::npos) {
+                    const int n = atoi(result.c_str() + colon + 1);
+                    const std::string base = trim(result.substr(0, colon));
+                    if (n < 1 || n > 64) fail("bad result count in " + result);
+                    for (int i = 0; i < n; i++) result_names.push_back(base + "#" + std::to_string(i));
+                } else {
+                    result_names = value_refs(result);
+                }
+            } else {
+                result_names.push_back(result);
+            }
+        }
         const std::string rest = t.substr(q);
         const size_t c = top_level_colon(rest);
         if (c == std::string::npos) fail("op '" + name + "' has no type signature");
@@ -571,9 +593,24 @@ struct Parser {
             outer = outer.substr(0, r0) + outer.substr(close + 1);
         }
         for (auto& v : value_refs(outer)) op.operands.push_back(value_id(v, false));
+        if (name == "call") {
+            const size_t at = op.attrs.find('@');
+            if (at == std::string::npos) fail("call without a callee");
+            size_t e = at + 1;
+            while (e < op.attrs.size() && (isalnum((unsigned char)op.attrs[e]) || op.attrs[e] == '_' || op.attrs[e] == '.' || op.attrs[e] == '$')) e++;
+            op.target = op.attrs.substr(at + 1, e - at - 1);
+            if (op.out_types.size() != result_names.size())
+                fail("call @" + op.target + " names " + std::to_string(result_names.size()) + " results, its signature has " +
+                     std::to_string(op.out_types.size()));
+            if (result_names.empty()) return;              // a call without results computes nothing here
+            op.result = value_id(result_names[0], true);
+            for (size_t i = 1; i < result_names.size(); i++) op.more_results.push_back(value_id(result_names[i], true));
+            fn.ops.push_back(std::move(op));
+            return;
+        }
         decode_attrs(op);
-        if (result.empty()) fail("op '" + name + "' has no result");
-        op.result = value_id(result, true);
+        if (result_names.empty()) fail("op '" + name + "' has no result");
+        op.result = value_id(result_names[0], true);
         fn.ops.push_back(std::move(op));
     }
 
@@ -657,14 +694,71 @@ struct Parser {
 
 }  // namespace
 
+// Replaces every call in `f` by the callee's operations (callees inlined first; recursion is an
+// error): the callee's arguments become the call's operands, its other values get fresh ids in the
+// caller, and uses of the call's results become uses of the values the callee returns.
+static void inline_calls(Function& f, const std::map<std::string, Function>& all, std::vector<std::string>& stack) {
+    bool any = false;
+    for (auto& op : f.ops) any |= op.name == "call";
+    if (!any) return;
+    if (stack.size() > 64) throw ParseError("calls nested deeper than 64 functions");
+    stack.push_back(f.name);
+    std::vector<Op> out;
+    std::map<int, int> subst;          // caller value -> the value that replaces it
+    auto mapped = [&](int v) { auto it = subst.find(v); return it == subst.end() ? v : it->second; };
+    for (auto& op : f.ops) {
+        for (int& v : op.operands) v = mapped(v);
+        if (op.name != "call") { out.push_back(std::move(op)); continue; }
+        auto it = all.find(op.target);
+        if (it == all.end()) throw ParseError("line " + std::to_string(op.line) + ": call of unknown function @" + op.target);
+        for (auto& s : stack)
+            if (s == op.target) throw ParseError("line " + std::to_string(op.line) + ": recursive call of @" + op.target);
+        Function callee = it->second;
+        inline_calls(callee, all, stack);
+        if (callee.arg_ids.size() != op.operands.size())
+            throw ParseError("line " + std::to_string(op.line) + ": @" + op.target + " takes " + std::to_string(callee.arg_ids.size()) +
+                             " arguments, the call passes " + std::to_string(op.operands.size()));
+        if (callee.returns.size() != op.out_types.size())
+            throw ParseError("line " + std::to_string(op.line) + ": @" + op.target + " returns " + std::to_string(callee.returns.size()) +
+                             " values, the call expects " + std::to_string(op.out_types.size()));
+        for (size_t i = 0; i < callee.arg_types.size(); i++)
+            if (!op.in_types.empty() && i < op.in_types.size() && !(op.in_types[i] == callee.arg_types[i]))
+                throw ParseError("line " + std::to_string(op.line) + ": argument " + std::to_string(i) + " of @" + op.target + " has another type");
+        std::map<int, int> local;      // callee value -> caller value
+        for (size_t i = 0; i < callee.arg_ids.size(); i++) local[callee.arg_ids[i]] = op.operands[i];
+        for (auto& c : callee.ops) {
+            Op n = c;
+            for (int& v : n.operands) v = local.at(v);
+            n.result = f.num_values++;
+            local[c.result] = n.result;
+            out.push_back(std::move(n));
+        }
+        std::vector<int> results = {op.result};
+        results.insert(results.end(), op.more_results.begin(), op.more_results.end());
+        for (size_t i = 0; i < results.size(); i++) {
+            if (!(callee.result_types.empty() || callee.result_types[i] == op.out_types[i]))
+                throw ParseError("line " + std::to_string(op.line) + ": result " + std::to_string(i) + " of @" + op.target + " has another type");
+            subst[results[i]] = local.at(callee.returns[i]);
+        }
+    }
+    for (int& r : f.returns) r = mapped(r);
+    f.ops = std::move(out);
+    stack.pop_back();
+}
+
 Function parse_module(const std::string& text) {
     Parser ps(text);
     std::vector<Function> fns;
     while (ps.parse_function()) fns.push_back(ps.fn);
     if (fns.empty()) throw ParseError("no func.func found in the module");
+    std::map<std::string, Function> all;
+    for (auto& f : fns) all.emplace(f.name, f);
+    Function* entry = &fns[0];
     for (auto& f : fns)
-        if (f.name == "main") return f;
-    return fns[0];
+        if (f.name == "main") { entry = &f; break; }
+    std::vector<std::string> stack;
+    inline_calls(*entry, all, stack);
+    return *entry;
 }
 
 // ---------------------------------------------------------------- backend_config

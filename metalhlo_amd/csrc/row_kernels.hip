@@ -493,8 +493,10 @@ __global__ __launch_bounds__(256) void softmax_strided_kernel(const T* __restric
 // ---------------------------------------------------------------------------
 // bias + GELU(tanh): pure streaming; the bias sits in LDS as fp32 planes.
 // ---------------------------------------------------------------------------
-template <typename T>
+// EXACT: 0.5 v (1 + erf(v / sqrt 2)) with the library's erff; otherwise the tanh approximation.
+template <typename T, bool EXACT = false>
 __device__ inline float gelu_tanh_f(float v) {
+    if (EXACT) return 0.5f * v * (1.f + erff(v * 0.7071067811865476f));
     if (sizeof(T) == 4) {
         const float inner = 0.7978845608028654f * (v + 0.044715f * v * v * v);
         return 0.5f * v * (1.f + tanhf(inner));
@@ -507,7 +509,7 @@ __device__ inline float gelu_tanh_f(float v) {
     return v * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(t));
 }
 
-template <typename T>
+template <typename T, bool EXACT>
 __global__ __launch_bounds__(256) void bias_gelu_vec_kernel(const T* __restrict__ x,
                                                             const T* __restrict__ bias,
                                                             T* __restrict__ y, int64_t nvec,
@@ -546,7 +548,7 @@ __global__ __launch_bounds__(256) void bias_gelu_vec_kernel(const T* __restrict_
 #pragma unroll
                 for (int e = 0; e < 4; e++)
                     o.v[4 * q + e] = Elem<T>::from_f32(
-                        gelu_tanh_f<T>(Elem<T>::to_f32(in.v[4 * q + e]) + bv[e]));
+                        gelu_tanh_f<T, EXACT>(Elem<T>::to_f32(in.v[4 * q + e]) + bv[e]));
             }
             store16_stream(y + i * E, o);
         }
@@ -556,7 +558,7 @@ __global__ __launch_bounds__(256) void bias_gelu_vec_kernel(const T* __restrict_
 // Tiles of R rows x 256 vectors, one workgroup each, workgroups in address order (the grid is
 // one-dimensional: row tile major, column block minor).  A thread keeps one column of the tile:
 // its bias vector is read once, the R loads are issued together, no index arithmetic per vector.
-template <typename T, int R>
+template <typename T, int R, bool EXACT>
 __global__ __launch_bounds__(256) void bias_gelu_tile_kernel(const T* __restrict__ x,
                                                              const T* __restrict__ bias,
                                                              T* __restrict__ y, int64_t rows,
@@ -580,13 +582,13 @@ __global__ __launch_bounds__(256) void bias_gelu_tile_kernel(const T* __restrict
             Vec16<T> o;
 #pragma unroll
             for (int e = 0; e < E; e++)
-                o.v[e] = Elem<T>::from_f32(gelu_tanh_f<T>(Elem<T>::to_f32(in[r].v[e]) + Elem<T>::to_f32(bv.v[e])));
+                o.v[e] = Elem<T>::from_f32(gelu_tanh_f<T, EXACT>(Elem<T>::to_f32(in[r].v[e]) + Elem<T>::to_f32(bv.v[e])));
             store16_stream(y + ((r0 + r) * nvec_row + c) * E, o);
         }
     }
 }
 
-template <typename T>
+template <typename T, bool EXACT>
 __global__ __launch_bounds__(256) void bias_gelu_scalar_kernel(const T* __restrict__ x,
                                                                const T* __restrict__ bias,
                                                                T* __restrict__ y, int64_t n,
@@ -595,7 +597,7 @@ __global__ __launch_bounds__(256) void bias_gelu_scalar_kernel(const T* __restri
     if (i >= n) return;
     float v = Elem<T>::to_f32(x[i]);
     if (bias) v += Elem<T>::to_f32(bias[i % cols]);
-    y[i] = Elem<T>::from_f32(gelu_tanh_f<T>(v));
+    y[i] = Elem<T>::from_f32(gelu_tanh_f<T, EXACT>(v));
 }
 
 // ---------------------------------------------------------------------------
@@ -706,7 +708,7 @@ static int row_entry(const char* name, void* stream, const void* x, const void* 
     }
 }
 
-template <typename T>
+template <typename T, bool EXACT>
 static int launch_gelu(hipStream_t s, const void* x, const void* bias, void* y, int64_t rows,
                        int64_t cols) {
     constexpr int E = Elem<T>::kPerVec;
@@ -724,7 +726,7 @@ static int launch_gelu(hipStream_t s, const void* x, const void* bias, void* y, 
         const int64_t tiles = bpr * ((rows + tile_rows - 1) / tile_rows);
         if (tiles <= 0x7FFFFFFFLL) {
 #define MHIP_GELU_TILE(R)                                                                              \
-    hipLaunchKernelGGL((bias_gelu_tile_kernel<T, R>), dim3((unsigned)tiles), dim3(256), 0, s, static_cast<const T*>(x), \
+    hipLaunchKernelGGL((bias_gelu_tile_kernel<T, R, EXACT>), dim3((unsigned)tiles), dim3(256), 0, s, static_cast<const T*>(x), \
                        static_cast<const T*>(bias), static_cast<T*>(y), rows, (int)nvec_row, (unsigned)bpr)
             if (tile_rows == 1) MHIP_GELU_TILE(1);
             else if (tile_rows == 2) MHIP_GELU_TILE(2);
@@ -734,7 +736,7 @@ static int launch_gelu(hipStream_t s, const void* x, const void* bias, void* y, 
             const int64_t want = (nvec + 511) / 512;
             const int64_t cap = (int64_t)compute_units() * tune_int("MHIP_GELU_BLOCKS_PER_CU", 64);
             const bool in_lds = bias && cols * sizeof(float) <= 48 * 1024;
-            hipLaunchKernelGGL((bias_gelu_vec_kernel<T>), dim3((unsigned)(want < cap ? want : cap)), dim3(256),
+            hipLaunchKernelGGL((bias_gelu_vec_kernel<T, EXACT>), dim3((unsigned)(want < cap ? want : cap)), dim3(256),
                                in_lds ? (size_t)cols * sizeof(float) : 0, s, static_cast<const T*>(x),
                                static_cast<const T*>(bias), static_cast<T*>(y), nvec, (int)nvec_row,
                                in_lds ? 1 : 0);
@@ -742,7 +744,7 @@ static int launch_gelu(hipStream_t s, const void* x, const void* bias, void* y, 
     } else {
         const int64_t grid = (n + 255) / 256;
         if (grid > 0x7FFFFFFFLL) return fail(MHIP_ERR_UNSUPPORTED, "bias_gelu: tensor too large");
-        hipLaunchKernelGGL((bias_gelu_scalar_kernel<T>), dim3((unsigned)grid), dim3(256), 0, s,
+        hipLaunchKernelGGL((bias_gelu_scalar_kernel<T, EXACT>), dim3((unsigned)grid), dim3(256), 0, s,
                            static_cast<const T*>(x), static_cast<const T*>(bias),
                            static_cast<T*>(y), n, cols);
     }
@@ -780,18 +782,29 @@ extern "C" int mhip_rms_norm(void* stream, const void* x, const void* gamma, voi
     return row_entry<kRmsNorm>("mhip_rms_norm", stream, x, gamma, nullptr, y, rows, cols, eps, dtype);
 }
 
-extern "C" int mhip_bias_gelu(void* stream, const void* x, const void* bias, void* y, int64_t rows,
-                              int64_t cols, int dtype) {
-    if (rows < 0 || cols < 0) return fail(MHIP_ERR_INVALID_ARGUMENT, "mhip_bias_gelu: negative size");
+template <bool EXACT>
+static int gelu_entry(const char* name, void* stream, const void* x, const void* bias, void* y, int64_t rows, int64_t cols,
+                      int dtype) {
+    if (rows < 0 || cols < 0) return fail(MHIP_ERR_INVALID_ARGUMENT, "%s: negative size", name);
     if (rows == 0 || cols == 0) return MHIP_OK;
-    if (!x || !y) return fail(MHIP_ERR_INVALID_ARGUMENT, "mhip_bias_gelu: NULL tensor pointer");
+    if (!x || !y) return fail(MHIP_ERR_INVALID_ARGUMENT, "%s: NULL tensor pointer", name);
     hipStream_t s = as_stream(stream);
     switch (dtype) {
-        case MHIP_F32: return launch_gelu<float>(s, x, bias, y, rows, cols);
-        case MHIP_BF16: return launch_gelu<bf16_t>(s, x, bias, y, rows, cols);
-        case MHIP_F16: return launch_gelu<f16_t>(s, x, bias, y, rows, cols);
-        default: return fail(MHIP_ERR_UNSUPPORTED, "mhip_bias_gelu: dtype %d", dtype);
+        case MHIP_F32: return launch_gelu<float, EXACT>(s, x, bias, y, rows, cols);
+        case MHIP_BF16: return launch_gelu<bf16_t, EXACT>(s, x, bias, y, rows, cols);
+        case MHIP_F16: return launch_gelu<f16_t, EXACT>(s, x, bias, y, rows, cols);
+        default: return fail(MHIP_ERR_UNSUPPORTED, "%s: dtype %d", name, dtype);
     }
+}
+
+extern "C" int mhip_bias_gelu(void* stream, const void* x, const void* bias, void* y, int64_t rows,
+                              int64_t cols, int dtype) {
+    return gelu_entry<false>("mhip_bias_gelu", stream, x, bias, y, rows, cols, dtype);
+}
+
+extern "C" int mhip_bias_gelu_erf(void* stream, const void* x, const void* bias, void* y, int64_t rows,
+                                  int64_t cols, int dtype) {
+    return gelu_entry<true>("mhip_bias_gelu_erf", stream, x, bias, y, rows, cols, dtype);
 }
 
 extern "C" int mhip_softmax_strided(void* stream, const void* x, void* y, int64_t outer,

@@ -130,8 +130,26 @@ def _softmax(operands, cfg):
 
 def _gelu(operands, cfg):
     _need(operands, 1)
-    # the reference emits the tanh form whatever `approximate` says (:694-707)
-    return [kernels.gelu(operands[0])]
+    # the reference emits the tanh form whatever `approximate` says (:694-707); the pattern
+    # recogniser of this build marks a decomposed erf GELU with "erf": true, which is exact
+    return [kernels.gelu(operands[0], exact=P.get_bool(cfg, "erf", False))]
+
+
+_ACTIVATION_ALIASES = {"gelu_approximate": "gelu", "geluApproximate": "gelu", "swish": "silu"}
+
+
+def _ffn(operands, cfg):
+    """act(x . up) . down, operands [x, up, down], config {activation: "gelu"}
+    (CustomCallHandlers.swift:849-910; "gelu_exact" is the erf form here)."""
+    _need(operands, 3)
+    x, up, down = operands[:3]
+    act = P.get_string(cfg, "activation", "gelu")
+    act = _ACTIVATION_ALIASES.get(act, act)
+    if act not in kernels.ACTIVATION_CODE:
+        raise CustomCallError(f"fused_ffn: unknown activation '{act}'")
+    if P.get_bool(cfg, "is_gated", False):
+        raise CustomCallError("fused_ffn: gated feed-forward blocks are not supported")
+    return [kernels.matmul(kernels.matmul(x, up, activation=act), down)]
 
 
 def _matmul_bias_act(operands, cfg):
@@ -139,6 +157,7 @@ def _matmul_bias_act(operands, cfg):
     x, w = operands[:2]
     bias = operands[2] if len(operands) > 2 else None
     act = P.get_string(cfg, "activation", "none")
+    act = _ACTIVATION_ALIASES.get(act, act)
     if act not in kernels.ACTIVATION_CODE:
         raise CustomCallError(f"fused_matmul_bias_activation: unknown activation '{act}'")
     return [kernels.matmul(x, w, bias=bias, activation=act,
@@ -158,6 +177,7 @@ class CustomCallRegistry:
             ("fused_softmax", _softmax),
             ("fused_gelu", _gelu),
             ("fused_matmul_bias_activation", _matmul_bias_act),
+            ("fused_ffn", _ffn),
         ):
             self.register(name, fn)
 
@@ -182,5 +202,5 @@ shared = CustomCallRegistry()
 
 # Targets the reference registers that lie outside the attention / GEMM / row-kernel
 # path (CustomCallHandlers.swift:75-89); asking for them raises UnsupportedTarget.
-NOT_ON_PATH = ("fused_batch_norm", "fused_conv_bias_act", "fused_rope", "fused_ffn",
+NOT_ON_PATH = ("fused_batch_norm", "fused_conv_bias_act", "fused_rope",
                "fused_elementwise", "fused_depth_attention")

@@ -23,7 +23,7 @@ DTYPE_CODE = {
     torch.float16: 0, torch.float32: 1, torch.float64: 2, torch.bfloat16: 3, torch.bool: 4,
     torch.int8: 5, torch.int16: 6, torch.int32: 7, torch.int64: 8, torch.uint8: 9,
 }
-ACTIVATION_CODE = {"none": 0, "relu": 1, "gelu": 2, "silu": 3, "tanh": 4, "sigmoid": 5}
+ACTIVATION_CODE = {"none": 0, "relu": 1, "gelu": 2, "silu": 3, "tanh": 4, "sigmoid": 5, "gelu_exact": 6}
 
 
 def _code(t: torch.Tensor) -> int:
@@ -95,20 +95,21 @@ def rms_norm(x, gamma=None, eps: float = 1e-5):
     return y
 
 
-def bias_gelu(x, bias=None):
+def bias_gelu(x, bias=None, exact: bool = False):
+    """gelu(x + bias): the tanh approximation, or with `exact` 0.5 v (1 + erf(v / sqrt 2))."""
     _dev(x, bias)
     lib = _lib.load()
     cols = x.shape[-1] if x.dim() else 1
     if bias is not None and (bias.numel() != cols or bias.dtype != x.dtype):
         raise ValueError("bias must have the row length and dtype of x")
     y = torch.empty_like(x)
-    _lib.check(lib.mhip_bias_gelu(_stream(), x.data_ptr(), _ptr(bias), y.data_ptr(),
-                                  x.numel() // max(cols, 1), cols, _code(x)))
+    fn = lib.mhip_bias_gelu_erf if exact else lib.mhip_bias_gelu
+    _lib.check(fn(_stream(), x.data_ptr(), _ptr(bias), y.data_ptr(), x.numel() // max(cols, 1), cols, _code(x)))
     return y
 
 
-def gelu(x):
-    return bias_gelu(x, None)
+def gelu(x, exact: bool = False):
+    return bias_gelu(x, None, exact)
 
 
 def matmul(a, b, bias=None, activation: str = "none", trans_a: bool = False,

@@ -148,6 +148,15 @@ def gelu_tanh(x) -> np.ndarray:
     return 0.5 * x * (1.0 + np.tanh(inner))
 
 
+def gelu_erf(x) -> np.ndarray:
+    """Exact GELU 0.5 x (1 + erf(x / sqrt 2)): the function the reference's handlers name
+    "gelu_exact" (Compiler/CustomCallHandlers.swift:893-894, where it falls back to the tanh
+    form for lack of an erf; this restatement is the function itself)."""
+    x = np.asarray(x, dtype=np.float64)
+    erf = np.vectorize(math.erf, otypes=[np.float64])
+    return 0.5 * x * (1.0 + erf(x / math.sqrt(2.0)))
+
+
 def bias_gelu(x, bias) -> np.ndarray:
     """gelu_tanh(x + bias[col]) — the epilogue of fused_matmul_bias_activation
     (Compiler/CodeGenerator.swift:4797-4850) applied as a stand-alone row op."""
@@ -155,6 +164,7 @@ def bias_gelu(x, bias) -> np.ndarray:
 
 
 ACTIVATIONS = {
+    "gelu_exact": lambda v: gelu_erf(v),
     # Compiler/IntegrationTypes.swift:328-355, CustomCallHandlers.swift:540-558
     "none": lambda v: v,
     "relu": lambda v: np.maximum(v, 0.0),
@@ -325,7 +335,15 @@ def custom_call(target: str, operands, backend_config: str = "") -> np.ndarray:
     if target == "fused_softmax":
         return softmax(operands[0], axis=int(cfg.get("axis", -1)))
     if target == "fused_gelu":
-        return gelu_tanh(operands[0])
+        # tanh form whatever `approximate` says (CustomCallHandlers.swift:694-707); "erf": true is this
+        # build's mark for a decomposed erf GELU and means the exact function
+        return gelu_erf(operands[0]) if cfg.get("erf") is True else gelu_tanh(operands[0])
+    if target == "fused_ffn":
+        if len(operands) < 3:
+            raise ValueError("expected 3 inputs")
+        act = str(cfg.get("activation", "gelu"))                  # CustomCallHandlers.swift:870
+        act = {"gelu_approximate": "gelu", "geluApproximate": "gelu", "swish": "silu"}.get(act, act)
+        return gemm(ACTIVATIONS[act](gemm(operands[0], operands[1])), operands[2])
     if target == "fused_matmul_bias_activation":
         bias = operands[2] if len(operands) > 2 else None
         return matmul_bias_act(operands[0], operands[1], bias,

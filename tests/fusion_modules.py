@@ -254,3 +254,93 @@ def masked_attention(form, B=2, H=2, S=64, D=32, dtype="f32"):
         f"  %p = stablehlo.divide %e, %sb : {st}",
         f"  %o = stablehlo.dot_general %p, %v, batching_dims = [0, 1] x [0, 1], contracting_dims = [3] x [2] : ({st}, {t}) -> {t}",
         f"  return %o : {t} }}"])
+
+
+# exact GELU the way jax.nn.gelu(approximate=False) lowers it: x * (erf(x / sqrt 2) + 1) / 2
+GELU_ERF = """func.func @main(%x: tensor<4x64xf32>) -> tensor<4x64xf32> {
+  %rt2 = stablehlo.constant dense<1.41421354> : tensor<4x64xf32>
+  %one = stablehlo.constant dense<1.0> : tensor<4x64xf32>
+  %two = stablehlo.constant dense<2.0> : tensor<4x64xf32>
+  %u = stablehlo.divide %x, %rt2 : tensor<4x64xf32>
+  %e = chlo.erf %u : tensor<4x64xf32> -> tensor<4x64xf32>
+  %p = stablehlo.add %e, %one : tensor<4x64xf32>
+  %xp = stablehlo.multiply %x, %p : tensor<4x64xf32>
+  %r = stablehlo.divide %xp, %two : tensor<4x64xf32>
+  return %r : tensor<4x64xf32> }"""
+
+# the other common spelling: 0.5 * x * (1 + erf(x * 0.70710678))
+GELU_ERF_MUL = """func.func @main(%x: tensor<4x64xf32>) -> tensor<4x64xf32> {
+  %k = stablehlo.constant dense<0.707106769> : tensor<4x64xf32>
+  %one = stablehlo.constant dense<1.0> : tensor<4x64xf32>
+  %half = stablehlo.constant dense<0.5> : tensor<4x64xf32>
+  %u = stablehlo.multiply %x, %k : tensor<4x64xf32>
+  %e = chlo.erf %u : tensor<4x64xf32> -> tensor<4x64xf32>
+  %p = stablehlo.add %one, %e : tensor<4x64xf32>
+  %hx = stablehlo.multiply %half, %x : tensor<4x64xf32>
+  %r = stablehlo.multiply %hx, %p : tensor<4x64xf32>
+  return %r : tensor<4x64xf32> }"""
+
+# LayerNorm with the one-pass variance mean(x^2) - mean(x)^2 (flax use_fast_variance, jnp.var)
+LAYER_NORM_ONE_PASS = """func.func @main(%x: tensor<16x64xf32>, %g: tensor<64xf32>, %b: tensor<64xf32>) -> tensor<16x64xf32> {
+  %zero = stablehlo.constant dense<0.0> : tensor<f32>
+  %n = stablehlo.constant dense<64.0> : tensor<16xf32>
+  %eps = stablehlo.constant dense<1.0e-5> : tensor<16xf32>
+  %s = stablehlo.reduce(%x init: %zero) applies stablehlo.add across dimensions = [1] : (tensor<16x64xf32>, tensor<f32>) -> tensor<16xf32>
+  %mean = stablehlo.divide %s, %n : tensor<16xf32>
+  %xx = stablehlo.multiply %x, %x : tensor<16x64xf32>
+  %s2 = stablehlo.reduce(%xx init: %zero) applies stablehlo.add across dimensions = [1] : (tensor<16x64xf32>, tensor<f32>) -> tensor<16xf32>
+  %m2 = stablehlo.divide %s2, %n : tensor<16xf32>
+  %mm = stablehlo.multiply %mean, %mean : tensor<16xf32>
+  %var = stablehlo.subtract %m2, %mm : tensor<16xf32>
+  %ve = stablehlo.add %var, %eps : tensor<16xf32>
+  %r = stablehlo.rsqrt %ve : tensor<16xf32>
+  %mb = stablehlo.broadcast_in_dim %mean, dims = [0] : (tensor<16xf32>) -> tensor<16x64xf32>
+  %c = stablehlo.subtract %x, %mb : tensor<16x64xf32>
+  %rb = stablehlo.broadcast_in_dim %r, dims = [0] : (tensor<16xf32>) -> tensor<16x64xf32>
+  %xn = stablehlo.multiply %c, %rb : tensor<16x64xf32>
+  %gb = stablehlo.broadcast_in_dim %g, dims = [1] : (tensor<64xf32>) -> tensor<16x64xf32>
+  %bb = stablehlo.broadcast_in_dim %b, dims = [1] : (tensor<64xf32>) -> tensor<16x64xf32>
+  %y = stablehlo.multiply %xn, %gb : tensor<16x64xf32>
+  %z = stablehlo.add %y, %bb : tensor<16x64xf32>
+  return %z : tensor<16x64xf32> }"""
+
+# a module the way a tracing front end writes it: private helpers, a call with two results
+# used as %r#0 / %r#1, a call nested inside a callee, the entry function not first
+CALLS = """module @jit_f {
+  func.func private @_where(%p: tensor<8x16xi1>, %a: tensor<8x16xf32>, %b: tensor<8x16xf32>) -> tensor<8x16xf32> {
+    %0 = stablehlo.select %p, %a, %b : tensor<8x16xi1>, tensor<8x16xf32>
+    return %0 : tensor<8x16xf32>
+  }
+  func.func private @relu_and_neg(%a: tensor<8x16xf32>) -> (tensor<8x16xf32>, tensor<8x16xf32>) {
+    %z = stablehlo.constant dense<0.0> : tensor<8x16xf32>
+    %p = stablehlo.compare GT, %a, %z, FLOAT : (tensor<8x16xf32>, tensor<8x16xf32>) -> tensor<8x16xi1>
+    %r = func.call @_where(%p, %a, %z) : (tensor<8x16xi1>, tensor<8x16xf32>, tensor<8x16xf32>) -> tensor<8x16xf32>
+    %n = stablehlo.negate %a : tensor<8x16xf32>
+    return %r, %n : tensor<8x16xf32>, tensor<8x16xf32>
+  }
+  func.func public @main(%x: tensor<8x16xf32>, %y: tensor<8x16xf32>) -> (tensor<8x16xf32>, tensor<8x16xf32>) {
+    %s = stablehlo.add %x, %y : tensor<8x16xf32>
+    %r:2 = call @relu_and_neg(%s) : (tensor<8x16xf32>) -> (tensor<8x16xf32>, tensor<8x16xf32>)
+    %t = stablehlo.multiply %r#0, %r#1 : tensor<8x16xf32>
+    %u = call @_where_wrapper(%r#1, %t) : (tensor<8x16xf32>, tensor<8x16xf32>) -> tensor<8x16xf32>
+    return %t, %u : tensor<8x16xf32>, tensor<8x16xf32>
+  }
+  func.func private @_where_wrapper(%a: tensor<8x16xf32>, %b: tensor<8x16xf32>) -> tensor<8x16xf32> {
+    %z = stablehlo.constant dense<0.0> : tensor<8x16xf32>
+    %p = stablehlo.compare LT, %a, %z, FLOAT : (tensor<8x16xf32>, tensor<8x16xf32>) -> tensor<8x16xi1>
+    %r = call @_where(%p, %a, %b) : (tensor<8x16xi1>, tensor<8x16xf32>, tensor<8x16xf32>) -> tensor<8x16xf32>
+    return %r : tensor<8x16xf32>
+  }
+}"""
+
+# softmax computed by a helper function: after inlining it is the ordinary pattern
+SOFTMAX_IN_CALLEE = """module {
+  func.func @main(%x: tensor<8x32xf32>) -> tensor<8x32xf32> {
+    %y = call @softmax(%x) : (tensor<8x32xf32>) -> tensor<8x32xf32>
+    return %y : tensor<8x32xf32>
+  }
+""" + SOFTMAX.replace("func.func @main", "  func.func private @softmax") + "\n}"
+
+FFN_CUSTOM_CALL = """func.func @main(%x: tensor<4x32x64xf32>, %up: tensor<64x256xf32>, %down: tensor<256x64xf32>) -> tensor<4x32x64xf32> {
+  %r = stablehlo.custom_call @fused_ffn(%x, %up, %down) {backend_config = "{\\"activation\\": \\"ACT\\"}"} : (tensor<4x32x64xf32>, tensor<64x256xf32>, tensor<256x64xf32>) -> tensor<4x32x64xf32>
+  return %r : tensor<4x32x64xf32> }"""

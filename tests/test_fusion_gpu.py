@@ -142,3 +142,43 @@ def test_matmul_bias_activation(sess):
     exp = oracle.matmul_bias_act(x.astype(np.float64), w.astype(np.float64), bias.astype(np.float64), "relu")
     close(a, exp, 1e-5)
     close(b, exp, 1e-5)
+
+
+def test_erf_gelu_one_pass_layer_norm_and_calls(sess):
+    rng = np.random.default_rng(84)
+    x = rng.uniform(-4, 4, (4, 64)).astype(np.float32)
+    for text in (M.GELU_ERF, M.GELU_ERF_MUL):
+        a, b = both(sess, text, [(x, "f32")], "fused_gelu")
+        close(a, oracle.gelu_erf(x.astype(np.float64)), 1e-5)
+        close(b, oracle.gelu_erf(x.astype(np.float64)), 1e-5)
+    # the exact form is not the tanh approximation: the two differ by more than the tolerance somewhere
+    assert np.max(np.abs(oracle.gelu_erf(x.astype(np.float64)) - oracle.gelu_tanh(x.astype(np.float64)))) > 1e-4
+    x = (3 + 2 * rng.standard_normal((16, 64))).astype(np.float32)
+    g = (1 + 0.1 * rng.standard_normal(64)).astype(np.float32)
+    bt = (0.1 * rng.standard_normal(64)).astype(np.float32)
+    a, b = both(sess, M.LAYER_NORM_ONE_PASS, [(x, "f32"), (g, "f32"), (bt, "f32")], "fused_layer_norm")
+    exp = oracle.layer_norm(x.astype(np.float64), g.astype(np.float64), bt.astype(np.float64), 1e-5)
+    close(a, exp, 1e-5)
+    close(b, exp, 1e-4)      # as written: mean(x^2) - mean(x)^2 in fp32 cancels (mean 3, deviation 2)
+    # calls: the flat program equals its own restatement
+    x = rng.standard_normal((8, 16)).astype(np.float32)
+    y = rng.standard_normal((8, 16)).astype(np.float32)
+    exe = sess.compile(M.CALLS)
+    t, u = sess.run(exe, [(x, "f32"), (y, "f32")])
+    sess.lib.mhlo_executable_destroy(exe)
+    s = x + y
+    r0, r1 = np.where(s > 0, s, 0), -s
+    assert np.array_equal(t, r0 * r1) and np.array_equal(u, np.where(r1 < 0, r1, r0 * r1))
+
+
+@pytest.mark.parametrize("act", ["gelu", "gelu_exact", "relu", "silu"])
+def test_fused_ffn(sess, act):
+    rng = np.random.default_rng(85)
+    x = rng.standard_normal((4, 32, 64)).astype(np.float32)
+    up = (0.2 * rng.standard_normal((64, 256))).astype(np.float32)
+    down = (0.2 * rng.standard_normal((256, 64))).astype(np.float32)
+    exe = sess.compile(M.FFN_CUSTOM_CALL.replace("ACT", act))
+    (got,) = sess.run(exe, [(x, "f32"), (up, "f32"), (down, "f32")])
+    sess.lib.mhlo_executable_destroy(exe)
+    h = oracle.ACTIVATIONS[act](oracle.gemm(x.astype(np.float64).reshape(-1, 64), up.astype(np.float64)))
+    close(got, oracle.gemm(h, down.astype(np.float64)).reshape(x.shape), 2e-5)

@@ -209,3 +209,78 @@ def test_declared_result_types_are_checked_at_compile_time(sess, name, level):
     with pytest.raises(capi.MHLOError) as e:
         ops(sess, BAD_RESULT_TYPES[name], level)
     assert e.value.code == 3, (e.value.code, str(e.value))      # MHLO_ERROR_PARSE_FAILED
+
+
+def test_erf_gelu_becomes_the_exact_fused_form(sess):
+    """Both common spellings of 0.5 x (1 + erf(x / sqrt 2)) become a fused_gelu marked "erf": true
+    (the executor then runs the exact function, not the tanh approximation); a wrong constant
+    leaves the program as written; behind matmul + bias it is the "gelu_exact" epilogue."""
+    assert ops(sess, M.GELU_ERF) == ["fused_gelu"] and ops(sess, M.GELU_ERF_MUL) == ["fused_gelu"]
+    assert "erf" in ops(sess, M.GELU_ERF, 0)
+    assert "fused_gelu" not in ops(sess, M.GELU_ERF.replace("1.41421354", "1.5"))
+    assert "fused_gelu" not in ops(sess, M.GELU_ERF_MUL.replace("0.707106769", "0.7978845608"))
+    assert "fused_gelu" not in ops(sess, M.GELU_ERF.replace("dense<2.0>", "dense<3.0>"))
+    t = "tensor<32x128xf32>"
+    text = (f"func.func @main(%x: tensor<32x64xf32>, %w: tensor<64x128xf32>, %b: tensor<128xf32>) -> {t} {{\n"
+            f"  %d = stablehlo.dot_general %x, %w, contracting_dims = [1] x [0] : (tensor<32x64xf32>, tensor<64x128xf32>) -> {t}\n"
+            f"  %bb = stablehlo.broadcast_in_dim %b, dims = [1] : (tensor<128xf32>) -> {t}\n"
+            f"  %h = stablehlo.add %d, %bb : {t}\n"
+            f"  %k = stablehlo.constant dense<0.707106769> : {t}\n  %one = stablehlo.constant dense<1.0> : {t}\n"
+            f"  %half = stablehlo.constant dense<0.5> : {t}\n  %u = stablehlo.multiply %h, %k : {t}\n"
+            f"  %e = chlo.erf %u : {t} -> {t}\n  %p = stablehlo.add %one, %e : {t}\n"
+            f"  %hx = stablehlo.multiply %half, %h : {t}\n  %r = stablehlo.multiply %hx, %p : {t}\n  return %r : {t} }}")
+    assert ops(sess, text) == ["fused_matmul_bias_activation"]
+
+
+def test_one_pass_variance_layer_norm(sess):
+    assert ops(sess, M.LAYER_NORM_ONE_PASS) == ["fused_layer_norm"]
+    # the square of another mean, or a centring by another statistic, is not a LayerNorm
+    assert "fused_layer_norm" not in ops(sess, M.LAYER_NORM_ONE_PASS.replace("%mm = stablehlo.multiply %mean, %mean", "%mm = stablehlo.multiply %mean, %m2"))
+    assert "fused_layer_norm" not in ops(sess, M.LAYER_NORM_ONE_PASS.replace("broadcast_in_dim %mean, dims = [0]", "broadcast_in_dim %m2, dims = [0]"))
+
+
+def test_silu_epilogue_and_unshifted_softmax(sess):
+    t = "tensor<32x128xf32>"
+    text = (f"func.func @main(%x: tensor<32x64xf32>, %w: tensor<64x128xf32>, %b: tensor<128xf32>) -> {t} {{\n"
+            f"  %d = stablehlo.dot_general %x, %w, contracting_dims = [1] x [0] : (tensor<32x64xf32>, tensor<64x128xf32>) -> {t}\n"
+            f"  %bb = stablehlo.broadcast_in_dim %b, dims = [1] : (tensor<128xf32>) -> {t}\n"
+            f"  %h = stablehlo.add %d, %bb : {t}\n  %s = stablehlo.logistic %h : {t}\n"
+            f"  %r = stablehlo.multiply %h, %s : {t}\n  return %r : {t} }}")
+    assert ops(sess, text) == ["fused_matmul_bias_activation"]
+    # the sigmoid is also a result: it must still be produced
+    both = text.replace(f") -> {t} {{", f") -> ({t}, {t}) {{").replace(f"return %r : {t}", f"return %r, %s : {t}, {t}")
+    assert "logistic" in ops(sess, both)
+    unshifted = ("func.func @main(%x: tensor<8x32xf32>) -> tensor<8x32xf32> {\n"
+                 "  %e = stablehlo.exponential %x : tensor<8x32xf32>\n  %zero = stablehlo.constant dense<0.0> : tensor<f32>\n"
+                 "  %s = stablehlo.reduce(%e init: %zero) applies stablehlo.add across dimensions = [1] : (tensor<8x32xf32>, tensor<f32>) -> tensor<8xf32>\n"
+                 "  %sb = stablehlo.broadcast_in_dim %s, dims = [0] : (tensor<8xf32>) -> tensor<8x32xf32>\n"
+                 "  %r = stablehlo.divide %e, %sb : tensor<8x32xf32>\n  return %r : tensor<8x32xf32> }")
+    assert ops(sess, unshifted) == ["fused_softmax"]
+
+
+def test_calls_are_inlined(sess):
+    """Private helper functions, a two-result call used as %r#0 / %r#1, calls inside callees, the
+    entry function in the middle of the module: one flat program after parsing; a pattern that
+    lives in a callee is recognised after inlining."""
+    got = ops(sess, M.CALLS, 0)
+    assert "call" not in got and sorted(got) == sorted(["add", "constant", "compare", "select", "negate", "multiply",
+                                                        "constant", "compare", "select"])
+    assert ops(sess, M.SOFTMAX_IN_CALLEE) == ["fused_softmax"]
+    for bad, msg in ((M.CALLS.replace("call @relu_and_neg(%s)", "call @nowhere(%s)"), "unknown function"),
+                     (M.CALLS.replace("%r = call @_where(%p, %a, %b)", "%r = call @_where_wrapper(%a, %b)")
+                             .replace("(tensor<8x16xi1>, tensor<8x16xf32>, tensor<8x16xf32>) -> tensor<8x16xf32>\n    return %r : tensor<8x16xf32>\n  }\n}",
+                                      "(tensor<8x16xf32>, tensor<8x16xf32>) -> tensor<8x16xf32>\n    return %r : tensor<8x16xf32>\n  }\n}"), "recursive"),
+                     (M.CALLS.replace("%r:2 = call", "%r:3 = call"), "names 3 results"),
+                     (M.CALLS.replace("call @relu_and_neg(%s) : (tensor<8x16xf32>)", "call @relu_and_neg(%s, %s) : (tensor<8x16xf32>, tensor<8x16xf32>)"), "takes 1 arguments")):
+        with pytest.raises(capi.MHLOError) as e:
+            ops(sess, bad, 0)
+        assert e.value.code == 3 and msg in str(e.value), str(e.value)
+
+
+def test_fused_ffn_custom_call(sess):
+    assert ops(sess, M.FFN_CUSTOM_CALL.replace("ACT", "gelu")) == ["fused_ffn"]
+    assert ops(sess, M.FFN_CUSTOM_CALL.replace("ACT", "gelu_exact")) == ["fused_ffn"]
+    with pytest.raises(capi.MHLOError):
+        ops(sess, M.FFN_CUSTOM_CALL.replace("ACT", "mish"))
+    with pytest.raises(capi.MHLOError):         # the down projection does not follow the up projection
+        ops(sess, M.FFN_CUSTOM_CALL.replace("ACT", "gelu").replace("256x64xf32", "128x64xf32"))

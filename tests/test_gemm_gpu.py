@@ -96,7 +96,7 @@ def test_gemm_batched_bias_activation():
     assert_close(c, oracle.gemm(as_f64(a), as_f64(b)), 2e-2, "batched")
     x, w = _ab(200, 264, 128, torch.bfloat16, 30)
     bias = to_dev(rng.standard_normal(264) * 0.5, torch.bfloat16)
-    for act in ("none", "relu", "gelu", "silu", "tanh", "sigmoid"):
+    for act in ("none", "relu", "gelu", "silu", "tanh", "sigmoid", "gelu_exact"):
         y = kernels.matmul(x, w, bias=bias, activation=act)
         assert_close(y, oracle.matmul_bias_act(as_f64(x), as_f64(w), as_f64(bias), act), 2e-2, act)
     xf, wf = _ab(20, 24, 16, torch.float32, 31)

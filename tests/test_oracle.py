@@ -336,3 +336,20 @@ def test_gpt2_oracle_bf16_rounding_points_stay_near_f64():
     lo = oracle.gpt2_forward(ids, params, 4, "f64")
     lb = oracle.gpt2_forward(ids, params, 4, "bf16")
     assert np.sqrt(np.mean((lb - lo) ** 2)) < 2e-2 * np.sqrt(np.mean(lo ** 2))
+
+
+def test_gelu_erf_is_the_exact_gelu():
+    """Pins oracle.gelu_erf: closed values of x * Phi(x), torch's exact GELU in fp64, scipy's erf,
+    the identity gelu(x) - gelu(-x) = x, and that it is not the tanh approximation."""
+    import torch
+    from scipy.special import erf
+    assert oracle.gelu_erf(0.0) == 0.0
+    assert abs(oracle.gelu_erf(1.0) - 0.8413447460685429) < 1e-15
+    assert abs(oracle.gelu_erf(-1.0) + 0.15865525393145707) < 1e-15
+    x = np.linspace(-6, 6, 2001)
+    assert np.allclose(oracle.gelu_erf(x), torch.nn.functional.gelu(torch.from_numpy(x), approximate="none").numpy(), rtol=0, atol=1e-14)
+    assert np.allclose(oracle.gelu_erf(x), 0.5 * x * (1 + erf(x / np.sqrt(2))), rtol=0, atol=1e-15)
+    assert np.allclose(oracle.gelu_erf(x) - oracle.gelu_erf(-x), x, rtol=0, atol=1e-14)
+    assert np.max(np.abs(oracle.gelu_erf(x) - oracle.gelu_tanh(x))) > 1e-4
+    assert np.allclose(oracle.custom_call("fused_gelu", [x], '{"approximate": false, "erf": true}'), oracle.gelu_erf(x))
+    assert np.allclose(oracle.custom_call("fused_gelu", [x], '{"approximate": false}'), oracle.gelu_tanh(x))

@@ -147,3 +147,15 @@ def test_invariants_full_size():
     assert_close(ln[idx], oracle.layer_norm(as_f64(sub), 1.0, 0.0, 1e-5), 2e-2, "ln sampled rows")
     ge = kernels.bias_gelu(x, torch.zeros_like(gam))
     assert_close(ge[idx], oracle.gelu_tanh(as_f64(sub)), 2e-2, "gelu sampled rows")
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=lambda d: NAME[d])
+@pytest.mark.parametrize("shape", [(7, 4096), (33, 768), (5, 100), (4, 8), (9, 50257)], ids=lambda s: f"{s[0]}x{s[1]}")
+def test_bias_gelu_exact(shape, dtype):
+    """mhip_bias_gelu_erf: 0.5 v (1 + erf(v / sqrt 2)), v = x + bias."""
+    from metalhlo_amd import kernels
+    rng = np.random.default_rng(19)
+    x = _x(*shape, dtype, 20)
+    b = to_dev(0.02 * rng.standard_normal(shape[1]), dtype)
+    assert_close(kernels.bias_gelu(x, b, exact=True), oracle.gelu_erf(as_f64(x) + as_f64(b)), TOL[dtype], "bias_gelu exact")
+    assert_close(kernels.gelu(x, exact=True), oracle.gelu_erf(as_f64(x)), TOL[dtype], "gelu exact")
