@@ -95,6 +95,19 @@ def wl_gemm(torch, kernels, M=4096, N=4096, K=4096):
                 bytes=2.0 * (M * K + K * N + M * N), bound="mfma", kernel="gemm256_kernel")
 
 
+PEAK_F32_TFLOPS = 157.3    # MI355X dense fp32 MFMA
+
+
+def wl_gemm_f32(torch, kernels, M=4096, N=4096, K=4096):
+    g = torch.Generator(device="cuda").manual_seed(2)
+    a = torch.rand(M, K, generator=g, device="cuda") * 2 - 1
+    b = torch.rand(K, N, generator=g, device="cuda") * 2 - 1
+    c = torch.empty(M, N, dtype=torch.float32, device="cuda")
+    return dict(name=f"fp32 GEMM {M}x{N}x{K} (row-major A[M,K], B[K,N]; fp32 operands and accumulate on the fp32 matrix instruction)",
+                fn=lambda i: kernels.matmul(a, b, out=c), flops=2.0 * M * N * K, bytes=4.0 * (M * K + K * N + M * N),
+                bound="mfma", peak=PEAK_F32_TFLOPS, kernel="gemm_f32_mfma_kernel")
+
+
 def wl_attention(torch, kernels, B=4, H=32, S=4096, D=128, causal=True):
     g = torch.Generator(device="cuda").manual_seed(4)
     q, k, v = (torch.randn(B, H, S, D, generator=g, device="cuda").to(torch.bfloat16) for _ in range(3))
@@ -212,8 +225,9 @@ def measure(wl, steps, warmup, torch, key=None):
         sec = wall
     if wl["bound"] == "mfma":
         ach = wl["flops"] / sec / 1e12
-        roof = dict(bound="mfma", achieved=round(ach, 2), peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
-                    frac=round(ach / PEAK_BF16_TFLOPS, 4), traffic=MEASURED_TRAFFIC.get(key))
+        peak = wl.get("peak", PEAK_BF16_TFLOPS)
+        roof = dict(bound="mfma", achieved=round(ach, 2), peak=peak, unit="TFLOP/s",
+                    frac=round(ach / peak, 4), traffic=MEASURED_TRAFFIC.get(key))
         value, unit = ach, "TFLOP/s"
     else:
         ach = wl["bytes"] / sec / 1e9
@@ -264,12 +278,13 @@ def cpu_baseline_torch(name, torch):
     g = torch.Generator().manual_seed(7)
     bf = torch.bfloat16
     base = dict(cores=th, kind="port")
-    if name == "gemm":
-        a = (torch.rand(4096, 4096, generator=g) * 2 - 1).to(bf)
-        b = (torch.rand(4096, 4096, generator=g) * 2 - 1).to(bf)
+    if name in ("gemm", "gemm_f32"):
+        dt = bf if name == "gemm" else torch.float32
+        a = (torch.rand(4096, 4096, generator=g) * 2 - 1).to(dt)
+        b = (torch.rand(4096, 4096, generator=g) * 2 - 1).to(dt)
         t = _best_of(lambda: torch.matmul(a, b))
         return dict(base, value=round(2.0 * 4096 ** 3 / t / 1e12, 4), unit="TFLOP/s",
-                    sample=f"torch.matmul on CPU, bf16 4096^3 (the whole workload), best of 3: {t:.3f} s")
+                    sample=f"torch.matmul on CPU, {'bf16' if name == 'gemm' else 'fp32'} 4096^3 (the whole workload), best of 3: {t:.3f} s")
     if name in ("attention", "attention_full"):
         S, causal = (4096, True) if name == "attention" else (2048, False)
         q, k, v = (torch.randn(1, 1, S, 128, generator=g).to(bf) for _ in range(3))
@@ -328,8 +343,8 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="gemm",
-                    choices=["gemm", "attention", "attention_full", "softmax", "layer_norm", "rms_norm", "bias_gelu", "copy", "gpt2",
-                             "gpt2_capi"])
+                    choices=["gemm", "gemm_f32", "attention", "attention_full", "softmax", "layer_norm", "rms_norm", "bias_gelu", "copy",
+                             "gpt2", "gpt2_capi"])
     ap.add_argument("--ramp-ms", type=float, default=150.0,
                     help="milliseconds of untimed launches of the same kernel in front of the warm-up steps (0 = none)")
     ap.add_argument("--only", action="store_true", help="time only --workload (for profiling runs)")
@@ -351,6 +366,8 @@ def main():
     def build(name):
         if name == "gemm":
             return wl_gemm(torch, kernels)
+        if name == "gemm_f32":
+            return wl_gemm_f32(torch, kernels)
         if name == "attention":
             return wl_attention(torch, kernels, causal=True)
         if name == "attention_full":
@@ -379,7 +396,7 @@ def main():
     head = run(args.workload)
     others = {}
     if not args.only:
-        for name in ["gemm", "attention", "attention_full", "softmax", "layer_norm", "rms_norm", "bias_gelu", "gpt2", "gpt2_capi"]:
+        for name in ["gemm", "gemm_f32", "attention", "attention_full", "softmax", "layer_norm", "rms_norm", "bias_gelu", "gpt2", "gpt2_capi"]:
             if name == args.workload:
                 continue
             others[name] = run(name)

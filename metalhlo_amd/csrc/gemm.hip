@@ -400,6 +400,9 @@ static int launch_mfma(hipStream_t s, GemmArgs g, int64_t batch) {
 // gemm256.hip: 4-wave 256x256 kernel with a hand-scheduled main loop.
 bool gemm256_eligible(const GemmArgs& g, int64_t batch, int dtype, int bw = 256);
 int launch_gemm256(hipStream_t s, const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype, int bw = 256);
+// gemm_f32.hip: fp32 operands on the fp32 matrix instruction, 128x128 tiles.
+bool gemm_f32_mfma_wanted(const GemmArgs& g);
+int launch_gemm_f32_mfma(hipStream_t s, const GemmArgs& g, int64_t batch, int trans_a, int trans_b);
 // tuning.hip: variant prescribed by the tuning table for this problem, 0 = none.
 int tuned_gemm_variant(const GemmArgs& g, int64_t batch, int ta, int tb, int dtype);
 
@@ -509,7 +512,9 @@ static int gemm_entry(void* stream, const void* a, const void* b, const void* bi
         return pick_layout<f16_t>(s, g, batch, trans_a, trans_b);
     }
     switch (dtype) {
-        case MHIP_F32: return launch_simple<float>(s, g, batch, trans_a, trans_b);
+        case MHIP_F32:
+            if (gemm_f32_mfma_wanted(g)) return launch_gemm_f32_mfma(s, g, batch, trans_a, trans_b);
+            return launch_simple<float>(s, g, batch, trans_a, trans_b);
         case MHIP_BF16: return launch_simple<bf16_t>(s, g, batch, trans_a, trans_b);
         case MHIP_F16: return launch_simple<f16_t>(s, g, batch, trans_a, trans_b);
         case MHIP_I32: return launch_exact<int32_t>(s, g, batch, trans_a, trans_b);

@@ -54,6 +54,48 @@ def test_gemm_f32(shape):
         assert_close(c, oracle.gemm(as_f64(a), as_f64(b), ta, tb), 1e-5, f"gemm f32 {shape}")
 
 
+@pytest.mark.parametrize("layout", [(False, False), (False, True), (True, False), (True, True)], ids=["nn", "nt", "tn", "tt"])
+@pytest.mark.parametrize("shape", [(128, 128, 64), (256, 384, 128), (300, 200, 72), (130, 70, 50), (64, 65, 17), (1000, 136, 256)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_gemm_f32_matrix_cores(shape, layout):
+    """fp32 operands on v_mfma_f32_32x32x2_f32 (128x128 tiles): every layout, ragged M / N / K, leading
+    dimensions that are no multiple of 4 (scalar staging), bias + activation + residual."""
+    from metalhlo_amd import kernels
+    M, N, K = shape
+    ta, tb = layout
+    a, b = _ab(M, N, K, torch.float32, 41, ta, tb)
+    c = kernels.matmul(a, b, trans_a=ta, trans_b=tb)
+    assert_close(c, oracle.gemm(as_f64(a), as_f64(b), ta, tb), 1e-5, f"gemm f32 mfma {shape} {layout}")
+    rng = np.random.default_rng(42)
+    bias = to_dev(rng.standard_normal(N), torch.float32)
+    r = to_dev(rng.standard_normal((M, N)), torch.float32)
+    y = kernels.matmul(a, b, bias=bias, activation="gelu", trans_a=ta, trans_b=tb, residual=r)
+    exp = oracle.matmul_bias_act(as_f64(a), as_f64(b), as_f64(bias), "gelu", ta, tb) + as_f64(r)
+    assert_close(y, exp, 1e-5, f"gemm f32 mfma epilogue {shape} {layout}")
+
+
+def test_gemm_f32_matrix_cores_long_k_and_batch():
+    """K = 4096: the rounding of a 4096-term fp32 sum exceeds 1e-5 of a result that happens to be
+    small, for any summation order; the bound that holds is the forward error bound of a dot
+    product, |c - c_exact| <= 1e-5 (|a| . |b|) -- still five digits of every product.  Also a batched
+    problem, and the matrix-core kernel against the plain fp32 kernel."""
+    import os
+    from metalhlo_amd import kernels
+    a, b = _ab(512, 384, 4096, torch.float32, 43)
+    c = as_f64(kernels.matmul(a, b))
+    A, B = as_f64(a), as_f64(b)
+    assert np.all(np.abs(c - A @ B) <= 1e-5 * (np.abs(A) @ np.abs(B)))
+    a, b = _ab(200, 136, 96, torch.float32, 44, batch=(3,))
+    c = kernels.matmul(a, b)
+    assert_close(c, oracle.gemm(as_f64(a), as_f64(b)), 1e-5, "batched f32")
+    os.environ["MHIP_GEMM_F32_MFMA"] = "2"
+    try:
+        plain = kernels.matmul(a, b)
+    finally:
+        del os.environ["MHIP_GEMM_F32_MFMA"]
+    assert_close(plain, as_f64(c), 1e-5, "plain vs matrix-core fp32 kernel")
+
+
 def test_gemm_unaligned_falls_back():
     """K or N not a multiple of 8 (e.g. vocab 50257) cannot use 16-byte loads."""
     from metalhlo_amd import kernels
