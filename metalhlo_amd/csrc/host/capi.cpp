@@ -55,10 +55,9 @@ MHLOStatusCode compile_text(MHLOClientRef client, const std::string& text, const
         exe = new Executable();
         exe->client = static_cast<Client*>(client);
         exe->opt_level = cfg ? (int)cfg->optimization_level : (int)MHLO_OPT_O2;
-        exe->fn = parse_module(text);
         // O0 runs the module as written; every other level recognises the fused patterns
         // (Sources/MetalHLO/CompilationConfig.swift:232-263 enables the fusion passes from O1)
-        if (exe->opt_level >= (int)MHLO_OPT_O1) fuse_patterns(exe->fn);
+        exe->fn = build_function(text, exe->opt_level);
         compile(*exe);
     });
     if (st != MHLO_OK) { delete exe; return st; }

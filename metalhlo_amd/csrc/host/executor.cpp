@@ -881,6 +881,7 @@ static void ensure_arena(Executable& exe, size_t bytes) {
 // a graph.  False when the capture or the instantiation fails; the stream is usable again then.
 static bool capture_graph(Executable& exe, const std::vector<DeviceTensor>& inputs, Executable::CapturedGraph& out) {
     Client& c = *exe.client;
+    std::lock_guard<std::mutex> stream_lock(c.stream_mu);       // no other thread enqueues on the stream meanwhile
     if (hipStreamBeginCapture(c.stream, hipStreamCaptureModeThreadLocal) != hipSuccess) {
         (void)hipGetLastError();
         return false;

@@ -75,6 +75,10 @@ struct Client {
     int device = -1;          // -1: created without a device (host-only operations)
     std::string device_name;
     hipStream_t stream = nullptr;
+    // Held while the stream is being captured into a graph, and by every other thread that
+    // enqueues work on the stream (the PJRT plugin's transfers): work enqueued from another thread
+    // during a capture would become part of the graph instead of running.
+    std::mutex stream_mu;
     DevicePool pool;
     DeviceTensor allocate(const TensorType& t);
 };

@@ -14,6 +14,8 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <stdlib.h>
+
 #include <algorithm>
 #include <set>
 
@@ -874,7 +876,7 @@ struct Rewriter {
 
 }  // namespace
 
-int fuse_patterns(Function& fn) {
+int fuse_patterns(Function& fn, const std::set<std::string>* disabled) {
     // malformed operations are reported by the validation that follows; do not look inside them
     static const std::map<std::string, size_t> kArity = {
         {"add", 2}, {"subtract", 2}, {"multiply", 2}, {"divide", 2}, {"maximum", 2}, {"minimum", 2}, {"dot", 2},
@@ -887,10 +889,62 @@ int fuse_patterns(Function& fn) {
             if (v < 0 || v >= fn.num_values) return 0;
     }
     Rewriter rw(fn);
-    rw.pass([&](size_t i) { rw.softmax(i) || rw.gelu(i) || rw.gelu_erf(i) || rw.norm(i); });
-    rw.pass([&](size_t i) { rw.attention(i) || rw.matmul_bias_act(i); });
-    rw.pass([&](size_t i) { rw.attention_views(i) || rw.matmul_residual(i); });
+    // The passes under the names the reference gives its pattern-fusion passes
+    // (Compiler/PassManager.swift:154-201), so that METALHLO_DISABLED_PASSES means the same thing.
+    // Later passes build on earlier ones: attention needs the fused softmax, the GELU epilogue the
+    // fused GELU, the residual epilogue the fused matmul.  METALHLO_DEBUG_PASSES=1 prints one line
+    // per pass, `[*] name ops: N -> M` (asterisk = the pass changed the program; PassManager.swift:255-278).
+    const char* dbg = getenv("METALHLO_DEBUG_PASSES");
+    const bool debug = dbg && !strcmp(dbg, "1");
+    auto run = [&](const char* name, auto&& try_at) {
+        if (disabled && disabled->count(name)) return;
+        const size_t before = fn.ops.size();
+        const int fused_before = rw.fused;
+        rw.pass(try_at);
+        if (debug) fprintf(stderr, "[%c] %s ops: %zu -> %zu\n", rw.fused != fused_before ? '*' : ' ', name, before, fn.ops.size());
+    };
+    run("softmax-fusion", [&](size_t i) { rw.softmax(i); });
+    run("gelu-fusion", [&](size_t i) { rw.gelu(i) || rw.gelu_erf(i); });
+    run("norm-fusion", [&](size_t i) { rw.norm(i); });
+    run("attention-fusion", [&](size_t i) { rw.attention(i); });
+    run("matmul-bias-act-fusion", [&](size_t i) { rw.matmul_bias_act(i); });
+    run("transpose-folding", [&](size_t i) { rw.attention_views(i); });
+    run("residual-chain-fusion", [&](size_t i) { rw.matmul_residual(i); });
     return rw.fused;
+}
+
+// The text front end with the environment's diagnostics: parse (calls inlined), recognise the
+// fused patterns unless the level is O0, write the result to the file METALHLO_DUMP_OPTIMIZED
+// names (one line per operation: result = name inputs=[...]; Compiler/MetalHLOCompiler.swift:205-218).
+// METALHLO_DISABLED_PASSES (comma-separated pass names) is honoured on every surface.
+Function build_function(const std::string& text, int opt_level) {
+    Function fn = parse_module(text);
+    std::set<std::string> disabled;
+    if (const char* d = getenv("METALHLO_DISABLED_PASSES")) {
+        std::string cur;
+        for (const char* c = d;; c++) {
+            if (*c == ',' || *c == 0) {
+                if (!cur.empty()) disabled.insert(cur);
+                cur.clear();
+                if (!*c) break;
+            } else if (*c != ' ') {
+                cur += *c;
+            }
+        }
+    }
+    if (opt_level >= 1) fuse_patterns(fn, &disabled);
+    if (const char* path = getenv("METALHLO_DUMP_OPTIMIZED")) {
+        if (FILE* f = fopen(path, "w")) {
+            fprintf(f, "// optimized IR -- %zu ops\n", fn.ops.size());
+            for (const Op& op : fn.ops) {
+                fprintf(f, "%%%d = %s inputs=[", op.result, op.name == "custom_call" ? op.target.c_str() : op.name.c_str());
+                for (size_t i = 0; i < op.operands.size(); i++) fprintf(f, "%s%%%d", i ? "," : "", op.operands[i]);
+                fprintf(f, "]%s%s\n", op.backend_config.empty() ? "" : " config=", op.backend_config.c_str());
+            }
+            fclose(f);
+        }
+    }
+    return fn;
 }
 
 }  // namespace mhlo

@@ -8,6 +8,7 @@
 #include <stdint.h>
 
 #include <map>
+#include <set>
 #include <stdexcept>
 #include <string>
 #include <vector>
@@ -82,7 +83,12 @@ Function parse_module(const std::string& text);
 // Rewrites decomposed softmax / GELU(tanh) / LayerNorm / RMSNorm / attention /
 // matmul+bias+activation subgraphs into the fused custom_calls (fusion.cpp); returns the
 // number of rewrites.  Values used outside a pattern are never absorbed.
-int fuse_patterns(Function& fn);
+int fuse_patterns(Function& fn, const std::set<std::string>* disabled = nullptr);
+
+// parse_module + fuse_patterns (unless `opt_level` is 0) with the environment's switches:
+// METALHLO_DISABLED_PASSES (comma-separated names of the reference's fusion passes),
+// METALHLO_DEBUG_PASSES=1 (one line per pass on stderr), METALHLO_DUMP_OPTIMIZED=<file>.
+Function build_function(const std::string& text, int opt_level);
 
 // Flat JSON object {"k": number | bool | "string" | [numbers]} as used by
 // backend_config (Compiler/CustomCallHandlers.swift:102-168).  Anything that

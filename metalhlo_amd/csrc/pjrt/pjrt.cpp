@@ -21,6 +21,7 @@
 #include <unistd.h>
 
 #include <atomic>
+#include <algorithm>
 #include <chrono>
 #include <condition_variable>
 #include <deque>
@@ -374,9 +375,17 @@ PJRT_Error* build_program(PJRT_Client* client, const std::string& text, std::sha
     auto prog = std::make_shared<Program>();
     PJRT_Error* err = guarded([&] {
         prog->exe.client = &client->host;
-        prog->exe.opt_level = 2;
-        prog->exe.fn = parse_module(text);
-        fuse_patterns(prog->exe.fn);
+        // METALHLO_OPT_LEVEL = O0 | O1 | O2 | O3, default O2 (PJRTExecutable.swift:1755-1765)
+        const char* lvl = getenv("METALHLO_OPT_LEVEL");
+        prog->exe.opt_level = !lvl ? 2 : !strcmp(lvl, "O0") ? 0 : !strcmp(lvl, "O1") ? 1 : !strcmp(lvl, "O3") ? 3 : 2;
+        // METALHLO_DUMP_MLIR = <directory>: the program as received, mlir_<lines>_<time>.txt (:1701-1706)
+        if (const char* dir = getenv("METALHLO_DUMP_MLIR")) {
+            const long lines = (long)std::count(text.begin(), text.end(), '\n') + 1;
+            const std::string path = std::string(dir) + "/mlir_" + std::to_string(lines) + "_" +
+                                     std::to_string(std::chrono::steady_clock::now().time_since_epoch().count()) + ".txt";
+            if (FILE* f = fopen(path.c_str(), "w")) { fwrite(text.data(), 1, text.size(), f); fclose(f); }
+        }
+        prog->exe.fn = build_function(text, prog->exe.opt_level);
         compile(prog->exe);
     });
     if (err) return err;
@@ -659,6 +668,7 @@ PJRT_Error* Client_BufferFromHostBuffer(PJRT_Client_BufferFromHostBuffer_Args* a
         if (staged) {
             // the caller's memory is read here and never again; the DMA runs behind this call
             memcpy(staged, a->data, n);
+            std::lock_guard<std::mutex> stream_lock(c->host.stream_mu);     // not into a graph capture
             if (hipMemcpyAsync(d.data(), staged, n, hipMemcpyHostToDevice, c->host.stream) != hipSuccess) {
                 (void)hipGetLastError();
                 c->transfers.unstage(staged, n);
@@ -672,6 +682,7 @@ PJRT_Error* Client_BufferFromHostBuffer(PJRT_Client_BufferFromHostBuffer_Args* a
                 finish();
             }
         } else if (n) {
+            std::lock_guard<std::mutex> stream_lock(c->host.stream_mu);
             if (hipMemcpyAsync(d.data(), a->data, n, hipMemcpyHostToDevice, c->host.stream) != hipSuccess ||
                 hipStreamSynchronize(c->host.stream) != hipSuccess) {
                 (void)hipGetLastError();
@@ -1015,6 +1026,7 @@ PJRT_Error* copy_to_host(PJRT_Buffer& b, void* dst, size_t offset, size_t bytes,
     PJRT_Client* c = b.client;
     const char* src = static_cast<const char*>(b.tensor.data()) + offset;
     void* staged = bytes <= TransferEngine::kStageMax && c->transfers.running ? c->transfers.stage(bytes) : nullptr;
+    std::lock_guard<std::mutex> stream_lock(c->host.stream_mu);     // not into a graph capture
     if (staged) {
         if (hipMemcpyAsync(staged, src, bytes, hipMemcpyDeviceToHost, c->host.stream) != hipSuccess) {
             (void)hipGetLastError();
@@ -1068,6 +1080,7 @@ PJRT_Error* clone_buffer(PJRT_Buffer& b, PJRT_Buffer** out) {
     PJRT_Error* err = guarded([&] {
         DeviceTensor d = b.client->host.allocate(b.tensor.type);
         const size_t n = b.tensor.type.bytes();
+        std::lock_guard<std::mutex> stream_lock(b.client->host.stream_mu);
         if (n && (hipMemcpyAsync(d.data(), b.tensor.data(), n, hipMemcpyDeviceToDevice, b.client->host.stream) != hipSuccess ||
                   hipStreamSynchronize(b.client->host.stream) != hipSuccess)) {
             (void)hipGetLastError();

@@ -16,6 +16,7 @@
 
 #include <atomic>
 #include <string>
+#include <thread>
 #include <vector>
 
 #include "pjrt_abi.h"
@@ -746,6 +747,49 @@ static void case_execute(PJRT_Client* c) {
     printf("ok execute\n");
 }
 
+// Executions that are replayed as a HIP graph (METALHLO_HIP_GRAPH=1: the second execution captures the
+// client's stream, later ones replay) while a second thread keeps uploading and downloading on
+// the same client: a capture holds the stream lock that every transfer takes, so no transfer is
+// recorded into a graph or left without its completion event.  Every result of both threads is
+// checked.  Without graph replay the case is the same traffic on the eager path.
+static void case_execute_while_transferring(PJRT_Client* c) {
+    std::string prog = "func.func @main(%x: tensor<256xf32>) -> tensor<256xf32> {\n  %c = stablehlo.constant dense<1.0> : tensor<256xf32>\n";
+    std::string cur = "%x";
+    for (int i = 0; i < 24; i++) {           // a chain long enough for the replay threshold
+        prog += "  %v" + std::to_string(i) + " = stablehlo.add " + cur + ", %c : tensor<256xf32>\n";
+        cur = "%v" + std::to_string(i);
+    }
+    prog += "  return " + cur + " : tensor<256xf32>\n}\n";
+    PJRT_LoadedExecutable* le = nullptr;
+    OK(compile(c, prog, "mlir", &le));
+    std::atomic<bool> stop{false};
+    std::atomic<int> round_trips{0};
+    std::thread mover([&] {
+        std::vector<float> src(4096), dst(4096);
+        for (int it = 0; !stop.load(); it++) {
+            for (size_t i = 0; i < src.size(); i++) src[i] = (float)(it * 7 + (int)i);
+            PJRT_Buffer* b = upload(c, src.data(), PJRT_Buffer_Type_F32, {4096});
+            download(b, dst.data(), dst.size() * sizeof(float));
+            destroy_buffer(b);
+            CHECK(dst == src);
+            round_trips++;
+        }
+    });
+    std::vector<float> x(256);
+    for (int it = 0; it < 40; it++) {
+        for (int i = 0; i < 256; i++) x[i] = (float)(it + i);
+        PJRT_Buffer* bx = upload(c, x.data(), PJRT_Buffer_Type_F32, {256});
+        std::vector<float> y = run1(le, {bx}, 256);
+        for (int i = 0; i < 256; i++) CHECK(y[i] == x[i] + 24.f);
+        destroy_buffer(bx);
+    }
+    while (round_trips.load() < 8) usleep(1000);
+    stop = true;
+    mover.join();
+    destroy_loaded(le);
+    printf("ok execute_while_transferring\n");
+}
+
 int main(int argc, char** argv) {
     if (argc < 3) { printf("usage: pjrt_driver <plugin.so> host|gpu\n"); return 2; }
     void* lib = dlopen(argv[1], RTLD_NOW | RTLD_LOCAL);
@@ -765,6 +809,7 @@ int main(int argc, char** argv) {
         case_round_trip(c);
         case_execute(c);
         case_async_transfers(c);
+        case_execute_while_transferring(c);
     } else {
         case_no_device_buffers(c);
     }

@@ -284,3 +284,36 @@ def test_fused_ffn_custom_call(sess):
         ops(sess, M.FFN_CUSTOM_CALL.replace("ACT", "mish"))
     with pytest.raises(capi.MHLOError):         # the down projection does not follow the up projection
         ops(sess, M.FFN_CUSTOM_CALL.replace("ACT", "gelu").replace("256x64xf32", "128x64xf32"))
+
+
+def test_environment_switches_of_the_front_end(sess, tmp_path, capfd):
+    """METALHLO_DISABLED_PASSES takes the reference's pass names (Compiler/PassManager.swift:154-201),
+    METALHLO_DEBUG_PASSES=1 prints one line per pass, METALHLO_DUMP_OPTIMIZED=<file> receives the
+    operation list after recognition."""
+    block = M.transformer_block(2, 64, 4, 64, 256, "bf16")
+    full = ops(sess, block)
+    os.environ["METALHLO_DISABLED_PASSES"] = "residual-chain-fusion, transpose-folding"
+    try:
+        got = ops(sess, block)
+        assert got.count("add") == 2 and "transpose" in got and got.count("fused_matmul_bias_activation") == 4
+    finally:
+        del os.environ["METALHLO_DISABLED_PASSES"]
+    os.environ["METALHLO_DISABLED_PASSES"] = "softmax-fusion"
+    try:
+        got = ops(sess, block)        # no fused softmax, hence no fused attention either
+        assert "fused_scaled_dot_product_attention" not in got and "exponential" in got and "fused_layer_norm" in got
+    finally:
+        del os.environ["METALHLO_DISABLED_PASSES"]
+    assert ops(sess, block) == full
+    dump = tmp_path / "opt.txt"
+    os.environ["METALHLO_DUMP_OPTIMIZED"] = str(dump)
+    os.environ["METALHLO_DEBUG_PASSES"] = "1"
+    try:
+        capfd.readouterr()
+        ops(sess, M.SOFTMAX)
+        err = capfd.readouterr().err
+    finally:
+        del os.environ["METALHLO_DUMP_OPTIMIZED"], os.environ["METALHLO_DEBUG_PASSES"]
+    assert "[*] softmax-fusion ops: 9 -> 1" in err and "[ ] norm-fusion ops: 1 -> 1" in err
+    text = dump.read_text()
+    assert text.startswith("// optimized IR -- 1 ops") and "fused_softmax inputs=[%0]" in text and '"axis": 1' in text

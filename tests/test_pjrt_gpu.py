@@ -17,11 +17,13 @@ pytestmark = pytest.mark.gpu
 @pytest.mark.parametrize("sync,graph", [("0", "0"), ("1", "0"), ("0", "1")], ids=["async", "sync", "async+graph"])
 def test_driver_gpu_cases(sync, graph):
     """The third run replays executions as HIP graphs (captured on the stream the transfer thread's
-    copies also use) while transfers are asynchronous."""
+    copies also use) while transfers are asynchronous; its last case executes while a second
+    thread uploads and downloads on the same client."""
     assert os.path.exists(PLUGIN) and os.path.exists(DRIVER), "plugin / driver not built"
     env = dict(os.environ, METALHLO_PJRT_SYNC_TRANSFERS=sync, METALHLO_HIP_GRAPH=graph)
     r = subprocess.run([DRIVER, PLUGIN, "gpu"], capture_output=True, text=True, timeout=120, env=env)
     assert r.returncode == 0, r.stdout[-3000:] + r.stderr[-3000:]
-    for case in ("table", "errors", "platform", "compile", "round_trip", "execute", "async_transfers", "all"):
+    for case in ("table", "errors", "platform", "compile", "round_trip", "execute", "async_transfers",
+                 "execute_while_transferring", "all"):
         assert f"ok {case}\n" in r.stdout, r.stdout
     print(r.stdout)
