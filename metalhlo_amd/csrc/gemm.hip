@@ -400,13 +400,15 @@ static int launch_mfma(hipStream_t s, GemmArgs g, int64_t batch) {
 // gemm256.hip: 4-wave 256x256 kernel with a hand-scheduled main loop.
 bool gemm256_eligible(const GemmArgs& g, int64_t batch, int dtype, int bw = 256);
 int launch_gemm256(hipStream_t s, const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype, int bw = 256);
+bool gemm_stream_eligible(const GemmArgs& g, int64_t batch, int trans_a, int dtype);
+int launch_gemm_stream(hipStream_t s, const GemmArgs& g, int trans_b, int dtype);
 // gemm_f32.hip: fp32 operands on the fp32 matrix instruction, 128x128 tiles.
 bool gemm_f32_mfma_wanted(const GemmArgs& g);
 int launch_gemm_f32_mfma(hipStream_t s, const GemmArgs& g, int64_t batch, int trans_a, int trans_b);
 // tuning.hip: variant prescribed by the tuning table for this problem, 0 = none.
 int tuned_gemm_variant(const GemmArgs& g, int64_t batch, int ta, int tb, int dtype);
 
-// Which kernel serves a 16-bit problem (MHIP_GEMM_TILE = 128 | 256 | 2560 | 2561 forces one):
+// Which kernel serves a 16-bit problem (MHIP_GEMM_TILE = 128 | 256 | 2560 | 2561 | 2562 forces one):
 //   * the four-wave ring kernel (gemm256.hip) on 256x256 tiles (2560) or 256x128 tiles
 //     (2561) when K >= 512 and the problem is eligible: one workgroup per CU, so its time is
 //     rounds x (stages x per-stage time + prologue and epilogue), rounds = ceil(tiles / 256 CUs);
@@ -415,6 +417,15 @@ int tuned_gemm_variant(const GemmArgs& g, int64_t batch, int ta, int tb, int dty
 //     fragment reads for every four MFMAs instead of two), prologue + epilogue about 700 and
 //     500 -- figures fitted to seven measured shapes (4096^3: wide; [8192,768] x K 3072
 //     or 768, [8192,2304..3072] x K 768: narrow);
+//   * the same 256x128 kernel as persistent workgroups that store a tile inside the loop of the
+//     next one (2562; gemm_stream_kernel) when the problem meets that kernel's conditions, B is
+//     stored [K, N] and there are two to four rounds of narrow tiles.  Fitted to measured shapes
+//     (us): a streamed tile costs 0.3875 per K stage + 3.8, plus 5 once; a wide tile 0.6625 per
+//     stage + 13.8 (its epilogue is exposed in every round).  Streamed tiles always beat the plain
+//     narrow form, but the narrow tile asks the L2 for 1.5 times the operand bytes of the wide one,
+//     and from about eight rounds on that outweighs the hidden epilogues: [8192,3072] x K 768
+//     58 -> 51 us and [8192,2304] x K 768 48 -> 41, but [8192,16384] x K 768 216 against 203 on
+//     wide tiles; with B stored [N, K] the gain is within noise;
 //   * the eight-wave 256x256 kernel for large problems the ring kernel cannot take whose
 //     rows of C are not 16-byte aligned (odd N): its eight waves hide the narrow stores;
 //   * otherwise 128x128 tiles, two workgroups per CU (short K, few tiles).
@@ -426,6 +437,9 @@ static int pick_tile(hipStream_t s, const GemmArgs& g, int64_t batch) {
     constexpr int dt = std::is_same<T, bf16_t>::value ? MHIP_BF16 : MHIP_F16;
     int force = tune_int("MHIP_GEMM_TILE", 0);
     if (force == 0) force = tuned_gemm_variant(g, batch, TA, TB, dt);   // tuning table / running tuner
+    if (force == 2562) {
+        if (gemm_stream_eligible(g, batch, TA, dt)) return launch_gemm_stream(s, g, TB, dt);
+    }
     if (force == 2561) {
         if (gemm256_eligible(g, batch, dt, 128)) return launch_gemm256(s, g, batch, TA, TB, dt, 128);
     }
@@ -436,6 +450,12 @@ static int pick_tile(hipStream_t s, const GemmArgs& g, int64_t batch) {
         constexpr int cus = 256;                       // compute units of the device this is written for
         const int64_t narrow = tiles_m * ((g.N + 127) / 128) * batch, stages = g.K / 32;
         const bool wide_ok = gemm256_eligible(g, batch, dt), narrow_ok = gemm256_eligible(g, batch, dt, 128);
+        if (!TB && (narrow + cus - 1) / cus <= 4 && tune_int("MHIP_GEMM_STREAM", 1) != 2 &&    // 2 = off
+            gemm_stream_eligible(g, batch, TA, dt)) {
+            const double stream_us = (double)((narrow + cus - 1) / cus) * (stages * 0.3875 + 3.8) + 5.0;
+            const double wide_us = (double)((big + cus - 1) / cus) * (stages * 0.6625 + 13.8);
+            if (!wide_ok || stream_us < wide_us) return launch_gemm_stream(s, g, TB, dt);
+        }
         const int64_t wide_cost = ((big + cus - 1) / cus) * (stages * 32 + 700);
         const int64_t narrow_cost = ((narrow + cus - 1) / cus) * (stages * 18 + 500);
         if (narrow_ok && (!wide_ok || narrow_cost < wide_cost)) return launch_gemm256(s, g, batch, TA, TB, dt, 128);

@@ -24,6 +24,8 @@
 
 namespace mhip {
 
+typedef uint32_t u32x16 __attribute__((ext_vector_type(16)));
+
 #include "gemm256_loop.inc"
 
 namespace {
@@ -117,50 +119,16 @@ __device__ inline void main_loop(f32x16 (&acc)[BW / 16], u32x4 ra, u32x4 rb, u32
 #undef MHIP_LOOP
 }
 
-// BW = 256: the 256x256 tile (each wave 128x128).  BW = 128: a 256x128 tile (each wave
-// 128x64, half the accumulators, a 24 KB stage) for problems whose 256x256 tiling would
-// leave compute units idle or a last round nearly empty.
-template <typename T, bool TA, bool TB, int BW>
-__global__ __launch_bounds__(256) void gemm256_kernel(GemmArgs g) {
-    extern __shared__ __attribute__((aligned(16))) char smem[];
-    using LA = typename std::conditional<TA, MnMajor<256>, KMajor>::type;
-    using LB = typename std::conditional<TB, KMajor, MnMajor<BW>>::type;
+// Epilogue of one tile: bias, activation, conversion, then through LDS (the ring, free after the
+// loop's last barrier) so that every store instruction writes whole 16-byte chunks of C rows.
+template <typename T, int BW>
+__device__ __forceinline__ void store_tile(f32x16 (&acc)[BW / 16], char* smem, const GemmArgs& g, T* c, const T* res,
+                                  int m0, int n0) {
     constexpr int WN = BW / 2;            // columns per wave
     constexpr int NBF = BW / 64;          // 32-column accumulator blocks per wave
-
-    int tm, tn;
-    tile_of(blockIdx.x, gridDim.x, g.tiles_m, g.tiles_n, tm, tn);
-    const int m0 = tm * 256, n0 = tn * BW;
-    const int64_t batch = blockIdx.y;
-    const char* a = reinterpret_cast<const char*>(static_cast<const T*>(g.a) + batch * g.sa);
-    const char* b = reinterpret_cast<const char*>(static_cast<const T*>(g.b) + batch * g.sb);
-    T* c = static_cast<T*>(g.c) + batch * g.sc;
-    const T* res = g.residual ? static_cast<const T*>(g.residual) + batch * g.sc : nullptr;
-    const uint32_t a_bytes = (uint32_t)((int64_t)(TA ? g.K : g.M) * g.lda * 2);
-    const uint32_t b_bytes = (uint32_t)((int64_t)(TB ? g.N : g.K) * g.ldb * 2);
-
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const int lrow = lane & 31, lhalf = lane >> 5;
-    // LDS byte address of the dynamic segment
-    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
-
-    const u32x4 ra = LA::raddr(lane, wm * 128, lds0);
-    const u32x4 rb = LB::raddr(lane, wn * WN, lds0 + kOperBytes);
-    u32x2 misc;
-    misc.x = LA::goff(lane, wave, m0, g.lda, g.M);
-    misc.y = LB::goff(lane, wave, n0, g.ldb, g.N);
-    // LDS address of this wave's 1 KB slot in pass 0 of buffer 0 (wave-uniform)
-    const uint32_t m0b = __builtin_amdgcn_readfirstlane(lds0 + (uint32_t)wave * 1024u);
-    const __amdgpu_buffer_rsrc_t rsa =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(a), 0, a_bytes, 0x00020000);
-    const __amdgpu_buffer_rsrc_t rsb =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(b), 0, b_bytes, 0x00020000);
-
-    f32x16 acc[4 * NBF];
-    main_loop<T, TA, TB, BW>(acc, ra, rb, misc, rsa, rsb, LA::pass_stride(g.lda), LB::pass_stride(g.ldb),
-                             LA::stage_stride(g.lda), LB::stage_stride(g.ldb), m0b, (uint32_t)(g.K / 32));
-
     // The loop ends with every wave's outstanding loads landed and a barrier, so the
     // ring may be reused as the staging area below.  Waves may still have (unused)
     // fragment reads of a stage past the end in flight; overwriting those is harmless.
@@ -235,6 +203,217 @@ __global__ __launch_bounds__(256) void gemm256_kernel(GemmArgs g) {
     }
 }
 
+// BW = 256: the 256x256 tile (each wave 128x128).  BW = 128: a 256x128 tile (each wave
+// 128x64, half the accumulators, a 24 KB stage) for problems whose 256x256 tiling would
+// leave compute units idle or a last round nearly empty.
+template <typename T, bool TA, bool TB, int BW>
+__global__ __launch_bounds__(256) void gemm256_kernel(GemmArgs g) {
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    using LA = typename std::conditional<TA, MnMajor<256>, KMajor>::type;
+    using LB = typename std::conditional<TB, KMajor, MnMajor<BW>>::type;
+    constexpr int WN = BW / 2;            // columns per wave
+    constexpr int NBF = BW / 64;          // 32-column accumulator blocks per wave
+
+    int tm, tn;
+    tile_of(blockIdx.x, gridDim.x, g.tiles_m, g.tiles_n, tm, tn);
+    const int m0 = tm * 256, n0 = tn * BW;
+    const int64_t batch = blockIdx.y;
+    const char* a = reinterpret_cast<const char*>(static_cast<const T*>(g.a) + batch * g.sa);
+    const char* b = reinterpret_cast<const char*>(static_cast<const T*>(g.b) + batch * g.sb);
+    T* c = static_cast<T*>(g.c) + batch * g.sc;
+    const T* res = g.residual ? static_cast<const T*>(g.residual) + batch * g.sc : nullptr;
+    const uint32_t a_bytes = (uint32_t)((int64_t)(TA ? g.K : g.M) * g.lda * 2);
+    const uint32_t b_bytes = (uint32_t)((int64_t)(TB ? g.N : g.K) * g.ldb * 2);
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int lrow = lane & 31, lhalf = lane >> 5;
+    // LDS byte address of the dynamic segment
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
+
+    const u32x4 ra = LA::raddr(lane, wm * 128, lds0);
+    const u32x4 rb = LB::raddr(lane, wn * WN, lds0 + kOperBytes);
+    u32x2 misc;
+    misc.x = LA::goff(lane, wave, m0, g.lda, g.M);
+    misc.y = LB::goff(lane, wave, n0, g.ldb, g.N);
+    // LDS address of this wave's 1 KB slot in pass 0 of buffer 0 (wave-uniform)
+    const uint32_t m0b = __builtin_amdgcn_readfirstlane(lds0 + (uint32_t)wave * 1024u);
+    const __amdgpu_buffer_rsrc_t rsa =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(a), 0, a_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsb =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(b), 0, b_bytes, 0x00020000);
+
+    f32x16 acc[4 * NBF];
+    main_loop<T, TA, TB, BW>(acc, ra, rb, misc, rsa, rsb, LA::pass_stride(g.lda), LB::pass_stride(g.ldb),
+                             LA::stage_stride(g.lda), LB::stage_stride(g.ldb), m0b, (uint32_t)(g.K / 32));
+
+    store_tile<T, BW>(acc, smem, g, c, res, m0, n0);
+}
+
+// ---- streamed tiles ------------------------------------------------------------------------------
+// The 256x128 kernel as a persistent workgroup: one workgroup per compute unit runs tile after tile,
+// and the stores of a tile travel inside the main loop of the NEXT one (gemm_stream_loop_* of the
+// generated file), so that the matrix pipes do not idle through a burst of C stores at the end of
+// every round, nor through the load latency at the start of one: the loads of the next tile's first
+// stages are issued before the finished accumulators are converted.  Between two tiles only that
+// conversion (bias, activation, rounding to 16 bits: 64 registers of packed results) is exposed.
+// LDS: the ring of five 24 KB stage buffers, a 4 KB transposition area per wave, two 256-byte
+// buffers for the bias values of the current and the previous tile.
+// Served: A with k contiguous, M a multiple of 256, N of 128 (no ragged tiles: the in-loop stores
+// carry no bounds checks), no residual, one batch, K >= 640.  Tile 0 of a workgroup runs the
+// ordinary loop, the last one the ordinary epilogue; results are those of gemm256_kernel bit for bit.
+constexpr int kStreamWorkgroups = 256;          // one per compute unit of the device this is written for
+constexpr uint32_t kStreamRing = 5 * 24 * 1024;
+constexpr uint32_t kStreamXpose = kStreamRing;                 // 4 waves x 4 KB
+constexpr uint32_t kStreamBias = kStreamRing + 4 * 4096;       // 2 x 256 bytes
+constexpr uint32_t kStreamSmem = kStreamBias + 512;
+
+template <typename T, bool TB>
+__device__ __forceinline__ void stream_prologue(u32x2& misc, __amdgpu_buffer_rsrc_t rsa, __amdgpu_buffer_rsrc_t rsb,
+                                       uint32_t pa, uint32_t pb, uint32_t ta, uint32_t tb, uint32_t m0b,
+                                       __amdgpu_buffer_rsrc_t rsbias, uint32_t m0bias, uint32_t vbias) {
+    constexpr bool bf = std::is_same<T, bf16_t>::value;
+    if constexpr (bf && !TB) gemm_stream_loop_nn_bf16_prologue(misc, rsa, rsb, pa, pb, ta, tb, m0b, rsbias, m0bias, vbias);
+    if constexpr (bf && TB) gemm_stream_loop_nt_bf16_prologue(misc, rsa, rsb, pa, pb, ta, tb, m0b, rsbias, m0bias, vbias);
+    if constexpr (!bf && !TB) gemm_stream_loop_nn_f16_prologue(misc, rsa, rsb, pa, pb, ta, tb, m0b, rsbias, m0bias, vbias);
+    if constexpr (!bf && TB) gemm_stream_loop_nt_f16_prologue(misc, rsa, rsb, pa, pb, ta, tb, m0b, rsbias, m0bias, vbias);
+}
+
+template <typename T, bool TB>
+__device__ __forceinline__ void stream_loop(f32x16 (&acc)[8], u32x4 ra, u32x4 rb, u32x2& misc, __amdgpu_buffer_rsrc_t rsa,
+                                   __amdgpu_buffer_rsrc_t rsb, uint32_t pa, uint32_t pb, uint32_t ta, uint32_t tb,
+                                   uint32_t m0b, uint32_t kt, const u32x16 (&pk)[4], u32x4 xaddr, uint64_t cptr,
+                                   uint32_t srow) {
+    constexpr bool bf = std::is_same<T, bf16_t>::value;
+    if constexpr (bf && !TB) gemm_stream_loop_nn_bf16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt, pk, xaddr, cptr, srow);
+    if constexpr (bf && TB) gemm_stream_loop_nt_bf16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt, pk, xaddr, cptr, srow);
+    if constexpr (!bf && !TB) gemm_stream_loop_nn_f16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt, pk, xaddr, cptr, srow);
+    if constexpr (!bf && TB) gemm_stream_loop_nt_f16(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt, pk, xaddr, cptr, srow);
+}
+
+// Bias, activation and rounding of a finished tile, in the arithmetic of store_tile; the bias values
+// come from the LDS buffer the tile's prologue filled.  pk[i][2 c], pk[i][2 c + 1]: accumulator block
+// i (32 rows), columns 8 c + 4 (lane >> 5) .. + 3 of the wave's 64.
+template <typename T>
+__device__ __forceinline__ void pack_tile(const f32x16 (&acc)[8], const char* bias_lds, int act, int wn, int lhalf,
+                                 u32x16 (&pk)[4]) {
+    dispatch_act(act, [&](auto act_tag) {
+    constexpr int ACT = decltype(act_tag)::value;
+    static_for<8>([&](auto c_tag) {
+        constexpr int cidx = decltype(c_tag)::value, j = cidx >> 2, q = cidx & 3;
+        const Pack4<T> t = __builtin_bit_cast(
+            Pack4<T>, *reinterpret_cast<const u32x2*>(bias_lds + (wn * 64 + 8 * cidx + 4 * lhalf) * 2));
+        float bv[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) bv[e] = Elem<T>::to_f32(t.v[e]);
+        static_for<4>([&](auto i_tag) {
+            constexpr int i = decltype(i_tag)::value;
+            Pack4<T> o;
+            static_for<4>([&](auto e_tag) {
+                constexpr int e = decltype(e_tag)::value;
+                float v = acc[i * 2 + j][4 * q + e] + bv[e];
+                v = apply_act_c<ACT>(v);
+                o.v[e] = Elem<T>::from_f32(v);
+            });
+            const u32x2 w = __builtin_bit_cast(u32x2, o);
+            pk[i][2 * cidx] = w.x;
+            pk[i][2 * cidx + 1] = w.y;
+        });
+        __builtin_amdgcn_sched_barrier(0);
+    });
+    });
+}
+
+template <typename T, bool TB>
+__global__ __launch_bounds__(256) void gemm_stream_kernel(GemmArgs g, int total) {
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    using LA = KMajor;
+    using LB = typename std::conditional<TB, KMajor, MnMajor<128>>::type;
+    const char* a = reinterpret_cast<const char*>(g.a);
+    const char* b = reinterpret_cast<const char*>(g.b);
+    T* c = static_cast<T*>(g.c);
+    const T* bias = static_cast<const T*>(g.bias);
+    const uint32_t a_bytes = (uint32_t)((int64_t)g.M * g.lda * 2);
+    const uint32_t b_bytes = (uint32_t)((int64_t)(TB ? g.N : g.K) * g.ldb * 2);
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int lrow = lane & 31, lhalf = lane >> 5;
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
+    const u32x4 ra = LA::raddr(lane, wm * 128, lds0);
+    const u32x4 rb = LB::raddr(lane, wn * 64, lds0 + kOperBytes);
+    const uint32_t m0b = __builtin_amdgcn_readfirstlane(lds0 + (uint32_t)wave * 1024u);
+    const __amdgpu_buffer_rsrc_t rsa =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(a), 0, a_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsb =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(b), 0, b_bytes, 0x00020000);
+    // without a bias: an empty buffer, whose loads put zeros into LDS
+    const __amdgpu_buffer_rsrc_t rsbias = __builtin_amdgcn_make_buffer_rsrc(
+        bias ? const_cast<T*>(bias) : c, 0, bias ? (uint32_t)g.N * 2u : 0u, 0x00020000);
+    const uint32_t pa = LA::pass_stride(g.lda), pb = LB::pass_stride(g.ldb);
+    const uint32_t ta = LA::stage_stride(g.lda), tb = LB::stage_stride(g.ldb);
+    const uint32_t kt = (uint32_t)(g.K / 32);
+    // transposition area of this wave: write address of this lane's row (chunk 0), read address
+    const uint32_t xbase = lds0 + kStreamXpose + (uint32_t)wave * 4096u;
+    u32x4 xaddr;
+    xaddr.x = xbase + (uint32_t)(lrow * 128 + 8 * lhalf + (((lrow >> 1) & 7) << 4));
+    xaddr.y = xbase + (uint32_t)lane * 16u;
+    const uint32_t srow = (uint32_t)g.N * 16u;            // eight rows of C, in bytes
+    const int chunk_even = (lane & 7) ^ ((lane >> 4) & 3);
+
+    f32x16 acc[8];
+    u32x16 pk[4];
+    int m0 = 0, n0 = 0, it = 0;
+    for (int vp = blockIdx.x; vp < total; vp += gridDim.x, it++) {
+        const int pm0 = m0, pn0 = n0;
+        int tm, tn;
+        tile_of(vp, total, g.tiles_m, g.tiles_n, tm, tn);
+        m0 = tm * 256; n0 = tn * 128;
+        u32x2 misc;
+        misc.x = LA::goff(lane, wave, m0, g.lda, g.M);
+        misc.y = LB::goff(lane, wave, n0, g.ldb, g.N);
+        if (it == 0) {
+            if (wave == 0)
+                *reinterpret_cast<uint32_t*>(smem + kStreamBias + lane * 4) =
+                    bias ? *reinterpret_cast<const uint32_t*>(bias + n0 + 2 * lane) : 0u;
+            main_loop<T, false, TB, 128>(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt);
+        } else {
+            const uint32_t m0bias = __builtin_amdgcn_readfirstlane(lds0 + kStreamBias + (uint32_t)(it & 1) * 256u);
+            stream_prologue<T, TB>(misc, rsa, rsb, pa, pb, ta, tb, m0b, rsbias, m0bias,
+                                   (uint32_t)(n0 * 2 + lane * 4));
+            pack_tile<T>(acc, smem + kStreamBias + ((it - 1) & 1) * 256, g.act, wn, lhalf, pk);
+            // where the previous tile's rows go: this lane's chunk of row (lane / 8) of each 8-row group
+            const uint32_t off_even =
+                (uint32_t)((((int64_t)(pm0 + wm * 128 + (lane >> 3)) * g.N) + pn0 + wn * 64 + chunk_even * 8) * 2);
+            xaddr.z = off_even;
+            xaddr.w = off_even ^ 64u;
+            stream_loop<T, TB>(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt, pk, xaddr,
+                               (uint64_t)reinterpret_cast<uintptr_t>(c), srow);
+        }
+    }
+    store_tile<T, 128>(acc, smem, g, c, static_cast<const T*>(nullptr), m0, n0);
+}
+
+template <typename T, bool TB>
+int launch_stream(hipStream_t s, GemmArgs g) {
+    auto kern = gemm_stream_kernel<T, TB>;
+    static std::once_flag once;
+    static hipError_t attr_err = hipSuccess;
+    std::call_once(once, [&] {
+        attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)kStreamSmem);
+    });
+    if (attr_err != hipSuccess)
+        return fail(MHIP_ERR_LAUNCH, "gemm_stream: cannot reserve %u bytes of LDS: %s", kStreamSmem,
+                    hipGetErrorString(attr_err));
+    g.tiles_m = g.M / 256;
+    g.tiles_n = g.N / 128;
+    const int total = g.tiles_m * g.tiles_n;
+    const int grid = total < kStreamWorkgroups ? total : kStreamWorkgroups;
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), kStreamSmem, s, g, total);
+    return check_launch("gemm_stream");
+}
+
 template <typename T, bool TA, bool TB, int BW>
 int launch256(hipStream_t s, GemmArgs g, int64_t batch) {
     constexpr int kSmem = 5 * (16 + BW / 16) * 1024;   // ring of five stage buffers; the epilogue staging reuses it
@@ -290,6 +469,21 @@ int launch_gemm256(hipStream_t s, const GemmArgs& g, int64_t batch, int trans_a,
     }
     if (dtype == MHIP_BF16) return layout256<bf16_t, 256>(s, g, batch, trans_a, trans_b);
     return layout256<f16_t, 256>(s, g, batch, trans_a, trans_b);
+}
+
+// Streamed tiles (persistent workgroups, stores inside the next tile's loop): see gemm_stream_kernel.
+// Worth it from the second round on, i.e. with more tiles than compute units.
+bool gemm_stream_eligible(const GemmArgs& g, int64_t batch, int trans_a, int dtype) {
+    if (!gemm256_eligible(g, batch, dtype, 128)) return false;
+    if (trans_a || batch != 1 || g.residual) return false;
+    if (g.M % 256 != 0 || g.N % 128 != 0 || g.K < 640) return false;
+    if ((int64_t)g.M * g.N * 2 >= 0xFFFFFFFFLL) return false;          // 32-bit byte offsets into C
+    return (int64_t)(g.M / 256) * (g.N / 128) > kStreamWorkgroups;
+}
+
+int launch_gemm_stream(hipStream_t s, const GemmArgs& g, int trans_b, int dtype) {
+    if (dtype == MHIP_BF16) return trans_b ? launch_stream<bf16_t, true>(s, g) : launch_stream<bf16_t, false>(s, g);
+    return trans_b ? launch_stream<f16_t, true>(s, g) : launch_stream<f16_t, false>(s, g);
 }
 
 }  // namespace mhip

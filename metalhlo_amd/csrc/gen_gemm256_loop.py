@@ -212,7 +212,7 @@ def drop(lines, prefix):
     return [l for l in lines if not l.startswith(prefix)]
 
 
-def stage_iteration(mnem, kinds, t, vmcnt):
+def stage_iteration(mnem, kinds, t, vmcnt, extra=(), extra_mid=()):
     g, nxt = t % NST, (t + 1) % NST
     r0 = all_frag_reads(kinds, nxt, 0, (2 * t + 2) % 4)
     r1 = all_frag_reads(kinds, nxt, 1, (2 * t + 3) % 4)
@@ -222,10 +222,12 @@ def stage_iteration(mnem, kinds, t, vmcnt):
     # k-step 0: its fragments were read one stage ago; only the previous k-step's reads
     # (LDS operations retire in order) may still be outstanding
     out.append(f"s_waitcnt lgkmcnt({min(len(r1), 15)})")
+    out += list(extra)      # older than every fragment read of this stage: the waits below cover them
     out += interleave(mfmas(mnem, (2 * t) % 4), r0, prev_second)
     # k-step 1
     out.append(f"s_waitcnt vmcnt({min(vmcnt, 63)}) lgkmcnt({min(len(r0), 15)})")
     out.append("s_barrier")
+    out += list(extra_mid)
     out += interleave(mfmas(mnem, (2 * t + 1) % 4), r1, this_first)
     if "noload" in EXP:
         out = [l for l in drop(drop(out, "buffer_load"), "s_add_u32 m0") if l != "s_nop 0"]
@@ -287,10 +289,179 @@ def body(mnem, kinds):
     return out
 
 
+# ---- streamed tiles ------------------------------------------------------------------------------
+# A persistent workgroup of the 256x128 kernel runs tile after tile.  From its second tile on, the
+# loop below also stores the PREVIOUS tile, which the caller hands over as packed 16-bit values in
+# v[128:191] (accumulator block i, 8-byte group c = 4 j + q at v[128 + 16 i + 2 c : +1]: row
+# 32 i + (lane & 31), columns 8 c + 4 (lane >> 5) .. + 3 of the wave's 128x64 sub-tile).  The first
+# 16 stages carry it, one 32-row block per four stages, through a 4 KB transposition area per wave:
+#   stage 4i   : eight ds_write_b64 (row = 128 bytes, 16-byte chunk c at position c ^ ((row >> 1) & 7))
+#   stage 4i+1 : four ds_read_b128, lane l <- row 8 p + l / 8, position l % 8
+#   stage 4i+2 : four global_store_dwordx4 of 8 rows x 128 bytes each, right behind the barrier: an
+#                even stage's wait is the tight one (it leaves only the youngest loads outstanding and
+#                would have to sit out a store still in flight), and from there the next one is two
+#                stages away
+# The prologue (the loads of the first stages, and the tile's 128 bias values straight into LDS) is a
+# function of its own, so that the caller can issue it BEFORE it converts the previous accumulators:
+# the load latency then hides behind that conversion.  The caller must issue no vector memory
+# instruction between the two functions (the waits below count the prologue's loads).
+# Extra registers: v[220:235] chunk temporaries, v236 transposition write address (this lane's row,
+# chunk 0), v237 read address, v238 / v239 byte offset into C of this lane's chunk for even / odd
+# p, v[240:247] write addresses of the eight chunks, s[82:83] running row pointer into C.
+STRAIGHT = 20         # stages emitted straight-line at the start of a streamed tile (2 x UNROLL)
+XSTAGES = 16          # the first 16 of them carry the previous tile
+PK, TMP, XA, WA, SC = 128, 220, 236, 240, 82
+
+
+def stream_extras(t):
+    """(lines in front of the stage's first MFMA, lines behind its barrier)"""
+    i, ph = divmod(t, 4)
+    first, mid = [], []
+    if ph == 0:
+        for c in range(8):
+            r = PK + 16 * i + 2 * c
+            first.append(f"ds_write_b64 v{WA + c}, v[{r}:{r + 1}]")
+    elif ph == 1:
+        for p in range(4):
+            first.append(f"ds_read_b128 {vr(TMP + 4 * p, 4)}, v{XA + 1} offset:{p * 1024}")
+    elif ph == 2:
+        for p in range(4):
+            # ordinary stores: with the streaming hint (nt) this kernel gained up to 7 %, but the next
+            # kernel, which reads C, lost more than that (GPT-2 FFN-down after FFN-up: 54 -> 67 us)
+            mid.append(f"global_store_dwordx4 v{XA + 2 + (p & 1)}, {vr(TMP + 4 * p, 4)}, s[{SC}:{SC + 1}]")
+            mid.append(f"s_add_u32 s{SC}, s{SC}, %[srow]")
+            mid.append(f"s_addc_u32 s{SC + 1}, s{SC + 1}, 0")
+    return first, mid
+
+
+def simulate_stream(kinds):
+    """vmcnt of the prologue wait and of each straight-line stage of a streamed tile.  The stores
+    of the previous tile are left out of the count on purpose: a store may be acknowledged before
+    an older load has landed, so a wait that allowed for them could pass too early, while a wait
+    that ignores them at worst also waits for a few younger loads."""
+    tr = Tracker()
+    tr.order.append(-100)                       # the bias load, first of the prologue
+    for t in range(-NST, -1):
+        tr.issue(trigger_group(kinds, t))
+    first, pending = halves(trigger_group(kinds, -1))
+    tr.issue(first)
+    pro = tr.allowed(1)
+    counts = []
+    for t in range(STRAIGHT):
+        tr.issue(pending)
+        counts.append(tr.allowed(t + 2))
+        first, pending = halves(trigger_group(kinds, t))
+        tr.issue(first)
+    return pro, counts
+
+
+def stream_prologue(kinds):
+    out = [f"s_mov_b32 s{ST + 1}, m0"]
+    for which, pin in (("A", "%[pa]"), ("B", "%[pb]")):
+        for i in range(1, 4):
+            out.append(f"s_mul_i32 s{SP[which] + i - 1}, {pin}, {i}")
+        out.append(f"v_add_u32 v{GOFF2[which]}, 64, v{GOFF[which]}")
+    out += ["s_mov_b32 m0, %[m0bias]", "s_nop 0", "buffer_load_dword %[vbias], %[rsbias], 0 offen lds"]
+    for t in range(-NST, -1):
+        for ld in trigger_group(kinds, t):
+            out += ld["lines"]
+    first, _ = halves(trigger_group(kinds, -1))
+    for ld in first:
+        out += ld["lines"]
+    out.append(f"s_mov_b32 m0, s{ST + 1}")
+    return out
+
+
+def stream_body(mnem, kinds):
+    pro_vmcnt, straight = simulate_stream(kinds)
+    _, vmcnts = simulate(kinds)
+    out = [f"s_mov_b32 s{ST + 1}, m0"]
+    for r in range(64 * NBF):
+        out.append(f"v_accvgpr_write_b32 a{r}, 0")
+    for which, pin in (("A", "%[pa]"), ("B", "%[pb]")):
+        for i in range(1, 4):
+            out.append(f"s_mul_i32 s{SP[which] + i - 1}, {pin}, {i}")
+    for which, base in (("A", RA), ("B", RB)):
+        n = 2 if kinds[which] == "K" else 4
+        for h in (1, 2):
+            for e in range(n):
+                out.append(f"v_add_u32 v{base + n * h + e}, {h * 2 * STAGE}, v{base + e}")
+        out.append(f"v_add_u32 v{GOFF2[which]}, 64, v{GOFF[which]}")
+    for c in range(8):
+        out.append(f"v_xor_b32 v{WA + c}, {16 * c}, v{XA}")
+    out.append(f"s_mov_b64 s[{SC}:{SC + 1}], %[cptr]")
+    out.append(f"s_waitcnt vmcnt({pro_vmcnt})")           # stages 0 and 1 landed
+    out.append("s_barrier")
+    out += all_frag_reads(kinds, 0, 0, 0)
+    out += all_frag_reads(kinds, 0, 1, 1)
+    out.append("s_waitcnt lgkmcnt(0)")
+    for t in range(STRAIGHT):
+        first, mid = stream_extras(t) if t < XSTAGES else ((), ())
+        out += stage_iteration(mnem, kinds, t, straight[t], first, mid)
+    out.append(f"s_mov_b32 s{ST}, {STRAIGHT}")
+    out.append(f"s_cmp_ge_u32 s{ST}, %[kt]")
+    out.append("s_cbranch_scc1 L_gemm256_done_%=")
+    out.append("L_gemm256_loop_%=:")
+    for t in range(UNROLL):
+        out += stage_iteration(mnem, kinds, STRAIGHT + t, vmcnts[t])
+        out.append(f"s_add_u32 s{ST}, s{ST}, 1")
+        if t < UNROLL - 1:
+            out.append(f"s_cmp_ge_u32 s{ST}, %[kt]")
+            out.append("s_cbranch_scc1 L_gemm256_done_%=")
+        else:
+            out.append(f"s_cmp_lt_u32 s{ST}, %[kt]")
+            out.append("s_cbranch_scc1 L_gemm256_loop_%=")
+    out.append("L_gemm256_done_%=:")
+    out.append("s_waitcnt vmcnt(0) lgkmcnt(0)")
+    out.append("s_barrier")
+    out.append(f"s_mov_b32 m0, s{ST + 1}")
+    out += ["s_nop 15", "s_nop 15"]
+    return out
+
+
+def emit_stream(name, mnem, ka, kb):
+    kinds = {"A": ka, "B": kb}
+    print(f"// {name}_prologue: loads of the first stages of a streamed tile and its bias values")
+    print(f"__device__ __forceinline__ void {name}_prologue(u32x2& goff, __amdgpu_buffer_rsrc_t rsa,")
+    print("        __amdgpu_buffer_rsrc_t rsb, uint32_t pa, uint32_t pb, uint32_t ta, uint32_t tb, uint32_t m0b,")
+    print("        __amdgpu_buffer_rsrc_t rsbias, uint32_t m0bias, uint32_t vbias) {")
+    print("    asm volatile(")
+    for ln in stream_prologue(kinds):
+        print(f'        "{ln}\\n"')
+    print(f'        : "+{{v[{GOFF["A"]}:{GOFF["B"]}]}}"(goff)')
+    print('        : [rsa] "s"(rsa), [rsb] "s"(rsb), [pa] "s"(pa), [pb] "s"(pb), [ta] "s"(ta), [tb] "s"(tb),')
+    print('          [m0b] "s"(m0b), [rsbias] "s"(rsbias), [m0bias] "s"(m0bias), [vbias] "v"(vbias)')
+    clob = [f'"v{GOFF2["A"]}"', f'"v{GOFF2["B"]}"'] + [f'"s{i}"' for i in range(SP["A"], ST + 2)] + ['"scc"', '"memory"']
+    print("        : " + ", ".join(clob) + ");")
+    print("}\n")
+    print(f"// {name}: main loop of a streamed tile ({mnem}); stores the previous tile on the way")
+    print(f"__device__ __forceinline__ void {name}(f32x16 (&acc)[{4 * NBF}], u32x4& ra, u32x4& rb, u32x2& goff,")
+    print("        __amdgpu_buffer_rsrc_t rsa, __amdgpu_buffer_rsrc_t rsb, uint32_t pa, uint32_t pb,")
+    print("        uint32_t ta, uint32_t tb, uint32_t m0b, uint32_t kt, const u32x16 (&pk)[4], u32x4 xaddr,")
+    print("        uint64_t cptr, uint32_t srow) {")
+    print("    asm volatile(")
+    for ln in stream_body(mnem, kinds):
+        print(f'        "{ln}\\n"')
+    outs = ", ".join(f'"={{a[{16 * i}:{16 * i + 15}]}}"(acc[{i}])' for i in range(4 * NBF))
+    print(f"        : {outs},")
+    print(f'          "+{{v[{GOFF["A"]}:{GOFF["B"]}]}}"(goff), "+{{v[{RA}:{RA + 3}]}}"(ra), "+{{v[{RB}:{RB + 3}]}}"(rb)')
+    print('        : [rsa] "s"(rsa), [rsb] "s"(rsb), [pa] "s"(pa), [pb] "s"(pb), [ta] "s"(ta), [tb] "s"(tb),')
+    print('          [m0b] "s"(m0b), [kt] "s"(kt),')
+    pks = ", ".join(f'"{{v[{PK + 16 * i}:{PK + 16 * i + 15}]}}"(pk[{i}])' for i in range(4))
+    print(f"          {pks},")
+    print(f'          "{{v[{XA}:{XA + 3}]}}"(xaddr), [cptr] "s"(cptr), [srow] "s"(srow)')
+    vclob = (list(range(128)) + list(range(RA + 4, RB)) + list(range(RB + 4, GOFF["A"])) + [GOFF2["A"], GOFF2["B"]]
+             + list(range(TMP, TMP + 16)) + list(range(WA, WA + 8)))
+    clob = ([f'"v{i}"' for i in vclob] + [f'"s{i}"' for i in range(SP["A"], ST + 2)] + [f'"s{SC}"', f'"s{SC + 1}"']
+            + ['"scc"', '"memory"'])
+    print("        : " + ", ".join(clob) + ");")
+    print("}\n")
+
+
 def emit(name, mnem, ka, kb):
     lines = body(mnem, {"A": ka, "B": kb})
     print(f"// {name}: A operand {ka}-major, B operand {kb}-major, {mnem}")
-    print(f"__device__ __forceinline__ void {name}(f32x16 (&acc)[{4 * NBF}], u32x4 ra, u32x4 rb, u32x2& goff,")
+    print(f"__device__ __forceinline__ void {name}(f32x16 (&acc)[{4 * NBF}], u32x4& ra, u32x4& rb, u32x2& goff,")
     print("        __amdgpu_buffer_rsrc_t rsa, __amdgpu_buffer_rsrc_t rsb, uint32_t pa, uint32_t pb,")
     print("        uint32_t ta, uint32_t tb, uint32_t m0b, uint32_t kt) {")
     print("    asm volatile(")
@@ -298,9 +469,10 @@ def emit(name, mnem, ka, kb):
         print(f'        "{ln}\\n"')
     outs = ", ".join(f'"={{a[{16 * i}:{16 * i + 15}]}}"(acc[{i}])' for i in range(4 * NBF))
     print(f"        : {outs},")
-    print(f'          "+{{v[{GOFF["A"]}:{GOFF["B"]}]}}"(goff)')
-    print(f'        : "{{v[{RA}:{RA + 3}]}}"(ra), "{{v[{RB}:{RB + 3}]}}"(rb),')
-    print('          [rsa] "s"(rsa), [rsb] "s"(rsb), [pa] "s"(pa), [pb] "s"(pb), [ta] "s"(ta), [tb] "s"(tb),')
+    # ra / rb are written too: the addresses of the other ring buffers of a k-contiguous operand
+    # are derived into their upper elements
+    print(f'          "+{{v[{GOFF["A"]}:{GOFF["B"]}]}}"(goff), "+{{v[{RA}:{RA + 3}]}}"(ra), "+{{v[{RB}:{RB + 3}]}}"(rb)')
+    print('        : [rsa] "s"(rsa), [rsb] "s"(rsb), [pa] "s"(pa), [pb] "s"(pb), [ta] "s"(ta), [tb] "s"(tb),')
     print('          [m0b] "s"(m0b), [kt] "s"(kt)')
     vclob = list(range(128)) + list(range(RA + 4, RB)) + list(range(RB + 4, GOFF["A"])) + [GOFF2["A"], GOFF2["B"]]
     clob = [f'"v{i}"' for i in vclob] + [f'"s{i}"' for i in range(SP["A"], ST + 2)] + ['"scc"', '"memory"']
@@ -317,6 +489,11 @@ def main():
         for tname, mnem in (("bf16", "v_mfma_f32_32x32x16_bf16"), ("f16", "v_mfma_f32_32x32x16_f16")):
             for lname, ka, kb in (("nn", "K", "MN"), ("nt", "K", "K"), ("tn", "MN", "MN"), ("tt", "MN", "K")):
                 emit(f"{stem}_{lname}_{tname}", mnem, ka, kb)
+    # streamed tiles: the 256x128 kernel as a persistent workgroup, for A with k contiguous
+    configure(128)
+    for tname, mnem in (("bf16", "v_mfma_f32_32x32x16_bf16"), ("f16", "v_mfma_f32_32x32x16_f16")):
+        for lname, ka, kb in (("nn", "K", "MN"), ("nt", "K", "K")):
+            emit_stream(f"gemm_stream_loop_{lname}_{tname}", mnem, ka, kb)
 
 
 if __name__ == "__main__":

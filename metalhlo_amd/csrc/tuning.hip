@@ -28,6 +28,7 @@
 namespace mhip {
 
 bool gemm256_eligible(const GemmArgs& g, int64_t batch, int dtype, int bw = 256);
+bool gemm_stream_eligible(const GemmArgs& g, int64_t batch, int trans_a, int dtype);
 
 namespace {
 struct Entry { std::string choice; float us; };
@@ -83,7 +84,7 @@ bool valid_choice(const char* line, const std::string& choice) {
     int a = 0, b = 0, c = 0, d = 0;
     if (!strncmp(line, "gemm ", 5)) {
         const int v = atoi(choice.c_str());
-        return v == 128 || v == 256 || v == 2560 || v == 2561;
+        return v == 128 || v == 256 || v == 2560 || v == 2561 || v == 2562;
     }
     if (!strncmp(line, "row ", 4))
         return sscanf(choice.c_str(), "%d %d %d %d", &a, &b, &c, &d) == 4 && (a == 1 || a == 2) && (b == 1 || b == 2) &&
@@ -172,7 +173,7 @@ int tuned_gemm_variant(const GemmArgs& g, int64_t batch, int ta, int tb, int dty
     std::string c;
     if (!have_entries() || !lookup(gemm_key(g.M, g.N, g.K, batch, ta, tb, dtype), &c)) return 0;
     const int v = atoi(c.c_str());
-    return (v == 128 || v == 256 || v == 2560 || v == 2561) ? v : 0;
+    return (v == 128 || v == 256 || v == 2560 || v == 2561 || v == 2562) ? v : 0;
 }
 
 bool tuned_row_launch(int op, int dtype, int64_t rows, int64_t cols, bool has_gamma, bool has_beta, RowLaunch* out) {
@@ -212,12 +213,13 @@ extern "C" int mhip_gemm_autotune(void* stream, const void* a, const void* b, co
     g.a = a; g.b = b; g.bias = bias; g.c = c;
     g.M = (int)M; g.N = (int)N; g.K = (int)K;
     g.sa = stride_a; g.sb = stride_b; g.sc = stride_c;
-    const int candidates[4] = {128, 256, 2560, 2561};
+    const int candidates[5] = {128, 256, 2560, 2561, 2562};
     int best = 0;
     float best_us = 0.f;
     for (int v : candidates) {
         if (v == 2560 && !gemm256_eligible(g, batch, dtype)) continue;    // validity filter
         if (v == 2561 && !gemm256_eligible(g, batch, dtype, 128)) continue;
+        if (v == 2562 && !gemm_stream_eligible(g, batch, trans_a, dtype)) continue;
         g_forced_gemm = v;
         const float us = t.time(s, iters, [&] {
             return mhip_gemm(stream, a, b, bias, c, M, N, K, batch, stride_a, stride_b, stride_c, trans_a, trans_b, activation, dtype);

@@ -256,6 +256,56 @@ def test_gemm_ring_kernel_rows_of_c_at_any_alignment(tile, dtype, monkeypatch):
         assert_close(c[rows], exp, TOL[dtype], f"odd N + residual {(M, N, K)}")
 
 
+# More 256x128 tiles than compute units, M a multiple of 256, N of 128, K >= 640: the persistent
+# workgroups that store a tile inside the loop of the next one (several tiles per workgroup, a
+# last round that is not full, K that leaves the straight-line part at once or after some trips).
+STREAMED = [(8192, 3072, 768), (2304, 4096, 640), (4096, 8320, 1024), (8192, 2304, 2080)]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=lambda d: NAME[d])
+@pytest.mark.parametrize("tb", [False, True], ids=["nn", "nt"])
+@pytest.mark.parametrize("shape", STREAMED, ids=lambda s: "x".join(map(str, s)))
+def test_gemm_streamed_tiles(shape, tb, dtype, monkeypatch):
+    """Forced, and compared with the oracle on sampled rows of every tile row and bit for bit with
+    the plain 256x128 kernel; with and without bias, GELU epilogue; nothing written outside C."""
+    from metalhlo_amd import kernels
+    M, N, K = shape
+    a, b = _ab(M, N, K, dtype, 61, False, tb)
+    rng = np.random.default_rng(62)
+    bias = to_dev(rng.standard_normal(N) * 0.5, dtype)
+    for use_bias, act in ((True, "gelu"), (False, "none")):
+        bb = bias if use_bias else None
+        monkeypatch.setenv("MHIP_GEMM_TILE", "2562")
+        guard = torch.full((M * N + 4096,), 7.0, dtype=dtype, device="cuda")
+        c = kernels.matmul(a, b, bb, act, trans_b=tb, out=guard[2048:2048 + M * N].view(M, N))
+        assert torch.all(guard[:2048] == 7.0) and torch.all(guard[2048 + M * N:] == 7.0)
+        monkeypatch.setenv("MHIP_GEMM_TILE", "2561")
+        plain = kernels.matmul(a, b, bb, act, trans_b=tb)
+        assert torch.equal(c, plain), (shape, tb, use_bias)
+        rows = np.unique(np.r_[np.arange(0, M, 256), np.arange(255, M, 256), rng.integers(0, M, 24)])
+        B = as_f64(b).T if tb else as_f64(b)
+        exp = oracle.matmul_bias_act(as_f64(a)[rows], B, as_f64(bias) if use_bias else None, act)
+        assert_close(c[rows], exp, TOL[dtype], f"streamed gemm {shape} nt={tb} bias={use_bias}")
+
+
+def test_gemm_streamed_tiles_is_the_default_where_it_wins(lib):
+    """The default choice for a GPT-2-shaped product [8192, 768] x [768, 3072] is the streamed
+    kernel (same bits as forcing it), and a problem it cannot take (ragged N) still runs."""
+    from metalhlo_amd import kernels
+    a, b = _ab(8192, 3072, 768, torch.bfloat16, 63)
+    os.environ.pop("MHIP_GEMM_TILE", None)
+    c = kernels.matmul(a, b, None, "gelu")
+    os.environ["MHIP_GEMM_TILE"] = "2562"
+    try:
+        forced = kernels.matmul(a, b, None, "gelu")
+        a2, b2 = _ab(8192, 3000, 768, torch.bfloat16, 64)
+        ragged = kernels.matmul(a2, b2)
+    finally:
+        del os.environ["MHIP_GEMM_TILE"]
+    assert torch.equal(c, forced)
+    assert torch.equal(ragged, kernels.matmul(a2, b2))
+
+
 def test_gemm_large_exact_small_integers():
     """Integer-valued operands with exactly representable partial sums: bit-exact."""
     from metalhlo_amd import kernels
