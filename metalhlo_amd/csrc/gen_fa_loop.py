@@ -164,14 +164,18 @@ def rescale_block(tag):
     return out
 
 
-def k_read(f, slot):
+RING = 8           # fragment ring slots (v[96:127]); a slot holds one K or one V fragment
+VAHEAD = 6         # V fragments (two reads each) in flight at most: the LDS counter holds 15 operations
+
+
+def k_read(f, slot, ring=4):
     st, t = f // 2, f % 2
-    return f"ds_read_b128 {v(KF + 4 * (f % 4), 4)}, {v(KADDR + st)} offset:{slot * KTILE + t * 8192}"
+    return f"ds_read_b128 {v(KF + 4 * (f % ring), 4)}, {v(KADDR + st)} offset:{slot * KTILE + t * 8192}"
 
 
-def v_reads(g, slot):
+def v_reads(g, slot, ring=4):
     u, dt = g // 4, g % 4
-    base = VF + 4 * (g % 4)
+    base = VF + 4 * (g % ring)
     off = slot * KTILE + u * 4096
     return [f"ds_read_b64_tr_b16 {v(base, 2)}, {v(VADDR + dt)} offset:{off}",
             f"ds_read_b64_tr_b16 {v(base + 2, 2)}, {v(VADDR + dt)} offset:{off + 2048}"]
@@ -184,8 +188,40 @@ def v_prefetch(slot):
     return out
 
 
-def body(n):
-    """Body n of the unrolled loop handles block j = n (mod 4)."""
+class LdsOrder:
+    """LDS reads in program order, to size the lgkmcnt waits: a wait for fragment X may leave
+    outstanding exactly the reads issued after X's last one (they return in order)."""
+
+    def __init__(self):
+        self.tags = []
+
+    def issue(self, tag, lines):
+        self.tags += [tag] * len(lines)
+        return lines
+
+    def wait_for(self, tags):
+        last = max(i for i, t in enumerate(self.tags) if t in tags)
+        return f"s_waitcnt lgkmcnt({min(len(self.tags) - 1 - last, 15)})"
+
+
+def loop_prefetch(order, body_no, slot):
+    """The first VAHEAD V fragments of body `body_no` (ring buffer `slot`)."""
+    out = []
+    for g in range(VAHEAD):
+        out += order.issue(("V", body_no, g), v_reads(g, slot, RING))
+    return out
+
+
+def body(n, order, uid):
+    """Body n of the unrolled loop handles block j = n (mod 4).  `uid` numbers the bodies in
+    emission order (tags of the fragment reads, which run ahead across bodies).
+
+    Fragments go through a ring of eight register slots (fragment i of a phase in slot i % 8).
+    V fragments are read up to six ahead; the K fragments of phase A are read from the last
+    iterations of phase B on, i.e. BEFORE this step's barrier: the wait in front of the barrier
+    leaves only the youngest pair of loads in flight, so K(j+1) landed, for every wave, with the
+    barrier of the step before.  Phase A then starts with its first fragments in registers
+    instead of behind a full LDS latency."""
     slot_v = (n + 3) % 4             # V(j-1)
     slot_k = (n + 1) % 4             # K(j+1)
     load_k, load_v = n % 4, (n + 3) % 4          # K(j+4) replaces K(j), V(j+3) replaces V(j-1)
@@ -203,24 +239,26 @@ def body(n):
     # ---- phase B: O += V^T . P^T  ||  first half of the softmax
     k = 0
     for g2 in range(8):
-        out.append(f"s_waitcnt lgkmcnt({4 if g2 < 7 else 0})")       # two fragments (four reads) may be in flight
+        out.append(order.wait_for({("V", uid, 2 * g2), ("V", uid, 2 * g2 + 1)}))
         for g in (2 * g2, 2 * g2 + 1):
             u, dt = g // 4, g % 4
             for qi in range(NQ):
                 acc = a(128 + 16 * (4 * qi + dt), 16)
-                out.append(f"{MN} {acc}, {v(VF + 4 * (g % 4), 4)}, {v(pprev + 4 * (4 * qi + u), 4)}, {acc}")
+                out.append(f"{MN} {acc}, {v(VF + 4 * (g % RING), 4)}, {v(pprev + 4 * (4 * qi + u), 4)}, {acc}")
                 out += head[k]
                 k += 1
-        for g in (2 * g2 + 4, 2 * g2 + 5):
+        for g in (2 * g2 + VAHEAD, 2 * g2 + VAHEAD + 1):
             if g < 16:
-                out += v_reads(g, slot_v)
+                out += order.issue(("V", uid, g), v_reads(g, slot_v, RING))
+        # slots freed by the V fragments take the first eight K fragments of phase A
+        first_k = {5: range(0, 4), 6: range(4, 6), 7: range(6, 8)}.get(g2, ())
+        for f in first_k:
+            out += order.issue(("K", uid, f), [k_read(f, slot_k, RING)])
     # ---- end of B
     if "norescale" not in EXP:
-        out += rescale_block(f"{n}")
-    out.append("s_waitcnt vmcnt(16)")
+        out += rescale_block(f"{uid}")
+    out.append("s_waitcnt vmcnt(8)")
     out.append("s_barrier")
-    for f in range(4):
-        out.append(k_read(f, slot_k))
     # the eight loads of K(j+4), V(j+3): M0 (the LDS target) is written one MFMA ahead of its load
     loads = []
     for i in range(4):
@@ -230,7 +268,7 @@ def body(n):
     # ---- phase A: S(j+1) = K . Q^T  ||  second half of the softmax
     k = 0
     for f2 in range(8):
-        out.append(f"s_waitcnt lgkmcnt({2 if f2 < 7 else 0})")       # two fragments may be in flight
+        out.append(order.wait_for({("K", uid, 2 * f2), ("K", uid, 2 * f2 + 1)}))
         for f in (2 * f2, 2 * f2 + 1):
             st, t = f // 2, f % 2
             for qi in range(NQ):
@@ -238,7 +276,7 @@ def body(n):
                     out.append(loads[k][0])
                 d = v(s_out + 16 * (2 * qi + t), 16)
                 c = "0" if st == 0 else d
-                out.append(f"{MN} {d}, {v(KF + 4 * (f % 4), 4)}, {a(4 * (8 * qi + st), 4)}, {c}")
+                out.append(f"{MN} {d}, {v(KF + 4 * (f % RING), 4)}, {a(4 * (8 * qi + st), 4)}, {c}")
                 out += tail[k]
                 if k < len(loads):
                     out.append(loads[k][1])
@@ -246,19 +284,29 @@ def body(n):
                     out.append(f"v_add_u32 {v(GK)}, {KTILE}, {v(GK)}")
                     out.append(f"v_add_u32 {v(GV)}, {KTILE}, {v(GV)}")
                 k += 1
-        for f in (2 * f2 + 4, 2 * f2 + 5):
+        for f in (2 * f2 + 8, 2 * f2 + 9):
             if f < 16:
-                out.append(k_read(f, slot_k))
-    out += v_prefetch(n % 4)                  # V(j): the first fragments of the next body
+                out += order.issue(("K", uid, f), [k_read(f, slot_k, RING)])
+        # V(j): the first fragments of the next body, into the slots the K fragments leave
+        nxt = {4: (0, 1), 5: (2, 3), 6: (4, 5)}.get(f2, ())
+        for g in nxt:
+            out += order.issue(("V", uid + 1, g), v_reads(g, n % 4, RING))
     return out
 
 
 def loop():
     out = ["s_mov_b32 s72, 4096", "s_mov_b32 s73, 8192", "s_mov_b32 s74, 12288", "s_mov_b32 s76, 0", "s_mov_b32 s77, m0"]
-    out += v_prefetch(3)
+    # the waits are those of the steady state: a first trip through the four bodies sets up the order
+    # of the reads in flight, the second one is emitted (on entry fewer reads are in flight than the
+    # waits allow for, which only makes them stricter)
+    order = LdsOrder()
+    warm = loop_prefetch(order, 0, 3)
+    for n in range(4):
+        body(n, order, n)
+    out += warm
     out.append("L_fa_loop_%=:")
     for n in range(4):
-        out += body(n)
+        out += body(n, order, 4 + n)
         out.append("s_add_u32 s76, s76, 1")
         if n < 3:
             out.append("s_cmp_ge_u32 s76, %[count]")
@@ -372,6 +420,7 @@ def clobbers(vregs, sregs=()):
 
 O_OPS = '"+{a[128:159]}"(o0), "+{a[160:191]}"(o1), "+{a[192:223]}"(o2), "+{a[224:255]}"(o3)'
 FRAGS = list(range(KF, KF + 16))
+RING_FRAGS = list(range(KF, KF + 4 * RING))
 TEMPS = list(range(ALPHA, ALPHA + 14))
 
 
@@ -401,7 +450,7 @@ def emit_all(dt):
     print(f'          "+{{v[{GK}:{GV}]}}"(goff)')
     print(f'        : "{{a[0:31]}}"(q0), "{{a[32:63]}}"(q1), "{{v[{KADDR}:{KADDR + 7}]}}"(kaddr), "{{v[{VADDR}:{VADDR + 3}]}}"(vaddr),')
     print('          [rk] "s"(rk), [rv] "s"(rv), [c] "s"(c), [m0b] "s"(m0b), [count] "s"(count)')
-    print("        : " + clobbers(FRAGS + TEMPS, range(72, 86)) + ");")
+    print("        : " + clobbers(RING_FRAGS + TEMPS, range(72, 86)) + ");")
     print("}\n")
     # ---- last block
     print("// Last block of a wave: raw scores in (s0, s1), probabilities of the block before it in py,")
