@@ -108,13 +108,17 @@ def wl_gemm_f32(torch, kernels, M=4096, N=4096, K=4096):
                 bound="mfma", peak=PEAK_F32_TFLOPS, kernel="gemm_f32_mfma_kernel")
 
 
-def wl_attention(torch, kernels, B=4, H=32, S=4096, D=128, causal=True):
+def wl_attention(torch, kernels, B=4, H=32, S=4096, D=128, causal=True, fp32=False):
     g = torch.Generator(device="cuda").manual_seed(4)
-    q, k, v = (torch.randn(B, H, S, D, generator=g, device="cuda").to(torch.bfloat16) for _ in range(3))
+    dt = torch.float32 if fp32 else torch.bfloat16
+    q, k, v = (torch.randn(B, H, S, D, generator=g, device="cuda").to(dt) for _ in range(3))
     flops = 4.0 * B * H * S * S * D * (0.5 if causal else 1.0)
-    return dict(name=f"bf16 flash-attention fwd B{B} H{H} S{S} D{D} {'causal' if causal else 'full'}",
-                fn=lambda i: kernels.flash_attention(q, k, v, is_causal=causal), flops=flops,
-                bytes=4.0 * B * H * S * D * 2, bound="mfma", kernel="fa_pipe_kernel")
+    r = dict(name=f"{'fp32' if fp32 else 'bf16'} flash-attention fwd B{B} H{H} S{S} D{D} {'causal' if causal else 'full'}",
+             fn=lambda i: kernels.flash_attention(q, k, v, is_causal=causal), flops=flops,
+             bytes=4.0 * B * H * S * D * (4 if fp32 else 2), bound="mfma", kernel="fa_f32_mfma_kernel" if fp32 else "fa_pipe_kernel")
+    if fp32:
+        r["peak"] = PEAK_F32_TFLOPS
+    return r
 
 
 def _rows(torch, rows=32768, cols=4096, nbuf=3):
@@ -285,13 +289,13 @@ def cpu_baseline_torch(name, torch):
         t = _best_of(lambda: torch.matmul(a, b))
         return dict(base, value=round(2.0 * 4096 ** 3 / t / 1e12, 4), unit="TFLOP/s",
                     sample=f"torch.matmul on CPU, {'bf16' if name == 'gemm' else 'fp32'} 4096^3 (the whole workload), best of 3: {t:.3f} s")
-    if name in ("attention", "attention_full"):
-        S, causal = (4096, True) if name == "attention" else (2048, False)
-        q, k, v = (torch.randn(1, 1, S, 128, generator=g).to(bf) for _ in range(3))
+    if name in ("attention", "attention_full", "attention_f32"):
+        S, causal = (4096, True) if name == "attention" else (2048, name == "attention_f32")
+        q, k, v = (torch.randn(1, 1, S, 128, generator=g).to(torch.float32 if name == "attention_f32" else bf) for _ in range(3))
         t = _best_of(lambda: F.scaled_dot_product_attention(q, k, v, is_causal=causal))
         flops = 4.0 * S * S * 128 * (0.5 if causal else 1.0)
         return dict(base, value=round(flops / t / 1e12, 4), unit="TFLOP/s",
-                    sample=f"torch scaled_dot_product_attention on CPU, bf16, ONE of the 128 (batch, head) slices "
+                    sample=f"torch scaled_dot_product_attention on CPU, {'fp32' if name == 'attention_f32' else 'bf16'}, ONE of the 128 (batch, head) slices "
                            f"(S {S}, D 128, {'causal' if causal else 'full'}), best of 3: {t:.3f} s; the rate carries over, "
                            f"the whole workload is 128 such slices")
     if name in ("softmax", "layer_norm", "rms_norm", "bias_gelu"):
@@ -343,7 +347,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="gemm",
-                    choices=["gemm", "gemm_f32", "attention", "attention_full", "softmax", "layer_norm", "rms_norm", "bias_gelu", "copy",
+                    choices=["gemm", "gemm_f32", "attention", "attention_full", "attention_f32", "softmax", "layer_norm", "rms_norm", "bias_gelu", "copy",
                              "gpt2", "gpt2_capi"])
     ap.add_argument("--ramp-ms", type=float, default=150.0,
                     help="milliseconds of untimed launches of the same kernel in front of the warm-up steps (0 = none)")
@@ -372,6 +376,8 @@ def main():
             return wl_attention(torch, kernels, causal=True)
         if name == "attention_full":
             return wl_attention(torch, kernels, S=2048, causal=False)
+        if name == "attention_f32":
+            return wl_attention(torch, kernels, S=2048, causal=True, fp32=True)
         if name == "copy":
             return wl_copy(torch, kernels)
         if name == "gpt2":
@@ -396,7 +402,8 @@ def main():
     head = run(args.workload)
     others = {}
     if not args.only:
-        for name in ["gemm", "gemm_f32", "attention", "attention_full", "softmax", "layer_norm", "rms_norm", "bias_gelu", "gpt2", "gpt2_capi"]:
+        for name in ["gemm", "gemm_f32", "attention", "attention_full", "attention_f32", "softmax", "layer_norm", "rms_norm", "bias_gelu",
+                     "gpt2", "gpt2_capi"]:
             if name == args.workload:
                 continue
             others[name] = run(name)
@@ -418,7 +425,7 @@ def main():
         "value": head["value"], "unit": head["unit"], "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(head["us_per_launch"] / 1e3, 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16", "data": "synthetic",
+        "dtype": "f32" if args.workload.endswith("_f32") else "bf16", "data": "synthetic",
         "config": {"workload": head["workload"], "kernel": head["kernel"]},
         "clock_ramp_ms": args.ramp_ms,
         "roofline": head["roofline"],

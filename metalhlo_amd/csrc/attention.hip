@@ -351,6 +351,9 @@ namespace mhip {
 // attention_pipe.hip: head size 128, four waves x 64 query rows, matrix / softmax overlap in one wave.
 bool fa_pipe_eligible(const FaArgs& a, int64_t D, int dtype, bool has_mask, int variant);
 int launch_fa_pipe(hipStream_t s, const FaArgs& a, int dtype, bool causal, int pair);
+// attention_f32.hip: fp32 tensors on the fp32 matrix instruction.
+bool fa_f32_mfma_eligible(const FaArgs& a, int64_t D);
+int launch_fa_f32_mfma(hipStream_t s, const FaArgs& a, int64_t D, float scale);
 }  // namespace mhip
 
 using namespace mhip;
@@ -415,7 +418,9 @@ static int fa_entry(const char* name, void* stream, const void* q, const void* k
         return fail(MHIP_ERR_UNSUPPORTED, "%s: strided layouts need bf16 / f16, head_dim 64 or 128, 16-byte aligned pointers and "
                                           "strides that are multiples of 8 elements", name);
     switch (dtype) {
-        case MHIP_F32: return launch_fa_scalar<float>(s, a, (int)D, scale);
+        case MHIP_F32:
+            if (fa_f32_mfma_eligible(a, D)) return launch_fa_f32_mfma(s, a, D, scale);
+            return launch_fa_scalar<float>(s, a, (int)D, scale);
         case MHIP_BF16: return launch_fa_scalar<bf16_t>(s, a, (int)D, scale);
         case MHIP_F16: return launch_fa_scalar<f16_t>(s, a, (int)D, scale);
         default: return fail(MHIP_ERR_UNSUPPORTED, "%s: dtype %d", name, dtype);

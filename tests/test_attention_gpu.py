@@ -39,6 +39,57 @@ def test_c1_fp32_causal_sdpa():
     assert_close(o[:, :, 0], as_f64(v)[:, :, 0], 1e-6, "row 0 == V[0]")
 
 
+F32_CASES = [  # B, H, Sq, Skv, D, causal -- the fp32 matrix-instruction kernel (head sizes 32 .. 128)
+    (1, 4, 128, 128, 64, True), (2, 2, 256, 256, 128, False), (1, 3, 200, 333, 96, False),
+    (1, 2, 77, 333, 64, True), (1, 2, 333, 77, 32, True), (1, 1, 1, 1, 128, True), (2, 2, 130, 31, 64, False),
+    (1, 2, 1024, 1024, 64, True),
+]
+
+
+@pytest.mark.parametrize("case", F32_CASES, ids=lambda c: "B%dH%dq%dk%dD%d%s" % (*c[:5], "c" if c[5] else ""))
+def test_attention_f32_matrix_cores(case, monkeypatch):
+    """fp32 tensors on v_mfma_f32_32x32x2_f32: 1e-5 against the oracle (ragged query and key counts,
+    causal with more queries than keys and the other way round), and the scalar kernel it
+    replaces stays within the same bar of it."""
+    from metalhlo_amd import kernels
+    B, H, Sq, Skv, D, causal = case
+    q, k, v = _qkv(B, H, Sq, Skv, D, torch.float32, 71)
+    exp = oracle.attention(as_f64(q), as_f64(k), as_f64(v), is_causal=causal)
+    o = kernels.flash_attention(q, k, v, is_causal=causal)
+    assert_close(o, exp, 1e-5, f"fp32 attention {case}")
+    monkeypatch.setenv("MHIP_FA_F32_MFMA", "2")
+    scalar = kernels.flash_attention(q, k, v, is_causal=causal)
+    assert_close(scalar, exp, 1e-5, f"fp32 scalar attention {case}")
+    assert not torch.equal(o, scalar) or Sq * Skv <= 1        # two kernels, two summation orders
+
+
+def test_attention_f32_matrix_cores_mask_and_scale():
+    from metalhlo_amd import kernels
+    rng = np.random.default_rng(72)
+    q, k, v = _qkv(2, 3, 160, 200, 64, torch.float32, 73)
+    for shape in [(2, 3, 160, 200), (2, 1, 160, 200), (1, 1, 160, 200)]:
+        m = rng.standard_normal(shape)
+        m[..., :, 150:] = -np.inf
+        md = to_dev(m, torch.float32)
+        o = kernels.flash_attention(q, k, v, mask=md, scale=0.07)
+        exp = oracle.attention(as_f64(q), as_f64(k), as_f64(v), scale=0.07, mask=as_f64(md))
+        assert_close(o, exp, 1e-5, f"fp32 mask {shape}")
+    m = np.zeros((1, 1, 160, 200)); m[..., 7, :] = -np.inf
+    md = to_dev(m, torch.float32)
+    o = kernels.flash_attention(q, k, v, mask=md, is_causal=True, scale=-0.1)
+    exp = oracle.attention(as_f64(q), as_f64(k), as_f64(v), scale=-0.1, is_causal=True, mask=as_f64(md))
+    assert_close(o, exp, 1e-5, "fp32 mask + causal, negative scale")
+    assert torch.count_nonzero(o[:, :, 7]) == 0                # a fully masked row gives zeros
+    # large logits: the running maximum keeps the exponentials in range (the fp32 rounding of a
+    # logit of size L alone is worth about L * 1e-6 relative in its probability, so 1e-5 holds
+    # for logits of the usual size only; at 30 x 30 the result must still be finite and close)
+    big = kernels.flash_attention(q * 3, k * 3, v)
+    assert_close(big, oracle.attention(as_f64(q) * 3, as_f64(k) * 3, as_f64(v)), 1e-4, "fp32 larger logits")
+    huge = kernels.flash_attention(q * 30, k * 30, v)
+    assert torch.isfinite(huge).all()
+    assert_close(huge, oracle.attention(as_f64(q) * 30, as_f64(k) * 30, as_f64(v)), 2e-3, "fp32 huge logits")
+
+
 CASES = [  # B, H, Sq, Skv, D, causal
     (1, 2, 128, 128, 128, False), (1, 2, 128, 128, 128, True),
     (2, 3, 256, 256, 64, True), (2, 3, 256, 256, 64, False),
