@@ -40,13 +40,15 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by what the same
 # counter reads for the 'copy' workload (256 MiB in, 256 MiB out); see profiles/<workload>.txt.
 MEASURED_TRAFFIC = {
-    "gemm": 238901384,
-    "attention": 773135522,
-    "attention_full": 268909839,
-    "softmax": 536709952,
-    "layer_norm": 536897658,
-    "rms_norm": 536783693,
-    "bias_gelu": 536757341,
+    "gemm": 237446022,
+    "gemm_f32": 1803825891,
+    "attention": 752630452,
+    "attention_full": 268946537,
+    "attention_f32": 1979773872,
+    "softmax": 536779900,
+    "layer_norm": 536936179,
+    "rms_norm": 536839114,
+    "bias_gelu": 536823915,
     "copy": 536870912,
 }
 
@@ -242,6 +244,73 @@ def measure(wl, steps, warmup, torch, key=None):
                 us_per_launch=round(sec * 1e6, 2), wall_us_per_launch=round(wall * 1e6, 2), roofline=roof)
 
 
+# ---------------------------------------------------------------- shader clock under load
+def clock_probe(torch, kernels, seconds=2.0):
+    """The device lowers its shader clock when a kernel would exceed the board's power limit, and
+    how far depends on the operand bits.  For the two matrix workloads: launches back to back for
+    `seconds` while `rocm-smi --showclocks` is sampled from a second thread, once on the
+    benchmark's random operands and once on zeros (which switch almost nothing and leave the
+    clock at its maximum), then the time of 20 launches.  Prints one JSON object."""
+    import re
+    import subprocess
+    import threading
+
+    def sample(stop, out):
+        while not stop.is_set():
+            r = subprocess.run(["/opt/rocm/bin/rocm-smi", "--showclocks"], capture_output=True, text=True)
+            m = re.search(r"sclk clock level: \d+: \((\d+)Mhz\)", r.stdout)
+            if m:
+                out.append(int(m.group(1)))
+            time.sleep(0.2)
+
+    def run(fn):
+        stop, mhz = threading.Event(), []
+        th = threading.Thread(target=sample, args=(stop, mhz))
+        th.start()
+        t0 = time.time()
+        while time.time() - t0 < seconds:
+            for _ in range(20):
+                fn()
+            torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(20):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        stop.set()
+        th.join()
+        tail = mhz[len(mhz) // 2:] or [0]
+        return dict(us_per_launch=round(e0.elapsed_time(e1) / 20 * 1e3, 1), sclk_mhz=round(sum(tail) / len(tail)))
+
+    res = {}
+    M = 4096
+    g = torch.Generator(device="cuda").manual_seed(2)
+    c = torch.empty(M, M, dtype=torch.bfloat16, device="cuda")
+    for tag in ("uniform", "zeros"):
+        if tag == "uniform":
+            a = (torch.rand(M, M, generator=g, device="cuda") * 2 - 1).to(torch.bfloat16)
+            b = (torch.rand(M, M, generator=g, device="cuda") * 2 - 1).to(torch.bfloat16)
+        else:
+            a = torch.zeros(M, M, dtype=torch.bfloat16, device="cuda")
+            b = torch.zeros(M, M, dtype=torch.bfloat16, device="cuda")
+        r = run(lambda: kernels.matmul(a, b, out=c))
+        r["tflops"] = round(2.0 * M ** 3 / r["us_per_launch"] / 1e6, 1)
+        res[f"gemm 4096^3 bf16, {tag} operands"] = r
+    B, H, S, D = 4, 32, 4096, 128
+    for tag in ("normal", "zeros"):
+        if tag == "normal":
+            q, k, v = (torch.randn(B, H, S, D, generator=g, device="cuda").to(torch.bfloat16) for _ in range(3))
+        else:
+            q, k, v = (torch.zeros(B, H, S, D, dtype=torch.bfloat16, device="cuda") for _ in range(3))
+        r = run(lambda: kernels.flash_attention(q, k, v, is_causal=True))
+        r["tflops"] = round(2.0 * B * H * S * S * D / r["us_per_launch"] / 1e6, 1)
+        res[f"causal attention B4 H32 S4096 D128 bf16, {tag} operands"] = r
+    x = torch.randn(32768, 4096, generator=g, device="cuda").to(torch.bfloat16)
+    res["softmax [32768,4096] bf16"] = run(lambda: kernels.softmax(x))
+    print(json.dumps({"clock_probe": res, "seconds_of_load_before_timing": seconds}))
+
+
 # ---------------------------------------------------------------- CPU baselines
 def _best_of(fn, reps=3):
     fn()                                    # warm-up
@@ -353,6 +422,9 @@ def main():
                     help="milliseconds of untimed launches of the same kernel in front of the warm-up steps (0 = none)")
     ap.add_argument("--only", action="store_true", help="time only --workload (for profiling runs)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--clock-probe", action="store_true",
+                    help="instead of the benchmark: shader clock and time per launch of the matrix workloads under "
+                         "sustained load, on random and on all-zero operands")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (the reference is single-device and "
@@ -366,6 +438,9 @@ def main():
     from metalhlo_amd import _lib, kernels
     _lib.load()
     torch.cuda.set_device(0)
+    if args.clock_probe:
+        clock_probe(torch, kernels)
+        return
 
     def build(name):
         if name == "gemm":
