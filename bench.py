@@ -44,7 +44,7 @@ MEASURED_TRAFFIC = {
     "gemm_f32": 1803825891,
     "attention": 752630452,
     "attention_full": 268946537,
-    "attention_f32": 1979773872,
+    "attention_f32": 1994907876,
     "softmax": 536779900,
     "layer_norm": 536936179,
     "rms_norm": 536839114,

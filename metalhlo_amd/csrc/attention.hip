@@ -18,28 +18,22 @@
 
 namespace mhip {
 
-template <typename T, int D, bool CAUSAL, bool HAS_MASK>
+// NB: depth of the K and of the V ring in LDS.  Two everywhere: with head size 64 a ring of three or
+// four measured 8 to 13 % slower (B8 H12 S1024: 38.5 / 40.5 against 35.7 us) -- it costs the third
+// resident workgroup per CU, which hides more latency than the deeper prefetch does.
+template <typename T, int D, bool CAUSAL, bool HAS_MASK, int NB>
 __global__ __launch_bounds__(256, 2) void fa_fwd_kernel(FaArgs a) {
     constexpr int CPR = D / 8;                  // 16-byte chunks per row
     constexpr int kTile = kBKV * D * 2;         // bytes of one K (or V) tile
     constexpr int kRowsPerInst = 64 / CPR;      // tile rows one wave-wide LDS-DMA load fills
     constexpr int kInst = kBKV / kRowsPerInst / 4;   // such loads per wave per tile
     constexpr int ND = D / 32, NS = D / 16;
-    __shared__ __attribute__((aligned(1024))) char smem[4 * kTile];   // K0 K1 V0 V1
+    constexpr int kLoadsPerTile = 2 * kInst;    // per wave
+    __shared__ __attribute__((aligned(1024))) char smem[2 * NB * kTile];   // K ring, then V ring
 
-    // ---- which (batch*head, query block) -----------------------------------
+    // ---- which (batch*head, query block): see tile_of_workgroup
     int bh, qb;
-    {
-        const int id = blockIdx.x;
-        if (a.xcd_map) {
-            const int xcd = id & 7, local = id >> 3;
-            bh = (local / a.nqb) * 8 + xcd;
-            qb = a.nqb - 1 - local % a.nqb;   // long (late) causal rows first
-        } else {
-            bh = id / a.nqb;
-            qb = a.nqb - 1 - id % a.nqb;
-        }
-    }
+    tile_of_workgroup<CAUSAL>(a, blockIdx.x, bh, qb);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int lrow = lane & 31, lhalf = lane >> 5;
     const int qblk0 = qb * kBQ;
@@ -78,21 +72,26 @@ __global__ __launch_bounds__(256, 2) void fa_fwd_kernel(FaArgs a) {
     // of a tile (lane l lands at byte 16*l of that KB); the swizzle is applied by
     // choosing which global chunk each lane fetches.  Keys past the end read 0.
     const int ld_row = lane / CPR, ld_pos = lane % CPR;
+    // (a block past the last one this workgroup needs is "loaded" all the same, out of bounds:
+    // the waits below count loads, so every step issues the same number)
+    const int kv_end = min(nkv * kBKV, a.Skv);
     auto load_tile = [&](int kv0, int buf) {
 #pragma unroll
         for (int i = 0; i < kInst; i++) {
             const int blk = i * 4 + wave;                 // which KB of the tile
             const int row = blk * kRowsPerInst + ld_row;
             const int key = kv0 + row;
-            const uint32_t koff = key < a.Skv ? (uint32_t)((key * k_rs + ((ld_pos ^ k_swz<D>(row)) << 3)) * 2) : kOobA;
-            const uint32_t voff = key < a.Skv ? (uint32_t)((key * v_rs + ((ld_pos ^ v_swz<D>(row)) << 3)) * 2) : kOobA;
+            const uint32_t koff = key < kv_end ? (uint32_t)((key * k_rs + ((ld_pos ^ k_swz<D>(row)) << 3)) * 2) : kOobA;
+            const uint32_t voff = key < kv_end ? (uint32_t)((key * v_rs + ((ld_pos ^ v_swz<D>(row)) << 3)) * 2) : kOobA;
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, (fa_lds_void*)(smem + buf * kTile + blk * 1024), 16, koff, 0, 0, 0);
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, (fa_lds_void*)(smem + (2 + buf) * kTile + blk * 1024), 16, voff, 0, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, (fa_lds_void*)(smem + (NB + buf) * kTile + blk * 1024), 16, voff, 0, 0, 0);
         }
     };
+    // loads land in program order: the next block has landed when only the NB - 2 blocks issued
+    // behind it are still in flight
     auto tiles_ready = [&]() {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NB - 2) * kLoadsPerTile) : "memory");
+        __builtin_amdgcn_s_barrier();
     };
 
     // V^T fragment addresses: lane i of a 16-lane group supplies key row i/4 and
@@ -108,17 +107,18 @@ __global__ __launch_bounds__(256, 2) void fa_fwd_kernel(FaArgs a) {
         for (int r = 0; r < 16; r++) oacc[i][r] = 0.f;
     float m_run = -INFINITY, l_run = 0.f;   // running max in the log2 domain, running sum
 
-    load_tile(0, 0);
+#pragma unroll
+    for (int p = 0; p < NB - 1; p++) load_tile(p * kBKV, p);
     tiles_ready();
 
     for (int it = 0; it < nkv; it++) {
-        const int cur = it & 1, kv0 = it * kBKV;
-        if (it + 1 < nkv) load_tile(kv0 + kBKV, cur ^ 1);
+        const int cur = it % NB, kv0 = it * kBKV;
+        load_tile(kv0 + (NB - 1) * kBKV, (it + NB - 1) % NB);
 
         const bool wave_active = !CAUSAL || kv0 <= qw + 31;
         if (wave_active) {
             const char* kt = smem + cur * kTile;
-            const char* vt = smem + (2 + cur) * kTile;
+            const char* vt = smem + (NB + cur) * kTile;
             // ---- S^T = K . Q^T ---------------------------------------------
             f32x16 sacc[2];
 #pragma unroll
@@ -232,6 +232,7 @@ __global__ __launch_bounds__(256, 2) void fa_fwd_kernel(FaArgs a) {
         }
         if (it + 1 < nkv) tiles_ready();
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // nothing may land in LDS after the workgroup ends
 
     // ---- normalise and store: lane holds 4 consecutive d per register group -
     const float l_tot = half_sum(l_run);
@@ -323,11 +324,12 @@ template <typename T, int D>
 static int launch_fa(hipStream_t s, FaArgs a, bool causal, bool has_mask) {
     a.nqb = (a.Sq + kBQ - 1) / kBQ;
     const int64_t bh = (int64_t)a.B * a.H;
-    a.xcd_map = (bh % 8 == 0) ? 1 : 0;
+    set_tile_order(a);
     const int64_t grid = bh * a.nqb;
     if (grid > 0x7FFFFFFFLL) return fail(MHIP_ERR_UNSUPPORTED, "flash_attention: grid too large");
+    constexpr int NB = 2;
 #define MHIP_FA(C, M)                                                                       \
-    hipLaunchKernelGGL((fa_fwd_kernel<T, D, C, M>), dim3((unsigned)grid), dim3(256), 0, s, a)
+    hipLaunchKernelGGL((fa_fwd_kernel<T, D, C, M, NB>), dim3((unsigned)grid), dim3(256), 0, s, a)
     if (causal && has_mask) MHIP_FA(true, true);
     else if (causal) MHIP_FA(true, false);
     else if (has_mask) MHIP_FA(false, true);
@@ -378,7 +380,7 @@ static int fa_entry(const char* name, void* stream, const void* q, const void* k
     a.negate_q = scale < 0.f;
     a.is_causal = is_causal ? 1 : 0;
     a.mask_sb = mask_stride_b; a.mask_sh = mask_stride_h;
-    a.nqb = 0; a.xcd_map = 0; a.pair_tiles = 0;
+    a.nqb = 0; a.xcd_map = 0; a.pair_tiles = 0; a.cu_group = 1;
     const int64_t packed[12] = {H * Sq * D, Sq * D, D, H * Skv * D, Skv * D, D, H * Skv * D, Skv * D, D, H * Sq * D, Sq * D, D};
     bool is_packed = true;
     int64_t max_row = D, max_span = 0;

@@ -25,10 +25,46 @@ struct FaArgs {
     int nqb;          // query blocks per (batch, head)
     int xcd_map;      // 1: (batch*head) % 8 == 0, use the XCD-aware block order
     int pair_tiles;   // pipelined kernel, causal: a workgroup takes two query tiles (first + last, ...)
+    int cu_group;     // 128-row kernel: CUs a run of consecutive workgroup ids is dealt over (per XCD, or all)
     // Element strides {batch, head, row} of q, k, v, o (the last axis is contiguous).  Only
     // fa_fwd_kernel reads them; every other kernel is given the packed [B,H,S,D] layout.
     int64_t qs[3], ks[3], vs[3], os[3];
 };
+
+// Which (batch * head, query tile) a workgroup of the one-tile-per-workgroup kernels takes.
+// Workgroup ids go round-robin over the 8 XCDs and, inside an XCD, round-robin over its CUs
+// (measured: with three workgroups resident per CU, a CU holds XCD-local indices c, c + 32,
+// c + 64).  A causal tile's work grows with its position, so the order decides the balance:
+// walking one head's tiles after the other puts the SAME tile position of three heads on a CU
+// (a tile count of 8 divides 32) -- three longest tiles here, three shortest there, and the
+// launch takes as long as the non-causal one.  Instead: all tiles of the XCD sorted longest
+// first and dealt to the CUs in rounds of cu_group, every other round in reverse (a snake
+// draft), which balances the resident set and is the longest-first rule for what is
+// dispatched later (B8 H12 S1024 D64 causal: 35.4 -> 23.7 us).
+template <bool CAUSAL>
+__device__ inline void tile_of_workgroup(const FaArgs& a, int id, int& bh, int& qb) {
+    const int groups = a.xcd_map ? 8 : 1;
+    const int xcd = a.xcd_map ? (id & 7) : 0, local = a.xcd_map ? (id >> 3) : id;
+    const int heads = (a.B * a.H) / groups;          // heads of this XCD
+    if (CAUSAL) {
+        const int total = heads * a.nqb;
+        const int round = local / a.cu_group, c = local % a.cu_group;
+        const int in_round = min(a.cu_group, total - round * a.cu_group);
+        const int e = round * a.cu_group + ((round & 1) ? in_round - 1 - c : c);   // place in the longest-first list
+        qb = a.nqb - 1 - e / heads;
+        bh = (e % heads) * groups + xcd;
+    } else {
+        bh = (local / a.nqb) * groups + xcd;
+        qb = local % a.nqb;
+    }
+}
+
+// host side: a.nqb set; fills xcd_map and cu_group
+inline void set_tile_order(FaArgs& a) {
+    a.xcd_map = (((int64_t)a.B * a.H) % 8 == 0) ? 1 : 0;
+    a.cu_group = a.xcd_map ? compute_units() / 8 : compute_units();
+    if (a.cu_group < 1) a.cu_group = 1;
+}
 
 template <typename T> struct Mfma32A;
 template <> struct Mfma32A<bf16_t> {

@@ -37,8 +37,8 @@ __global__ __launch_bounds__(256) void fa_f32_mfma_kernel(FaArgs a, float scale)
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int ln = lane & 31, h = lane >> 5;
-    const int nqb = (a.Sq + kFBQ - 1) / kFBQ;
-    const int bh = blockIdx.x / nqb, qb = blockIdx.x % nqb;
+    int bh, qb;
+    tile_of_workgroup<CAUSAL>(a, blockIdx.x, bh, qb);
     const int q0 = qb * kFBQ + wave * 32;
     const int qpos = q0 + ln;                       // this lane's query row
     const bool q_live = qpos < a.Sq;
@@ -168,8 +168,10 @@ __global__ __launch_bounds__(256) void fa_f32_mfma_kernel(FaArgs a, float scale)
 }
 
 template <int D>
-int launch_f32(hipStream_t s, const FaArgs& a, float scale, bool causal, bool has_mask) {
-    const int64_t grid = (int64_t)a.B * a.H * ((a.Sq + kFBQ - 1) / kFBQ);
+int launch_f32(hipStream_t s, FaArgs a, float scale, bool causal, bool has_mask) {
+    a.nqb = (a.Sq + kFBQ - 1) / kFBQ;
+    set_tile_order(a);
+    const int64_t grid = (int64_t)a.B * a.H * a.nqb;
     if (grid > 0x7FFFFFFFLL) return fail(MHIP_ERR_UNSUPPORTED, "flash_attention: grid too large");
 #define MHIP_FA32(C, M) \
     hipLaunchKernelGGL((fa_f32_mfma_kernel<D, C, M>), dim3((unsigned)grid), dim3(256), 0, s, a, scale)
