@@ -80,6 +80,7 @@ struct Allocator {
     ArenaPlan* plan = nullptr;
     char* base = nullptr;
     bool escaping_in_arena = false;
+    std::vector<std::shared_ptr<DeviceMem>>* presets = nullptr;   // by slot: storage allocated ahead for the escaping slots
     size_t next = 0;
 
     DeviceTensor allocate(const TensorType& t) {
@@ -100,8 +101,12 @@ struct Allocator {
         }
         if (next >= plan->slots.size() || plan->slots[next].bytes != rounded)
             throw ExecError("the execution does not follow the memory plan made at compile time");
+        const size_t slot_no = next;
         const ArenaPlan::Slot& sl = plan->slots[next++];
-        if (sl.escapes && !escaping_in_arena) {
+        if (sl.escapes && presets) {
+            d.mem = (*presets)[slot_no];
+            if (!d.mem) throw ExecError("the execution does not follow the memory plan made at compile time");
+        } else if (sl.escapes && !escaping_in_arena) {
             d.mem->pool = &client->pool;
             d.mem->ptr = client->pool.alloc(d.mem->bytes);
         } else {
@@ -879,8 +884,31 @@ static void ensure_arena(Executable& exe, size_t bytes) {
 
 // Captures one walk over the program (every value, results included, at its arena address) into
 // a graph.  False when the capture or the instantiation fails; the stream is usable again then.
+// True when every returned value is an allocation of its own (no input, constant or alias among the
+// results, none returned twice): the results of a captured graph can then live in buffers of their own.
+static bool direct_results(const Executable& exe) {
+    size_t escaping = 0;
+    for (auto& sl : exe.plan.slots) escaping += sl.escapes;
+    return escaping == exe.fn.returns.size() && env_flag("METALHLO_GRAPH_DIRECT_RESULTS", true);
+}
+
 static bool capture_graph(Executable& exe, const std::vector<DeviceTensor>& inputs, Executable::CapturedGraph& out) {
     Client& c = *exe.client;
+    // storage of the results, allocated before the capture begins (nothing may allocate inside it)
+    std::vector<std::shared_ptr<DeviceMem>> presets;
+    const bool direct = direct_results(exe);
+    if (direct) {
+        presets.resize(exe.plan.slots.size());
+        for (size_t i = 0; i < exe.plan.slots.size(); i++) {
+            if (!exe.plan.slots[i].escapes) continue;
+            auto m = std::make_shared<DeviceMem>();
+            m->bytes = exe.plan.slots[i].bytes;             // the slot's size (the value's, rounded up to 256)
+            m->pool = &c.pool;
+            m->ptr = c.pool.alloc(m->bytes);
+            m->replay_result = true;
+            presets[i] = m;
+        }
+    }
     std::lock_guard<std::mutex> stream_lock(c.stream_mu);       // no other thread enqueues on the stream meanwhile
     if (hipStreamBeginCapture(c.stream, hipStreamCaptureModeThreadLocal) != hipSuccess) {
         (void)hipGetLastError();
@@ -891,7 +919,8 @@ static bool capture_graph(Executable& exe, const std::vector<DeviceTensor>& inpu
     al.client = &c;
     al.plan = &exe.plan;
     al.base = static_cast<char*>(exe.arena);
-    al.escaping_in_arena = true;
+    al.escaping_in_arena = !direct;
+    if (direct) al.presets = &presets;
     std::vector<DeviceTensor> rets;
     bool ok = true;
     try { rets = run_ops(exe, inputs, al, false); } catch (const std::exception&) { ok = false; }
@@ -908,7 +937,18 @@ static bool capture_graph(Executable& exe, const std::vector<DeviceTensor>& inpu
     out.inputs.clear();
     for (auto& t : inputs) out.inputs.push_back(t.data());
     out.returns.clear();
-    for (auto& r : rets) out.returns.emplace_back(r.data(), r.type);
+    out.results.clear();
+    if (direct) {
+        for (auto& r : rets) {
+            if (!r.mem || !r.mem->replay_result) {          // not what the plan promised: keep this program eager
+                (void)hipGraphExecDestroy(ex);
+                return false;
+            }
+            out.results.push_back(r);
+        }
+    } else {
+        for (auto& r : rets) out.returns.emplace_back(r.data(), r.type);
+    }
     return true;
 }
 
@@ -933,7 +973,7 @@ std::vector<DeviceTensor> execute(Executable& exe, const std::vector<DeviceTenso
     const auto t0 = std::chrono::steady_clock::now();
     std::vector<DeviceTensor> rets;
     bool replayed = false;
-    if (use_arena) ensure_arena(exe, want_graph ? exe.plan.full_bytes : exe.plan.core_bytes);
+    if (use_arena) ensure_arena(exe, want_graph && !direct_results(exe) ? exe.plan.full_bytes : exe.plan.core_bytes);
     // the first execution runs eagerly (kernels set their attributes, tuning tables load); from the
     // second on the op list is one graph per set of input addresses
     if (want_graph && !exe.graph_failed && exe.eager_runs > 0) {
@@ -943,7 +983,13 @@ std::vector<DeviceTensor> execute(Executable& exe, const std::vector<DeviceTenso
             for (size_t i = 0; same && i < inputs.size(); i++) same = g.inputs[i] == inputs[i].data();
             if (same) { hit = &g; break; }
         }
-        if (!hit) {
+        // a graph with result buffers of its own can run again only when the caller has released
+        // what the previous replay handed out; this execution is eager otherwise
+        bool busy = false;
+        if (hit)
+            for (auto& r : hit->results) busy = busy || r.mem.use_count() > 1;
+        if (busy) hit = nullptr;
+        if (!hit && !busy) {
             Executable::CapturedGraph g;
             if (capture_graph(exe, inputs, g)) {
                 if (exe.graphs.size() >= 8) {
@@ -964,6 +1010,7 @@ std::vector<DeviceTensor> execute(Executable& exe, const std::vector<DeviceTenso
                 throw ExecError(std::string("graph launch failed: ") + hipGetErrorString(e));
             }
             exe.graph_replays++;
+            for (auto& r : hit->results) rets.push_back(r);
             for (auto& r : hit->returns) {
                 DeviceTensor t;
                 t.type = r.second;
@@ -1002,7 +1049,7 @@ std::vector<DeviceTensor> execute(Executable& exe, const std::vector<DeviceTenso
         if (!o.mem) throw ExecError("a returned value was never produced");
         // an output must own its storage: inputs, constants, aliases, repeated results and
         // values that lie in the arena are copied out
-        const bool shared = o.mem.use_count() > 1 || !o.mem->pool;
+        const bool shared = !o.mem->replay_result && (o.mem.use_count() > 1 || !o.mem->pool);
         if (shared) {
             DeviceTensor cpy = c.allocate(o.type);
             if (mhip_copy(c.stream, o.data(), cpy.data(), (int64_t)o.type.bytes()) != MHIP_OK) throw ExecError(mhip_last_error());

@@ -59,6 +59,7 @@ struct DeviceMem {
     size_t bytes = 0;
     ArenaPlan* recorder = nullptr;   // dry run: note the release time of slot `slot`
     int slot = -1;
+    bool replay_result = false;      // result buffer of a captured graph: the graph keeps one reference, the caller gets the other
     ~DeviceMem() {
         if (recorder) recorder->slots[slot].end = recorder->clock++;
         else if (pool && ptr) pool->release(ptr, bytes);
@@ -101,7 +102,11 @@ struct Executable {
     struct CapturedGraph {
         std::vector<const void*> inputs;                     // device addresses the graph was captured with
         hipGraphExec_t exec = nullptr;
-        std::vector<std::pair<const void*, TensorType>> returns;   // where each result lies after a replay
+        std::vector<std::pair<const void*, TensorType>> returns;   // where each result lies after a replay (arena form)
+        // Direct form: the graph writes its results into buffers of their own, which are handed to the
+        // caller as they are (no copy out of the arena).  A replay needs all of them back, i.e. released
+        // by the caller of the previous one; otherwise that execution runs eagerly.
+        std::vector<DeviceTensor> results;
     };
     std::vector<CapturedGraph> graphs;
     int64_t graph_captures = 0, graph_replays = 0, eager_runs = 0;

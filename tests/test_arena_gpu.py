@@ -157,3 +157,52 @@ def test_attention_program_replays(sess, monkeypatch):
     for b in bufs:
         sess.lib.mhlo_buffer_destroy(b)
     sess.lib.mhlo_executable_destroy(exe)
+
+
+def test_replay_results_are_handed_out_without_a_copy_and_never_overwritten(sess, monkeypatch):
+    """A captured graph writes its results into buffers of their own.  While the caller still holds
+    the results of the previous replay the next execution must not run that graph (it would
+    overwrite them): it runs eagerly, the held buffers keep their contents, and once they are
+    released the graph is replayed again.  Programs that return an input or an alias keep the
+    copy-out form (covered by 'pass_through' above)."""
+    monkeypatch.setenv("METALHLO_ARENA", "1")
+    monkeypatch.setenv("METALHLO_HIP_GRAPH", "1")
+    rng = np.random.default_rng(21)
+    ins = inputs_for(rng, FAN)
+    exe = sess.compile(FAN)
+    bufs = [sess.buffer(a, t) for a, t in ins]
+    other = [sess.buffer(a + 1.0, t) for a, t in ins]           # a second set of inputs -> a second graph
+    want = run_with(sess, exe, bufs)                             # the first execution is eager
+    want_other = run_with(sess, exe, other)                      # captured and replayed at once
+    for i in range(3):                                           # capture, then replays: results released each time
+        got = run_with(sess, exe, bufs)
+        assert all(np.array_equal(g, w) for g, w in zip(got, want)), f"replay {i}"
+    base = sess.plan(exe)
+    assert base["graph_captures"] == 2 and base["graph_replays"] == 4 and base["eager_runs"] == 1
+
+    def execute_keep(inputs):
+        outs = (C.c_void_p * 2)()
+        n = C.c_int32()
+        arr = (C.c_void_p * len(inputs))(*inputs)
+        assert sess.lib.mhlo_execute(exe, arr, len(inputs), outs, C.byref(n)) == 0, sess.lib.mhlo_get_last_error()
+        return [outs[i] for i in range(n.value)]
+
+    held = execute_keep(bufs)                                    # a replay whose results stay with the caller
+    assert sess.plan(exe)["graph_replays"] == 5
+    again = execute_keep(bufs)                                   # must not touch `held`: eager
+    after = sess.plan(exe)
+    assert after["graph_replays"] == 5 and after["eager_runs"] == 2 and after["graph_captures"] == 2
+    got_other = run_with(sess, exe, other)                       # other inputs: their own graph, their own result buffers
+    assert all(np.array_equal(g, w) for g, w in zip(got_other, want_other))
+    for hs in (held, again):
+        vals = [sess.to_numpy(h) for h in hs]
+        assert all(np.array_equal(g, w) for g, w in zip(vals, want))
+    for h in held + again:
+        sess.lib.mhlo_buffer_destroy(h)
+    got = run_with(sess, exe, bufs)                              # released: the graph runs again
+    assert all(np.array_equal(g, w) for g, w in zip(got, want))
+    end = sess.plan(exe)
+    assert end["graph_replays"] == 7 and end["eager_runs"] == 2 and end["graph_captures"] == 2
+    for b in bufs + other:
+        sess.lib.mhlo_buffer_destroy(b)
+    sess.lib.mhlo_executable_destroy(exe)
