@@ -175,29 +175,52 @@ __device__ __forceinline__ void store_tile(f32x16 (&acc)[BW / 16], char* smem, c
     constexpr int kRowsPerPass = 64 / kChunks;
     const int cc = lane % kChunks, rr = lane / kChunks;
     const bool rows_aligned = g.N % 8 == 0;
-#pragma unroll 4
-    for (int p = 0; p < 128 / kRowsPerPass; p++) {
-        const int ml = p * kRowsPerPass + rr;
-        const int m = m0 + wm * 128 + ml;
-        const int n = n0 + wn * WN + cc * 8;
-        if (m < g.M && n + 8 <= g.N) {
-            u32x4 w = *reinterpret_cast<const u32x4*>(stage + ml * kRowPad + cc * 16);
-            if (rows_aligned) {
-                if (res) w = add_chunk<T>(w, *reinterpret_cast<const u32x4*>(res + (int64_t)m * g.N + n));
-                *reinterpret_cast<u32x4*>(c + (int64_t)m * g.N + n) = w;
-            } else {
-                // N is no multiple of 8: rows of C start at any even byte.  The device takes 16-byte
-                // accesses at such addresses (alignment is not enforced for global memory); the type
-                // says so, so the compiler assumes nothing more.
-                if (res) w = add_chunk<T>(w, *reinterpret_cast<const u32x4_unaligned*>(res + (int64_t)m * g.N + n));
-                *reinterpret_cast<u32x4_unaligned*>(c + (int64_t)m * g.N + n) = w;
+    // A wave whose 128 x WN sub-tile lies inside C, rows on 16-byte boundaries, nothing to add:
+    // no per-row conditions, so the reads from LDS run eight passes ahead of the stores (the
+    // general loop below waits for each read before its store).  Same values, same addresses.
+    const bool interior = rows_aligned && !res && m0 + wm * 128 + 128 <= g.M && n0 + wn * WN + WN <= g.N;
+    if (__builtin_amdgcn_readfirstlane(interior)) {
+        constexpr int kPasses = 128 / kRowsPerPass, kAhead = 8;
+        T* cw = c + (int64_t)(m0 + wm * 128 + rr) * g.N + (n0 + wn * WN + cc * 8);
+        const char* sp = stage + rr * kRowPad + cc * 16;
+        const int64_t step = (int64_t)kRowsPerPass * g.N;
+#pragma unroll
+        for (int p0 = 0; p0 < kPasses; p0 += kAhead) {
+            u32x4 w[kAhead];
+#pragma unroll
+            for (int u = 0; u < kAhead; u++)
+                w[u] = *reinterpret_cast<const u32x4*>(sp + (p0 + u) * kRowsPerPass * kRowPad);
+#pragma unroll
+            for (int u = 0; u < kAhead; u++) {
+                *reinterpret_cast<u32x4*>(cw) = w[u];
+                cw += step;
             }
-        } else if (m < g.M && n < g.N) {         // the last, partial chunk of a row
-            const T* sv = reinterpret_cast<const T*>(stage + ml * kRowPad + cc * 16);
-            for (int e = 0; e < g.N - n; e++) {
-                T val = sv[e];
-                if (res) val = Elem<T>::from_f32(Elem<T>::to_f32(val) + Elem<T>::to_f32(res[(int64_t)m * g.N + n + e]));
-                c[(int64_t)m * g.N + n + e] = val;
+        }
+    } else {
+#pragma unroll 4
+        for (int p = 0; p < 128 / kRowsPerPass; p++) {
+            const int ml = p * kRowsPerPass + rr;
+            const int m = m0 + wm * 128 + ml;
+            const int n = n0 + wn * WN + cc * 8;
+            if (m < g.M && n + 8 <= g.N) {
+                u32x4 w = *reinterpret_cast<const u32x4*>(stage + ml * kRowPad + cc * 16);
+                if (rows_aligned) {
+                    if (res) w = add_chunk<T>(w, *reinterpret_cast<const u32x4*>(res + (int64_t)m * g.N + n));
+                    *reinterpret_cast<u32x4*>(c + (int64_t)m * g.N + n) = w;
+                } else {
+                    // N is no multiple of 8: rows of C start at any even byte.  The device takes 16-byte
+                    // accesses at such addresses (alignment is not enforced for global memory); the type
+                    // says so, so the compiler assumes nothing more.
+                    if (res) w = add_chunk<T>(w, *reinterpret_cast<const u32x4_unaligned*>(res + (int64_t)m * g.N + n));
+                    *reinterpret_cast<u32x4_unaligned*>(c + (int64_t)m * g.N + n) = w;
+                }
+            } else if (m < g.M && n < g.N) {         // the last, partial chunk of a row
+                const T* sv = reinterpret_cast<const T*>(stage + ml * kRowPad + cc * 16);
+                for (int e = 0; e < g.N - n; e++) {
+                    T val = sv[e];
+                    if (res) val = Elem<T>::from_f32(Elem<T>::to_f32(val) + Elem<T>::to_f32(res[(int64_t)m * g.N + n + e]));
+                    c[(int64_t)m * g.N + n + e] = val;
+                }
             }
         }
     }
