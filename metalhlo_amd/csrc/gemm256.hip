@@ -119,6 +119,17 @@ __device__ inline void main_loop(f32x16 (&acc)[BW / 16], u32x4 ra, u32x4 rb, u32
 #undef MHIP_LOOP
 }
 
+// One accumulator value, moved out of the accumulation registers where it is used.  Left to
+// itself the compiler copies all 256 of them into ordinary registers right behind the loop
+// (the copies are common to every activation's branch), which leaves no register for
+// anything else: addresses then sit in scratch memory and every register group waits for a
+// reload.
+__device__ __forceinline__ float acc_value(float in_agpr) {
+    float v;
+    asm("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(in_agpr));
+    return v;
+}
+
 // Epilogue of one tile: bias, activation, conversion, then through LDS (the ring, free after the
 // loop's last barrier) so that every store instruction writes whole 16-byte chunks of C rows.
 template <typename T, int BW>
@@ -138,28 +149,45 @@ __device__ __forceinline__ void store_tile(f32x16 (&acc)[BW / 16], char* smem, c
     const T* bias = static_cast<const T*>(g.bias);
     constexpr int kRowPad = WN * 2 + 16;
     char* stage = smem + wave * (128 * kRowPad);
+    // The bias of all the lane's columns, fetched before the first register group needs it (a
+    // load inside each group would be waited for sixteen times); zero without a bias and for
+    // columns past N.
+    Pack4<T> bq[4 * NBF];
+    static_for<4 * NBF>([&](auto jq_tag) {
+        constexpr int jq = decltype(jq_tag)::value;
+        bq[jq] = __builtin_bit_cast(Pack4<T>, u32x2{0u, 0u});
+    });
+    if (bias) {
+        const int nw = n0 + wn * WN + 4 * lhalf;
+        if (__builtin_amdgcn_readfirstlane(n0 + wn * WN + WN <= g.N)) {
+            static_for<4 * NBF>([&](auto jq_tag) {
+                constexpr int jq = decltype(jq_tag)::value;
+                bq[jq] = __builtin_bit_cast(Pack4<T>, *reinterpret_cast<const u32x2*>(bias + nw + (jq >> 2) * 32 + 8 * (jq & 3)));
+            });
+        } else {
+            static_for<4 * NBF>([&](auto jq_tag) {
+                constexpr int jq = decltype(jq_tag)::value;
+                const int n = nw + (jq >> 2) * 32 + 8 * (jq & 3);
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    if (n + e < g.N) bq[jq].v[e] = bias[n + e];
+            });
+        }
+    }
     dispatch_act(g.act, [&](auto act_tag) {
     constexpr int ACT = decltype(act_tag)::value;
     static_for<4 * NBF>([&](auto jq_tag) {
         constexpr int j = decltype(jq_tag)::value >> 2, q = decltype(jq_tag)::value & 3;
         const int nl = j * 32 + 8 * q + 4 * lhalf;
-        const int n = n0 + wn * WN + nl;
-        float bv[4] = {0.f, 0.f, 0.f, 0.f};
-        if (bias && n + 4 <= g.N) {
-            const Pack4<T> t = __builtin_bit_cast(Pack4<T>, *reinterpret_cast<const u32x2*>(bias + n));
+        float bv[4];
 #pragma unroll
-            for (int e = 0; e < 4; e++) bv[e] = Elem<T>::to_f32(t.v[e]);
-        } else if (bias) {                       // the last columns of an N that is no multiple of 4
-#pragma unroll
-            for (int e = 0; e < 4; e++)
-                if (n + e < g.N) bv[e] = Elem<T>::to_f32(bias[n + e]);
-        }
+        for (int e = 0; e < 4; e++) bv[e] = Elem<T>::to_f32(bq[j * 4 + q].v[e]);
         static_for<4>([&](auto i_tag) {
             constexpr int i = decltype(i_tag)::value;
             Pack4<T> o;
             static_for<4>([&](auto e_tag) {
                 constexpr int e = decltype(e_tag)::value;
-                float v = acc[i * NBF + j][4 * q + e] + bv[e];
+                float v = acc_value(acc[i * NBF + j][4 * q + e]) + bv[e];
                 v = apply_act_c<ACT>(v);
                 o.v[e] = Elem<T>::from_f32(v);
             });
@@ -334,7 +362,7 @@ __device__ __forceinline__ void pack_tile(const f32x16 (&acc)[8], const char* bi
             Pack4<T> o;
             static_for<4>([&](auto e_tag) {
                 constexpr int e = decltype(e_tag)::value;
-                float v = acc[i * 2 + j][4 * q + e] + bv[e];
+                float v = acc_value(acc[i * 2 + j][4 * q + e]) + bv[e];
                 v = apply_act_c<ACT>(v);
                 o.v[e] = Elem<T>::from_f32(v);
             });
