@@ -203,10 +203,10 @@ __device__ __forceinline__ void store_tile(f32x16 (&acc)[BW / 16], char* smem, c
     constexpr int kRowsPerPass = 64 / kChunks;
     const int cc = lane % kChunks, rr = lane / kChunks;
     const bool rows_aligned = g.N % 8 == 0;
-    // A wave whose 128 x WN sub-tile lies inside C, rows on 16-byte boundaries, nothing to add:
-    // no per-row conditions, so the reads from LDS run eight passes ahead of the stores (the
-    // general loop below waits for each read before its store).  Same values, same addresses.
-    const bool interior = rows_aligned && !res && m0 + wm * 128 + 128 <= g.M && n0 + wn * WN + WN <= g.N;
+    // A wave whose 128 x WN sub-tile lies inside C with nothing to add: no per-row conditions,
+    // so the reads from LDS run eight passes ahead of the stores (the general loop below waits
+    // for each read before its store).  Same values, same addresses.
+    const bool interior = !res && m0 + wm * 128 + 128 <= g.M && n0 + wn * WN + WN <= g.N;
     if (__builtin_amdgcn_readfirstlane(interior)) {
         constexpr int kPasses = 128 / kRowsPerPass, kAhead = 8;
         T* cw = c + (int64_t)(m0 + wm * 128 + rr) * g.N + (n0 + wn * WN + cc * 8);
@@ -220,7 +220,9 @@ __device__ __forceinline__ void store_tile(f32x16 (&acc)[BW / 16], char* smem, c
                 w[u] = *reinterpret_cast<const u32x4*>(sp + (p0 + u) * kRowsPerPass * kRowPad);
 #pragma unroll
             for (int u = 0; u < kAhead; u++) {
-                *reinterpret_cast<u32x4*>(cw) = w[u];
+                // (rows at any even byte when N is no multiple of 8: see below)
+                if (rows_aligned) *reinterpret_cast<u32x4*>(cw) = w[u];
+                else *reinterpret_cast<u32x4_unaligned*>(cw) = w[u];
                 cw += step;
             }
         }

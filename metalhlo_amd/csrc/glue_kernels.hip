@@ -144,26 +144,44 @@ __global__ __launch_bounds__(256) void to_bool_kernel(const S* __restrict__ x, u
     else y[i] = Cvt<S>::ld(x, i) != 0.0;
 }
 
-// fp32 -> 16-bit float, eight elements per lane (two 16-byte loads, one 16-byte store)
+// fp32 -> 16-bit float.  A workgroup narrows 2048 consecutive elements as two rows of 256
+// four-element groups: every load instruction of a wave reads 1 KB that is contiguous across its
+// lanes (16 bytes each) and every store writes 512 contiguous bytes, the access form of the plain
+// copy above.  The fp32 source is read once and never again (non-temporal); the result is what
+// the next kernels read, so it is stored the ordinary way.
+template <typename D> struct alignas(8) Narrow4 { D v[4]; };
+
+template <typename D>
+__device__ __forceinline__ void narrow_group(const float* __restrict__ x, D* __restrict__ y) {
+    const f32x4 a = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(x));
+    Narrow4<D> o;
+#pragma unroll
+    for (int e = 0; e < 4; e++) o.v[e] = Elem<D>::from_f32(a[e]);
+    *reinterpret_cast<u32x2*>(y) = __builtin_bit_cast(u32x2, o);
+}
+
 template <typename D>
 __global__ __launch_bounds__(256) void narrow_vec_kernel(const float* __restrict__ x,
-                                                         D* __restrict__ y, int64_t nvec) {
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= nvec) return;
-    const f32x4 a = *reinterpret_cast<const f32x4*>(x + i * 8);
-    const f32x4 b = *reinterpret_cast<const f32x4*>(x + i * 8 + 4);
-    Vec16<D> o;
+                                                         D* __restrict__ y, int64_t ngroups) {
+    const int64_t g0 = (int64_t)blockIdx.x * 512 + threadIdx.x, g1 = g0 + 256;
+    // both loads are issued before either is converted
+    f32x4 a = {0.f, 0.f, 0.f, 0.f}, b = a;
+    if (g0 < ngroups) a = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(x + g0 * 4));
+    if (g1 < ngroups) b = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(x + g1 * 4));
+    Narrow4<D> oa, ob;
 #pragma unroll
     for (int e = 0; e < 4; e++) {
-        o.v[e] = Elem<D>::from_f32(a[e]);
-        o.v[4 + e] = Elem<D>::from_f32(b[e]);
+        oa.v[e] = Elem<D>::from_f32(a[e]);
+        ob.v[e] = Elem<D>::from_f32(b[e]);
     }
-    store16(y + i * 8, o);
+    if (g0 < ngroups) *reinterpret_cast<u32x2*>(y + g0 * 4) = __builtin_bit_cast(u32x2, oa);
+    if (g1 < ngroups) *reinterpret_cast<u32x2*>(y + g1 * 4) = __builtin_bit_cast(u32x2, ob);
 }
 
 // fp32 -> 16-bit float for up to kBatchMax tensors in one launch (a model's parameters: many
 // of them small).  The table travels in the kernel arguments; a workgroup handles 2048
-// consecutive elements of one tensor, which it finds by bisecting the running block counts.
+// consecutive elements of one tensor (in the access form of narrow_vec_kernel), which it finds
+// by bisecting the running block counts.
 constexpr int kBatchMax = 96;
 struct ConvertBatch {
     const float* x[kBatchMax];
@@ -184,21 +202,15 @@ __global__ __launch_bounds__(256) void narrow_batch_kernel(ConvertBatch b) {
     const float* x = b.x[lo];
     D* y = static_cast<D*>(b.y[lo]);
     const int64_t n = b.n[lo];
-    const int64_t i = ((int64_t)(blockIdx.x - b.first_block[lo]) * 256 + threadIdx.x) * 8;
-    if (i >= n) return;
-    const bool vec = i + 8 <= n && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15) == 0;
-    if (vec) {
-        const f32x4 p = *reinterpret_cast<const f32x4*>(x + i);
-        const f32x4 q = *reinterpret_cast<const f32x4*>(x + i + 4);
-        Vec16<D> o;
+    const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15) == 0;
+    const int64_t base = (int64_t)(blockIdx.x - b.first_block[lo]) * 2048;
 #pragma unroll
-        for (int e = 0; e < 4; e++) {
-            o.v[e] = Elem<D>::from_f32(p[e]);
-            o.v[4 + e] = Elem<D>::from_f32(q[e]);
-        }
-        store16(y + i, o);
-    } else {
-        for (int64_t e = i; e < n && e < i + 8; e++) y[e] = Elem<D>::from_f32(x[e]);
+    for (int h = 0; h < 2; h++) {                  // (the two loads are independent: both in flight)
+        const int64_t i = base + (int64_t)(h * 256 + threadIdx.x) * 4;
+        if (i >= n) continue;
+        if (aligned && i + 4 <= n) narrow_group<D>(x + i, y + i);
+        else
+            for (int64_t e = i; e < n && e < i + 4; e++) y[e] = Elem<D>::from_f32(x[e]);
     }
 }
 
@@ -440,14 +452,14 @@ extern "C" int mhip_convert(void* stream, const void* x, void* y, int64_t n, int
     hipStream_t s = as_stream(stream);
     if (src_dtype == MHIP_F32 && (dst_dtype == MHIP_BF16 || dst_dtype == MHIP_F16) && n >= 8 &&
         ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15) == 0) {
-        const int64_t nvec = n / 8;
+        const int64_t ngroups = n / 4;
         unsigned grid;
-        if (grid_for(nvec, 256, &grid)) return MHIP_ERR_UNSUPPORTED;
+        if (grid_for(ngroups, 512, &grid)) return MHIP_ERR_UNSUPPORTED;
         if (dst_dtype == MHIP_BF16)
-            hipLaunchKernelGGL((narrow_vec_kernel<bf16_t>), dim3(grid), dim3(256), 0, s, (const float*)x, (bf16_t*)y, nvec);
+            hipLaunchKernelGGL((narrow_vec_kernel<bf16_t>), dim3(grid), dim3(256), 0, s, (const float*)x, (bf16_t*)y, ngroups);
         else
-            hipLaunchKernelGGL((narrow_vec_kernel<f16_t>), dim3(grid), dim3(256), 0, s, (const float*)x, (f16_t*)y, nvec);
-        const int64_t done = nvec * 8;
+            hipLaunchKernelGGL((narrow_vec_kernel<f16_t>), dim3(grid), dim3(256), 0, s, (const float*)x, (f16_t*)y, ngroups);
+        const int64_t done = ngroups * 4;
         if (done == n) return check_launch("convert");
         const int es = 2;
         return mhip_convert(stream, (const char*)x + done * 4, (char*)y + done * es, n - done, src_dtype, dst_dtype);
