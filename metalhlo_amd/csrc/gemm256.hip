@@ -149,6 +149,27 @@ __device__ __forceinline__ void store_tile(f32x16 (&acc)[BW / 16], char* smem, c
     const T* bias = static_cast<const T*>(g.bias);
     constexpr int kRowPad = WN * 2 + 16;
     char* stage = smem + wave * (128 * kRowPad);
+    constexpr int kChunks = WN / 8;                      // 16-byte chunks per row of the wave's sub-tile
+    constexpr int kRowsPerPass = 64 / kChunks;
+    constexpr int kPasses = 128 / kRowsPerPass;
+    const int cc = lane % kChunks, rr = lane / kChunks;
+    const bool rows_aligned = g.N % 8 == 0;
+    // A wave whose 128 x WN sub-tile lies inside C stores it without per-row conditions (below).
+    const bool interior = __builtin_amdgcn_readfirstlane(m0 + wm * 128 + 128 <= g.M && n0 + wn * WN + WN <= g.N);
+    const int64_t first = (int64_t)(m0 + wm * 128 + rr) * g.N + (n0 + wn * WN + cc * 8);   // the lane's chunk of pass 0
+    const int64_t step = (int64_t)kRowsPerPass * g.N;
+    // Its residual chunks are asked for now: they come from memory (the tensor was written
+    // several kernels ago), and a load in front of each store would be waited for pass by pass.
+    u32x4 rv[kPasses];
+    if (interior && res) {
+        const T* rp = res + first;
+#pragma unroll
+        for (int p = 0; p < kPasses; p++) {
+            rv[p] = rows_aligned ? *reinterpret_cast<const u32x4*>(rp) : *reinterpret_cast<const u32x4_unaligned*>(rp);
+            rp += step;
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
     // The bias of all the lane's columns, fetched before the first register group needs it (a
     // load inside each group would be waited for sixteen times); zero without a bias and for
     // columns past N.
@@ -199,19 +220,12 @@ __device__ __forceinline__ void store_tile(f32x16 (&acc)[BW / 16], char* smem, c
     });
     });
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // a wave re-reads only its own rows
-    constexpr int kChunks = WN / 8;                      // 16-byte chunks per row of the wave's sub-tile
-    constexpr int kRowsPerPass = 64 / kChunks;
-    const int cc = lane % kChunks, rr = lane / kChunks;
-    const bool rows_aligned = g.N % 8 == 0;
-    // A wave whose 128 x WN sub-tile lies inside C with nothing to add: no per-row conditions,
-    // so the reads from LDS run eight passes ahead of the stores (the general loop below waits
-    // for each read before its store).  Same values, same addresses.
-    const bool interior = !res && m0 + wm * 128 + 128 <= g.M && n0 + wn * WN + WN <= g.N;
-    if (__builtin_amdgcn_readfirstlane(interior)) {
-        constexpr int kPasses = 128 / kRowsPerPass, kAhead = 8;
-        T* cw = c + (int64_t)(m0 + wm * 128 + rr) * g.N + (n0 + wn * WN + cc * 8);
+    // Interior sub-tile: the reads from LDS run eight passes ahead of the stores (the general
+    // loop below waits for each read before its store).  Same values, same addresses.
+    if (interior) {
+        constexpr int kAhead = 8;
+        T* cw = c + first;
         const char* sp = stage + rr * kRowPad + cc * 16;
-        const int64_t step = (int64_t)kRowsPerPass * g.N;
 #pragma unroll
         for (int p0 = 0; p0 < kPasses; p0 += kAhead) {
             u32x4 w[kAhead];
@@ -220,6 +234,7 @@ __device__ __forceinline__ void store_tile(f32x16 (&acc)[BW / 16], char* smem, c
                 w[u] = *reinterpret_cast<const u32x4*>(sp + (p0 + u) * kRowsPerPass * kRowPad);
 #pragma unroll
             for (int u = 0; u < kAhead; u++) {
+                if (res) w[u] = add_chunk<T>(w[u], rv[p0 + u]);
                 // (rows at any even byte when N is no multiple of 8: see below)
                 if (rows_aligned) *reinterpret_cast<u32x4*>(cw) = w[u];
                 else *reinterpret_cast<u32x4_unaligned*>(cw) = w[u];
