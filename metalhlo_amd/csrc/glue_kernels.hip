@@ -147,8 +147,9 @@ __global__ __launch_bounds__(256) void to_bool_kernel(const S* __restrict__ x, u
 // fp32 -> 16-bit float.  A workgroup narrows 2048 consecutive elements as two rows of 256
 // four-element groups: every load instruction of a wave reads 1 KB that is contiguous across its
 // lanes (16 bytes each) and every store writes 512 contiguous bytes, the access form of the plain
-// copy above.  The fp32 source is read once and never again (non-temporal); the result is what
-// the next kernels read, so it is stored the ordinary way.
+// copy above.  Source and result are both streamed past the caches (non-temporal): the typical
+// call narrows a model's parameters, far more than the L2 holds, long before most of them are
+// read (measured on 124 M parameters: 133 -> 115 us against ordinary stores).
 template <typename D> struct alignas(8) Narrow4 { D v[4]; };
 
 template <typename D>
@@ -157,7 +158,7 @@ __device__ __forceinline__ void narrow_group(const float* __restrict__ x, D* __r
     Narrow4<D> o;
 #pragma unroll
     for (int e = 0; e < 4; e++) o.v[e] = Elem<D>::from_f32(a[e]);
-    *reinterpret_cast<u32x2*>(y) = __builtin_bit_cast(u32x2, o);
+    __builtin_nontemporal_store(__builtin_bit_cast(u32x2, o), reinterpret_cast<u32x2*>(y));
 }
 
 template <typename D>
@@ -174,8 +175,8 @@ __global__ __launch_bounds__(256) void narrow_vec_kernel(const float* __restrict
         oa.v[e] = Elem<D>::from_f32(a[e]);
         ob.v[e] = Elem<D>::from_f32(b[e]);
     }
-    if (g0 < ngroups) *reinterpret_cast<u32x2*>(y + g0 * 4) = __builtin_bit_cast(u32x2, oa);
-    if (g1 < ngroups) *reinterpret_cast<u32x2*>(y + g1 * 4) = __builtin_bit_cast(u32x2, ob);
+    if (g0 < ngroups) __builtin_nontemporal_store(__builtin_bit_cast(u32x2, oa), reinterpret_cast<u32x2*>(y + g0 * 4));
+    if (g1 < ngroups) __builtin_nontemporal_store(__builtin_bit_cast(u32x2, ob), reinterpret_cast<u32x2*>(y + g1 * 4));
 }
 
 // fp32 -> 16-bit float for up to kBatchMax tensors in one launch (a model's parameters: many
