@@ -398,7 +398,7 @@ static int launch_mfma(hipStream_t s, GemmArgs g, int64_t batch) {
 }
 
 // gemm256.hip: 4-wave 256x256 kernel with a hand-scheduled main loop.
-bool gemm256_eligible(const GemmArgs& g, int64_t batch, int dtype, int bw = 256);
+bool gemm256_eligible(const GemmArgs& g, int64_t batch, int dtype, int bw = 256, bool any_tile_count = false);
 int launch_gemm256(hipStream_t s, const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype, int bw = 256);
 bool gemm_stream_eligible(const GemmArgs& g, int64_t batch, int trans_a, int dtype);
 int launch_gemm_stream(hipStream_t s, const GemmArgs& g, int trans_b, int dtype);
@@ -408,7 +408,49 @@ int launch_gemm_f32_mfma(hipStream_t s, const GemmArgs& g, int64_t batch, int tr
 // tuning.hip: variant prescribed by the tuning table for this problem, 0 = none.
 int tuned_gemm_variant(const GemmArgs& g, int64_t batch, int ta, int tb, int dtype);
 
-// Which kernel serves a 16-bit problem (MHIP_GEMM_TILE = 128 | 256 | 2560 | 2561 | 2562 forces one):
+// A problem whose wide (256x256) tiles fill whole rounds of the device except for a narrow band
+// of columns is run as two launches: wide tiles on the first `n_wide` columns, 256x128 tiles on
+// the rest (one round at most) -- [8192,2304] x K 768: 256 wide + 64 narrow tiles instead of two
+// and a quarter rounds of narrow ones.  The slices are plain pointer offsets: B[:, n_wide:] (or B[n_wide:, :] when it is
+// stored [N, K]), bias, residual and C at column n_wide with the full row stride.
+// Returns -1 when the problem does not have that shape (the caller goes on to the other kernels).
+template <typename T, bool TA, bool TB>
+static int launch_column_split(hipStream_t s, const GemmArgs& g, int64_t batch, int dt, bool forced) {
+    constexpr int cus = 256;
+    if (batch != 1 || g.ldc != 0 || g.M % 256 != 0 || g.N % 8 != 0) return -1;
+    const int64_t tiles_m = g.M / 256, cols_w = g.N / 256;
+    // the largest number of wide tile columns that makes whole rounds
+    int64_t c = cols_w;
+    while (c > 0 && (tiles_m * c) % cus != 0) c--;
+    if (c == 0) return -1;
+    const int n_wide = (int)(c * 256), rest = g.N - n_wide;
+    if (rest <= 0) return -1;
+    const int64_t rest_tiles = tiles_m * ((rest + 127) / 128);
+    if (rest_tiles > cus) return -1;
+    if (!forced) {
+        // Measured inside a GPT-2 forward pass (operands from memory, K 768): a round of wide tiles
+        // takes 31 us where two rounds of streamed narrow tiles take 33, so the split only pays
+        // when it replaces a mostly empty last round of narrow tiles -- [8192,2304]: 64 tiles in
+        // the third round, 48.6 -> 45.8 us; [8192,3072], three full rounds: 56.8 -> 58.3, left alone.
+        const int64_t narrow = tiles_m * ((g.N + 127) / 128);
+        const int64_t last_round = narrow % cus;
+        if (last_round == 0 || last_round * 2 > cus || narrow < 2 * cus) return -1;
+    }
+    GemmArgs w = g, r = g;
+    w.N = n_wide; w.ldc = g.N;
+    r.N = rest; r.ldc = g.N;
+    const int64_t boff = TB ? (int64_t)n_wide * g.ldb : (int64_t)n_wide;
+    r.b = static_cast<const T*>(g.b) + boff;
+    if (g.bias) r.bias = static_cast<const T*>(g.bias) + n_wide;
+    if (g.residual) r.residual = static_cast<const T*>(g.residual) + n_wide;
+    r.c = static_cast<T*>(g.c) + n_wide;
+    if (!gemm256_eligible(w, 1, dt) || !gemm256_eligible(r, 1, dt, 128, /*any_tile_count=*/true)) return -1;
+    const int st = launch_gemm256(s, w, 1, TA, TB, dt);
+    if (st != MHIP_OK) return st;
+    return launch_gemm256(s, r, 1, TA, TB, dt, 128);
+}
+
+// Which kernel serves a 16-bit problem (MHIP_GEMM_TILE = 128 | 256 | 2560 | 2561 | 2562 | 2563 forces one):
 //   * the four-wave ring kernel (gemm256.hip) on 256x256 tiles (2560) or 256x128 tiles
 //     (2561) when K >= 512 and the problem is eligible: one workgroup per CU, so its time is
 //     rounds x (stages x per-stage time + prologue and epilogue), rounds = ceil(tiles / 256 CUs);
@@ -426,6 +468,8 @@ int tuned_gemm_variant(const GemmArgs& g, int64_t batch, int ta, int tb, int dty
 //     and from about eight rounds on that outweighs the hidden epilogues: [8192,3072] x K 768
 //     58 -> 51 us and [8192,2304] x K 768 48 -> 41, but [8192,16384] x K 768 216 against 203 on
 //     wide tiles; with B stored [N, K] the gain is within noise;
+//   * wide tiles on the columns that fill whole rounds and narrow tiles on the rest (2563;
+//     launch_column_split) where the problem has that shape;
 //   * the eight-wave 256x256 kernel for large problems the ring kernel cannot take whose
 //     rows of C are not 16-byte aligned (odd N): its eight waves hide the narrow stores;
 //   * otherwise 128x128 tiles, two workgroups per CU (short K, few tiles).
@@ -445,6 +489,10 @@ static int pick_tile(hipStream_t s, const GemmArgs& g, int64_t batch) {
     }
     if (force == 2560) {
         if (gemm256_eligible(g, batch, dt)) return launch_gemm256(s, g, batch, TA, TB, dt);
+    }
+    if (force == 2563 || (force == 0 && g.K >= 512 && tune_int("MHIP_GEMM_SPLIT", 1) != 2)) {    // 2 = off
+        const int st = launch_column_split<T, TA, TB>(s, g, batch, dt, force == 2563);
+        if (st >= 0) return st;
     }
     if (force == 0 && g.K >= 512) {
         constexpr int cus = 256;                       // compute units of the device this is written for

@@ -153,11 +153,12 @@ __device__ __forceinline__ void store_tile(f32x16 (&acc)[BW / 16], char* smem, c
     constexpr int kRowsPerPass = 64 / kChunks;
     constexpr int kPasses = 128 / kRowsPerPass;
     const int cc = lane % kChunks, rr = lane / kChunks;
-    const bool rows_aligned = g.N % 8 == 0;
+    const int ldc = g.ldc ? g.ldc : g.N;                 // (a column slice of a wider C: its row stride)
+    const bool rows_aligned = ldc % 8 == 0;
     // A wave whose 128 x WN sub-tile lies inside C stores it without per-row conditions (below).
     const bool interior = __builtin_amdgcn_readfirstlane(m0 + wm * 128 + 128 <= g.M && n0 + wn * WN + WN <= g.N);
-    const int64_t first = (int64_t)(m0 + wm * 128 + rr) * g.N + (n0 + wn * WN + cc * 8);   // the lane's chunk of pass 0
-    const int64_t step = (int64_t)kRowsPerPass * g.N;
+    const int64_t first = (int64_t)(m0 + wm * 128 + rr) * ldc + (n0 + wn * WN + cc * 8);   // the lane's chunk of pass 0
+    const int64_t step = (int64_t)kRowsPerPass * ldc;
     // Its residual chunks are asked for now: they come from memory (the tensor was written
     // several kernels ago), and a load in front of each store would be waited for pass by pass.
     u32x4 rv[kPasses];
@@ -250,21 +251,21 @@ __device__ __forceinline__ void store_tile(f32x16 (&acc)[BW / 16], char* smem, c
             if (m < g.M && n + 8 <= g.N) {
                 u32x4 w = *reinterpret_cast<const u32x4*>(stage + ml * kRowPad + cc * 16);
                 if (rows_aligned) {
-                    if (res) w = add_chunk<T>(w, *reinterpret_cast<const u32x4*>(res + (int64_t)m * g.N + n));
-                    *reinterpret_cast<u32x4*>(c + (int64_t)m * g.N + n) = w;
+                    if (res) w = add_chunk<T>(w, *reinterpret_cast<const u32x4*>(res + (int64_t)m * ldc + n));
+                    *reinterpret_cast<u32x4*>(c + (int64_t)m * ldc + n) = w;
                 } else {
                     // N is no multiple of 8: rows of C start at any even byte.  The device takes 16-byte
                     // accesses at such addresses (alignment is not enforced for global memory); the type
                     // says so, so the compiler assumes nothing more.
-                    if (res) w = add_chunk<T>(w, *reinterpret_cast<const u32x4_unaligned*>(res + (int64_t)m * g.N + n));
-                    *reinterpret_cast<u32x4_unaligned*>(c + (int64_t)m * g.N + n) = w;
+                    if (res) w = add_chunk<T>(w, *reinterpret_cast<const u32x4_unaligned*>(res + (int64_t)m * ldc + n));
+                    *reinterpret_cast<u32x4_unaligned*>(c + (int64_t)m * ldc + n) = w;
                 }
             } else if (m < g.M && n < g.N) {         // the last, partial chunk of a row
                 const T* sv = reinterpret_cast<const T*>(stage + ml * kRowPad + cc * 16);
                 for (int e = 0; e < g.N - n; e++) {
                     T val = sv[e];
-                    if (res) val = Elem<T>::from_f32(Elem<T>::to_f32(val) + Elem<T>::to_f32(res[(int64_t)m * g.N + n + e]));
-                    c[(int64_t)m * g.N + n + e] = val;
+                    if (res) val = Elem<T>::from_f32(Elem<T>::to_f32(val) + Elem<T>::to_f32(res[(int64_t)m * ldc + n + e]));
+                    c[(int64_t)m * ldc + n + e] = val;
                 }
             }
         }
@@ -290,8 +291,9 @@ __global__ __launch_bounds__(256) void gemm256_kernel(GemmArgs g) {
     const char* b = reinterpret_cast<const char*>(static_cast<const T*>(g.b) + batch * g.sb);
     T* c = static_cast<T*>(g.c) + batch * g.sc;
     const T* res = g.residual ? static_cast<const T*>(g.residual) + batch * g.sc : nullptr;
-    const uint32_t a_bytes = (uint32_t)((int64_t)(TA ? g.K : g.M) * g.lda * 2);
-    const uint32_t b_bytes = (uint32_t)((int64_t)(TB ? g.N : g.K) * g.ldb * 2);
+    // (extents to the last element: the matrices may be column slices of wider ones)
+    const uint32_t a_bytes = (uint32_t)(((int64_t)((TA ? g.K : g.M) - 1) * g.lda + (TA ? g.M : g.K)) * 2);
+    const uint32_t b_bytes = (uint32_t)(((int64_t)((TB ? g.N : g.K) - 1) * g.ldb + (TB ? g.K : g.N)) * 2);
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
@@ -517,16 +519,18 @@ int layout256(hipStream_t s, const GemmArgs& g, int64_t batch, int ta, int tb) {
 // they are then stored with unaligned 16-byte accesses), operands small enough for
 // 32-bit byte offsets including the prefetch overrun of five K stages, and enough
 // tiles (256 x `bw`) to occupy the device.
-bool gemm256_eligible(const GemmArgs& g, int64_t batch, int dtype, int bw) {
+bool gemm256_eligible(const GemmArgs& g, int64_t batch, int dtype, int bw, bool any_tile_count) {
     if (dtype != MHIP_BF16 && dtype != MHIP_F16) return false;
     if (g.K % 32 != 0 || g.K < 32) return false;
     if ((reinterpret_cast<uintptr_t>(g.c) & 15) != 0 || (batch > 1 && g.sc % 8 != 0)) return false;
     if (g.residual && (reinterpret_cast<uintptr_t>(g.residual) & 15) != 0) return false;
     if (g.bias && (reinterpret_cast<uintptr_t>(g.bias) & 7) != 0) return false;
-    const int64_t a_bytes = (int64_t)g.M * g.K * 2, b_bytes = (int64_t)g.N * g.K * 2;
+    // (an upper bound of the extents whichever way the operands are stored; a column slice keeps
+    // the row stride of the whole matrix)
+    const int64_t a_bytes = (int64_t)(g.M > g.K ? g.M : g.K) * g.lda * 2, b_bytes = (int64_t)(g.N > g.K ? g.N : g.K) * g.ldb * 2;
     if (a_bytes >= 0x70000000LL || b_bytes >= 0x70000000LL) return false;
     const int64_t tiles = (int64_t)((g.M + 255) / 256) * ((g.N + bw - 1) / bw) * batch;
-    return tiles >= 192 && tiles <= 0x7FFFFFFF && batch <= 65535;
+    return (tiles >= 192 || any_tile_count) && tiles <= 0x7FFFFFFF && batch <= 65535;
 }
 
 int launch_gemm256(hipStream_t s, const GemmArgs& g, int64_t batch, int trans_a, int trans_b,
@@ -542,9 +546,9 @@ int launch_gemm256(hipStream_t s, const GemmArgs& g, int64_t batch, int trans_a,
 // Streamed tiles (persistent workgroups, stores inside the next tile's loop): see gemm_stream_kernel.
 // Worth it from the second round on, i.e. with more tiles than compute units.
 bool gemm_stream_eligible(const GemmArgs& g, int64_t batch, int trans_a, int dtype) {
-    if (!gemm256_eligible(g, batch, dtype, 128)) return false;
+    if (!gemm256_eligible(g, batch, dtype, 128, false)) return false;
     if (trans_a || batch != 1 || g.residual) return false;
-    if (g.M % 256 != 0 || g.N % 128 != 0 || g.K < 640) return false;
+    if (g.M % 256 != 0 || g.N % 128 != 0 || g.K < 640 || g.ldc != 0) return false;
     if ((int64_t)g.M * g.N * 2 >= 0xFFFFFFFFLL) return false;          // 32-bit byte offsets into C
     return (int64_t)(g.M / 256) * (g.N / 128) > kStreamWorkgroups;
 }

@@ -27,7 +27,7 @@
 
 namespace mhip {
 
-bool gemm256_eligible(const GemmArgs& g, int64_t batch, int dtype, int bw = 256);
+bool gemm256_eligible(const GemmArgs& g, int64_t batch, int dtype, int bw = 256, bool any_tile_count = false);
 bool gemm_stream_eligible(const GemmArgs& g, int64_t batch, int trans_a, int dtype);
 
 namespace {
@@ -84,7 +84,7 @@ bool valid_choice(const char* line, const std::string& choice) {
     int a = 0, b = 0, c = 0, d = 0;
     if (!strncmp(line, "gemm ", 5)) {
         const int v = atoi(choice.c_str());
-        return v == 128 || v == 256 || v == 2560 || v == 2561 || v == 2562;
+        return v == 128 || v == 256 || v == 2560 || v == 2561 || v == 2562 || v == 2563;
     }
     if (!strncmp(line, "row ", 4))
         return sscanf(choice.c_str(), "%d %d %d %d", &a, &b, &c, &d) == 4 && (a == 1 || a == 2) && (b == 1 || b == 2) &&
@@ -173,7 +173,7 @@ int tuned_gemm_variant(const GemmArgs& g, int64_t batch, int ta, int tb, int dty
     std::string c;
     if (!have_entries() || !lookup(gemm_key(g.M, g.N, g.K, batch, ta, tb, dtype), &c)) return 0;
     const int v = atoi(c.c_str());
-    return (v == 128 || v == 256 || v == 2560 || v == 2561 || v == 2562) ? v : 0;
+    return (v == 128 || v == 256 || v == 2560 || v == 2561 || v == 2562 || v == 2563) ? v : 0;
 }
 
 bool tuned_row_launch(int op, int dtype, int64_t rows, int64_t cols, bool has_gamma, bool has_beta, RowLaunch* out) {

@@ -306,6 +306,46 @@ def test_gemm_streamed_tiles_is_the_default_where_it_wins(lib):
     assert torch.equal(ragged, kernels.matmul(a2, b2))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=lambda d: NAME[d])
+@pytest.mark.parametrize("tb", [False, True], ids=["nn", "nt"])
+@pytest.mark.parametrize("shape", [(8192, 2304, 768), (4096, 4360, 512), (2048, 8200, 96)], ids=lambda s: "x".join(map(str, s)))
+def test_gemm_wide_tiles_plus_a_narrow_band(shape, tb, dtype, monkeypatch):
+    """Forced: wide tiles on the columns that make whole rounds, 256x128 tiles on the rest (the
+    band ragged in two of the shapes).  Bit for bit the wide kernel's result, with bias + GELU and
+    with a residual; nothing written outside C; sampled rows against the oracle."""
+    from metalhlo_amd import kernels
+    M, N, K = shape
+    a, b = _ab(M, N, K, dtype, 65, False, tb)
+    rng = np.random.default_rng(66)
+    bias = to_dev(rng.standard_normal(N) * 0.5, dtype)
+    res = to_dev(rng.standard_normal((M, N)), dtype)
+    for use_bias, act, r in ((True, "gelu", None), (False, "none", res)):
+        bb = bias if use_bias else None
+        monkeypatch.setenv("MHIP_GEMM_TILE", "2563")
+        guard = torch.full((M * N + 4096,), 7.0, dtype=dtype, device="cuda")
+        c = kernels.matmul(a, b, bb, act, trans_b=tb, residual=r, out=guard[2048:2048 + M * N].view(M, N))
+        assert torch.all(guard[:2048] == 7.0) and torch.all(guard[2048 + M * N:] == 7.0)
+        monkeypatch.setenv("MHIP_GEMM_TILE", "2560")
+        wide = kernels.matmul(a, b, bb, act, trans_b=tb, residual=r)
+        assert torch.equal(c, wide), (shape, tb, use_bias)
+        if r is None:
+            rows = np.unique(np.r_[np.arange(0, M, 256), np.arange(255, M, 256), rng.integers(0, M, 24)])
+            B = as_f64(b).T if tb else as_f64(b)
+            exp = oracle.matmul_bias_act(as_f64(a)[rows], B, as_f64(bias) if use_bias else None, act)
+            assert_close(c[rows], exp, TOL[dtype], f"split gemm {shape} nt={tb}")
+
+
+def test_gemm_split_is_the_default_for_a_mostly_empty_last_round(lib, monkeypatch):
+    """[8192, 768] x [768, 2304] (two and a quarter rounds of narrow tiles) takes the split by
+    default: same bits as forcing it; [8192, 3072] (three full rounds) stays on streamed tiles."""
+    from metalhlo_amd import kernels
+    a, b = _ab(8192, 2304, 768, torch.bfloat16, 67)
+    monkeypatch.delenv("MHIP_GEMM_TILE", raising=False)
+    c = kernels.matmul(a, b)
+    monkeypatch.setenv("MHIP_GEMM_TILE", "2563")
+    assert torch.equal(c, kernels.matmul(a, b))
+
+
 def test_gemm_large_exact_small_integers():
     """Integer-valued operands with exactly representable partial sums: bit-exact."""
     from metalhlo_amd import kernels
