@@ -161,11 +161,14 @@ __device__ __forceinline__ void store_tile(f32x16 (&acc)[BW / 16], char* smem, c
     const int64_t step = (int64_t)kRowsPerPass * ldc;
     // Its residual chunks are asked for now: they come from memory (the tensor was written
     // several kernels ago), and a load in front of each store would be waited for pass by pass.
-    u32x4 rv[kPasses];
+    // (The wide tile has registers for half of them; the rest is fetched block by block.)
+    constexpr int kPB = kPasses / 4;                     // passes per 32-row block
+    constexpr int kAheadBlocks = BW == 256 ? 2 : 4;
+    u32x4 rv[kAheadBlocks * kPB];
     if (interior && res) {
         const T* rp = res + first;
 #pragma unroll
-        for (int p = 0; p < kPasses; p++) {
+        for (int p = 0; p < kAheadBlocks * kPB; p++) {
             rv[p] = rows_aligned ? *reinterpret_cast<const u32x4*>(rp) : *reinterpret_cast<const u32x4_unaligned*>(rp);
             rp += step;
         }
@@ -196,52 +199,66 @@ __device__ __forceinline__ void store_tile(f32x16 (&acc)[BW / 16], char* smem, c
             });
         }
     }
+    // The sub-tile goes through LDS one 32-row block at a time.  For an interior sub-tile the
+    // stores of a block are issued behind the conversion of the next one (its chunks were read
+    // back from LDS in front of it), so the store traffic overlaps the arithmetic instead of
+    // following it: same values, same addresses as the general loop below.
+    T* cw = c + first;
+    const T* rw = res + first;
+    const char* sp = stage + rr * kRowPad + cc * 16;
+    u32x4 w[kPB];
+    auto store_block = [&](auto i_tag) __attribute__((always_inline)) {
+        constexpr int i = decltype(i_tag)::value;
+        if (res) {
+#pragma unroll
+            for (int u = 0; u < kPB; u++) {
+                u32x4 r;
+                if constexpr (i < kAheadBlocks) r = rv[i * kPB + u];
+                else r = rows_aligned ? *reinterpret_cast<const u32x4*>(rw + (i * kPB + u) * step)
+                                      : *reinterpret_cast<const u32x4_unaligned*>(rw + (i * kPB + u) * step);
+                w[u] = add_chunk<T>(w[u], r);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kPB; u++) {
+            // (rows at any even byte when N is no multiple of 8: see below)
+            if (rows_aligned) *reinterpret_cast<u32x4*>(cw) = w[u];
+            else *reinterpret_cast<u32x4_unaligned*>(cw) = w[u];
+            cw += step;
+        }
+    };
     dispatch_act(g.act, [&](auto act_tag) {
     constexpr int ACT = decltype(act_tag)::value;
-    static_for<4 * NBF>([&](auto jq_tag) {
-        constexpr int j = decltype(jq_tag)::value >> 2, q = decltype(jq_tag)::value & 3;
-        const int nl = j * 32 + 8 * q + 4 * lhalf;
-        float bv[4];
-#pragma unroll
-        for (int e = 0; e < 4; e++) bv[e] = Elem<T>::to_f32(bq[j * 4 + q].v[e]);
-        static_for<4>([&](auto i_tag) {
-            constexpr int i = decltype(i_tag)::value;
+    static_for<4>([&](auto i_tag) {
+        constexpr int i = decltype(i_tag)::value;
+        static_for<4 * NBF>([&](auto jq_tag) {
+            constexpr int j = decltype(jq_tag)::value >> 2, q = decltype(jq_tag)::value & 3;
+            const int nl = j * 32 + 8 * q + 4 * lhalf;
             Pack4<T> o;
             static_for<4>([&](auto e_tag) {
                 constexpr int e = decltype(e_tag)::value;
-                float v = acc_value(acc[i * NBF + j][4 * q + e]) + bv[e];
+                float v = acc_value(acc[i * NBF + j][4 * q + e]) + Elem<T>::to_f32(bq[j * 4 + q].v[e]);
                 v = apply_act_c<ACT>(v);
                 o.v[e] = Elem<T>::from_f32(v);
             });
             *reinterpret_cast<u32x2*>(stage + (i * 32 + lrow) * kRowPad + nl * 2) =
                 __builtin_bit_cast(u32x2, o);
+            // one register group at a time: do not let all the accumulator reads pile up
+            __builtin_amdgcn_sched_barrier(0);
         });
-        // one register group at a time: do not let all the accumulator reads pile up
-        __builtin_amdgcn_sched_barrier(0);
-    });
-    });
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // a wave re-reads only its own rows
-    // Interior sub-tile: the reads from LDS run eight passes ahead of the stores (the general
-    // loop below waits for each read before its store).  Same values, same addresses.
-    if (interior) {
-        constexpr int kAhead = 8;
-        T* cw = c + first;
-        const char* sp = stage + rr * kRowPad + cc * 16;
+        if (interior) {
+            if constexpr (i > 0) store_block(std::integral_constant<int, i - 1>{});
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // a wave re-reads only its own rows
 #pragma unroll
-        for (int p0 = 0; p0 < kPasses; p0 += kAhead) {
-            u32x4 w[kAhead];
-#pragma unroll
-            for (int u = 0; u < kAhead; u++)
-                w[u] = *reinterpret_cast<const u32x4*>(sp + (p0 + u) * kRowsPerPass * kRowPad);
-#pragma unroll
-            for (int u = 0; u < kAhead; u++) {
-                if (res) w[u] = add_chunk<T>(w[u], rv[p0 + u]);
-                // (rows at any even byte when N is no multiple of 8: see below)
-                if (rows_aligned) *reinterpret_cast<u32x4*>(cw) = w[u];
-                else *reinterpret_cast<u32x4_unaligned*>(cw) = w[u];
-                cw += step;
-            }
+            for (int u = 0; u < kPB; u++)
+                w[u] = *reinterpret_cast<const u32x4*>(sp + (i * kPB + u) * kRowsPerPass * kRowPad);
+            __builtin_amdgcn_sched_barrier(0);
         }
+    });
+    });
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    if (interior) {
+        store_block(std::integral_constant<int, 3>{});
     } else {
 #pragma unroll 4
         for (int p = 0; p < 128 / kRowsPerPass; p++) {
