@@ -303,7 +303,8 @@ int mhip_fill(void* stream, void* y, int64_t n, uint64_t pattern, int elem_size)
  * and synchronise with the stream. */
 
 /* GEMM kernel variants (128x128 tiles / 4 waves, 256x256 / 8 waves, the four-wave LDS-ring kernel
- * on 256x256 and on 256x128 tiles): variant code 128 | 256 | 2560 | 2561, microseconds per launch. */
+ * on 256x256 and on 256x128 tiles, the latter also as persistent workgroups, and wide tiles plus a
+ * band of narrow ones): variant code 128 | 256 | 2560 | 2561 | 2562 | 2563, microseconds per launch. */
 int mhip_gemm_autotune(void* stream, const void* a, const void* b, const void* bias, void* c,
                        int64_t M, int64_t N, int64_t K, int64_t batch, int64_t stride_a,
                        int64_t stride_b, int64_t stride_c, int trans_a, int trans_b, int activation,

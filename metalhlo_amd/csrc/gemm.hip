@@ -414,19 +414,28 @@ int tuned_gemm_variant(const GemmArgs& g, int64_t batch, int ta, int tb, int dty
 // and a quarter rounds of narrow ones.  The slices are plain pointer offsets: B[:, n_wide:] (or B[n_wide:, :] when it is
 // stored [N, K]), bias, residual and C at column n_wide with the full row stride.
 // Returns -1 when the problem does not have that shape (the caller goes on to the other kernels).
+// The columns that go to wide tiles: the largest multiple of 256 whose tiles make whole rounds of
+// the device, leaving a band of at most one round of narrow tiles.  False: no such split.
+bool gemm_split_shape(const GemmArgs& g, int64_t batch, int* n_wide_out) {
+    constexpr int cus = 256;
+    if (batch != 1 || g.ldc != 0 || g.M % 256 != 0 || g.N % 8 != 0) return false;
+    const int64_t tiles_m = g.M / 256;
+    int64_t c = g.N / 256;
+    while (c > 0 && (tiles_m * c) % cus != 0) c--;
+    if (c == 0) return false;
+    const int64_t rest = g.N - c * 256;
+    if (rest <= 0 || tiles_m * ((rest + 127) / 128) > cus) return false;
+    if (n_wide_out) *n_wide_out = (int)(c * 256);
+    return true;
+}
+
 template <typename T, bool TA, bool TB>
 static int launch_column_split(hipStream_t s, const GemmArgs& g, int64_t batch, int dt, bool forced) {
     constexpr int cus = 256;
-    if (batch != 1 || g.ldc != 0 || g.M % 256 != 0 || g.N % 8 != 0) return -1;
-    const int64_t tiles_m = g.M / 256, cols_w = g.N / 256;
-    // the largest number of wide tile columns that makes whole rounds
-    int64_t c = cols_w;
-    while (c > 0 && (tiles_m * c) % cus != 0) c--;
-    if (c == 0) return -1;
-    const int n_wide = (int)(c * 256), rest = g.N - n_wide;
-    if (rest <= 0) return -1;
-    const int64_t rest_tiles = tiles_m * ((rest + 127) / 128);
-    if (rest_tiles > cus) return -1;
+    int n_wide = 0;
+    if (!gemm_split_shape(g, batch, &n_wide)) return -1;
+    const int64_t tiles_m = g.M / 256;
+    const int rest = g.N - n_wide;
     if (!forced) {
         // Measured inside a GPT-2 forward pass (operands from memory, K 768): a round of wide tiles
         // takes 31 us where two rounds of streamed narrow tiles take 33, so the split only pays

@@ -29,6 +29,7 @@ namespace mhip {
 
 bool gemm256_eligible(const GemmArgs& g, int64_t batch, int dtype, int bw = 256, bool any_tile_count = false);
 bool gemm_stream_eligible(const GemmArgs& g, int64_t batch, int trans_a, int dtype);
+bool gemm_split_shape(const GemmArgs& g, int64_t batch, int* n_wide_out);
 
 namespace {
 struct Entry { std::string choice; float us; };
@@ -212,14 +213,16 @@ extern "C" int mhip_gemm_autotune(void* stream, const void* a, const void* b, co
     GemmArgs g{};
     g.a = a; g.b = b; g.bias = bias; g.c = c;
     g.M = (int)M; g.N = (int)N; g.K = (int)K;
+    g.lda = (int)(trans_a ? M : K); g.ldb = (int)(trans_b ? K : N);
     g.sa = stride_a; g.sb = stride_b; g.sc = stride_c;
-    const int candidates[5] = {128, 256, 2560, 2561, 2562};
+    const int candidates[6] = {128, 256, 2560, 2561, 2562, 2563};
     int best = 0;
     float best_us = 0.f;
     for (int v : candidates) {
         if (v == 2560 && !gemm256_eligible(g, batch, dtype)) continue;    // validity filter
         if (v == 2561 && !gemm256_eligible(g, batch, dtype, 128)) continue;
         if (v == 2562 && !gemm_stream_eligible(g, batch, trans_a, dtype)) continue;
+        if (v == 2563 && !(gemm_split_shape(g, batch, nullptr) && gemm256_eligible(g, batch, dtype))) continue;
         g_forced_gemm = v;
         const float us = t.time(s, iters, [&] {
             return mhip_gemm(stream, a, b, bias, c, M, N, K, batch, stride_a, stride_b, stride_c, trans_a, trans_b, activation, dtype);
