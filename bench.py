@@ -41,7 +41,7 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # counter reads for the 'copy' workload (256 MiB in, 256 MiB out); see profiles/<workload>.txt.
 MEASURED_TRAFFIC = {
     "gemm": 237446022,
-    "gemm_f32": 1803825891,
+    "gemm_f32": 812745437,
     "attention": 752630452,
     "attention_full": 268946537,
     "attention_f32": 1994907876,

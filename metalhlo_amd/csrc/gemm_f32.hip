@@ -26,6 +26,12 @@ namespace {
 
 constexpr int kStep = 16;       // k per stage
 constexpr int kPad = 20;        // floats per LDS row (16 + 4: rows stay 16-byte aligned, banks spread)
+// Start of row r of a stage: 20 floats per row and four more after every sixteenth row.  The
+// transposing store below has the lanes of a wave sixteen row groups apart in steps of four
+// rows: 4 x 20 floats are 16 banks, so without the extra step lanes i and i + 4 (rows 16 apart
+// = 320 floats = five times around the 64 banks) would land on the same bank, four deep.
+__device__ __forceinline__ constexpr int lds_row(int r) { return r * kPad + 4 * (r >> 4); }
+constexpr int lds_floats(int rows) { return rows * kPad + 4 * (rows / 16); }
 
 // Copies this thread's share (NF = TILE / 16 floats) of one operand's [TILE x 16] stage into
 // registers.  K_CONTIG: element (row, k) at p[row * ld + k]; otherwise at p[k * ld + row].
@@ -68,13 +74,13 @@ __device__ inline void stage_store(float* lds, const float (&r)[NF]) {
     const int t = threadIdx.x;
     constexpr int TPR = 16 / NF;
     if (K_CONTIG) {
-        float* d = lds + (t / TPR) * kPad + (t % TPR) * NF;
+        float* d = lds + lds_row(t / TPR) + (t % TPR) * NF;
 #pragma unroll
         for (int h = 0; h < NF / 4; h++) *reinterpret_cast<f32x4*>(d + 4 * h) = f32x4{r[4 * h], r[4 * h + 1], r[4 * h + 2], r[4 * h + 3]};
     } else {
         const int k = t >> 4, row = (t & 15) * NF;
 #pragma unroll
-        for (int e = 0; e < NF; e++) lds[(row + e) * kPad + k] = r[e];
+        for (int e = 0; e < NF; e++) lds[lds_row(row + e) + k] = r[e];
     }
 }
 
@@ -82,7 +88,7 @@ __device__ inline void stage_store(float* lds, const float (&r)[NF]) {
 template <bool TA, bool TB, int WB>
 __global__ __launch_bounds__(256, 2) void gemm_f32_mfma_kernel(GemmArgs g, int vec_a, int vec_b) {
     constexpr int kTile = 64 * WB, NF = kTile / 16;
-    __shared__ __attribute__((aligned(16))) float lds[2][2][kTile * kPad];   // [stage][A | B]
+    __shared__ __attribute__((aligned(16))) float lds[2][2][lds_floats(kTile)];   // [stage][A | B]
     int tm, tn;
     tile_of(blockIdx.x, gridDim.x, g.tiles_m, g.tiles_n, tm, tn);
     const int m0 = tm * kTile, n0 = tn * kTile;
@@ -120,8 +126,8 @@ __global__ __launch_bounds__(256, 2) void gemm_f32_mfma_kernel(GemmArgs g, int v
         f32x4 fa[WB][2], fb[WB][2];
 #pragma unroll
         for (int i = 0; i < WB; i++) {
-            const float* pa = lds[cur][0] + (wm * 32 * WB + i * 32 + lrow) * kPad + lhalf * 8;
-            const float* pb = lds[cur][1] + (wn * 32 * WB + i * 32 + lrow) * kPad + lhalf * 8;
+            const float* pa = lds[cur][0] + lds_row(wm * 32 * WB + i * 32 + lrow) + lhalf * 8;
+            const float* pb = lds[cur][1] + lds_row(wn * 32 * WB + i * 32 + lrow) + lhalf * 8;
             fa[i][0] = *reinterpret_cast<const f32x4*>(pa);
             fa[i][1] = *reinterpret_cast<const f32x4*>(pa + 4);
             fb[i][0] = *reinterpret_cast<const f32x4*>(pb);
@@ -193,12 +199,16 @@ int launch_tile(hipStream_t s, GemmArgs g, int64_t batch) {
     return check_launch("gemm_f32_mfma");
 }
 
-// 64x64 tiles by default: with eight workgroups resident per CU they measured faster than
-// 128x128 tiles with three even where the latter fill the device (4096^3: 97 against 85 TFLOP/s);
-// MHIP_GEMM_F32_TILE = 128 takes the large tile.
+// 128x128 tiles (three workgroups resident per CU: 768 on the device) once there are enough of
+// them for a round and a quarter, 64x64 tiles (eight per CU) below that.  Measured (TFLOP/s,
+// 64 | 128): 4096^3 101 | 116, [8192,3072] x K 768 (1536 large tiles) 100 | 113; [3000,3000] x K 1000
+// (576) 89 | 73, [2048,2048] x K 2048 (256) 99 | 91, [8192,768] x K 3072 (384) 100 | 87, 1024^3 (64)
+// 62 | 23.  MHIP_GEMM_F32_TILE = 64 | 128 forces one.
 template <bool TA, bool TB>
 int launch(hipStream_t s, const GemmArgs& g, int64_t batch) {
-    if (tune_int("MHIP_GEMM_F32_TILE", 64) == 128) return launch_tile<TA, TB, 2>(s, g, batch);
+    const int forced = tune_int("MHIP_GEMM_F32_TILE", 0);
+    const int64_t large_tiles = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128) * batch;
+    if (forced == 128 || (forced != 64 && large_tiles >= 960)) return launch_tile<TA, TB, 2>(s, g, batch);
     return launch_tile<TA, TB, 1>(s, g, batch);
 }
 
