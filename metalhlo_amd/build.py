@@ -75,7 +75,8 @@ def build_kernels(verbose: bool = True) -> str:
     with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as ex:
         list(ex.map(one, zip(srcs, objs)))
     out = os.path.join(LIBDIR, "libmetalhlo_hip.so")
-    _run([hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out, *objs])
+    # (-z defs: a kernel whose host-side launch stub was not emitted must fail here, not at load time)
+    _run([hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-Wl,-z,defs", "-o", out, *objs])
     if verbose:
         print("  link ", os.path.relpath(out, ROOT), flush=True)
     return out

@@ -21,6 +21,17 @@ namespace mhip {
 // NB: depth of the K and of the V ring in LDS.  Two everywhere: with head size 64 a ring of three or
 // four measured 8 to 13 % slower (B8 H12 S1024: 38.5 / 40.5 against 35.7 us) -- it costs the third
 // resident workgroup per CU, which hides more latency than the deeper prefetch does.
+//
+// The softmax keeps a REFERENCE maximum per row (log2 domain) that moves only when a block's
+// maximum exceeds it by more than 8: probabilities are exp2(s - ref) <= 2^8, accumulated in fp32,
+// and the final division uses the sum taken with the same reference, so the result is the same
+// function.  What it saves is the rescaling of the output accumulators, which a strict running
+// maximum triggers in nearly every block when 32 rows share a wave.  (-inf + 8 = -inf: the first
+// finite block maximum always moves it; a block of masked scores never does.)
+__device__ __forceinline__ float moved_reference(float ref, float block_max) {
+    return block_max > ref + 8.f ? block_max : ref;
+}
+
 template <typename T, int D, bool CAUSAL, bool HAS_MASK, int NB>
 __global__ __launch_bounds__(256, 2) void fa_fwd_kernel(FaArgs a) {
     constexpr int CPR = D / 8;                  // 16-byte chunks per row
@@ -72,19 +83,26 @@ __global__ __launch_bounds__(256, 2) void fa_fwd_kernel(FaArgs a) {
     // of a tile (lane l lands at byte 16*l of that KB); the swizzle is applied by
     // choosing which global chunk each lane fetches.  Keys past the end read 0.
     const int ld_row = lane / CPR, ld_pos = lane % CPR;
-    // (a block past the last one this workgroup needs is "loaded" all the same, out of bounds:
-    // the waits below count loads, so every step issues the same number)
-    const int kv_end = min(nkv * kBKV, a.Skv);
+    // (a block past the last one this workgroup needs is loaded all the same: the waits below
+    // count loads, so every step issues the same number.)  Each lane's offsets inside block 0
+    // are computed once; a step adds the block's offset.  Keys past the end need no test: their
+    // offsets lie beyond the extent of the buffer descriptors above, and such loads put zeros
+    // into LDS (V rows of zeros, so that a probability of zero times them stays zero).
+    // (The swizzles repeat every sixteen rows and a wave's loads of a tile are 4 * kRowsPerInst
+    // = 16 or 32 rows apart, so load i differs from load 0 by a constant.)
+    const int wave_s = __builtin_amdgcn_readfirstlane(wave);
+    const int ld_row0 = wave_s * kRowsPerInst + ld_row;
+    const uint32_t koff0 = (uint32_t)((ld_row0 * k_rs + ((ld_pos ^ k_swz<D>(ld_row0)) << 3)) * 2);
+    const uint32_t voff0 = (uint32_t)((ld_row0 * v_rs + ((ld_pos ^ v_swz<D>(ld_row0)) << 3)) * 2);
     auto load_tile = [&](int kv0, int buf) {
 #pragma unroll
         for (int i = 0; i < kInst; i++) {
-            const int blk = i * 4 + wave;                 // which KB of the tile
-            const int row = blk * kRowsPerInst + ld_row;
-            const int key = kv0 + row;
-            const uint32_t koff = key < kv_end ? (uint32_t)((key * k_rs + ((ld_pos ^ k_swz<D>(row)) << 3)) * 2) : kOobA;
-            const uint32_t voff = key < kv_end ? (uint32_t)((key * v_rs + ((ld_pos ^ v_swz<D>(row)) << 3)) * 2) : kOobA;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, (fa_lds_void*)(smem + buf * kTile + blk * 1024), 16, koff, 0, 0, 0);
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, (fa_lds_void*)(smem + (NB + buf) * kTile + blk * 1024), 16, voff, 0, 0, 0);
+            const int blk = i * 4 + wave_s;               // which KB of the tile
+            const int row = kv0 + i * 4 * kRowsPerInst;   // (scalar)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, (fa_lds_void*)(smem + buf * kTile + blk * 1024), 16,
+                                                     koff0 + (uint32_t)(row * k_rs * 2), 0, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, (fa_lds_void*)(smem + (NB + buf) * kTile + blk * 1024), 16,
+                                                     voff0 + (uint32_t)(row * v_rs * 2), 0, 0, 0);
         }
     };
     // loads land in program order: the next block has landed when only the NB - 2 blocks issued
@@ -105,7 +123,7 @@ __global__ __launch_bounds__(256, 2) void fa_fwd_kernel(FaArgs a) {
     for (int i = 0; i < ND; i++)
 #pragma unroll
         for (int r = 0; r < 16; r++) oacc[i][r] = 0.f;
-    float m_run = -INFINITY, l_run = 0.f;   // running max in the log2 domain, running sum
+    float m_run = -INFINITY, l_run = 0.f;   // reference maximum in the log2 domain (see moved_reference), running sum
 
 #pragma unroll
     for (int p = 0; p < NB - 1; p++) load_tile(p * kBKV, p);
@@ -171,7 +189,7 @@ __global__ __launch_bounds__(256, 2) void fa_fwd_kernel(FaArgs a) {
 #pragma unroll
                 for (int i = 1; i < 32; i++) mloc = fmaxf(mloc, sv[i]);
                 mloc = half_max(mloc);
-                m_new = fmaxf(m_run, mloc);
+                m_new = moved_reference(m_run, mloc);
                 const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
 #pragma unroll
                 for (int i = 0; i < 32; i++) sv[i] = __builtin_amdgcn_exp2f(sv[i] - m_use);
@@ -182,7 +200,7 @@ __global__ __launch_bounds__(256, 2) void fa_fwd_kernel(FaArgs a) {
 #pragma unroll
                 for (int i = 1; i < 32; i++) mloc = fmaxf(mloc, sv[i]);
                 mloc = half_max(mloc);
-                m_new = fmaxf(m_run, mloc * a.c);
+                m_new = moved_reference(m_run, mloc * a.c);
                 const float neg_m = -m_new;     // finite: an interior block has no masked score
 #pragma unroll
                 for (int i = 0; i < 32; i++) sv[i] = __builtin_amdgcn_exp2f(fmaf(sv[i], a.c, neg_m));

@@ -186,7 +186,8 @@ def test_attention_pipelined_scale_and_extremes(force_pipelined):
     force_pipelined.setenv("MHIP_FA_PIPE", "2")
     b = kernels.flash_attention(q, k, v, is_causal=True)
     assert_close(a, as_f64(b), 2e-2, "pipelined == 128-row kernel")
-    assert not torch.equal(a, b)         # two different kernels ran (their roundings differ)
+    # (both keep the same lazily moving reference maximum, so they usually agree to the last bit;
+    # their row sums are taken in different orders, so that is not required)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=lambda d: NAME[d])
