@@ -21,16 +21,6 @@ namespace mhip {
 // NB: depth of the K and of the V ring in LDS.  Two everywhere: with head size 64 a ring of three or
 // four measured 8 to 13 % slower (B8 H12 S1024: 38.5 / 40.5 against 35.7 us) -- it costs the third
 // resident workgroup per CU, which hides more latency than the deeper prefetch does.
-//
-// The softmax keeps a REFERENCE maximum per row (log2 domain) that moves only when a block's
-// maximum exceeds it by more than 8: probabilities are exp2(s - ref) <= 2^8, accumulated in fp32,
-// and the final division uses the sum taken with the same reference, so the result is the same
-// function.  What it saves is the rescaling of the output accumulators, which a strict running
-// maximum triggers in nearly every block when 32 rows share a wave.  (-inf + 8 = -inf: the first
-// finite block maximum always moves it; a block of masked scores never does.)
-__device__ __forceinline__ float moved_reference(float ref, float block_max) {
-    return block_max > ref + 8.f ? block_max : ref;
-}
 
 template <typename T, int D, bool CAUSAL, bool HAS_MASK, int NB>
 __global__ __launch_bounds__(256, 2) void fa_fwd_kernel(FaArgs a) {

@@ -94,6 +94,16 @@ __device__ inline __amdgpu_buffer_rsrc_t fa_rsrc(const void* p, uint32_t bytes) 
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
 }
 
+// The softmax keeps a REFERENCE maximum per row (log2 domain) that moves only when a block's
+// maximum exceeds it by more than 8: probabilities are exp2(s - ref) <= 2^8, accumulated in fp32,
+// and the final division uses the sum taken with the same reference, so the result is the same
+// function.  What it saves is the rescaling of the output accumulators, which a strict running
+// maximum triggers in nearly every block when 32 rows share a wave.  (-inf + 8 = -inf: the first
+// finite block maximum always moves it; a block of masked scores never does.)
+__device__ __forceinline__ float moved_reference(float ref, float block_max) {
+    return block_max > ref + 8.f ? block_max : ref;
+}
+
 // K and V tiles sit in LDS as they lie in memory, [64 keys][D], 16-byte chunks
 // XOR-swizzled inside each row.  K is read as the A operand of S^T = K.Q^T with
 // ds_read_b128 (lane = key row, eight consecutive d); V is read as the A operand

@@ -127,7 +127,8 @@ __global__ __launch_bounds__(256) void fa_f32_mfma_kernel(FaArgs a, float scale)
             m_blk = fmaxf(m_blk, t[i]);
         }
         m_blk = half_max(m_blk);
-        const float m_new = fmaxf(m_run, m_blk);
+        // (a reference maximum that moves only when the block exceeds it by 2^8: see moved_reference)
+        const float m_new = moved_reference(m_run, m_blk);
         const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
         const float alpha = exp2f(m_run - m_use);
         m_run = m_new;
@@ -138,10 +139,12 @@ __global__ __launch_bounds__(256) void fa_f32_mfma_kernel(FaArgs a, float scale)
             psum += t[i];
         }
         l_run = l_run * alpha + psum;
+        if (__any(alpha != 1.f)) {                     // rare once the reference has settled
 #pragma unroll
-        for (int d = 0; d < ND; d++)
+            for (int d = 0; d < ND; d++)
 #pragma unroll
-            for (int i = 0; i < 16; i++) o[d][i] *= alpha;
+                for (int i = 0; i < 16; i++) o[d][i] *= alpha;
+        }
 
         // ---- O^T += V^T . P^T
 #pragma unroll
