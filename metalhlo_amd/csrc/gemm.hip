@@ -437,13 +437,13 @@ static int launch_column_split(hipStream_t s, const GemmArgs& g, int64_t batch, 
     const int64_t tiles_m = g.M / 256;
     const int rest = g.N - n_wide;
     if (!forced) {
-        // Measured inside a GPT-2 forward pass (operands from memory, K 768): a round of wide tiles
-        // takes 31 us where two rounds of streamed narrow tiles take 33, so the split only pays
-        // when it replaces a mostly empty last round of narrow tiles -- [8192,2304]: 64 tiles in
-        // the third round, 48.6 -> 45.8 us; [8192,3072], three full rounds: 56.8 -> 58.3, left alone.
+        // Worth it from a third round of narrow tiles on.  Measured inside a GPT-2 forward pass
+        // (operands from memory, K 768; a round of wide tiles takes 31 us there, a streamed narrow
+        // tile 14-17): [8192,2304], whose third narrow round holds 64 tiles, 48.6 -> 45.8 us;
+        // [8192,3072], three full rounds, 2 us better than streamed or plain narrow tiles (the
+        // whole pass 3.385 -> 3.362 ms).
         const int64_t narrow = tiles_m * ((g.N + 127) / 128);
-        const int64_t last_round = narrow % cus;
-        if (last_round == 0 || last_round * 2 > cus || narrow < 2 * cus) return -1;
+        if (narrow <= 2 * cus) return -1;
     }
     GemmArgs w = g, r = g;
     w.N = n_wide; w.ldc = g.N;

@@ -289,10 +289,11 @@ def test_gemm_streamed_tiles(shape, tb, dtype, monkeypatch):
 
 
 def test_gemm_streamed_tiles_is_the_default_where_it_wins(lib):
-    """The default choice for a GPT-2-shaped product [8192, 768] x [768, 3072] is the streamed
-    kernel (same bits as forcing it), and a problem it cannot take (ragged N) still runs."""
+    """The default choice for [8192, 768] x [768, 3584] (three and a half rounds of narrow tiles,
+    no column split with a band of at most one round) is the streamed kernel (same bits as forcing
+    it), and a problem it cannot take (ragged N) still runs."""
     from metalhlo_amd import kernels
-    a, b = _ab(8192, 3072, 768, torch.bfloat16, 63)
+    a, b = _ab(8192, 3584, 768, torch.bfloat16, 63)
     os.environ.pop("MHIP_GEMM_TILE", None)
     c = kernels.matmul(a, b, None, "gelu")
     os.environ["MHIP_GEMM_TILE"] = "2562"
@@ -335,15 +336,16 @@ def test_gemm_wide_tiles_plus_a_narrow_band(shape, tb, dtype, monkeypatch):
             assert_close(c[rows], exp, TOL[dtype], f"split gemm {shape} nt={tb}")
 
 
-def test_gemm_split_is_the_default_for_a_mostly_empty_last_round(lib, monkeypatch):
-    """[8192, 768] x [768, 2304] (two and a quarter rounds of narrow tiles) takes the split by
-    default: same bits as forcing it; [8192, 3072] (three full rounds) stays on streamed tiles."""
+def test_gemm_split_is_the_default_from_a_third_round_on(lib, monkeypatch):
+    """[8192, 768] x [768, 2304] and x [768, 3072] (more than two rounds of narrow tiles, a band of
+    at most one round) take the split by default: same bits as forcing it."""
     from metalhlo_amd import kernels
-    a, b = _ab(8192, 2304, 768, torch.bfloat16, 67)
-    monkeypatch.delenv("MHIP_GEMM_TILE", raising=False)
-    c = kernels.matmul(a, b)
-    monkeypatch.setenv("MHIP_GEMM_TILE", "2563")
-    assert torch.equal(c, kernels.matmul(a, b))
+    for N in (2304, 3072):
+        a, b = _ab(8192, N, 768, torch.bfloat16, 67)
+        monkeypatch.delenv("MHIP_GEMM_TILE", raising=False)
+        c = kernels.matmul(a, b, None, "gelu")
+        monkeypatch.setenv("MHIP_GEMM_TILE", "2563")
+        assert torch.equal(c, kernels.matmul(a, b, None, "gelu"))
 
 
 def test_gemm_large_exact_small_integers():
