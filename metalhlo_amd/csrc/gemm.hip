@@ -469,14 +469,9 @@ static int launch_column_split(hipStream_t s, const GemmArgs& g, int64_t batch, 
 //     500 -- figures fitted to seven measured shapes (4096^3: wide; [8192,768] x K 3072
 //     or 768, [8192,2304..3072] x K 768: narrow);
 //   * the same 256x128 kernel as persistent workgroups that store a tile inside the loop of the
-//     next one (2562; gemm_stream_kernel) when the problem meets that kernel's conditions, B is
-//     stored [K, N] and there are two to four rounds of narrow tiles.  Fitted to measured shapes
-//     (us): a streamed tile costs 0.3875 per K stage + 3.8, plus 5 once; a wide tile 0.6625 per
-//     stage + 13.8 (its epilogue is exposed in every round).  Streamed tiles always beat the plain
-//     narrow form, but the narrow tile asks the L2 for 1.5 times the operand bytes of the wide one,
-//     and from about eight rounds on that outweighs the hidden epilogues: [8192,3072] x K 768
-//     58 -> 51 us and [8192,2304] x K 768 48 -> 41, but [8192,16384] x K 768 216 against 203 on
-//     wide tiles; with B stored [N, K] the gain is within noise;
+//     next one (2562; gemm_stream_kernel): forced, recorded by the tuner, or with
+//     MHIP_GEMM_STREAM=1 for two to four rounds of narrow tiles with B stored [K, N] (see below
+//     why it is no longer a default);
 //   * wide tiles on the columns that fill whole rounds and narrow tiles on the rest (2563;
 //     launch_column_split) where the problem has that shape;
 //   * the eight-wave 256x256 kernel for large problems the ring kernel cannot take whose
@@ -507,7 +502,13 @@ static int pick_tile(hipStream_t s, const GemmArgs& g, int64_t batch) {
         constexpr int cus = 256;                       // compute units of the device this is written for
         const int64_t narrow = tiles_m * ((g.N + 127) / 128) * batch, stages = g.K / 32;
         const bool wide_ok = gemm256_eligible(g, batch, dt), narrow_ok = gemm256_eligible(g, batch, dt, 128);
-        if (!TB && (narrow + cus - 1) / cus <= 4 && tune_int("MHIP_GEMM_STREAM", 1) != 2 &&    // 2 = off
+        // (The streamed form of the narrow tile, 2562, is no longer chosen here: it is 5 % ahead of
+        // wide tiles on a few shapes when the operands sit in the L2 -- [4096,8320] x K 1024 77 against
+        // 81 us, [8192,4608] x K 768 67 against 71 -- and 10 to 15 % behind on the same shapes when
+        // they come from memory, 92 against 84 and 83 against 72, which is how a GEMM inside a
+        // model finds them; [8192,3584] x K 768: 58 / 66 us streamed, 48 / 53 on wide tiles.  The tuner
+        // still times it and records it where it wins; MHIP_GEMM_STREAM=1 restores the old choice.)
+        if (!TB && (narrow + cus - 1) / cus <= 4 && tune_int("MHIP_GEMM_STREAM", 2) == 1 &&
             gemm_stream_eligible(g, batch, TA, dt)) {
             const double stream_us = (double)((narrow + cus - 1) / cus) * (stages * 0.3875 + 3.8) + 5.0;
             const double wide_us = (double)((big + cus - 1) / cus) * (stages * 0.6625 + 13.8);

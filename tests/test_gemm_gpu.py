@@ -288,10 +288,10 @@ def test_gemm_streamed_tiles(shape, tb, dtype, monkeypatch):
         assert_close(c[rows], exp, TOL[dtype], f"streamed gemm {shape} nt={tb} bias={use_bias}")
 
 
-def test_gemm_streamed_tiles_is_the_default_where_it_wins(lib):
-    """The default choice for [8192, 768] x [768, 3584] (three and a half rounds of narrow tiles,
-    no column split with a band of at most one round) is the streamed kernel (same bits as forcing
-    it), and a problem it cannot take (ragged N) still runs."""
+def test_gemm_streamed_tiles_agree_with_the_default_choice(lib):
+    """[8192, 768] x [768, 3584] (three and a half rounds of narrow tiles, no column split with a
+    band of at most one round): the default choice (wide tiles) and the streamed kernel give the
+    same bits, and a problem the streamed kernel cannot take (ragged N) still runs when it is forced."""
     from metalhlo_amd import kernels
     a, b = _ab(8192, 3584, 768, torch.bfloat16, 63)
     os.environ.pop("MHIP_GEMM_TILE", None)
