@@ -25,7 +25,7 @@ constexpr int kFBK = 32;      // keys per block
 __device__ __forceinline__ int f32_key(int i, int h) { return 8 * (i >> 2) + 4 * h + (i & 3); }
 
 template <int D, bool CAUSAL, bool HAS_MASK>
-__global__ __launch_bounds__(256) void fa_f32_mfma_kernel(FaArgs a, float scale) {
+__global__ __launch_bounds__(256, 2) void fa_f32_mfma_kernel(FaArgs a, float scale) {
     // K rows padded to D + 2 floats (lane = key reads fall on distinct banks), V rows to D + 8
     // (the two halves of a wave read rows four apart)
     constexpr int KS = D + 2, VS = D + 8;
