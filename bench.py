@@ -44,7 +44,7 @@ MEASURED_TRAFFIC = {
     "gemm_f32": 812745437,
     "attention": 752630452,
     "attention_full": 268946537,
-    "attention_f32": 2029700000,
+    "attention_f32": 1823030837,
     "softmax": 536779900,
     "layer_norm": 536936179,
     "rms_norm": 536839114,

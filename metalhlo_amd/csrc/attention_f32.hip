@@ -130,12 +130,14 @@ __global__ __launch_bounds__(256, 2) void fa_f32_mfma_kernel(FaArgs a, float sca
         // (a reference maximum that moves only when the block exceeds it by 2^8: see moved_reference)
         const float m_new = moved_reference(m_run, m_blk);
         const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = exp2f(m_run - m_use);
+        // (v_exp_f32 itself, about 1 ulp: the library exp2f wraps it in five more instructions that
+        // only serve results below 2^-126, which are zeros here either way)
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
         m_run = m_new;
         float psum = 0.f;
 #pragma unroll
         for (int i = 0; i < 16; i++) {
-            t[i] = exp2f(t[i] - m_use);
+            t[i] = __builtin_amdgcn_exp2f(t[i] - m_use);
             psum += t[i];
         }
         l_run = l_run * alpha + psum;
