@@ -66,13 +66,25 @@ __global__ __launch_bounds__(256) void embed_kernel(const int32_t* __restrict__ 
                                                     const P* __restrict__ wte,
                                                     const P* __restrict__ wpe,
                                                     O* __restrict__ out, int64_t S, int64_t d,
-                                                    int64_t vocab) {
+                                                    int64_t vocab, int vec4) {
     const int64_t tok = blockIdx.x;  // over B*S
     int64_t id = ids[tok];
     id = id < 0 ? 0 : (id > vocab - 1 ? vocab - 1 : id);
     const P* te = wte + id * d;
     const P* pe = wpe + (tok % S) * d;
     O* o = out + tok * d;
+    if (vec4) {       // rows of all three tensors start on 16-byte (params) / 8-byte (result) boundaries
+        struct alignas(4 * sizeof(P)) P4 { P v[4]; };
+        struct alignas(4 * sizeof(O)) O4 { O v[4]; };
+        for (int64_t c = (int64_t)threadIdx.x * 4; c < d; c += 1024) {
+            const P4 t = *reinterpret_cast<const P4*>(te + c), q = *reinterpret_cast<const P4*>(pe + c);
+            O4 r;
+#pragma unroll
+            for (int e = 0; e < 4; e++) r.v[e] = Elem<O>::from_f32(Elem<P>::to_f32(t.v[e]) + Elem<P>::to_f32(q.v[e]));
+            *reinterpret_cast<O4*>(o + c) = r;
+        }
+        return;
+    }
     for (int64_t c = threadIdx.x; c < d; c += 256)
         o[c] = Elem<O>::from_f32(Elem<P>::to_f32(te[c]) + Elem<P>::to_f32(pe[c]));
 }
@@ -361,9 +373,12 @@ extern "C" int mhip_embed_tokens(void* stream, const void* ids, const void* wte,
     if (B * S > 0x7FFFFFFFLL) return fail(MHIP_ERR_UNSUPPORTED, "mhip_embed_tokens: too many tokens");
     hipStream_t s = as_stream(stream);
     const dim3 grid((unsigned)(B * S)), blk(256);
+    // four elements per lane when every row starts on a 16-byte boundary (in either element size)
+    const int vec4 = d_model % 4 == 0 && ((reinterpret_cast<uintptr_t>(wte) | reinterpret_cast<uintptr_t>(wpe) |
+                                            reinterpret_cast<uintptr_t>(out)) & 15) == 0;
 #define MHIP_EMB(P, O)                                                                      \
     hipLaunchKernelGGL((embed_kernel<P, O>), grid, blk, 0, s, (const int32_t*)ids,          \
-                       (const P*)wte, (const P*)wpe, (O*)out, S, d_model, vocab)
+                       (const P*)wte, (const P*)wpe, (O*)out, S, d_model, vocab, vec4)
     if (param_dtype == MHIP_F32 && out_dtype == MHIP_BF16) MHIP_EMB(float, bf16_t);
     else if (param_dtype == MHIP_F32 && out_dtype == MHIP_F16) MHIP_EMB(float, f16_t);
     else if (param_dtype == MHIP_F32 && out_dtype == MHIP_F32) MHIP_EMB(float, float);
