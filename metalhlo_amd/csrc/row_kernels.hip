@@ -276,7 +276,13 @@ void row_split_kernel(const T* __restrict__ x, const T* __restrict__ gamma, cons
             v[r] = t;
         }
     };
-    const int64_t first = chunk > 0 ? (int64_t)blockIdx.x * chunk * RPB : (int64_t)blockIdx.x * RPB;
+    // chunk < 0: one iteration per workgroup, and the workgroups of XCD x (ids x, x + 8, ...: the
+    // dispatcher deals ids round-robin over the eight XCDs) take the x-th eighth of the rows -- the
+    // rows whose tiles a GEMM on [rows, cols] has just written from that XCD, and whose tiles the
+    // next GEMM reads on it, so a tensor that fits the L2s is found there (grid a multiple of 8).
+    const unsigned bid = chunk < 0 ? (blockIdx.x % 8u) * (gridDim.x / 8u) + blockIdx.x / 8u : blockIdx.x;
+    if (chunk < 0) chunk = 1;
+    const int64_t first = chunk > 0 ? (int64_t)bid * chunk * RPB : (int64_t)bid * RPB;
     const int64_t stop = chunk > 0 ? (first + (int64_t)chunk * RPB < rows ? first + (int64_t)chunk * RPB : rows) : rows;
     const int64_t step = chunk > 0 ? RPB : (int64_t)gridDim.x * RPB;
     for (int64_t base = first; base < stop; base += step) {
@@ -624,12 +630,16 @@ static void launch_split(const RowLaunch& c, hipStream_t s, const T* xp, const T
     const int rpb = 4 / WPR * (c.r == 2 ? 2 : 1);
     const int64_t units = (rows + rpb - 1) / rpb;
     if (c.ordered) {
+        // a tensor small enough to sit in the L2s between two kernels: rows by XCD (see the kernel)
+        const bool by_xcd = units % 8 == 0 && (int64_t)rows * cols * (int64_t)sizeof(T) <= (16 << 20) &&
+                            tune_int("MHIP_ROW_XCD", 1) != 2;      // 2 = off
+        const int chunk = by_xcd ? -1 : 1;
         if (c.r == 2)
             hipLaunchKernelGGL((row_split_kernel<T, OP, NVS, WPR, 2>), dim3((unsigned)units), dim3(256), 0, s, xp, gp, bp, yp,
-                               rows, cols, eps, 1);
+                               rows, cols, eps, chunk);
         else
             hipLaunchKernelGGL((row_split_kernel<T, OP, NVS, WPR, 1>), dim3((unsigned)units), dim3(256), 0, s, xp, gp, bp, yp,
-                               rows, cols, eps, 1);
+                               rows, cols, eps, chunk);
     } else if (c.r == 2) {
         launch_persistent(row_split_kernel<T, OP, NVS, WPR, 2>, 0, c.per_cu, units, s, xp, gp, bp, yp, rows, cols, eps, 0);
     } else {
