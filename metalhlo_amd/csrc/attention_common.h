@@ -23,7 +23,7 @@ struct FaArgs {
     int is_causal;    // read by the scalar path (the MFMA path is templated on it)
     int64_t mask_sb, mask_sh;
     int nqb;          // query blocks per (batch, head)
-    int xcd_map;      // 1: (batch*head) % 8 == 0, use the XCD-aware block order
+    int xcd_map;      // (batch*head) % 8 == 0: the XCD-aware block order, 1 = an XCD takes a contiguous eighth of the heads, 2 = every eighth head
     int pair_tiles;   // pipelined kernel, causal: a workgroup takes two query tiles (first + last, ...)
     int cu_group;     // 128-row kernel: CUs a run of consecutive workgroup ids is dealt over (per XCD, or all)
     // Element strides {batch, head, row} of q, k, v, o (the last axis is contiguous).  Only
@@ -41,6 +41,10 @@ struct FaArgs {
 // first and dealt to the CUs in rounds of cu_group, every other round in reverse (a snake
 // draft), which balances the resident set and is the longest-first rule for what is
 // dispatched later (B8 H12 S1024 D64 causal: 35.4 -> 23.7 us).
+// An XCD takes a contiguous eighth of the (batch, head) pairs: with the fused projection of a
+// transformer layer in front ([B*S, 3*H*D], whose row tiles a GEMM writes XCD by XCD in eighths
+// of the rows) and the output projection behind, a batch's heads then read what its own XCD's
+// L2 may still hold and leave their output where the next GEMM looks for it.
 template <bool CAUSAL>
 __device__ inline void tile_of_workgroup(const FaArgs& a, int id, int& bh, int& qb) {
     const int groups = a.xcd_map ? 8 : 1;
@@ -52,16 +56,17 @@ __device__ inline void tile_of_workgroup(const FaArgs& a, int id, int& bh, int& 
         const int in_round = min(a.cu_group, total - round * a.cu_group);
         const int e = round * a.cu_group + ((round & 1) ? in_round - 1 - c : c);   // place in the longest-first list
         qb = a.nqb - 1 - e / heads;
-        bh = (e % heads) * groups + xcd;
+        bh = a.xcd_map == 2 ? (e % heads) * groups + xcd : xcd * heads + e % heads;
     } else {
-        bh = (local / a.nqb) * groups + xcd;
+        bh = a.xcd_map == 2 ? (local / a.nqb) * groups + xcd : xcd * heads + local / a.nqb;
         qb = local % a.nqb;
     }
 }
 
 // host side: a.nqb set; fills xcd_map and cu_group
 inline void set_tile_order(FaArgs& a) {
-    a.xcd_map = (((int64_t)a.B * a.H) % 8 == 0) ? 1 : 0;
+    // (MHIP_FA_HEADS=2: the heads dealt round-robin over the XCDs instead of in contiguous eighths)
+    a.xcd_map = (((int64_t)a.B * a.H) % 8 == 0) ? (tune_int("MHIP_FA_HEADS", 1) == 2 ? 2 : 1) : 0;
     a.cu_group = a.xcd_map ? compute_units() / 8 : compute_units();
     if (a.cu_group < 1) a.cu_group = 1;
 }
