@@ -454,9 +454,16 @@ static int launch_column_split(hipStream_t s, const GemmArgs& g, int64_t batch, 
     if (g.residual) r.residual = static_cast<const T*>(g.residual) + n_wide;
     r.c = static_cast<T*>(g.c) + n_wide;
     if (!gemm256_eligible(w, 1, dt) || !gemm256_eligible(r, 1, dt, 128, /*any_tile_count=*/true)) return -1;
-    const int st = launch_gemm256(s, w, 1, TA, TB, dt);
+    // The band first (MHIP_GEMM_SPLIT=3: last): what the wide tiles store at their common end is
+    // then the freshest content of the L2s when the next kernel starts at column 0.
+    if (tune_int("MHIP_GEMM_SPLIT", 1) == 3) {
+        const int st = launch_gemm256(s, w, 1, TA, TB, dt);
+        if (st != MHIP_OK) return st;
+        return launch_gemm256(s, r, 1, TA, TB, dt, 128);
+    }
+    const int st = launch_gemm256(s, r, 1, TA, TB, dt, 128);
     if (st != MHIP_OK) return st;
-    return launch_gemm256(s, r, 1, TA, TB, dt, 128);
+    return launch_gemm256(s, w, 1, TA, TB, dt);
 }
 
 // Which kernel serves a 16-bit problem (MHIP_GEMM_TILE = 128 | 256 | 2560 | 2561 | 2562 | 2563 forces one):

@@ -67,7 +67,9 @@ __global__ __launch_bounds__(256) void embed_kernel(const int32_t* __restrict__ 
                                                     const P* __restrict__ wpe,
                                                     O* __restrict__ out, int64_t S, int64_t d,
                                                     int64_t vocab, int vec4) {
-    const int64_t tok = blockIdx.x;  // over B*S
+    // over B*S; with a grid that is a multiple of 8, XCD x (workgroup ids x, x + 8, ...) takes the
+    // x-th eighth of the tokens: the rows a following row kernel or GEMM handles on that XCD
+    const int64_t tok = gridDim.x % 8 == 0 ? (int64_t)(blockIdx.x % 8u) * (gridDim.x / 8u) + blockIdx.x / 8u : blockIdx.x;
     int64_t id = ids[tok];
     id = id < 0 ? 0 : (id > vocab - 1 ? vocab - 1 : id);
     const P* te = wte + id * d;
