@@ -132,7 +132,7 @@ __device__ __forceinline__ float acc_value(float in_agpr) {
 
 // Epilogue of one tile: bias, activation, conversion, then through LDS (the ring, free after the
 // loop's last barrier) so that every store instruction writes whole 16-byte chunks of C rows.
-template <typename T, int BW>
+template <typename T, int BW, bool STREAM_C = false>
 __device__ __forceinline__ void store_tile(f32x16 (&acc)[BW / 16], char* smem, const GemmArgs& g, T* c, const T* res,
                                   int m0, int n0) {
     constexpr int WN = BW / 2;            // columns per wave
@@ -222,8 +222,13 @@ __device__ __forceinline__ void store_tile(f32x16 (&acc)[BW / 16], char* smem, c
 #pragma unroll
         for (int u = 0; u < kPB; u++) {
             // (rows at any even byte when N is no multiple of 8: see below)
-            if (rows_aligned) *reinterpret_cast<u32x4*>(cw) = w[u];
-            else *reinterpret_cast<u32x4_unaligned*>(cw) = w[u];
+            if constexpr (STREAM_C) {
+                if (rows_aligned) __builtin_nontemporal_store(w[u], reinterpret_cast<u32x4*>(cw));
+                else __builtin_nontemporal_store(w[u], reinterpret_cast<u32x4_unaligned*>(cw));
+            } else {
+                if (rows_aligned) *reinterpret_cast<u32x4*>(cw) = w[u];
+                else *reinterpret_cast<u32x4_unaligned*>(cw) = w[u];
+            }
             cw += step;
         }
     };
@@ -334,7 +339,9 @@ __global__ __launch_bounds__(256) void gemm256_kernel(GemmArgs g) {
     main_loop<T, TA, TB, BW>(acc, ra, rb, misc, rsa, rsb, LA::pass_stride(g.lda), LB::pass_stride(g.ldb),
                              LA::stage_stride(g.lda), LB::stage_stride(g.ldb), m0b, (uint32_t)(g.K / 32));
 
-    store_tile<T, BW>(acc, smem, g, c, res, m0, n0);
+    // (a compile-time variant: the same branch inside the epilogue upsets the compiler)
+    if (g.stream_c) store_tile<T, BW, true>(acc, smem, g, c, res, m0, n0);
+    else store_tile<T, BW, false>(acc, smem, g, c, res, m0, n0);
 }
 
 // ---- streamed tiles ------------------------------------------------------------------------------
@@ -516,6 +523,12 @@ int launch256(hipStream_t s, GemmArgs g, int64_t batch) {
                     hipGetErrorString(attr_err));
     g.tiles_m = (g.M + 255) / 256;
     g.tiles_n = (g.N + BW - 1) / BW;
+    // A result of more than 256 MB passes through the L2s (32 MB) and the memory-side cache once and
+    // is gone before anything reads it; stored the ordinary way it evicts the operands on its way.
+    const int stream_mode = tune_int("MHIP_GEMM_STREAM_C", 1);                     // 2 = never, 3 = always
+    // (only rows on 16-byte boundaries: with N = 50257 the hint cost 55 us where with 50304 it gains 50)
+    g.stream_c = stream_mode == 3 || ((int64_t)g.M * g.N * batch * 2 > (256ll << 20) && stream_mode != 2 &&
+                                      (g.ldc ? g.ldc : g.N) % 8 == 0);
     hipLaunchKernelGGL(kern, dim3((unsigned)(g.tiles_m * g.tiles_n), (unsigned)batch), dim3(256),
                        kSmem, s, g);
     return check_launch("gemm256");

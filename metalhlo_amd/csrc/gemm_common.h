@@ -24,6 +24,7 @@ struct GemmArgs {
     int tiles_m, tiles_n;
     const void* residual = nullptr;   // C's layout and batch stride; added after the activation (may alias c)
     int ldc = 0;                      // row stride of C and the residual in elements; 0 = N (gemm256.hip only: a column slice of a wider C)
+    int stream_c = 0;                 // gemm256.hip: C is far larger than the L2s, store it with the streaming hint
 };
 
 template <typename T> struct Mfma32;

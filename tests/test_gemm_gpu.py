@@ -348,6 +348,27 @@ def test_gemm_split_is_the_default_from_a_third_round_on(lib, monkeypatch):
         assert torch.equal(c, kernels.matmul(a, b, None, "gelu"))
 
 
+def test_gemm_streaming_stores_of_a_large_result(monkeypatch):
+    """A result of more than 256 MB is stored with the streaming hint; forced here on small
+    problems (both tile widths, aligned and odd N, with a residual): the same bits, nothing
+    written outside C."""
+    from metalhlo_amd import kernels
+    rng = np.random.default_rng(68)
+    for (M, N, K, tile, tb) in [(4096, 4096, 256, "2560", False), (8192, 768, 512, "2561", False), (2048, 6145, 128, "2560", True)]:
+        a, b = _ab(M, N, K, torch.bfloat16, 69, False, tb)
+        bias = to_dev(rng.standard_normal(N) * 0.5, torch.bfloat16)
+        res = to_dev(rng.standard_normal((M, N)), torch.bfloat16)
+        monkeypatch.setenv("MHIP_GEMM_TILE", tile)
+        for r in (None, res):
+            monkeypatch.setenv("MHIP_GEMM_STREAM_C", "2")
+            plain = kernels.matmul(a, b, bias, "gelu", trans_b=tb, residual=r)
+            monkeypatch.setenv("MHIP_GEMM_STREAM_C", "3")
+            guard = torch.full((M * N + 4096,), 7.0, dtype=torch.bfloat16, device="cuda")
+            c = kernels.matmul(a, b, bias, "gelu", trans_b=tb, residual=r, out=guard[2048:2048 + M * N].view(M, N))
+            assert torch.all(guard[:2048] == 7.0) and torch.all(guard[2048 + M * N:] == 7.0)
+            assert torch.equal(c, plain), (M, N, K, tile)
+
+
 def test_gemm_large_exact_small_integers():
     """Integer-valued operands with exactly representable partial sums: bit-exact."""
     from metalhlo_amd import kernels
