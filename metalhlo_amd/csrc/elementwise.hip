@@ -407,9 +407,31 @@ extern "C" int mhip_strided_copy(void* stream, const void* x, void* y, int rank,
     }
     if (n == 0) return MHIP_OK;
     if (!x || !y) return fail(MHIP_ERR_INVALID_ARGUMENT, "%s: NULL pointer", what);
+    hipStream_t s = as_stream(stream);
+    // Whole 16-byte groups: when the innermost axis is contiguous in the source and everything
+    // else (its length, the other strides, the offset, both pointers) is a multiple of V = 16 /
+    // elem_size elements, the copy is the same copy of 16-byte elements with that axis V times
+    // shorter -- a broadcast, a slice of rows or a transpose of outer axes then moves 16 bytes per
+    // lane and does its index arithmetic once per group ([8,1024,768] f32 broadcast: 20 -> 7 us).
+    if (rank >= 1 && (elem_size == 1 || elem_size == 2 || elem_size == 4 || elem_size == 8)) {
+        const int64_t V = 16 / elem_size;
+        bool ok = in_strides[rank - 1] == 1 && out_shape[rank - 1] % V == 0 && in_offset % V == 0 &&
+                  ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15) == 0;
+        for (int d = 0; ok && d < rank - 1; d++) ok = in_strides[d] % V == 0;
+        if (ok) {
+            StridedArgs v = a;
+            v.out_shape[rank - 1] /= V;
+            for (int d = 0; d < rank - 1; d++) v.in_stride[d] /= V;
+            v.in_offset /= V;
+            const int64_t nv = n / V;
+            unsigned gridv;
+            if (ew_grid(nv, &gridv)) return MHIP_ERR_UNSUPPORTED;
+            hipLaunchKernelGGL((strided_copy_kernel<u32x4>), dim3(gridv), dim3(256), 0, s, (const u32x4*)x, (u32x4*)y, nv, v);
+            return check_launch(what);
+        }
+    }
     unsigned grid;
     if (ew_grid(n, &grid)) return MHIP_ERR_UNSUPPORTED;
-    hipStream_t s = as_stream(stream);
 #define MHIP_SC(W) hipLaunchKernelGGL((strided_copy_kernel<W>), dim3(grid), dim3(256), 0, s, (const W*)x, (W*)y, n, a)
     switch (elem_size) {
         case 1: MHIP_SC(uint8_t); break;
