@@ -630,9 +630,12 @@ static void launch_split(const RowLaunch& c, hipStream_t s, const T* xp, const T
     const int rpb = 4 / WPR * (c.r == 2 ? 2 : 1);
     const int64_t units = (rows + rpb - 1) / rpb;
     if (c.ordered) {
-        // a tensor small enough to sit in the L2s between two kernels: rows by XCD (see the kernel)
-        const bool by_xcd = units % 8 == 0 && (int64_t)rows * cols * (int64_t)sizeof(T) <= (16 << 20) &&
-                            tune_int("MHIP_ROW_XCD", 1) != 2;      // 2 = off
+        // a tensor small enough to sit in the L2s between two kernels: rows by XCD (see the kernel).
+        // Not for large ones: eight separate windows of memory in flight instead of one cost the
+        // [32768, 4096] benchmarks 4 to 17 % (softmax 0.80 -> 0.71 of the HBM peak, RMSNorm 0.79 -> 0.65).
+        const int xcd_mode = tune_int("MHIP_ROW_XCD", 1);          // 2 = never, 3 = whatever the size
+        const bool by_xcd = units % 8 == 0 && xcd_mode != 2 &&
+                            (xcd_mode == 3 || (int64_t)rows * cols * (int64_t)sizeof(T) <= (16 << 20));
         const int chunk = by_xcd ? -1 : 1;
         if (c.r == 2)
             hipLaunchKernelGGL((row_split_kernel<T, OP, NVS, WPR, 2>), dim3((unsigned)units), dim3(256), 0, s, xp, gp, bp, yp,
