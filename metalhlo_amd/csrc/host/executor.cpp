@@ -163,7 +163,8 @@ static const std::map<std::string, int> kActivation = {{"none", MHIP_ACT_NONE}, 
                                                        {"swish", MHIP_ACT_SILU}, {"gelu_exact", MHIP_ACT_GELU_ERF}};
 // custom_call targets served by a kernel (Compiler/CustomCallHandlers.swift:75-89)
 static const char* kTargets[] = {"fused_scaled_dot_product_attention", "fused_layer_norm", "fused_rms_norm",
-                                 "fused_softmax", "fused_gelu", "fused_matmul_bias_activation", "fused_ffn"};
+                                 "fused_softmax", "fused_gelu", "fused_matmul_bias_activation", "fused_ffn",
+                                 "fused_token_embedding"};
 
 static std::string where(const Op& op) { return "line " + std::to_string(op.line) + " (stablehlo." + op.name + "): "; }
 
@@ -388,6 +389,19 @@ static std::vector<int64_t> dot_result_shape(const Op& op, const TensorType& lt,
 static void check_custom_call_types(const Op& op, const std::vector<TensorType>& vt) {
     auto in = [&](size_t i) -> const TensorType& { return vt[op.operands.at(i)]; };
     const int dt = op.out.dtype;
+    if (op.target == "fused_token_embedding") {
+        // ids [B, S] i32, table [vocab, d] f32, positions [P, d] f32 -> [B, S, d]; token (b, s)
+        // gets table[ids[b, s]] + positions[first_position + s]
+        const TensorType &ids = in(0), &table = in(1), &pos = in(2);
+        const int64_t p0 = parse_config(op.backend_config).get_int("first_position", 0);
+        if (ids.dtype != I32 || ids.shape.size() != 2 || table.dtype != F32 || table.shape.size() != 2 || table.shape[0] < 1 ||
+            pos.dtype != F32 || pos.shape.size() != 2 || pos.shape[1] != table.shape[1])
+            throw ParseError(where(op) + "expected ids [B, S] i32, table [vocab, d] f32 and positions [P, d] f32");
+        if (p0 < 0 || p0 + ids.shape[1] > pos.shape[0]) throw ParseError(where(op) + "positions outside their table");
+        if (op.out.shape != std::vector<int64_t>{ids.shape[0], ids.shape[1], table.shape[1]})
+            throw ParseError(where(op) + "the result shape is not [B, S, d]");
+        return;
+    }
     for (size_t i = 0; i < op.operands.size(); i++)
         if (in(i).dtype != dt) throw ParseError(where(op) + "every operand must have the result's element type");
     const Config cfg = parse_config(op.backend_config);
@@ -533,11 +547,13 @@ void compile(Executable& exe) {
             bool ok = false;
             for (auto t : kTargets) ok |= op.target == t;
             if (!ok) throw UnsupportedOp(where(op) + "Unsupported custom call target: " + op.target);
-            const size_t need = op.target == "fused_scaled_dot_product_attention" || op.target == "fused_layer_norm" || op.target == "fused_ffn" ? 3
+            const size_t need = op.target == "fused_scaled_dot_product_attention" || op.target == "fused_layer_norm" || op.target == "fused_ffn" ||
+                                        op.target == "fused_token_embedding" ? 3
                               : op.target == "fused_rms_norm" || op.target == "fused_matmul_bias_activation" ? 2 : 1;
             if (op.operands.size() < need)
                 throw ParseError(where(op) + "Invalid input count: expected " + std::to_string(need) + ", got " + std::to_string(op.operands.size()));
-            if (!is_kernel_float(in(0).dtype)) throw UnsupportedOp(where(op) + "element type not supported");
+            if (!is_kernel_float(op.target == "fused_token_embedding" ? op.out.dtype : in(0).dtype))
+                throw UnsupportedOp(where(op) + "element type not supported");
             if (op.target == "fused_matmul_bias_activation" &&
                 !kActivation.count(parse_config(op.backend_config).get_string("activation", "none")))
                 throw UnsupportedOp(where(op) + "unknown activation");
@@ -701,7 +717,12 @@ static std::vector<DeviceTensor> run_ops(Executable& exe, const std::vector<Devi
                 const TensorType& xt = in(0).type;
                 const int64_t cols = xt.shape.empty() ? 1 : xt.shape.back();
                 const int64_t rows = cols ? xt.numel() / cols : 0;
-                if (op.target == "fused_softmax") {
+                if (op.target == "fused_token_embedding") {
+                    const TensorType &ids = in(0).type, &table = in(1).type;
+                    const int64_t d = table.shape[1], p0 = cfg.get_int("first_position", 0);
+                    RUN(mhip_embed_tokens(s, in(0).data(), in(1).data(), static_cast<const float*>(in(2).data()) + p0 * d, out.data(),
+                                          ids.shape[0], ids.shape[1], d, table.shape[0], MHIP_F32, dt));
+                } else if (op.target == "fused_softmax") {
                     int64_t axis = cfg.get_int("axis", -1);
                     if (axis < 0) axis += (int64_t)xt.shape.size();
                     if (axis < 0 || axis >= (int64_t)xt.shape.size()) throw ExecError(where(op) + "softmax axis out of range");

@@ -199,6 +199,57 @@ struct Rewriter {
         fused++;
     }
 
+    // ------------------------------------------------------------------ token + position embedding
+    // convert(add(gather(table, ids), broadcast_in_dim(positions, dims = [1, 2]))) -- or the add
+    // alone where the program computes in f32: whole rows of an f32 table [vocab, d] picked by
+    // ids [B, S] (i32), plus f32 positions [S, d] repeated over the batch, the positions possibly
+    // rows p0 .. p0+S of a longer table (slice with unit strides over whole rows).  One kernel
+    // reads both rows, adds them in f32 and rounds once, as the three operations in a row do.
+    bool embedding(size_t ri) {
+        const Op& root = fn.ops[ri];
+        std::set<size_t> nodes{ri};
+        const Op* sum = root.name == "add" ? &root : root.name == "convert" ? op_named(root.operands[0], "add") : nullptr;
+        if (!sum || sum->out.dtype != F32 || sum->out.shape.size() != 3 || !fused_float(root.out.dtype) || root.out.shape != sum->out.shape)
+            return false;
+        nodes.insert(index_of(sum));
+        const int64_t B = sum->out.shape[0], S = sum->out.shape[1], d = sum->out.shape[2];
+        if (B < 1 || S < 1 || d < 1) return false;
+        for (int k = 0; k < 2; k++) {
+            const Op* g = op_named(sum->operands[k], "gather");
+            const Op* b = op_named(sum->operands[1 - k], "broadcast_in_dim");
+            if (!g || !b || g->operands.size() != 2) continue;
+            const TensorType &tt = type.at(g->operands[0]), &it = type.at(g->operands[1]);
+            // the whole-row form of gather, indices without a trailing unit dim
+            if (tt.dtype != F32 || tt.shape.size() != 2 || tt.shape[1] != d || tt.shape[0] < 1 || it.dtype != I32 ||
+                it.shape != std::vector<int64_t>{B, S} || g->dims != std::vector<int64_t>{0} ||
+                g->starts != std::vector<int64_t>{0} || g->limits != std::vector<int64_t>{1, d} || !g->lhs_batch.empty() ||
+                !g->rhs_batch.empty() || g->iota_dim != 2 || g->strides != std::vector<int64_t>{2})
+                continue;
+            int pos = b->operands[0];
+            const TensorType& pt = type.at(pos);
+            if (b->dims != std::vector<int64_t>{1, 2} || pt.dtype != F32 || pt.shape != std::vector<int64_t>{S, d}) continue;
+            std::set<size_t> all = nodes;
+            all.insert(index_of(g));
+            all.insert(index_of(b));
+            int64_t p0 = 0;
+            if (const Op* sl = op_named(pos, "slice")) {
+                const TensorType& st = type.at(sl->operands[0]);
+                if (st.dtype == F32 && st.shape.size() == 2 && st.shape[1] == d && sl->strides == std::vector<int64_t>{1, 1} &&
+                    sl->starts.size() == 2 && sl->limits.size() == 2 && sl->starts[1] == 0 && sl->limits[1] == d &&
+                    sl->starts[0] >= 0 && sl->limits[0] == sl->starts[0] + S && sl->limits[0] <= st.shape[0]) {
+                    p0 = sl->starts[0];
+                    pos = sl->operands[0];
+                    all.insert(index_of(sl));
+                }
+            }
+            if (!closed(all, ri)) continue;
+            replace(ri, all, "fused_token_embedding", {g->operands[1], g->operands[0], pos},
+                    "{\"first_position\": " + std::to_string(p0) + "}");
+            return true;
+        }
+        return false;
+    }
+
     // ------------------------------------------------------------------ softmax
     // divide(e, bcast(reduce_add(e))), e = exp(subtract(x, bcast(reduce_max(x))))
     bool softmax(size_t ri) {
@@ -910,6 +961,8 @@ int fuse_patterns(Function& fn, const std::set<std::string>* disabled) {
     run("matmul-bias-act-fusion", [&](size_t i) { rw.matmul_bias_act(i); });
     run("transpose-folding", [&](size_t i) { rw.attention_views(i); });
     run("residual-chain-fusion", [&](size_t i) { rw.matmul_residual(i); });
+    // no counterpart among the reference's passes: the lookup at the head of a language model
+    run("embedding-fusion", [&](size_t i) { rw.embedding(i); });
     return rw.fused;
 }
 

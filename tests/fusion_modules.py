@@ -344,3 +344,25 @@ SOFTMAX_IN_CALLEE = """module {
 FFN_CUSTOM_CALL = """func.func @main(%x: tensor<4x32x64xf32>, %up: tensor<64x256xf32>, %down: tensor<256x64xf32>) -> tensor<4x32x64xf32> {
   %r = stablehlo.custom_call @fused_ffn(%x, %up, %down) {backend_config = "{\\"activation\\": \\"ACT\\"}"} : (tensor<4x32x64xf32>, tensor<64x256xf32>, tensor<256x64xf32>) -> tensor<4x32x64xf32>
   return %r : tensor<4x32x64xf32> }"""
+
+
+def embedding(B=2, S=16, d=64, vocab=50, n_pos=24, dtype="bf16", first=0, ids_type="i32", keep_tokens=False, cols=None):
+    """Token gather + positions [first, first+S) of a longer table, repeated over the batch, summed
+    in f32 and (for a 16-bit `dtype`) rounded once.  `keep_tokens` also returns the gathered rows;
+    `cols` slices fewer columns of a wider position table (not whole rows)."""
+    x3f, out_t = f"tensor<{B}x{S}x{d}xf32>", f"tensor<{B}x{S}x{d}x{dtype}>"
+    wp = cols or d
+    res = f"({out_t}, {x3f})" if keep_tokens else out_t
+    L = [f"func.func @main(%ids: tensor<{B}x{S}x{ids_type}>, %wte: tensor<{vocab}x{d}xf32>, %wpe: tensor<{n_pos}x{wp}xf32>) -> {res} {{",
+         f'  %tok = "stablehlo.gather"(%wte, %ids) {{ dimension_numbers = #stablehlo.gather<offset_dims = [2], collapsed_slice_dims = [0], '
+         f'start_index_map = [0], index_vector_dim = 2>, slice_sizes = array<i64: 1, {d}>, indices_are_sorted = false }} '
+         f": (tensor<{vocab}x{d}xf32>, tensor<{B}x{S}x{ids_type}>) -> {x3f}",
+         f"  %pos = stablehlo.slice %wpe [{first}:{first + S}, 0:{d}] : (tensor<{n_pos}x{wp}xf32>) -> tensor<{S}x{d}xf32>",
+         f"  %posb = stablehlo.broadcast_in_dim %pos, dims = [1, 2] : (tensor<{S}x{d}xf32>) -> {x3f}",
+         f"  %emb = stablehlo.add %posb, %tok : {x3f}"]
+    last = "%emb"
+    if dtype != "f32":
+        L.append(f"  %h = stablehlo.convert %emb : ({x3f}) -> {out_t}")
+        last = "%h"
+    L.append(f"  return {last}, %tok : {out_t}, {x3f} }}" if keep_tokens else f"  return {last} : {out_t} }}")
+    return "\n".join(L)

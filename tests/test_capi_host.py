@@ -111,6 +111,13 @@ def test_error_codes(lib, client):
       %0 = stablehlo.custom_call @fused_layer_norm(%a) {backend_config = "{}"} : (tensor<4x8xf32>) -> tensor<4x8xf32>
       return %0 : tensor<4x8xf32> }"""
     assert lib.mhlo_compile(client, few.encode(), C.byref(exe)) == 3 and b"expected 3, got 1" in lib.mhlo_get_last_error()
+    emb = """func.func @main(%i: tensor<2x8xi32>, %t: tensor<10x16xf32>, %p: tensor<12x16xf32>) -> tensor<2x8x16xbf16> {
+      %0 = stablehlo.custom_call @fused_token_embedding(%i, %t, %p) {backend_config = "{\\"first_position\\": FIRST}"} : (tensor<2x8xi32>, tensor<10x16xf32>, tensor<12x16xf32>) -> tensor<2x8x16xbf16>
+      return %0 : tensor<2x8x16xbf16> }"""
+    assert lib.mhlo_compile(client, emb.replace("FIRST", "4").encode(), C.byref(exe)) == 0
+    lib.mhlo_executable_destroy(exe)
+    assert lib.mhlo_compile(client, emb.replace("FIRST", "5").encode(), C.byref(exe)) == 3 and b"positions outside" in lib.mhlo_get_last_error()
+    assert lib.mhlo_compile(client, emb.replace("FIRST", "0").replace("2x8xi32", "2x8xi64").encode(), C.byref(exe)) == 3
     # without a device: buffers and execution report NO_DEVICE, nothing crashes
     buf = C.c_void_p()
     shape = (C.c_int64 * 1)(4)

@@ -182,3 +182,24 @@ def test_fused_ffn(sess, act):
     sess.lib.mhlo_executable_destroy(exe)
     h = oracle.ACTIVATIONS[act](oracle.gemm(x.astype(np.float64).reshape(-1, 64), up.astype(np.float64)))
     close(got, oracle.gemm(h, down.astype(np.float64)).reshape(x.shape), 2e-5)
+
+
+@pytest.mark.parametrize("dtype,first,d", [("bf16", 0, 64), ("bf16", 5, 48), ("f32", 3, 64), ("f16", 0, 30)])
+def test_token_embedding(sess, dtype, first, d):
+    """The embedding head as one kernel and as written give the same bits (one fp32 sum, one
+    rounding), ids outside the table clamped as gather clamps them; both equal
+    table[ids] + positions[first + s] rounded to the result type."""
+    B, S, vocab, n_pos = 3, 16, 50, 24
+    rng = np.random.default_rng(97)
+    ids = rng.integers(0, vocab, (B, S)).astype(np.int32)
+    ids[0, 0], ids[1, 3], ids[2, 15] = -7, vocab, vocab + 1000
+    wte = rng.standard_normal((vocab, d)).astype(np.float32)
+    wpe = rng.standard_normal((n_pos, d)).astype(np.float32)
+    text = M.embedding(B, S, d, vocab, n_pos, dtype, first)
+    a, b = both(sess, text, [(ids, "i32"), (wte, "f32"), (wpe, "f32")], "fused_token_embedding")
+    assert np.array_equal(a, b)
+    exp = wte[np.clip(ids, 0, vocab - 1)] + wpe[None, first:first + S]          # fp32 sum
+    if dtype == "bf16":
+        assert np.array_equal(a, oracle.bf16_round_bits(exp))
+    else:
+        assert np.array_equal(np.asarray(a, dtype=np.float32), exp.astype({"f32": np.float32, "f16": np.float16}[dtype]).astype(np.float32))

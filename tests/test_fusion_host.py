@@ -317,3 +317,19 @@ def test_environment_switches_of_the_front_end(sess, tmp_path, capfd):
     assert "[*] softmax-fusion ops: 9 -> 1" in err and "[ ] norm-fusion ops: 1 -> 1" in err
     text = dump.read_text()
     assert text.startswith("// optimized IR -- 1 ops") and "fused_softmax inputs=[%0]" in text and '"axis": 1' in text
+
+
+def test_token_and_position_embedding_is_one_call(sess):
+    """gather of whole table rows + a slice of the position table spread over the batch + the
+    rounding: one kernel; the positions' first row travels in the configuration.  Left alone when
+    the ids are i64, the gathered rows are a result too, or the slice cuts rows of the table."""
+    assert ops(sess, M.embedding()) == ["fused_token_embedding"]
+    assert ops(sess, M.embedding(dtype="f32", first=3)) == ["fused_token_embedding"]
+    assert len(ops(sess, M.embedding(), 0)) == 5
+    assert "fused_token_embedding" not in ops(sess, M.embedding(ids_type="i64"))
+    assert "fused_token_embedding" not in ops(sess, M.embedding(keep_tokens=True))
+    got = ops(sess, M.embedding(cols=80))
+    assert got == ["slice", "fused_token_embedding"]          # the cut rows are made first, then used whole
+    from metalhlo_amd import programs
+    head = ops(sess, programs.gpt2_program(2, 64, 1, 4, 64, 1024, 1000, 128, "bf16"))
+    assert head.count("fused_token_embedding") == 1 and "gather" not in head
