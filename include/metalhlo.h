@@ -190,8 +190,9 @@ char* mhlo_ext_executable_ops(MHLOExecutableRef executable);
 /* Extension, not part of the reference's header: the memory plan and launch statistics of an
  * executable, "key=value" pairs separated by commas: planned (0/1), arena_bytes (one arena
  * holds every intermediate; lifetimes that do not overlap share bytes), slots, unshared_bytes
- * (what one allocation per intermediate would take), result_bytes, graph_captures,
- * graph_replays, eager_runs.  The plan plays the part of the reference's StaticMemoryPlanner
+ * (what one allocation per intermediate would take), result_bytes, overlaps (pairs of slots
+ * alive together whose bytes intersect; 0 in a sound plan), graph_captures, graph_replays,
+ * eager_runs.  The plan plays the part of the reference's StaticMemoryPlanner
  * (Sources/MetalHLOCore/Memory/StaticMemoryPlanner.swift:144-250).  Returns a malloc'd
  * string; release with mhlo_free_string. */
 char* mhlo_ext_executable_plan(MHLOExecutableRef executable);

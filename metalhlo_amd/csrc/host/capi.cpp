@@ -379,15 +379,22 @@ char* mhlo_ext_executable_ops(MHLOExecutableRef executable) {
 // Extension (not in the reference's header): the memory plan and launch statistics of an
 // executable as "key=value" pairs separated by commas: arena_bytes (the planned arena for
 // intermediates), slots, unshared_bytes (one allocation per intermediate would take this),
-// result_bytes, graph_captures, graph_replays, eager_runs.  Caller frees with mhlo_free_string.
+// result_bytes, overlaps (pairs of slots alive at the same time whose bytes intersect: 0 in a
+// sound plan), graph_captures, graph_replays, eager_runs.  Caller frees with mhlo_free_string.
 char* mhlo_ext_executable_plan(MHLOExecutableRef executable) {
     if (!executable) { set_error(MHLO_ERROR_INVALID_ARGUMENT, "executable is null"); return nullptr; }
     Executable* exe = static_cast<Executable*>(executable);
     std::lock_guard<std::mutex> lk(exe->run_mu);
     const ArenaPlan& p = exe->plan;
+    size_t overlaps = 0;
+    for (size_t i = 0; i < p.slots.size(); i++)
+        for (size_t j = i + 1; j < p.slots.size(); j++) {
+            const ArenaPlan::Slot &a = p.slots[i], &b = p.slots[j];
+            overlaps += a.begin <= b.end && b.begin <= a.end && a.offset < b.offset + b.bytes && b.offset < a.offset + a.bytes;
+        }
     std::string out = "planned=" + std::to_string(p.valid ? 1 : 0) + ",arena_bytes=" + std::to_string(p.core_bytes) +
                       ",slots=" + std::to_string(p.slots.size()) + ",unshared_bytes=" + std::to_string(p.sum_bytes) +
-                      ",result_bytes=" + std::to_string(p.full_bytes - p.core_bytes) +
+                      ",result_bytes=" + std::to_string(p.full_bytes - p.core_bytes) + ",overlaps=" + std::to_string(overlaps) +
                       ",graph_captures=" + std::to_string(exe->graph_captures) +
                       ",graph_replays=" + std::to_string(exe->graph_replays) + ",eager_runs=" + std::to_string(exe->eager_runs);
     return strdup(out.c_str());

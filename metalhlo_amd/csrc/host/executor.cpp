@@ -144,6 +144,62 @@ static size_t place_slots(ArenaPlan& plan, bool escaping, size_t floor) {
     return top;
 }
 
+// The same slots placed in the order the execution allocates them, each in the block of its own
+// size that was released last (else the smallest larger block, split; else new bytes at the top,
+// after merging free neighbours).  A value then tends to land where its predecessor in the
+// program was read a moment ago, bytes that are still in the caches, instead of at the lowest
+// address that happens to be free.  May need more bytes than place_slots; the caller compares.
+static size_t place_slots_recent(ArenaPlan& plan, bool escaping, size_t floor) {
+    struct Event { int time; int slot; bool release; };
+    std::vector<Event> ev;
+    for (int i = 0; i < (int)plan.slots.size(); i++) {
+        if (plan.slots[i].escapes != escaping) continue;
+        ev.push_back({plan.slots[i].begin, i, false});
+        ev.push_back({plan.slots[i].end, i, true});
+    }
+    // a release at the time of an allocation (cannot happen with the recording clock) comes second
+    std::stable_sort(ev.begin(), ev.end(), [](const Event& a, const Event& b) { return a.time != b.time ? a.time < b.time : a.release < b.release; });
+    struct Block { size_t offset, bytes; int released; };
+    std::vector<Block> free_blocks;
+    size_t top = floor;
+    auto merge = [&]() {
+        std::sort(free_blocks.begin(), free_blocks.end(), [](const Block& a, const Block& b) { return a.offset < b.offset; });
+        std::vector<Block> out;
+        for (const Block& b : free_blocks) {
+            if (!out.empty() && out.back().offset + out.back().bytes == b.offset) {
+                out.back().bytes += b.bytes;
+                out.back().released = std::max(out.back().released, b.released);
+            } else out.push_back(b);
+        }
+        if (!out.empty() && out.back().offset + out.back().bytes == top) { top = out.back().offset; out.pop_back(); }
+        free_blocks.swap(out);
+    };
+    auto take = [&](size_t bytes, size_t& offset) {
+        int best = -1;
+        for (int i = 0; i < (int)free_blocks.size(); i++)
+            if (free_blocks[i].bytes == bytes && (best < 0 || free_blocks[i].released > free_blocks[best].released)) best = i;
+        if (best < 0)
+            for (int i = 0; i < (int)free_blocks.size(); i++)
+                if (free_blocks[i].bytes > bytes && (best < 0 || free_blocks[i].bytes < free_blocks[best].bytes)) best = i;
+        if (best < 0) return false;
+        offset = free_blocks[best].offset;
+        if (free_blocks[best].bytes == bytes) free_blocks.erase(free_blocks.begin() + best);
+        else { free_blocks[best].offset += bytes; free_blocks[best].bytes -= bytes; }
+        return true;
+    };
+    size_t high = floor;
+    for (const Event& e : ev) {
+        ArenaPlan::Slot& s = plan.slots[e.slot];
+        if (e.release) { free_blocks.push_back({s.offset, s.bytes, e.time}); continue; }
+        if (!take(s.bytes, s.offset)) {
+            merge();
+            if (!take(s.bytes, s.offset)) { s.offset = top; top += s.bytes; }
+        }
+        high = std::max(high, std::max(top, s.offset + s.bytes));
+    }
+    return high;
+}
+
 // ---------------------------------------------------------------- op tables
 static const std::map<std::string, int> kUnary = {
     {"exponential", MHIP_UN_EXP}, {"tanh", MHIP_UN_TANH}, {"rsqrt", MHIP_UN_RSQRT}, {"sqrt", MHIP_UN_SQRT},
@@ -877,7 +933,18 @@ static void plan_memory(Executable& exe) {
             if (sl.escapes) sl.end = 0x7FFFFFFF;
             else exe.plan.sum_bytes += sl.bytes;
         }
-        exe.plan.core_bytes = place_slots(exe.plan, false, 0);
+        // Both placements are made; the one by recency is kept unless it needs over a quarter more
+        // bytes than the packed one (METALHLO_ARENA_PLACEMENT=packed keeps the packed one regardless).
+        // GPT-2-small forward, B8 S1024: 361 MB against 319 MB, and 0.02-0.03 ms of 3.5 ms faster.
+        const char* how = getenv("METALHLO_ARENA_PLACEMENT");
+        const size_t packed = place_slots(exe.plan, false, 0);
+        exe.plan.core_bytes = packed;
+        if (!how || strcmp(how, "packed")) {
+            const std::vector<ArenaPlan::Slot> keep = exe.plan.slots;
+            const size_t recent = place_slots_recent(exe.plan, false, 0);
+            if (recent <= packed + packed / 4) exe.plan.core_bytes = recent;
+            else exe.plan.slots = keep;
+        }
         exe.plan.full_bytes = place_slots(exe.plan, true, exe.plan.core_bytes);
         exe.plan.valid = true;
     } catch (const std::exception&) {

@@ -100,3 +100,24 @@ def test_unfused_layer_norm_shares_bytes(sess):
     assert p0["arena_bytes"] < p0["unshared_bytes"]
     p2 = plan_of(sess, fm.LAYER_NORM, opt=2)
     assert p2["slots"] == 1 and p2["arena_bytes"] == 0
+
+
+@pytest.mark.parametrize("placement", ["recent", "packed"])
+def test_both_placements_keep_live_slots_apart(sess, placement, monkeypatch):
+    """Slots are placed where a block of their size was released last (bytes still in the caches)
+    unless that takes over a quarter more than packing them at the lowest free address;
+    METALHLO_ARENA_PLACEMENT=packed keeps the packed plan.  Either way no two slots alive at the
+    same time share a byte, on programs with many sizes and lifetimes."""
+    from metalhlo_amd import programs
+    monkeypatch.setenv("METALHLO_ARENA_PLACEMENT", placement)
+    sizes = {}
+    for name, text, opt in [("block", fm.transformer_block(), 2), ("block_as_written", fm.transformer_block(), 0),
+                            ("gpt2", programs.gpt2_program(2, 64, 3, 4, 64, 1024, 1000, 128, "bf16"), 2),
+                            ("attention", fm.attention(with_mask=True), 0)]:
+        p = plan_of(sess, text, opt)
+        assert p["planned"] == 1 and p["overlaps"] == 0, name
+        assert p["arena_bytes"] <= p["unshared_bytes"]
+        sizes[name] = p["arena_bytes"]
+    monkeypatch.setenv("METALHLO_ARENA_PLACEMENT", "packed")
+    for name, text, opt in [("block", fm.transformer_block(), 2), ("gpt2", programs.gpt2_program(2, 64, 3, 4, 64, 1024, 1000, 128, "bf16"), 2)]:
+        assert sizes[name] <= plan_of(sess, text, opt)["arena_bytes"] * 5 // 4
