@@ -222,7 +222,7 @@ def wl_gpt2_capi(torch, kernels, B=8, S=1024):
     return dict(name=f"GPT-2-small forward B{B} S{S} from one plain StableHLO module through mhlo_compile / mhlo_execute "
                      f"(fp32 parameters converted every step, {len(sess.ops(exe))} operations after pattern recognition)",
                 fn=step, flops=GPT2.flops(cfg, B, S), bytes=0.0, bound="mfma", host_timed=True, keep=(sess, bufs),
-                kernel="mhlo_execute (HIP graph replay): batched converts, gather, 12 x 7 fused kernels, LN, logits GEMM")
+                kernel="mhlo_execute (HIP graph replay): batched converts, embedding, 12 x 7 fused kernels, LN, logits GEMM")
 
 
 def measure(wl, steps, warmup, torch, key=None):
