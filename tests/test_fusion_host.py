@@ -333,3 +333,8 @@ def test_token_and_position_embedding_is_one_call(sess):
     from metalhlo_amd import programs
     head = ops(sess, programs.gpt2_program(2, 64, 1, 4, 64, 1024, 1000, 128, "bf16"))
     assert head.count("fused_token_embedding") == 1 and "gather" not in head
+    os.environ["METALHLO_DISABLED_PASSES"] = "embedding-fusion"
+    try:
+        assert ops(sess, M.embedding()) == ["gather", "slice", "broadcast_in_dim", "add", "convert"]
+    finally:
+        del os.environ["METALHLO_DISABLED_PASSES"]
