@@ -36,9 +36,12 @@ sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+PEAK_CLOCK_MHZ = 2400.0     # the shader clock the matrix peak is quoted at
 
 # HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by what the same
 # counter reads for the 'copy' workload (256 MiB in, 256 MiB out); see profiles/<workload>.txt.
+# TRAFFIC_COMMIT: the commit of this repository the counter runs were taken at (the profiles say so too).
+TRAFFIC_COMMIT = "aabac17"
 MEASURED_TRAFFIC = {
     "gemm": 237446022,
     "gemm_f32": 812745437,
@@ -70,27 +73,113 @@ def _ramp(fn, torch):
 
 
 def _time_launches(fn, steps, warmup, torch):
-    """Mean seconds per launch of fn(i) over `steps` launches (HIP events on the
-    current stream), after `warmup` untimed launches."""
+    """Times exactly `steps` launches of fn(i) after `warmup` untimed ones, with HIP events on the
+    current stream: one event in front of the first launch and one behind every launch.  Returns
+    (mean seconds per launch from the first event to the last, host wall seconds per launch,
+    sorted per-launch seconds from consecutive events, (t0, t1) host clock around the timed region)."""
     for i in range(warmup):
         fn(i)
     torch.cuda.synchronize()
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
     t0 = time.perf_counter()
-    start.record()
+    ev[0].record()
     for i in range(steps):
         fn(i)
-    stop.record()
+        ev[i + 1].record()
     torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    return start.elapsed_time(stop) * 1e-3 / steps, wall / steps
+    t1 = time.perf_counter()
+    each = sorted(ev[i].elapsed_time(ev[i + 1]) * 1e-3 for i in range(steps))
+    return ev[0].elapsed_time(ev[steps]) * 1e-3 / steps, (t1 - t0) / steps, each, (t0, t1)
+
+
+class DeviceSampler:
+    """Board power and shader clock from the amdgpu hwmon files of the first card that has them,
+    read by a side thread every millisecond or so while a workload runs.  The controller averages
+    power over milliseconds, so the figures describe the steady state of the loop the sampler runs
+    beside (ramp, warm-up and timed launches of one kernel), not a single launch."""
+
+    def __init__(self):
+        import glob
+        self.power = self.cap = self.freq = self.dpm = None
+        for d in sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*")):
+            for name in ("power1_average", "power1_input"):
+                if self.power is None and os.path.exists(os.path.join(d, name)):
+                    self.power = os.path.join(d, name)
+            if self.power and self.power.startswith(d):
+                if os.path.exists(os.path.join(d, "power1_cap")):
+                    self.cap = os.path.join(d, "power1_cap")
+                if os.path.exists(os.path.join(d, "freq1_input")):
+                    self.freq = os.path.join(d, "freq1_input")
+                else:       # the level table of the shader clock; the current level carries a star
+                    dpm = os.path.join(os.path.dirname(os.path.dirname(d)), "pp_dpm_sclk")
+                    self.dpm = dpm if os.path.exists(dpm) else None
+                break
+        self.samples = []
+        self._stop = None
+
+    @staticmethod
+    def _read(path):
+        try:
+            with open(path) as f:
+                return float(f.read().strip())
+        except (OSError, ValueError):
+            return None
+
+    def _clock_hz(self):
+        if self.freq:
+            return self._read(self.freq)
+        if self.dpm:
+            try:
+                with open(self.dpm) as f:
+                    for line in f:
+                        if "*" in line:
+                            return float(line.split(":")[1].strip().split("Mhz")[0]) * 1e6
+            except (OSError, ValueError, IndexError):
+                return None
+        return None
+
+    def available(self):
+        return self.power is not None and self._read(self.power) is not None
+
+    def start(self):
+        import threading
+        self.samples = []
+        self._stop = threading.Event()
+
+        def loop():
+            while not self._stop.is_set():
+                w = self._read(self.power)
+                f = self._clock_hz()
+                self.samples.append((time.perf_counter(), w, f))
+                time.sleep(0.001)
+        self._th = threading.Thread(target=loop, daemon=True)
+        self._th.start()
+
+    def stop(self, since=None):
+        """Mean power (W) and clock (MHz) of the samples taken after host time `since`."""
+        self._stop.set()
+        self._th.join()
+        sel = [s for s in self.samples if since is None or s[0] >= since] or self.samples[-3:]
+        ws = [s[1] for s in sel if s[1] is not None]
+        fs = [s[2] for s in sel if s[2] is not None]
+        cap = self._read(self.cap) if self.cap else None
+        return dict(power_w=round(sum(ws) / len(ws) / 1e6, 1) if ws else None,
+                    power_cap_w=round(cap / 1e6, 1) if cap else None,
+                    clock_mhz=round(sum(fs) / len(fs) / 1e6) if fs else None, samples=len(sel))
 
 
 # ---------------------------------------------------------------- workloads
+def _rng_dev(torch, draw, dtype):
+    """A host array drawn from numpy's generator (the seeds and distributions of the benchmark
+    configurations) -> device tensor of `dtype`, rounded to nearest even."""
+    return torch.from_numpy(draw).to("cuda").to(dtype)
+
+
 def wl_gemm(torch, kernels, M=4096, N=4096, K=4096):
-    g = torch.Generator(device="cuda").manual_seed(2)
-    a = (torch.rand(M, K, generator=g, device="cuda") * 2 - 1).to(torch.bfloat16)
-    b = (torch.rand(K, N, generator=g, device="cuda") * 2 - 1).to(torch.bfloat16)
+    import numpy as np
+    rng = np.random.default_rng(2)
+    a = _rng_dev(torch, rng.uniform(-1, 1, (M, K)).astype(np.float32), torch.bfloat16)
+    b = _rng_dev(torch, rng.uniform(-1, 1, (K, N)).astype(np.float32), torch.bfloat16)
     c = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
     return dict(name=f"bf16 GEMM {M}x{N}x{K} (row-major A[M,K], B[K,N]; fp32 accumulate, bf16 out)",
                 fn=lambda i: kernels.matmul(a, b, out=c), flops=2.0 * M * N * K,
@@ -101,9 +190,10 @@ PEAK_F32_TFLOPS = 157.3    # MI355X dense fp32 MFMA
 
 
 def wl_gemm_f32(torch, kernels, M=4096, N=4096, K=4096):
-    g = torch.Generator(device="cuda").manual_seed(2)
-    a = torch.rand(M, K, generator=g, device="cuda") * 2 - 1
-    b = torch.rand(K, N, generator=g, device="cuda") * 2 - 1
+    import numpy as np
+    rng = np.random.default_rng(2)
+    a = _rng_dev(torch, rng.uniform(-1, 1, (M, K)).astype(np.float32), torch.float32)
+    b = _rng_dev(torch, rng.uniform(-1, 1, (K, N)).astype(np.float32), torch.float32)
     c = torch.empty(M, N, dtype=torch.float32, device="cuda")
     return dict(name=f"fp32 GEMM {M}x{N}x{K} (row-major A[M,K], B[K,N]; fp32 operands and accumulate on the fp32 matrix instruction)",
                 fn=lambda i: kernels.matmul(a, b, out=c), flops=2.0 * M * N * K, bytes=4.0 * (M * K + K * N + M * N),
@@ -111,9 +201,10 @@ def wl_gemm_f32(torch, kernels, M=4096, N=4096, K=4096):
 
 
 def wl_attention(torch, kernels, B=4, H=32, S=4096, D=128, causal=True, fp32=False):
-    g = torch.Generator(device="cuda").manual_seed(4)
+    import numpy as np
+    rng = np.random.default_rng(4)
     dt = torch.float32 if fp32 else torch.bfloat16
-    q, k, v = (torch.randn(B, H, S, D, generator=g, device="cuda").to(dt) for _ in range(3))
+    q, k, v = (_rng_dev(torch, rng.standard_normal((B, H, S, D), dtype=np.float32), dt) for _ in range(3))
     flops = 4.0 * B * H * S * S * D * (0.5 if causal else 1.0)
     r = dict(name=f"{'fp32' if fp32 else 'bf16'} flash-attention fwd B{B} H{H} S{S} D{D} {'causal' if causal else 'full'}",
              fn=lambda i: kernels.flash_attention(q, k, v, is_causal=causal), flops=flops,
@@ -126,11 +217,13 @@ def wl_attention(torch, kernels, B=4, H=32, S=4096, D=128, causal=True, fp32=Fal
 def _rows(torch, rows=32768, cols=4096, nbuf=3):
     # several input sets, visited round-robin, so that a launch cannot find its
     # input still resident in the 256 MB last-level cache from the previous one
-    g = torch.Generator(device="cuda").manual_seed(3)
-    xs = [torch.randn(rows, cols, generator=g, device="cuda").to(torch.bfloat16) for _ in range(nbuf)]
-    gam = (1 + 0.1 * torch.randn(cols, generator=g, device="cuda")).to(torch.bfloat16)
-    bet = (0.1 * torch.randn(cols, generator=g, device="cuda")).to(torch.bfloat16)
-    bias = (0.02 * torch.randn(cols, generator=g, device="cuda")).to(torch.bfloat16)
+    import numpy as np
+    rng = np.random.default_rng(3)
+    bf = torch.bfloat16
+    xs = [_rng_dev(torch, rng.standard_normal((rows, cols), dtype=np.float32), bf) for _ in range(nbuf)]
+    gam = _rng_dev(torch, (1 + 0.1 * rng.standard_normal(cols)).astype(np.float32), bf)
+    bet = _rng_dev(torch, (0.1 * rng.standard_normal(cols)).astype(np.float32), bf)
+    bias = _rng_dev(torch, (0.02 * rng.standard_normal(cols)).astype(np.float32), bf)
     return xs, gam, bet, bias
 
 
@@ -178,8 +271,8 @@ def wl_gpt2(torch, kernels, B=8, S=1024):
     from metalhlo_amd.gpt2 import GPT2, GPT2Config, init_params
     cfg = GPT2Config()
     model = GPT2(cfg, init_params(cfg, seed=5))
-    g = torch.Generator(device="cuda").manual_seed(5)
-    ids = torch.randint(0, cfg.vocab, (B, S), generator=g, device="cuda", dtype=torch.int32)
+    import numpy as np
+    ids = torch.from_numpy(np.random.default_rng(5).integers(0, cfg.vocab, (B, S)).astype(np.int32)).cuda()
     graphed = model.capture(ids)     # one HIP graph replay per step instead of ~135 host launches
     return dict(name=f"GPT-2-small forward B{B} S{S}, bf16 compute / fp32 params (converted every step), HIP graph replay",
                 fn=lambda i: graphed(ids), flops=GPT2.flops(cfg, B, S), bytes=0.0, bound="mfma",
@@ -226,23 +319,43 @@ def wl_gpt2_capi(torch, kernels, B=8, S=1024):
 
 
 def measure(wl, steps, warmup, torch, key=None):
+    sampler = DeviceSampler() if wl["bound"] == "mfma" else None
+    if sampler is not None and sampler.available():
+        sampler.start()
+    else:
+        sampler = None
+    t_begin = time.perf_counter()
     _ramp(wl["fn"], torch)
-    sec, wall = _time_launches(wl["fn"], steps, warmup, torch)
+    sec, wall, each, (t0, t1) = _time_launches(wl["fn"], steps, warmup, torch)
+    # power and clock: the samples of the second half of ramp + warm-up + timed launches (one kernel
+    # throughout, so the steady state the timed launches run in)
+    dev = sampler.stop(since=t_begin + 0.5 * (t1 - t_begin)) if sampler else None
     if wl.get("host_timed"):        # the calls are synchronous and run on the library's own stream
         sec = wall
+    med, low = each[len(each) // 2], each[0]
     if wl["bound"] == "mfma":
         ach = wl["flops"] / sec / 1e12
         peak = wl.get("peak", PEAK_BF16_TFLOPS)
         roof = dict(bound="mfma", achieved=round(ach, 2), peak=peak, unit="TFLOP/s",
                     frac=round(ach / peak, 4), traffic=MEASURED_TRAFFIC.get(key))
+        if dev:
+            roof.update(power_w=dev["power_w"], power_cap_w=dev["power_cap_w"], clock_mhz=dev["clock_mhz"],
+                        device_samples=dev["samples"])
+            if dev["clock_mhz"]:
+                # what the same cycles would give at the 2400 MHz the peak figure is quoted for
+                roof["frac_at_clock"] = round(ach / peak * PEAK_CLOCK_MHZ / dev["clock_mhz"], 4)
         value, unit = ach, "TFLOP/s"
     else:
         ach = wl["bytes"] / sec / 1e9
         roof = dict(bound="hbm", achieved=round(ach, 1), peak=PEAK_HBM_GBS, unit="GB/s",
                     frac=round(ach / PEAK_HBM_GBS, 4), traffic=MEASURED_TRAFFIC.get(key))
         value, unit = ach, "GB/s"
-    return dict(workload=wl["name"], kernel=wl["kernel"], value=round(value, 2), unit=unit,
-                us_per_launch=round(sec * 1e6, 2), wall_us_per_launch=round(wall * 1e6, 2), roofline=roof)
+    roof["traffic_commit"] = TRAFFIC_COMMIT if MEASURED_TRAFFIC.get(key) else None
+    r = dict(workload=wl["name"], kernel=wl["kernel"], value=round(value, 2), unit=unit,
+             us_per_launch=round(sec * 1e6, 2), wall_us_per_launch=round(wall * 1e6, 2), roofline=roof)
+    if not wl.get("host_timed"):
+        r.update(median_us=round(med * 1e6, 2), min_us=round(low * 1e6, 2))
+    return r
 
 
 # ---------------------------------------------------------------- shader clock under load
@@ -257,18 +370,26 @@ def clock_probe(torch, kernels, seconds=2.0):
     import threading
 
     def sample(stop, out):
+        # fallback where the hwmon files are not readable: the command-line tool, a few samples a second
         while not stop.is_set():
-            r = subprocess.run(["/opt/rocm/bin/rocm-smi", "--showclocks"], capture_output=True, text=True)
+            r = subprocess.run(["/opt/rocm/bin/rocm-smi", "--showclocks", "--showpower"], capture_output=True, text=True)
             m = re.search(r"sclk clock level: \d+: \((\d+)Mhz\)", r.stdout)
+            w = re.search(r"Power \(W\): ([0-9.]+)", r.stdout)
             if m:
-                out.append(int(m.group(1)))
+                out.append((int(m.group(1)), float(w.group(1)) if w else None))
             time.sleep(0.2)
 
     def run(fn):
-        stop, mhz = threading.Event(), []
-        th = threading.Thread(target=sample, args=(stop, mhz))
-        th.start()
+        hw = DeviceSampler()
+        stop, smi = threading.Event(), []
+        if hw.available():
+            hw.start()
+            th = None
+        else:
+            th = threading.Thread(target=sample, args=(stop, smi))
+            th.start()
         t0 = time.time()
+        t_half = time.perf_counter() + seconds / 2
         while time.time() - t0 < seconds:
             for _ in range(20):
                 fn()
@@ -279,10 +400,18 @@ def clock_probe(torch, kernels, seconds=2.0):
             fn()
         e1.record()
         torch.cuda.synchronize()
-        stop.set()
-        th.join()
-        tail = mhz[len(mhz) // 2:] or [0]
-        return dict(us_per_launch=round(e0.elapsed_time(e1) / 20 * 1e3, 1), sclk_mhz=round(sum(tail) / len(tail)))
+        out = dict(us_per_launch=round(e0.elapsed_time(e1) / 20 * 1e3, 1))
+        if th is None:
+            d = hw.stop(since=t_half)
+            out.update(sclk_mhz=d["clock_mhz"], power_w=d["power_w"], power_cap_w=d["power_cap_w"], source="hwmon")
+        else:
+            stop.set()
+            th.join()
+            tail = smi[len(smi) // 2:] or [(0, None)]
+            ws = [w for _, w in tail if w is not None]
+            out.update(sclk_mhz=round(sum(c for c, _ in tail) / len(tail)),
+                       power_w=round(sum(ws) / len(ws), 1) if ws else None, source="rocm-smi")
+        return out
 
     res = {}
     M = 4096

@@ -22,6 +22,12 @@
 extern "C" {
 #endif
 
+/* Everything declared here is the library's public surface: the library itself is built with
+ * hidden visibility, and only these names (and the two mhlo_ext_* extensions) are exported. */
+#if defined(__GNUC__)
+#pragma GCC visibility push(default)
+#endif
+
 /* metalhlo.h:23 — static string, never freed. */
 const char* mhlo_version(void);
 
@@ -196,6 +202,19 @@ char* mhlo_ext_executable_ops(MHLOExecutableRef executable);
  * (Sources/MetalHLOCore/Memory/StaticMemoryPlanner.swift:144-250).  Returns a malloc'd
  * string; release with mhlo_free_string. */
 char* mhlo_ext_executable_plan(MHLOExecutableRef executable);
+
+/* Extension: per-operation device time of the last profiled execution (mhlo_execute_with_profile
+ * profiles the execution it makes; METALHLO_PROFILE_GPU=1 profiles every execution and also prints
+ * the lines to stderr): one "<operation> <result shape> <microseconds>" line per operation in
+ * program order, measured with HIP events around the operation's launches on an eager run.  The
+ * counterpart of the reference's METALHLO_PROFILE_GPU / METALHLO_DEBUG_DISPATCH output
+ * (Runtime/MetalExecutor.swift:289-316, IntegratedExecutor.swift:411-478).  Returns a malloc'd
+ * string (empty when nothing was profiled); release with mhlo_free_string. */
+char* mhlo_ext_executable_profile(MHLOExecutableRef executable);
+
+#if defined(__GNUC__)
+#pragma GCC visibility pop
+#endif
 
 #ifdef __cplusplus
 }

@@ -310,6 +310,11 @@ int mhip_gemm_autotune(void* stream, const void* a, const void* b, const void* b
                        int64_t stride_b, int64_t stride_c, int trans_a, int trans_b, int activation,
                        int dtype, int iters, int* out_variant, float* out_us);
 
+/* The kernel variant (codes above; 0 = none of them: fp32, integer, f64 or unaligned operands) that
+ * the calling thread's most recent mhip_gemm / mhip_gemm_residual call launched.  The tuner's
+ * effect and the heuristic's choice can be observed with it. */
+int mhip_gemm_last_variant(void);
+
 /* Row operators (op 0 softmax, 1 LayerNorm, 2 RMSNorm; arguments as for the operator itself).
  * Searched: one wave per row with the parameters in LDS on a persistent grid (resident workgroups
  * per CU 0 = occupancy query, 2, 4, 6, 8) or a row split over the waves of a workgroup (one or two

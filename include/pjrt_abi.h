@@ -471,6 +471,10 @@ typedef struct PJRT_Api {
 } PJRT_Api;
 
 /* The one exported symbol (PJRTApi.swift:170-173): the table lives for the whole process. */
+/* The one exported symbol of the plugin (it is built with hidden visibility). */
+#if defined(__GNUC__)
+__attribute__((visibility("default")))
+#endif
 const PJRT_Api* GetPjrtApi(void);
 
 #ifdef __cplusplus

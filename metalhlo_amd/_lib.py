@@ -52,6 +52,7 @@ SIGNATURES = {
     "mhip_reduce": (_i32, [_vp, _i32, _vp, _vp, _i64, _i64, _i64, C.c_double, _i32]),
     "mhip_fill": (_i32, [_vp, _vp, _i64, C.c_uint64, _i32]),
     "mhip_argmax": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32]),
+    "mhip_gemm_last_variant": (_i32, []),
     "mhip_gemm_autotune": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _i32,
                                   _i32, _i32, C.POINTER(C.c_int), C.POINTER(C.c_float)]),
     "mhip_row_autotune": (_i32, [_vp, _i32, _vp, _vp, _vp, _vp, _i64, _i64, C.c_float, _i32, _i32, C.POINTER(C.c_int),

@@ -42,6 +42,11 @@ def hipcc() -> str:
     return "hipcc"
 
 
+def _exports(lib: str) -> str:
+    """Linker option that limits a library's dynamic symbols to its C-ABI (csrc/exports/<lib>.map)."""
+    return "-Wl,--version-script=" + os.path.join(CSRC, "exports", lib + ".map")
+
+
 def generate_sources(verbose: bool = True) -> None:
     """Regenerates the hand-scheduled loops included by gemm256.hip and attention_pipe.hip."""
     for script, target in (("gen_gemm256_loop.py", "gemm256_loop.inc"), ("gen_fa_loop.py", "fa_loop.inc")):
@@ -76,7 +81,7 @@ def build_kernels(verbose: bool = True) -> str:
         list(ex.map(one, zip(srcs, objs)))
     out = os.path.join(LIBDIR, "libmetalhlo_hip.so")
     # (-z defs: a kernel whose host-side launch stub was not emitted must fail here, not at load time)
-    _run([hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-Wl,-z,defs", "-o", out, *objs])
+    _run([hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-Wl,-z,defs", _exports("libmetalhlo_hip"), "-o", out, *objs])
     if verbose:
         print("  link ", os.path.relpath(out, ROOT), flush=True)
     return out
@@ -92,9 +97,9 @@ def build_host(verbose: bool = True) -> list:
     if not srcs:
         return outs
     out = os.path.join(LIBDIR, "libCMetalHLO.so")
-    _run([hipcc(), "-x", "c++", "-O2", "-std=c++17", "-fPIC", "-D__HIP_PLATFORM_AMD__", "-Wall",
+    _run([hipcc(), "-x", "c++", "-O2", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-D__HIP_PLATFORM_AMD__", "-Wall",
           "-I", os.path.join(ROOT, "include"), "-I", "/opt/rocm/include", *srcs,
-          "-shared", "-o", out, "-L", LIBDIR, "-lmetalhlo_hip", "-L", "/opt/rocm/lib", "-lamdhip64",
+          "-shared", _exports("libCMetalHLO"), "-o", out, "-L", LIBDIR, "-lmetalhlo_hip", "-L", "/opt/rocm/lib", "-lamdhip64",
           "-Wl,-rpath,$ORIGIN", "-Wl,-rpath,/opt/rocm/lib"])
     if verbose:
         print("  link ", os.path.relpath(out, ROOT), flush=True)
@@ -103,10 +108,10 @@ def build_host(verbose: bool = True) -> list:
     pjrt = os.path.join(CSRC, "pjrt", "pjrt.cpp")
     if os.path.exists(pjrt):
         out = os.path.join(LIBDIR, "libPJRTMetalHLO.so")
-        _run([hipcc(), "-x", "c++", "-O2", "-std=c++17", "-fPIC", "-D__HIP_PLATFORM_AMD__", "-Wall",
+        _run([hipcc(), "-x", "c++", "-O2", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-D__HIP_PLATFORM_AMD__", "-Wall",
               "-I", os.path.join(ROOT, "include"), "-I", "/opt/rocm/include", pjrt,
               *[f for f in srcs if os.path.basename(f) != "capi.cpp"],
-              "-shared", "-o", out, "-L", LIBDIR, "-lmetalhlo_hip", "-L", "/opt/rocm/lib", "-lamdhip64",
+              "-shared", _exports("libPJRTMetalHLO"), "-o", out, "-L", LIBDIR, "-lmetalhlo_hip", "-L", "/opt/rocm/lib", "-lamdhip64",
               "-Wl,-rpath,$ORIGIN", "-Wl,-rpath,/opt/rocm/lib"])
         if verbose:
             print("  link ", os.path.relpath(out, ROOT), flush=True)

@@ -68,6 +68,7 @@ SIGNATURES = {
     "mhlo_free_string": (None, [_vp]),
     "mhlo_ext_executable_ops": (_vp, [_vp]),     # extension: op list after pattern recognition
     "mhlo_ext_executable_plan": (_vp, [_vp]),    # extension: memory plan and launch statistics
+    "mhlo_ext_executable_profile": (_vp, [_vp]), # extension: per-operation device time of the last profiled execution
 }
 
 _lib = None
@@ -137,6 +138,19 @@ class Session:
             return {k: int(v) for k, v in (kv.split("=") for kv in C.string_at(p).decode().split(","))} if p else {}
         finally:
             self.lib.mhlo_free_string(p)
+
+    def profile(self, exe) -> list:
+        """(operation, result shape, microseconds) of the last profiled execution."""
+        p = self.lib.mhlo_ext_executable_profile(exe)
+        try:
+            lines = C.string_at(p).decode().splitlines() if p else []
+        finally:
+            self.lib.mhlo_free_string(p)
+        out = []
+        for ln in lines:
+            name, shape, us = ln.rsplit(" ", 2)
+            out.append((name, shape, float(us)))
+        return out
 
     def buffer(self, array: np.ndarray, element_type: str):
         a = np.ascontiguousarray(array)

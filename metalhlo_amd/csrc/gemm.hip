@@ -398,9 +398,9 @@ static int launch_mfma(hipStream_t s, GemmArgs g, int64_t batch) {
 }
 
 // gemm256.hip: 4-wave 256x256 kernel with a hand-scheduled main loop.
-bool gemm256_eligible(const GemmArgs& g, int64_t batch, int dtype, int bw = 256, bool any_tile_count = false);
+bool gemm256_eligible(const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype, int bw = 256, bool any_tile_count = false);
 int launch_gemm256(hipStream_t s, const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype, int bw = 256);
-bool gemm_stream_eligible(const GemmArgs& g, int64_t batch, int trans_a, int dtype);
+bool gemm_stream_eligible(const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype);
 int launch_gemm_stream(hipStream_t s, const GemmArgs& g, int trans_b, int dtype);
 // gemm_f32.hip: fp32 operands on the fp32 matrix instruction, 128x128 tiles.
 bool gemm_f32_mfma_wanted(const GemmArgs& g);
@@ -453,7 +453,7 @@ static int launch_column_split(hipStream_t s, const GemmArgs& g, int64_t batch, 
     if (g.bias) r.bias = static_cast<const T*>(g.bias) + n_wide;
     if (g.residual) r.residual = static_cast<const T*>(g.residual) + n_wide;
     r.c = static_cast<T*>(g.c) + n_wide;
-    if (!gemm256_eligible(w, 1, dt) || !gemm256_eligible(r, 1, dt, 128, /*any_tile_count=*/true)) return -1;
+    if (!gemm256_eligible(w, 1, TA, TB, dt) || !gemm256_eligible(r, 1, TA, TB, dt, 128, /*any_tile_count=*/true)) return -1;
     // The band first (MHIP_GEMM_SPLIT=3: last): what the wide tiles store at their common end is
     // then the freshest content of the L2s when the next kernel starts at column 0.
     if (tune_int("MHIP_GEMM_SPLIT", 1) == 3) {
@@ -485,6 +485,10 @@ static int launch_column_split(hipStream_t s, const GemmArgs& g, int64_t batch, 
 //     rows of C are not 16-byte aligned (odd N): its eight waves hide the narrow stores;
 //   * otherwise 128x128 tiles, two workgroups per CU (short K, few tiles).
 // An entry of the tuning table (mhip_gemm_autotune) for the problem overrides the heuristic.
+// The kernel the last mhip_gemm / mhip_gemm_residual call of this thread chose (mhip_gemm_last_variant).
+static thread_local int g_last_variant = 0;
+static inline int chose(int variant, int status) { g_last_variant = variant; return status; }
+
 template <typename T, bool TA, bool TB>
 static int pick_tile(hipStream_t s, const GemmArgs& g, int64_t batch) {
     const int64_t tiles_m = (g.M + 255) / 256;
@@ -493,22 +497,22 @@ static int pick_tile(hipStream_t s, const GemmArgs& g, int64_t batch) {
     int force = tune_int("MHIP_GEMM_TILE", 0);
     if (force == 0) force = tuned_gemm_variant(g, batch, TA, TB, dt);   // tuning table / running tuner
     if (force == 2562) {
-        if (gemm_stream_eligible(g, batch, TA, dt)) return launch_gemm_stream(s, g, TB, dt);
+        if (gemm_stream_eligible(g, batch, TA, TB, dt)) return chose(2562, launch_gemm_stream(s, g, TB, dt));
     }
     if (force == 2561) {
-        if (gemm256_eligible(g, batch, dt, 128)) return launch_gemm256(s, g, batch, TA, TB, dt, 128);
+        if (gemm256_eligible(g, batch, TA, TB, dt, 128)) return chose(2561, launch_gemm256(s, g, batch, TA, TB, dt, 128));
     }
     if (force == 2560) {
-        if (gemm256_eligible(g, batch, dt)) return launch_gemm256(s, g, batch, TA, TB, dt);
+        if (gemm256_eligible(g, batch, TA, TB, dt)) return chose(2560, launch_gemm256(s, g, batch, TA, TB, dt));
     }
     if (force == 2563 || (force == 0 && g.K >= 512 && tune_int("MHIP_GEMM_SPLIT", 1) != 2)) {    // 2 = off
         const int st = launch_column_split<T, TA, TB>(s, g, batch, dt, force == 2563);
-        if (st >= 0) return st;
+        if (st >= 0) return chose(2563, st);
     }
     if (force == 0 && g.K >= 512) {
         constexpr int cus = 256;                       // compute units of the device this is written for
         const int64_t narrow = tiles_m * ((g.N + 127) / 128) * batch, stages = g.K / 32;
-        const bool wide_ok = gemm256_eligible(g, batch, dt), narrow_ok = gemm256_eligible(g, batch, dt, 128);
+        const bool wide_ok = gemm256_eligible(g, batch, TA, TB, dt), narrow_ok = gemm256_eligible(g, batch, TA, TB, dt, 128);
         // (The streamed form of the narrow tile, 2562, is no longer chosen here: it is 5 % ahead of
         // wide tiles on a few shapes when the operands sit in the L2 -- [4096,8320] x K 1024 77 against
         // 81 us, [8192,4608] x K 768 67 against 71 -- and 10 to 15 % behind on the same shapes when
@@ -516,19 +520,19 @@ static int pick_tile(hipStream_t s, const GemmArgs& g, int64_t batch) {
         // model finds them; [8192,3584] x K 768: 58 / 66 us streamed, 48 / 53 on wide tiles.  The tuner
         // still times it and records it where it wins; MHIP_GEMM_STREAM=1 restores the old choice.)
         if (!TB && (narrow + cus - 1) / cus <= 4 && tune_int("MHIP_GEMM_STREAM", 2) == 1 &&
-            gemm_stream_eligible(g, batch, TA, dt)) {
+            gemm_stream_eligible(g, batch, TA, TB, dt)) {
             const double stream_us = (double)((narrow + cus - 1) / cus) * (stages * 0.3875 + 3.8) + 5.0;
             const double wide_us = (double)((big + cus - 1) / cus) * (stages * 0.6625 + 13.8);
-            if (!wide_ok || stream_us < wide_us) return launch_gemm_stream(s, g, TB, dt);
+            if (!wide_ok || stream_us < wide_us) return chose(2562, launch_gemm_stream(s, g, TB, dt));
         }
         const int64_t wide_cost = ((big + cus - 1) / cus) * (stages * 32 + 700);
         const int64_t narrow_cost = ((narrow + cus - 1) / cus) * (stages * 18 + 500);
-        if (narrow_ok && (!wide_ok || narrow_cost < wide_cost)) return launch_gemm256(s, g, batch, TA, TB, dt, 128);
-        if (wide_ok) return launch_gemm256(s, g, batch, TA, TB, dt);
+        if (narrow_ok && (!wide_ok || narrow_cost < wide_cost)) return chose(2561, launch_gemm256(s, g, batch, TA, TB, dt, 128));
+        if (wide_ok) return chose(2560, launch_gemm256(s, g, batch, TA, TB, dt));
     }
     const bool want256 = force == 256 || (force != 128 && big >= 192 && (g.K >= 1024 || g.N % 8 != 0));
-    if (want256) return launch_mfma<T, 256, 256, 2, 4, TA, TB>(s, g, batch);
-    return launch_mfma<T, 128, 128, 2, 2, TA, TB>(s, g, batch);
+    if (want256) return chose(256, launch_mfma<T, 256, 256, 2, 4, TA, TB>(s, g, batch));
+    return chose(128, launch_mfma<T, 128, 128, 2, 2, TA, TB>(s, g, batch));
 }
 
 template <typename T>
@@ -575,6 +579,7 @@ static int gemm_entry(void* stream, const void* a, const void* b, const void* bi
     if (M > 0x7FFFFFFF || N > 0x7FFFFFFF || K > 0x7FFFFFFF)
         return fail(MHIP_ERR_UNSUPPORTED, "mhip_gemm: dimension exceeds 2^31-1");
     hipStream_t s = as_stream(stream);
+    g_last_variant = 0;
     GemmArgs g;
     g.a = a; g.b = b; g.bias = bias; g.c = c;
     g.M = (int)M; g.N = (int)N; g.K = (int)K;
@@ -616,6 +621,8 @@ extern "C" int mhip_gemm(void* stream, const void* a, const void* b, const void*
     return gemm_entry(stream, a, b, bias, nullptr, c, M, N, K, batch, stride_a, stride_b, stride_c, trans_a, trans_b,
                       activation, dtype);
 }
+
+extern "C" int mhip_gemm_last_variant(void) { return g_last_variant; }
 
 extern "C" int mhip_gemm_residual(void* stream, const void* a, const void* b, const void* bias,
                                   const void* residual, void* c, int64_t M, int64_t N, int64_t K,

@@ -549,15 +549,16 @@ int layout256(hipStream_t s, const GemmArgs& g, int64_t batch, int ta, int tb) {
 // they are then stored with unaligned 16-byte accesses), operands small enough for
 // 32-bit byte offsets including the prefetch overrun of five K stages, and enough
 // tiles (256 x `bw`) to occupy the device.
-bool gemm256_eligible(const GemmArgs& g, int64_t batch, int dtype, int bw, bool any_tile_count) {
+bool gemm256_eligible(const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype, int bw, bool any_tile_count) {
     if (dtype != MHIP_BF16 && dtype != MHIP_F16) return false;
     if (g.K % 32 != 0 || g.K < 32) return false;
     if ((reinterpret_cast<uintptr_t>(g.c) & 15) != 0 || (batch > 1 && g.sc % 8 != 0)) return false;
     if (g.residual && (reinterpret_cast<uintptr_t>(g.residual) & 15) != 0) return false;
     if (g.bias && (reinterpret_cast<uintptr_t>(g.bias) & 7) != 0) return false;
-    // (an upper bound of the extents whichever way the operands are stored; a column slice keeps
-    // the row stride of the whole matrix)
-    const int64_t a_bytes = (int64_t)(g.M > g.K ? g.M : g.K) * g.lda * 2, b_bytes = (int64_t)(g.N > g.K ? g.N : g.K) * g.ldb * 2;
+    // (the extents the kernel puts into its buffer descriptors: the last stored row ends the operand;
+    // a column slice keeps the row stride of the whole matrix)
+    const int64_t a_bytes = ((int64_t)((trans_a ? g.K : g.M) - 1) * g.lda + (trans_a ? g.M : g.K)) * 2;
+    const int64_t b_bytes = ((int64_t)((trans_b ? g.N : g.K) - 1) * g.ldb + (trans_b ? g.K : g.N)) * 2;
     if (a_bytes >= 0x70000000LL || b_bytes >= 0x70000000LL) return false;
     const int64_t tiles = (int64_t)((g.M + 255) / 256) * ((g.N + bw - 1) / bw) * batch;
     return (tiles >= 192 || any_tile_count) && tiles <= 0x7FFFFFFF && batch <= 65535;
@@ -575,8 +576,8 @@ int launch_gemm256(hipStream_t s, const GemmArgs& g, int64_t batch, int trans_a,
 
 // Streamed tiles (persistent workgroups, stores inside the next tile's loop): see gemm_stream_kernel.
 // Worth it from the second round on, i.e. with more tiles than compute units.
-bool gemm_stream_eligible(const GemmArgs& g, int64_t batch, int trans_a, int dtype) {
-    if (!gemm256_eligible(g, batch, dtype, 128, false)) return false;
+bool gemm_stream_eligible(const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype) {
+    if (!gemm256_eligible(g, batch, trans_a, trans_b, dtype, 128, false)) return false;
     if (trans_a || batch != 1 || g.residual) return false;
     if (g.M % 256 != 0 || g.N % 128 != 0 || g.K < 640 || g.ldc != 0) return false;
     if ((int64_t)g.M * g.N * 2 >= 0xFFFFFFFFLL) return false;          // 32-bit byte offsets into C

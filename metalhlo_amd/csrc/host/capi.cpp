@@ -268,6 +268,7 @@ static MHLOStatusCode make_buffer(MHLOClientRef client, const void* data, size_t
         DeviceTensor d = c->allocate(t);
         if (init && t.bytes()) {
             // explicit host -> device copy on the client's stream (the reference relies on unified memory)
+            std::lock_guard<std::mutex> stream_lock(c->stream_mu);      // not into another thread's graph capture
             if (hipMemcpyAsync(d.data(), data, t.bytes(), hipMemcpyHostToDevice, c->stream) != hipSuccess ||
                 hipStreamSynchronize(c->stream) != hipSuccess) {
                 (void)hipGetLastError();
@@ -322,6 +323,7 @@ MHLOStatusCode mhlo_buffer_to_host(MHLOBufferRef buffer, void* out_data, size_t 
                                                           std::to_string(data_size));
     clear_error();
     if (need == 0) return MHLO_OK;
+    std::lock_guard<std::mutex> stream_lock(h->client->stream_mu);      // not into another thread's graph capture
     if (hipMemcpyAsync(out_data, h->t.data(), need, hipMemcpyDeviceToHost, h->client->stream) != hipSuccess ||
         hipStreamSynchronize(h->client->stream) != hipSuccess) {
         (void)hipGetLastError();
@@ -345,6 +347,8 @@ MHLOStatusCode mhlo_execute_with_profile(MHLOExecutableRef executable, const MHL
                                          MHLOBufferRef* out_outputs, int32_t* out_num_outputs,
                                          MHLOExecutionProfile* out_profile) {
     double enc = 0, gpu = 0, total = 0;
+    // this execution is timed operation by operation (mhlo_ext_executable_profile returns the list)
+    if (executable) static_cast<Executable*>(executable)->profile_next = true;
     MHLOStatusCode st = run(executable, inputs, num_inputs, out_outputs, out_num_outputs, &enc, &gpu, &total);
     if (st == MHLO_OK && out_profile) {
         out_profile->partition_count = 1;
@@ -397,6 +401,25 @@ char* mhlo_ext_executable_plan(MHLOExecutableRef executable) {
                       ",result_bytes=" + std::to_string(p.full_bytes - p.core_bytes) + ",overlaps=" + std::to_string(overlaps) +
                       ",graph_captures=" + std::to_string(exe->graph_captures) +
                       ",graph_replays=" + std::to_string(exe->graph_replays) + ",eager_runs=" + std::to_string(exe->eager_runs);
+    return strdup(out.c_str());
+}
+
+// Extension: the device time of every operation of the last profiled execution (the one made by
+// mhlo_execute_with_profile, or any execution under METALHLO_PROFILE_GPU=1), one
+// "<operation> <result shape> <microseconds>" line per launch group in program order.  The reference
+// prints the same breakdown from METALHLO_PROFILE_GPU / METALHLO_DEBUG_DISPATCH
+// (Runtime/MetalExecutor.swift:289-316, Runtime/IntegratedExecutor.swift:411-478).  Empty string when
+// no execution was profiled.  Caller frees with mhlo_free_string.
+char* mhlo_ext_executable_profile(MHLOExecutableRef executable) {
+    if (!executable) { set_error(MHLO_ERROR_INVALID_ARGUMENT, "executable is null"); return nullptr; }
+    Executable* exe = static_cast<Executable*>(executable);
+    std::lock_guard<std::mutex> lk(exe->run_mu);
+    std::string out;
+    char buf[64];
+    for (auto& t : exe->last_profile) {
+        snprintf(buf, sizeof buf, " %.1f\n", t.us);
+        out += t.name + " " + t.shape + buf;
+    }
     return strdup(out.c_str());
 }
 

@@ -522,6 +522,9 @@ void compile(Executable& exe) {
         if (n == "constant") {
             if (exe.client && exe.client->device >= 0) {
                 DeviceTensor d = exe.client->allocate(op.out);
+                // (the fill goes to the client's stream and the copy waits for it: neither while another
+                // thread captures that stream)
+                std::lock_guard<std::mutex> stream_lock(exe.client->stream_mu);
                 if (op.splat) {
                     if (mhip_fill(exe.client->stream, d.data(), op.out.numel(), op.splat_bits, dtype_bytes(op.out.dtype)) != MHIP_OK)
                         throw ExecError(std::string("constant fill failed: ") + mhip_last_error());
@@ -620,7 +623,10 @@ void compile(Executable& exe) {
             throw UnsupportedOp(where(op) + "operation is outside the supported subset");
         }
     }
-    if (exe.client && exe.client->device >= 0) (void)hipStreamSynchronize(exe.client->stream);
+    if (exe.client && exe.client->device >= 0) {
+        std::lock_guard<std::mutex> stream_lock(exe.client->stream_mu);     // another thread may be capturing the stream
+        (void)hipStreamSynchronize(exe.client->stream);
+    }
     plan_memory(exe);
 }
 
@@ -647,9 +653,23 @@ static DeviceTensor permuted_copy(Allocator& al, bool dry, void* stream, const D
 // the client's stream; with `dry` nothing is launched (the walk only shows `al` which
 // allocations an execution makes and when each is released).  Returns the value of each result.
 #define RUN(call) do { if (!dry) check((call), op); } while (0)
-static std::vector<DeviceTensor> run_ops(Executable& exe, const std::vector<DeviceTensor>& inputs, Allocator& al, bool dry) {
+// `marks` (optional): one HIP event is recorded on the stream in front of the first launch and one
+// behind every operation; marks[i].first = index of the operation the event closes (-1: the start).
+static std::vector<DeviceTensor> run_ops(Executable& exe, const std::vector<DeviceTensor>& inputs, Allocator& al, bool dry,
+                                         std::vector<std::pair<int, hipEvent_t>>* marks = nullptr) {
     const Function& fn = exe.fn;
     void* s = exe.client ? exe.client->stream : nullptr;
+    auto mark = [&](int op_index) {
+        if (!marks || dry) return;
+        hipEvent_t e = nullptr;
+        if (hipEventCreate(&e) != hipSuccess || hipEventRecord(e, static_cast<hipStream_t>(s)) != hipSuccess) {
+            (void)hipGetLastError();
+            if (e) (void)hipEventDestroy(e);
+            return;
+        }
+        marks->emplace_back(op_index, e);
+    };
+    mark(-1);
     std::vector<DeviceTensor> val(fn.num_values);
     for (size_t i = 0; i < inputs.size(); i++) val[fn.arg_ids[i]] = inputs[i];
     // last use of every value, so that intermediates return to the pool early
@@ -673,6 +693,7 @@ static std::vector<DeviceTensor> run_ops(Executable& exe, const std::vector<Devi
         }
         const Op& op = fn.ops[0];
         RUN(mhip_convert_batch(s, (int)xs.size(), xs.data(), ys.data(), ns.data(), F32, op.out.dtype));
+        mark((int)exe.batched_converts - 1);
     }
     for (size_t oi = exe.batched_converts; oi < fn.ops.size(); oi++) {
         const Op& op = fn.ops[oi];
@@ -903,6 +924,7 @@ static std::vector<DeviceTensor> run_ops(Executable& exe, const std::vector<Devi
             }
         }
         val[op.result] = out;
+        if (n != "constant" && n != "reshape") mark((int)oi);
         for (int v : op.operands)
             if (last[v] == (int)oi) val[v] = DeviceTensor();
     }
@@ -997,7 +1019,7 @@ static bool capture_graph(Executable& exe, const std::vector<DeviceTensor>& inpu
             presets[i] = m;
         }
     }
-    std::lock_guard<std::mutex> stream_lock(c.stream_mu);       // no other thread enqueues on the stream meanwhile
+    // the caller (execute) holds c.stream_mu: no other thread enqueues on the stream meanwhile
     if (hipStreamBeginCapture(c.stream, hipStreamCaptureModeThreadLocal) != hipSuccess) {
         (void)hipGetLastError();
         return false;
@@ -1055,40 +1077,63 @@ std::vector<DeviceTensor> execute(Executable& exe, const std::vector<DeviceTenso
     // from roughly twenty launches per execution on, so short programs stay eager by default
     size_t launches = 0;
     for (auto& op : fn.ops) launches += op.name != "constant" && op.name != "reshape";
-    const bool want_graph = use_arena && env_flag("METALHLO_HIP_GRAPH", exe.opt_level >= 3 && launches >= 16);
+    const bool profile_env = env_flag("METALHLO_PROFILE_GPU", false);
+    const bool profile = profile_env || exe.profile_next;          // a profiled execution is eager: events between the launches
+    exe.profile_next = false;
+    const bool want_graph = !profile && use_arena && env_flag("METALHLO_HIP_GRAPH", exe.opt_level >= 3 && launches >= 16);
+    std::vector<std::pair<int, hipEvent_t>> marks;
     std::unique_lock<std::mutex> run_lock(exe.run_mu, std::defer_lock);
     if (use_arena) run_lock.lock();          // the arena belongs to one execution at a time
     const auto t0 = std::chrono::steady_clock::now();
     std::vector<DeviceTensor> rets;
     bool replayed = false;
+    // Every call that touches the client's stream happens under its lock, from here to the end of the
+    // copy-out: the synchronisation in front of a new arena, eager launches, the capture, graph
+    // launches and the synchronisations.  Another thread that executes another program on this
+    // client (or a PJRT transfer) can then never launch into, or wait for, a stream that is being
+    // captured, where its work would be recorded into the graph instead of run.
+    std::unique_lock<std::mutex> stream_lock(c.stream_mu);
     if (use_arena) ensure_arena(exe, want_graph && !direct_results(exe) ? exe.plan.full_bytes : exe.plan.core_bytes);
     // the first execution runs eagerly (kernels set their attributes, tuning tables load); from the
     // second on the op list is one graph per set of input addresses
     if (want_graph && !exe.graph_failed && exe.eager_runs > 0) {
+        // A graph with result buffers of its own can run again only when the caller has released
+        // what its previous replay handed out.  A caller that still holds the results of step n when
+        // it starts step n + 1 (the usual pattern of a training or serving loop) gets a second and a
+        // third graph for the same inputs, each with its own result buffers, and the replays rotate
+        // over whichever is free; with all of them held this execution is eager.
+        constexpr size_t kResultSets = 3;
         Executable::CapturedGraph* hit = nullptr;
+        size_t same_inputs = 0;
         for (auto& g : exe.graphs) {
             bool same = g.inputs.size() == inputs.size();
             for (size_t i = 0; same && i < inputs.size(); i++) same = g.inputs[i] == inputs[i].data();
-            if (same) { hit = &g; break; }
+            if (!same) continue;
+            same_inputs++;
+            bool busy = false;
+            for (auto& r : g.results) busy = busy || r.mem.use_count() > 1;
+            if (!busy) { hit = &g; break; }
         }
-        // a graph with result buffers of its own can run again only when the caller has released
-        // what the previous replay handed out; this execution is eager otherwise
-        bool busy = false;
-        if (hit)
-            for (auto& r : hit->results) busy = busy || r.mem.use_count() > 1;
-        if (busy) hit = nullptr;
-        if (!hit && !busy) {
+        if (!hit && same_inputs < kResultSets) {
             Executable::CapturedGraph g;
             if (capture_graph(exe, inputs, g)) {
                 if (exe.graphs.size() >= 8) {
+                    // the oldest graph whose results the caller does not hold makes room
+                    size_t victim = exe.graphs.size();
+                    for (size_t i = 0; i < exe.graphs.size() && victim == exe.graphs.size(); i++) {
+                        bool busy = false;
+                        for (auto& r : exe.graphs[i].results) busy = busy || r.mem.use_count() > 1;
+                        if (!busy) victim = i;
+                    }
+                    if (victim == exe.graphs.size()) victim = 0;
                     (void)hipStreamSynchronize(c.stream);
-                    (void)hipGraphExecDestroy(exe.graphs.front().exec);
-                    exe.graphs.erase(exe.graphs.begin());
+                    (void)hipGraphExecDestroy(exe.graphs[victim].exec);
+                    exe.graphs.erase(exe.graphs.begin() + victim);
                 }
                 exe.graphs.push_back(std::move(g));
                 hit = &exe.graphs.back();
                 exe.graph_captures++;
-            } else {
+            } else if (same_inputs == 0) {
                 exe.graph_failed = true;     // this program stays on eager launches
             }
         }
@@ -1119,7 +1164,7 @@ std::vector<DeviceTensor> execute(Executable& exe, const std::vector<DeviceTenso
             al.base = static_cast<char*>(exe.arena);
             al.escaping_in_arena = false;
         }
-        rets = run_ops(exe, inputs, al, false);
+        rets = run_ops(exe, inputs, al, false, profile ? &marks : nullptr);
         exe.eager_runs++;
     }
     const auto t1 = std::chrono::steady_clock::now();
@@ -1128,6 +1173,23 @@ std::vector<DeviceTensor> execute(Executable& exe, const std::vector<DeviceTenso
         throw ExecError(std::string("execution failed: ") + hipGetErrorString(e));
     }
     const auto t2 = std::chrono::steady_clock::now();
+    if (profile) {
+        exe.last_profile.clear();
+        for (size_t i = 1; i < marks.size(); i++) {
+            float ms = 0.f;
+            if (hipEventElapsedTime(&ms, marks[i - 1].second, marks[i].second) != hipSuccess) { (void)hipGetLastError(); continue; }
+            const Op& op = fn.ops[marks[i].first];
+            Executable::OpTime t;
+            const bool batch = exe.batched_converts && marks[i].first == (int)exe.batched_converts - 1;
+            t.name = batch ? "convert x" + std::to_string(exe.batched_converts) : (op.name == "custom_call" ? op.target : op.name);
+            for (size_t d = 0; d < op.out.shape.size(); d++) t.shape += (d ? "x" : "") + std::to_string(op.out.shape[d]);
+            t.shape += (t.shape.empty() ? "" : "x") + std::string(dtype_name(op.out.dtype));
+            t.us = ms * 1e3;
+            if (profile_env) fprintf(stderr, "[metalhlo gpu] %3zu %-36s %-24s %9.1f us\n", i - 1, t.name.c_str(), t.shape.c_str(), t.us);
+            exe.last_profile.push_back(std::move(t));
+        }
+        for (auto& m : marks) (void)hipEventDestroy(m.second);
+    }
     if (encode_s) *encode_s = std::chrono::duration<double>(t1 - t0).count();
     if (gpu_s) *gpu_s = std::chrono::duration<double>(t2 - t0).count();
     std::vector<DeviceTensor> outs;

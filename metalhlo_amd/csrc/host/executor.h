@@ -111,6 +111,12 @@ struct Executable {
     std::vector<CapturedGraph> graphs;
     int64_t graph_captures = 0, graph_replays = 0, eager_runs = 0;
     bool graph_failed = false;
+    // Device time of every operation of the last profiled execution (METALHLO_PROFILE_GPU=1 or a call of
+    // mhlo_execute_with_profile): microseconds between the HIP events recorded in front of and
+    // behind the operation's launches on the client's stream.
+    struct OpTime { std::string name; std::string shape; double us = 0; };
+    std::vector<OpTime> last_profile;
+    bool profile_next = false;             // set by mhlo_execute_with_profile for one execution
     ~Executable();
 };
 
@@ -126,6 +132,11 @@ void compile(Executable& exe);
 // more launches; =0 switches it off) captures the op list into a
 // HIP graph on the second execution and replays it while the input addresses stay the same
 // (up to eight address sets are kept); results are then copied out of the arena.
+// Per-dispatch timing (the role of METALHLO_PROFILE_GPU / METALHLO_DEBUG_DISPATCH in the reference,
+// Runtime/MetalExecutor.swift:289-316, Runtime/IntegratedExecutor.swift:411-478): with
+// METALHLO_PROFILE_GPU=1, or for the one execution after exe.profile_next is set, the program runs
+// eagerly with a HIP event pair around every operation; the times land in exe.last_profile and,
+// with the environment variable, one line per operation goes to stderr.
 std::vector<DeviceTensor> execute(Executable& exe, const std::vector<DeviceTensor>& inputs,
                                   double* encode_s, double* gpu_s);
 

@@ -28,6 +28,10 @@ inline int dtype_bytes(int dt) {
         default: return 1;
     }
 }
+inline const char* dtype_name(int dt) {
+    static const char* const names[13] = {"f16", "f32", "f64", "bf16", "i1", "i8", "i16", "i32", "i64", "ui8", "ui16", "ui32", "ui64"};
+    return dt >= 0 && dt < 13 ? names[dt] : "?";
+}
 inline bool dtype_is_float(int dt) { return dt == F16 || dt == F32 || dt == F64 || dt == BF16; }
 
 struct TensorType {

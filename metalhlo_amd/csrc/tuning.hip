@@ -27,8 +27,8 @@
 
 namespace mhip {
 
-bool gemm256_eligible(const GemmArgs& g, int64_t batch, int dtype, int bw = 256, bool any_tile_count = false);
-bool gemm_stream_eligible(const GemmArgs& g, int64_t batch, int trans_a, int dtype);
+bool gemm256_eligible(const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype, int bw = 256, bool any_tile_count = false);
+bool gemm_stream_eligible(const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype);
 bool gemm_split_shape(const GemmArgs& g, int64_t batch, int* n_wide_out);
 
 namespace {
@@ -219,10 +219,10 @@ extern "C" int mhip_gemm_autotune(void* stream, const void* a, const void* b, co
     int best = 0;
     float best_us = 0.f;
     for (int v : candidates) {
-        if (v == 2560 && !gemm256_eligible(g, batch, dtype)) continue;    // validity filter
-        if (v == 2561 && !gemm256_eligible(g, batch, dtype, 128)) continue;
-        if (v == 2562 && !gemm_stream_eligible(g, batch, trans_a, dtype)) continue;
-        if (v == 2563 && !(gemm_split_shape(g, batch, nullptr) && gemm256_eligible(g, batch, dtype))) continue;
+        if (v == 2560 && !gemm256_eligible(g, batch, trans_a, trans_b, dtype)) continue;    // validity filter
+        if (v == 2561 && !gemm256_eligible(g, batch, trans_a, trans_b, dtype, 128)) continue;
+        if (v == 2562 && !gemm_stream_eligible(g, batch, trans_a, trans_b, dtype)) continue;
+        if (v == 2563 && !(gemm_split_shape(g, batch, nullptr) && gemm256_eligible(g, batch, trans_a, trans_b, dtype))) continue;
         g_forced_gemm = v;
         const float us = t.time(s, iters, [&] {
             return mhip_gemm(stream, a, b, bias, c, M, N, K, batch, stride_a, stride_b, stride_c, trans_a, trans_b, activation, dtype);

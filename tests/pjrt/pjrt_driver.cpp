@@ -52,7 +52,16 @@ static PJRT_Error_Code code_of(PJRT_Error* e, std::string* msg = nullptr) {
     api->PJRT_Error_Destroy(&d);
     return c.code;
 }
-#define OK(call) CHECK(code_of(call) == PJRT_Error_Code_OK)
+#define OK(call)                                                                                   \
+    do {                                                                                           \
+        std::string ok_msg;                                                                        \
+        const PJRT_Error_Code ok_code = code_of(call, &ok_msg);                                    \
+        if (ok_code != PJRT_Error_Code_OK) {                                                       \
+            printf("FAIL %s:%d: %s -> code %d: %s\n", __FILE__, __LINE__, #call, (int)ok_code, ok_msg.c_str()); \
+            fflush(stdout);                                                                        \
+            exit(1);                                                                               \
+        }                                                                                          \
+    } while (0)
 
 static const char* kAdd =
     "module @add {\n  func.func @main(%a: tensor<4xf32>, %b: tensor<4xf32>) -> tensor<4xf32> {\n"
@@ -790,6 +799,49 @@ static void case_execute_while_transferring(PJRT_Client* c) {
     printf("ok execute_while_transferring\n");
 }
 
+// Two programs executed from two threads on ONE client with graph replay on: while one thread's
+// second execution captures the client's stream, the other thread's launches must not be recorded
+// into that graph (they would never run and its results would be stale).  Every enqueue of an
+// execution happens under the client's stream lock; each thread checks every result, with inputs
+// that change from one execution to the next so that a launch that did not run is seen.
+static void case_two_programs_two_threads(PJRT_Client* c) {
+    auto chain = [](int n, const char* op, const char* cst) {
+        std::string prog = std::string("func.func @main(%x: tensor<512xf32>) -> tensor<512xf32> {\n  %c = stablehlo.constant dense<") + cst + "> : tensor<512xf32>\n";
+        std::string cur = "%x";
+        for (int i = 0; i < n; i++) {
+            prog += "  %v" + std::to_string(i) + " = stablehlo." + op + " " + cur + ", %c : tensor<512xf32>\n";
+            cur = "%v" + std::to_string(i);
+        }
+        return prog + "  return " + cur + " : tensor<512xf32>\n}\n";
+    };
+    PJRT_LoadedExecutable *la = nullptr, *lb = nullptr;
+    OK(compile(c, chain(24, "add", "1.0"), "mlir", &la));
+    OK(compile(c, chain(20, "subtract", "2.0"), "mlir", &lb));
+    std::atomic<int> failures{0};
+    auto worker = [&](PJRT_LoadedExecutable* le, float delta, int seed) {
+        std::vector<float> x(512);
+        for (int it = 0; it < 30; it++) {
+            for (int i = 0; i < 512; i++) x[i] = (float)(seed + 3 * it + i);
+            // a fresh input buffer every other execution: new addresses force new captures while
+            // the other thread is launching
+            PJRT_Buffer* bx = upload(c, x.data(), PJRT_Buffer_Type_F32, {512});
+            for (int rep = 0; rep < 2; rep++) {
+                std::vector<float> y = run1(le, {bx}, 512);
+                for (int i = 0; i < 512; i++)
+                    if (y[i] != x[i] + delta) failures++;
+            }
+            destroy_buffer(bx);
+        }
+    };
+    std::thread ta(worker, la, 24.f, 1), tb(worker, lb, -40.f, 1000);
+    ta.join();
+    tb.join();
+    CHECK(failures.load() == 0);
+    destroy_loaded(la);
+    destroy_loaded(lb);
+    printf("ok two_programs_two_threads\n");
+}
+
 int main(int argc, char** argv) {
     if (argc < 3) { printf("usage: pjrt_driver <plugin.so> host|gpu\n"); return 2; }
     void* lib = dlopen(argv[1], RTLD_NOW | RTLD_LOCAL);
@@ -810,6 +862,7 @@ int main(int argc, char** argv) {
         case_execute(c);
         case_async_transfers(c);
         case_execute_while_transferring(c);
+        case_two_programs_two_threads(c);
     } else {
         case_no_device_buffers(c);
     }

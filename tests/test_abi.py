@@ -70,3 +70,42 @@ def test_host_wrappers_refuse_cpu_tensors():
     from metalhlo_amd import kernels
     with pytest.raises(RuntimeError, match="no CPU path"):
         kernels.softmax(torch.zeros(2, 2))
+
+
+def _exported(libname):
+    import subprocess
+    path = os.path.join(ROOT, "metalhlo_amd", "lib", libname)
+    out = subprocess.run(["nm", "-D", "--defined-only", path], capture_output=True, text=True, check=True).stdout
+    return sorted(line.split()[-1] for line in out.splitlines() if line.strip())
+
+
+def test_libraries_export_their_c_abi_and_nothing_else():
+    """The sealed boundary: the kernel library exports exactly the mhip_* functions of include/mhip.h,
+    the C API library exactly the mhlo_* functions of include/metalhlo.h, the PJRT plugin the one
+    symbol GetPjrtApi (Sources/PJRTMetalHLO/PJRTApi.swift:170-173).  The C API library and the
+    plugin contain the same C++ host; with its symbols private, a process that loads both gets
+    two independent copies instead of one library's calls bound to the other's definitions."""
+    assert _exported("libmetalhlo_hip.so") == _declared("mhip.h")
+    assert _exported("libCMetalHLO.so") == _declared("metalhlo.h")
+    assert _exported("libPJRTMetalHLO.so") == ["GetPjrtApi"]
+
+
+def test_reference_c_example_builds_against_this_header_and_library(tmp_path):
+    """The reference's own C program (Examples/CExample/main.c, which includes "metalhlo.h" and
+    calls the mhlo_* API) compiles against include/metalhlo.h and links against libCMetalHLO.so
+    unchanged.  Needs the reference tree (METALHLO_REFERENCE, default /root/reference); the file
+    is read where it lies, never copied.  Running it needs a GPU and is not part of this check."""
+    import subprocess
+    ref = os.environ.get("METALHLO_REFERENCE", "/root/reference")
+    src = os.path.join(ref, "Examples", "CExample", "main.c")
+    if not os.path.exists(src):
+        pytest.skip("the reference tree is not present")
+    exe = str(tmp_path / "cexample")
+    libdir = os.path.join(ROOT, "metalhlo_amd", "lib")
+    r = subprocess.run(["gcc", "-std=c11", "-I", os.path.join(ROOT, "include"), src, "-o", exe,
+                        "-L", libdir, "-lCMetalHLO", "-Wl,-rpath," + libdir, "-Wl,-rpath-link," + libdir,
+                        "-Wl,-rpath-link,/opt/rocm/lib", "-lm"], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-3000:]
+    undefined = subprocess.run(["nm", "-u", exe], capture_output=True, text=True, check=True).stdout
+    used = sorted(set(re.findall(r"\b(mhlo_[a-z_]+)", undefined)))
+    assert len(used) >= 15 and set(used) <= set(_declared("metalhlo.h")), used

@@ -161,10 +161,12 @@ def test_attention_program_replays(sess, monkeypatch):
 
 def test_replay_results_are_handed_out_without_a_copy_and_never_overwritten(sess, monkeypatch):
     """A captured graph writes its results into buffers of their own.  While the caller still holds
-    the results of the previous replay the next execution must not run that graph (it would
-    overwrite them): it runs eagerly, the held buffers keep their contents, and once they are
-    released the graph is replayed again.  Programs that return an input or an alias keep the
-    copy-out form (covered by 'pass_through' above)."""
+    the results of a replay the next execution must not run that graph (it would overwrite them):
+    it gets a second and then a third graph with result buffers of their own (a loop that keeps
+    the previous step's output alive replays every step), with all three sets held it runs
+    eagerly, the held buffers keep their contents, and once they are released the graphs are
+    replayed again.  Programs that return an input or an alias keep the copy-out form (covered
+    by 'pass_through' above)."""
     monkeypatch.setenv("METALHLO_ARENA", "1")
     monkeypatch.setenv("METALHLO_HIP_GRAPH", "1")
     rng = np.random.default_rng(21)
@@ -187,22 +189,35 @@ def test_replay_results_are_handed_out_without_a_copy_and_never_overwritten(sess
         assert sess.lib.mhlo_execute(exe, arr, len(inputs), outs, C.byref(n)) == 0, sess.lib.mhlo_get_last_error()
         return [outs[i] for i in range(n.value)]
 
-    held = execute_keep(bufs)                                    # a replay whose results stay with the caller
+    held = [execute_keep(bufs)]                                  # a replay whose results stay with the caller
     assert sess.plan(exe)["graph_replays"] == 5
-    again = execute_keep(bufs)                                   # must not touch `held`: eager
+    held.append(execute_keep(bufs))                              # must not touch held[0]: a second result set
+    held.append(execute_keep(bufs))                              # ... and a third
+    p3 = sess.plan(exe)
+    assert p3["graph_replays"] == 7 and p3["eager_runs"] == 1 and p3["graph_captures"] == 4, p3
+    held.append(execute_keep(bufs))                              # all three sets held: eager
     after = sess.plan(exe)
-    assert after["graph_replays"] == 5 and after["eager_runs"] == 2 and after["graph_captures"] == 2
+    assert after["graph_replays"] == 7 and after["eager_runs"] == 2 and after["graph_captures"] == 4, after
     got_other = run_with(sess, exe, other)                       # other inputs: their own graph, their own result buffers
     assert all(np.array_equal(g, w) for g, w in zip(got_other, want_other))
-    for hs in (held, again):
+    for hs in held:
         vals = [sess.to_numpy(h) for h in hs]
         assert all(np.array_equal(g, w) for g, w in zip(vals, want))
-    for h in held + again:
+    # the pattern of a loop that holds step n while it runs step n + 1: every step is a replay
+    for h in held[1] + held[2] + held[3]:
         sess.lib.mhlo_buffer_destroy(h)
-    got = run_with(sess, exe, bufs)                              # released: the graph runs again
-    assert all(np.array_equal(g, w) for g, w in zip(got, want))
+    prev = held[0]
+    for i in range(6):
+        cur = execute_keep(bufs)
+        assert all(np.array_equal(sess.to_numpy(h), w) for h, w in zip(cur, want)), f"rotating replay {i}"
+        assert all(np.array_equal(sess.to_numpy(h), w) for h, w in zip(prev, want)), f"held result during rotating replay {i}"
+        for h in prev:
+            sess.lib.mhlo_buffer_destroy(h)
+        prev = cur
+    for h in prev:
+        sess.lib.mhlo_buffer_destroy(h)
     end = sess.plan(exe)
-    assert end["graph_replays"] == 7 and end["eager_runs"] == 2 and end["graph_captures"] == 2
+    assert end["graph_replays"] == 14 and end["eager_runs"] == 2 and end["graph_captures"] == 4, end
     for b in bufs + other:
         sess.lib.mhlo_buffer_destroy(b)
     sess.lib.mhlo_executable_destroy(exe)

@@ -222,3 +222,45 @@ def test_stats_timing_profile_and_errors(sess):
     for b in (ba, bb, wrong):
         lib.mhlo_buffer_destroy(b)
     lib.mhlo_executable_destroy(exe)
+
+
+def test_per_operation_device_times(sess, monkeypatch):
+    """mhlo_execute_with_profile times the execution it makes operation by operation (HIP events
+    around every operation's launches); mhlo_ext_executable_profile returns the list: one entry per
+    launched operation in program order with its result shape, all times positive and their sum
+    no more than the execution's total.  The results are those of an ordinary execution, and the
+    next ordinary execution is not profiled (at level 3 it may be replayed as a graph again)."""
+    from metalhlo_amd import capi
+    text = """func.func @main(%x: tensor<64x256xf32>, %w: tensor<256x128xf32>) -> tensor<64x128xf32> {
+        %0 = stablehlo.custom_call @fused_softmax(%x) {backend_config = "{\\"axis\\": -1}"} : (tensor<64x256xf32>) -> tensor<64x256xf32>
+        %1 = stablehlo.dot %0, %w : (tensor<64x256xf32>, tensor<256x128xf32>) -> tensor<64x128xf32>
+        %2 = stablehlo.tanh %1 : tensor<64x128xf32>
+        %3 = stablehlo.add %2, %1 : tensor<64x128xf32>
+        return %3 : tensor<64x128xf32> }"""
+    exe = sess.compile(text)
+    rng = np.random.default_rng(77)
+    x, w = rng.standard_normal((64, 256)).astype(np.float32), rng.standard_normal((256, 128)).astype(np.float32) * 0.1
+    (want,) = sess.run(exe, [(x, "f32"), (w, "f32")])
+    assert sess.profile(exe) == []
+    bufs = [sess.buffer(x, "f32"), sess.buffer(w, "f32")]
+    arr = (C.c_void_p * 2)(*bufs)
+    outs = (C.c_void_p * 1)()
+    n = C.c_int32()
+    prof = capi.ExecutionProfile()
+    assert sess.lib.mhlo_execute_with_profile(exe, arr, 2, outs, C.byref(n), C.byref(prof)) == 0
+    got = sess.to_numpy(outs[0])
+    sess.lib.mhlo_buffer_destroy(outs[0])
+    assert np.array_equal(got, want)
+    times = sess.profile(exe)
+    assert [t[0] for t in times] == ["fused_softmax", "dot", "tanh", "add"]
+    assert [t[1] for t in times] == ["64x256xf32", "64x128xf32", "64x128xf32", "64x128xf32"]
+    assert all(t[2] > 0 for t in times) and sum(t[2] for t in times) * 1e-3 <= prof.total_time_ms
+    assert prof.partition_count == 1 and prof.gpu_time_ms > 0
+    # METALHLO_PROFILE_GPU=1 profiles ordinary executions too
+    monkeypatch.setenv("METALHLO_PROFILE_GPU", "1")
+    assert sess.lib.mhlo_execute(exe, arr, 2, outs, C.byref(n)) == 0
+    sess.lib.mhlo_buffer_destroy(outs[0])
+    assert len(sess.profile(exe)) == 4
+    for b in bufs:
+        sess.lib.mhlo_buffer_destroy(b)
+    sess.lib.mhlo_executable_destroy(exe)

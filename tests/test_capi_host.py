@@ -39,7 +39,7 @@ def test_exports_every_declared_symbol(lib):
     src = open(os.path.join(ROOT, "include", "metalhlo.h")).read()
     src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
     names = sorted(set(re.findall(r"\b(mhlo_[a-z0-9_]+)\s*\(", src)))
-    assert len(names) == 33        # the reference's 31 + mhlo_ext_executable_ops + mhlo_ext_executable_plan
+    assert len(names) == 34        # the reference's 31 + mhlo_ext_executable_ops, _plan and _profile
     for n in names:
         assert hasattr(lib, n), n
     assert sorted(capi.SIGNATURES) == names

@@ -444,3 +444,22 @@ def test_gemm_errors(lib):
     assert lib.mhip_gemm(None, p, p, None, p, 4, 4, 4, 1, 0, 0, 0, 0, 0, 1, 7) == 2   # no activation on int32
     assert lib.mhip_gemm(None, p, p, None, p, 4, 4, 4, 1, 0, 0, 0, 0, 0, 99, 1) == 1  # bad activation
     assert lib.mhip_gemm(None, p, p, None, p, 0, 4, 4, 1, 0, 0, 0, 0, 0, 0, 1) == 0   # empty is a no-op
+
+
+def test_gemm_ring_kernel_takes_wide_and_deep_operands(lib):
+    """The ring kernels address their operands with 32-bit byte offsets, so eligibility is decided
+    by the operands' real extents: B stored [K, N] with N = 50304 (an untied vocabulary head,
+    77 MB) and [2048, 32768] x [32768, 8192] stay on the four-wave ring kernel (variant 2560 / 2561), and the
+    results follow the oracle on sampled rows."""
+    from metalhlo_amd import kernels
+    rng = np.random.default_rng(71)
+    for (M, N, K) in [(4096, 50304, 768), (2048, 8192, 32768)]:
+        a = to_dev(rng.uniform(-1, 1, (M, K)), torch.bfloat16)
+        b = to_dev(rng.uniform(-1, 1, (K, N)) * (K ** -0.5), torch.bfloat16)
+        c = kernels.matmul(a, b)
+        assert lib.mhip_gemm_last_variant() in (2560, 2561, 2563), (M, N, K, lib.mhip_gemm_last_variant())
+        rows = np.r_[0, 255, 256, M - 1, rng.integers(0, M, 12)]
+        assert_close(c[rows], as_f64(a[rows]) @ as_f64(b), 2e-2, f"gemm {M}x{N}x{K}")
+    # fp32 operands run none of the 16-bit variants
+    kernels.matmul(torch.ones(64, 64, device="cuda"), torch.ones(64, 64, device="cuda"))
+    assert lib.mhip_gemm_last_variant() == 0

@@ -123,30 +123,47 @@ def test_empty_and_errors(lib):
         kernels.softmax(xi)
 
 
-def test_invariants_full_size():
-    """The benchmark row-kernel shape [32768, 4096] bf16: size-independent properties."""
+def test_full_size_config_parameters():
+    """The row-kernel benchmark configuration as written: X [32768, 4096] ~ N(0,1) from
+    numpy.random.default_rng(3), gamma ~ N(1, 0.1), beta ~ N(0, 0.1), bias ~ N(0, 0.02), all rounded to
+    bf16; eps 1e-5 (LayerNorm) / 1e-6 (RMSNorm).  All four operators run on the whole tensor (the
+    launch form the benchmark times) and 40 sampled rows of each are compared with the oracle;
+    size-independent properties cover the rest of the rows."""
     from metalhlo_amd import kernels
-    g = torch.Generator(device="cuda").manual_seed(3)
-    x = torch.randn(32768, 4096, generator=g, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+    rng = np.random.default_rng(3)
+    rows, cols = 32768, 4096
+    x = to_dev(rng.standard_normal((rows, cols), dtype=np.float32), torch.bfloat16)
+    gam = to_dev(1 + 0.1 * rng.standard_normal(cols), torch.bfloat16)
+    bet = to_dev(0.1 * rng.standard_normal(cols), torch.bfloat16)
+    bias = to_dev(0.02 * rng.standard_normal(cols), torch.bfloat16)
+    idx = np.r_[0, 1, 2, 3, 4097, rows - 2, rows - 1, rng.integers(0, rows, 33)]
+    sub, g64, b64, bias64 = as_f64(x[idx]), as_f64(gam), as_f64(bet), as_f64(bias)
     y = kernels.softmax(x)
-    assert torch.allclose(y.float().sum(-1), torch.ones(32768, device="cuda"), atol=2e-2)
-    # shift invariance: softmax(x + c) == softmax(x) when x + c is exact in bf16
-    idx = [0, 1, 4097, 32767]
-    sub = x[idx]
-    assert_close(kernels.softmax(sub), oracle.softmax(as_f64(sub)), 2e-2, "softmax rows of full tensor")
-    assert_close(y[idx], oracle.softmax(as_f64(sub)), 2e-2, "softmax full launch, sampled rows")
-    gam = torch.ones(4096, device="cuda", dtype=torch.bfloat16)
+    assert_close(y[idx], oracle.softmax(sub), 2e-2, "softmax full launch, sampled rows")
+    assert torch.allclose(y.float().sum(-1), torch.ones(rows, device="cuda"), atol=2e-2)
+    assert_close(kernels.softmax(x[idx].contiguous()), oracle.softmax(sub), 2e-2, "softmax on the sampled rows alone")
+    del y
+    ln = kernels.layer_norm(x, gam, bet, eps=1e-5)
+    assert_close(ln[idx], oracle.layer_norm(sub, g64, b64, 1e-5), 2e-2, "LayerNorm full launch, sampled rows")
+    # affine invariance of the statistics: LN(2x) == LN(x) up to eps (a power-of-two scale is exact in bf16)
+    ln2 = kernels.layer_norm(x * 2, gam, bet, eps=4 * float(np.float32(1e-5)))
+    assert torch.equal(ln2, ln)
+    del ln, ln2
     r = kernels.rms_norm(x, gam, eps=1e-6)
-    ms = (r.float() ** 2).mean(-1)
-    assert torch.allclose(ms, torch.ones_like(ms), atol=2e-2)
-    # scale covariance: rms_norm(2x) == rms_norm(x) (power-of-two scale is exact in bf16)
-    r2 = kernels.rms_norm(x * 2, gam, eps=4e-6)
+    assert_close(r[idx], oracle.rms_norm(sub, g64, 1e-6), 2e-2, "RMSNorm full launch, sampled rows")
+    # scale covariance: rms_norm(2x, 4 eps) == rms_norm(x, eps)
+    r2 = kernels.rms_norm(x * 2, gam, eps=4 * float(np.float32(1e-6)))
     assert torch.equal(r2, r)
-    ln = kernels.layer_norm(x, gam, torch.zeros_like(gam), eps=1e-5)
-    assert ln.float().mean(-1).abs().max().item() < 2e-2
-    assert_close(ln[idx], oracle.layer_norm(as_f64(sub), 1.0, 0.0, 1e-5), 2e-2, "ln sampled rows")
-    ge = kernels.bias_gelu(x, torch.zeros_like(gam))
-    assert_close(ge[idx], oracle.gelu_tanh(as_f64(sub)), 2e-2, "gelu sampled rows")
+    # with gamma = 1 every row has mean square 1
+    r1 = kernels.rms_norm(x, torch.ones_like(gam), eps=1e-6)
+    ms = (r1.float() ** 2).mean(-1)
+    assert torch.allclose(ms, torch.ones_like(ms), atol=2e-2)
+    del r, r2, r1
+    ge = kernels.bias_gelu(x, bias)
+    assert_close(ge[idx], oracle.bias_gelu(sub, bias64), 2e-2, "bias+GELU full launch, sampled rows")
+    # every row sees the same bias: a row repeated elsewhere in the tensor gives the same result
+    x2 = x.clone(); x2[1000] = x[idx[7]]
+    assert torch.equal(kernels.bias_gelu(x2, bias)[1000], ge[idx[7]])
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=lambda d: NAME[d])
