@@ -120,7 +120,7 @@ def build_host(verbose: bool = True) -> list:
         drv_src = os.path.join(ROOT, "tests", "pjrt", "pjrt_driver.cpp")
         if os.path.exists(drv_src):
             drv = os.path.join(ROOT, "tests", "pjrt", "pjrt_driver")
-            _run(["g++", "-O1", "-std=c++17", "-Wall", "-pthread", "-I", os.path.join(ROOT, "include"), drv_src, "-o", drv, "-ldl"])
+            _run(["g++", "-O1", "-g", "-std=c++17", "-Wall", "-pthread", "-rdynamic", "-I", os.path.join(ROOT, "include"), drv_src, "-o", drv, "-ldl"])
             if verbose:
                 print("  link ", os.path.relpath(drv, ROOT), flush=True)
     return outs

@@ -656,9 +656,9 @@ static DeviceTensor permuted_copy(Allocator& al, bool dry, void* stream, const D
 // `marks` (optional): one HIP event is recorded on the stream in front of the first launch and one
 // behind every operation; marks[i].first = index of the operation the event closes (-1: the start).
 static std::vector<DeviceTensor> run_ops(Executable& exe, const std::vector<DeviceTensor>& inputs, Allocator& al, bool dry,
-                                         std::vector<std::pair<int, hipEvent_t>>* marks = nullptr) {
+                                         std::vector<std::pair<int, hipEvent_t>>* marks = nullptr, hipStream_t on_stream = nullptr) {
     const Function& fn = exe.fn;
-    void* s = exe.client ? exe.client->stream : nullptr;
+    void* s = on_stream ? on_stream : (exe.client ? exe.client->stream : nullptr);
     auto mark = [&](int op_index) {
         if (!marks || dry) return;
         hipEvent_t e = nullptr;
@@ -1019,8 +1019,17 @@ static bool capture_graph(Executable& exe, const std::vector<DeviceTensor>& inpu
             presets[i] = m;
         }
     }
-    // the caller (execute) holds c.stream_mu: no other thread enqueues on the stream meanwhile
-    if (hipStreamBeginCapture(c.stream, hipStreamCaptureModeThreadLocal) != hipSuccess) {
+    // The capture runs on the client's capture stream (see Client), in relaxed mode: nothing inside the
+    // capture allocates or synchronises (the replay tests hold every kernel wrapper to that), and
+    // what other threads call meanwhile -- the pool's hipMalloc, the transfer engine's pinned blocks
+    // and event waits -- cannot invalidate it.  The caller (execute) holds c.stream_mu.
+    if (c.capture_broken) return false;
+    if (!c.capture_stream && hipStreamCreateWithFlags(&c.capture_stream, hipStreamNonBlocking) != hipSuccess) {
+        (void)hipGetLastError();
+        c.capture_stream = nullptr;
+        return false;
+    }
+    if (hipStreamBeginCapture(c.capture_stream, hipStreamCaptureModeRelaxed) != hipSuccess) {
         (void)hipGetLastError();
         return false;
     }
@@ -1033,9 +1042,22 @@ static bool capture_graph(Executable& exe, const std::vector<DeviceTensor>& inpu
     if (direct) al.presets = &presets;
     std::vector<DeviceTensor> rets;
     bool ok = true;
-    try { rets = run_ops(exe, inputs, al, false); } catch (const std::exception&) { ok = false; }
+    std::string why;
+    try { rets = run_ops(exe, inputs, al, false, nullptr, c.capture_stream); } catch (const std::exception& x) { ok = false; why = x.what(); }
     hipGraph_t g = nullptr;
-    const hipError_t e = hipStreamEndCapture(c.stream, &g);
+    const hipError_t e = hipStreamEndCapture(c.capture_stream, &g);
+    if (e != hipSuccess || !ok) {
+        (void)hipGetLastError();
+        hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+        const hipError_t q = hipStreamIsCapturing(c.capture_stream, &st);
+        (void)hipGetLastError();
+        // a failed capture can leave its stream in the capturing state for good (seen with an
+        // invalidated capture); nothing more is captured on this client then
+        if (q != hipSuccess || st != hipStreamCaptureStatusNone) c.capture_broken = true;
+        if (getenv("METALHLO_DEBUG_GRAPH"))
+            fprintf(stderr, "[metalhlo] graph capture failed: launches: %s; end of capture: %s; stream capture status afterwards: %d (%s)\n",
+                    ok ? "ok" : why.c_str(), hipGetErrorString(e), (int)st, hipGetErrorString(q));
+    }
     hipGraphExec_t ex = nullptr;
     if (ok && e == hipSuccess && g && hipGraphInstantiate(&ex, g, nullptr, nullptr, 0) != hipSuccess) ex = nullptr;
     if (g) (void)hipGraphDestroy(g);

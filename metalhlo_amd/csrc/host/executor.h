@@ -80,6 +80,15 @@ struct Client {
     // enqueues work on the stream (the PJRT plugin's transfers): work enqueued from another thread
     // during a capture would become part of the graph instead of running.
     std::mutex stream_mu;
+    // Graphs are captured on a stream of their own (created at the first capture, non-blocking), never on
+    // `stream`: the launches of a capture do not run, so which stream records them is immaterial to
+    // the replays, and the events that other threads wait for on `stream` (the PJRT plugin's
+    // transfer completions) then never belong to a stream that is capturing -- waiting for such an
+    // event invalidates the capture.  `capture_broken`: a capture failed and left that stream in the
+    // capturing state; this client captures nothing further (every execution is eager).
+    hipStream_t capture_stream = nullptr;
+    bool capture_broken = false;
+    ~Client() { if (capture_stream && !capture_broken) (void)hipStreamDestroy(capture_stream); }
     DevicePool pool;
     DeviceTensor allocate(const TensorType& t);
 };

@@ -7,6 +7,8 @@
 // case_async_transfers has no counterpart there (the reference's transfers complete inside
 // the call): it covers the asynchronous uploads and downloads of this plugin.
 #include <dlfcn.h>
+#include <execinfo.h>
+#include <signal.h>
 #include <math.h>
 #include <stdio.h>
 #include <stdlib.h>
@@ -842,7 +844,21 @@ static void case_two_programs_two_threads(PJRT_Client* c) {
     printf("ok two_programs_two_threads\n");
 }
 
+// A crash inside the plugin names its call chain (module + offset per frame) before the process ends.
+static void on_crash(int sig) {
+    void* frames[48];
+    const int n = backtrace(frames, 48);
+    const char msg[] = "FAIL: fatal signal, call chain:\n";
+    (void)!write(1, msg, sizeof msg - 1);
+    backtrace_symbols_fd(frames, n, 1);
+    signal(sig, SIG_DFL);
+    raise(sig);
+}
+
 int main(int argc, char** argv) {
+    signal(SIGSEGV, on_crash);
+    signal(SIGABRT, on_crash);
+    setvbuf(stdout, nullptr, _IONBF, 0);       // every "ok" line reaches a pipe even when a later case crashes
     if (argc < 3) { printf("usage: pjrt_driver <plugin.so> host|gpu\n"); return 2; }
     void* lib = dlopen(argv[1], RTLD_NOW | RTLD_LOCAL);
     if (!lib) { printf("FAIL dlopen: %s\n", dlerror()); return 1; }
