@@ -304,11 +304,31 @@ int mhip_fill(void* stream, void* y, int64_t n, uint64_t pattern, int elem_size)
 
 /* GEMM kernel variants (128x128 tiles / 4 waves, 256x256 / 8 waves, the four-wave LDS-ring kernel
  * on 256x256 and on 256x128 tiles, the latter also as persistent workgroups, and wide tiles plus a
- * band of narrow ones): variant code 128 | 256 | 2560 | 2561 | 2562 | 2563, microseconds per launch. */
+ * band of narrow ones): variant code 128 | 256 | 2560 | 2561 | 2562 | 2563, and the other members of the
+ * generated ring-kernel family (tile width 256 / 128 x ring depth 4 / 5 / 6, those that fit 160 KB of
+ * LDS): 2564 = 256x128 with six stages, 2565 = 256x128 with four, 2566 = 256x256 with four;
+ * microseconds per launch. */
 int mhip_gemm_autotune(void* stream, const void* a, const void* b, const void* bias, void* c,
                        int64_t M, int64_t N, int64_t K, int64_t batch, int64_t stride_a,
                        int64_t stride_b, int64_t stride_c, int trans_a, int trans_b, int activation,
                        int dtype, int iters, int* out_variant, float* out_us);
+
+/* The same search as a GEMM inside a model meets its operands: before every timed launch `flush`
+ * (device memory the caller lends, at least 64 MB) is overwritten -- 64 to 128 MB empty the L2s and
+ * leave most of the memory-side cache, the state of weights written a millisecond earlier; 512 MB and
+ * more empty both -- and A is rewritten in place, as the kernel in front of the GEMM would have left
+ * it.  Each launch is timed on its own, the median of `iters` decides and is recorded under the
+ * same key as mhip_gemm_autotune (the later pass wins). */
+int mhip_gemm_autotune_in_model(void* stream, const void* a, const void* b, const void* bias, void* c,
+                                int64_t M, int64_t N, int64_t K, int64_t batch, int64_t stride_a,
+                                int64_t stride_b, int64_t stride_c, int trans_a, int trans_b, int activation,
+                                int dtype, int iters, void* flush, int64_t flush_bytes, int* out_variant,
+                                float* out_us);
+
+/* Records `variant` for a GEMM problem (0 removes the entry): for searches that time more than one
+ * kernel, such as `python -m metalhlo_amd.tune`, which times a whole GPT-2 forward pass per candidate. */
+int mhip_tuning_set_gemm(int64_t M, int64_t N, int64_t K, int64_t batch, int trans_a, int trans_b, int dtype,
+                         int variant, float us);
 
 /* The kernel variant (codes above; 0 = none of them: fp32, integer, f64 or unaligned operands) that
  * the calling thread's most recent mhip_gemm / mhip_gemm_residual call launched.  The tuner's
@@ -334,8 +354,10 @@ int mhip_attention_autotune(void* stream, const void* q, const void* k, const vo
 /* The tuning table as text, one "<operator> <device> <problem> = <choice> @ <microseconds>" line per
  * entry (Tuning/TuningDatabase.swift:109-150); <device> is the architecture name and the number
  * of compute units ("gfx950/256", TuningDatabase.swift:15-60 keys by device too), and only
- * entries of the current device are used.  Loading merges into the table; the file named by the
- * environment variable MHIP_TUNING_DB is loaded at first use. */
+ * entries of the current device are used.  Loading merges into the table.  At first use the
+ * library loads the table that ships with it for the device in use (../tuning/<arch>_<CUs>.txt beside
+ * the shared object, written by `python -m metalhlo_amd.tune`) and then the file the environment
+ * variable MHIP_TUNING_DB names; MHIP_TUNING_DB=none loads neither, mhip_tuning_clear empties the table. */
 int mhip_tuning_save(const char* path);
 int mhip_tuning_load(const char* path);
 void mhip_tuning_clear(void);

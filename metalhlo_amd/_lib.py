@@ -52,6 +52,9 @@ SIGNATURES = {
     "mhip_reduce": (_i32, [_vp, _i32, _vp, _vp, _i64, _i64, _i64, C.c_double, _i32]),
     "mhip_fill": (_i32, [_vp, _vp, _i64, C.c_uint64, _i32]),
     "mhip_argmax": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32]),
+    "mhip_gemm_autotune_in_model": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _i32,
+                                           _i32, _i32, _vp, _i64, C.POINTER(C.c_int), C.POINTER(C.c_float)]),
+    "mhip_tuning_set_gemm": (_i32, [_i64, _i64, _i64, _i64, _i32, _i32, _i32, _i32, C.c_float]),
     "mhip_gemm_last_variant": (_i32, []),
     "mhip_gemm_autotune": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _i32,
                                   _i32, _i32, C.POINTER(C.c_int), C.POINTER(C.c_float)]),

@@ -65,8 +65,8 @@ __device__ inline void tile_of_workgroup(const FaArgs& a, int id, int& bh, int& 
 
 // host side: a.nqb set; fills xcd_map and cu_group
 inline void set_tile_order(FaArgs& a) {
-    // (MHIP_FA_HEADS=2: the heads dealt round-robin over the XCDs instead of in contiguous eighths)
-    a.xcd_map = (((int64_t)a.B * a.H) % 8 == 0) ? (tune_int("MHIP_FA_HEADS", 1) == 2 ? 2 : 1) : 0;
+    // (an XCD takes a contiguous eighth of the (batch, head) pairs)
+    a.xcd_map = (((int64_t)a.B * a.H) % 8 == 0) ? 1 : 0;
     a.cu_group = a.xcd_map ? compute_units() / 8 : compute_units();
     if (a.cu_group < 1) a.cu_group = 1;
 }

@@ -399,7 +399,7 @@ static int launch_mfma(hipStream_t s, GemmArgs g, int64_t batch) {
 
 // gemm256.hip: 4-wave 256x256 kernel with a hand-scheduled main loop.
 bool gemm256_eligible(const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype, int bw = 256, bool any_tile_count = false);
-int launch_gemm256(hipStream_t s, const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype, int bw = 256);
+int launch_gemm256(hipStream_t s, const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype, int bw = 256, int ring = 5);
 bool gemm_stream_eligible(const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype);
 int launch_gemm_stream(hipStream_t s, const GemmArgs& g, int trans_b, int dtype);
 // gemm_f32.hip: fp32 operands on the fp32 matrix instruction, 128x128 tiles.
@@ -454,19 +454,16 @@ static int launch_column_split(hipStream_t s, const GemmArgs& g, int64_t batch, 
     if (g.residual) r.residual = static_cast<const T*>(g.residual) + n_wide;
     r.c = static_cast<T*>(g.c) + n_wide;
     if (!gemm256_eligible(w, 1, TA, TB, dt) || !gemm256_eligible(r, 1, TA, TB, dt, 128, /*any_tile_count=*/true)) return -1;
-    // The band first (MHIP_GEMM_SPLIT=3: last): what the wide tiles store at their common end is
+    // The band first: what the wide tiles store at their common end is
     // then the freshest content of the L2s when the next kernel starts at column 0.
-    if (tune_int("MHIP_GEMM_SPLIT", 1) == 3) {
-        const int st = launch_gemm256(s, w, 1, TA, TB, dt);
-        if (st != MHIP_OK) return st;
-        return launch_gemm256(s, r, 1, TA, TB, dt, 128);
-    }
     const int st = launch_gemm256(s, r, 1, TA, TB, dt, 128);
     if (st != MHIP_OK) return st;
     return launch_gemm256(s, w, 1, TA, TB, dt);
 }
 
-// Which kernel serves a 16-bit problem (MHIP_GEMM_TILE = 128 | 256 | 2560 | 2561 | 2562 | 2563 forces one):
+// Which kernel serves a 16-bit problem (MHIP_GEMM_TILE = 128 | 256 | 2560 ... 2566 forces one; 2564 / 2565 = the
+// 256x128 tile with a ring of six / four stages, 2566 = the 256x256 tile with four: members of the
+// generated family that only a forced choice or the tuning table selects):
 //   * the four-wave ring kernel (gemm256.hip) on 256x256 tiles (2560) or 256x128 tiles
 //     (2561) when K >= 512 and the problem is eligible: one workgroup per CU, so its time is
 //     rounds x (stages x per-stage time + prologue and epilogue), rounds = ceil(tiles / 256 CUs);
@@ -476,9 +473,8 @@ static int launch_column_split(hipStream_t s, const GemmArgs& g, int64_t batch, 
 //     500 -- figures fitted to seven measured shapes (4096^3: wide; [8192,768] x K 3072
 //     or 768, [8192,2304..3072] x K 768: narrow);
 //   * the same 256x128 kernel as persistent workgroups that store a tile inside the loop of the
-//     next one (2562; gemm_stream_kernel): forced, recorded by the tuner, or with
-//     MHIP_GEMM_STREAM=1 for two to four rounds of narrow tiles with B stored [K, N] (see below
-//     why it is no longer a default);
+//     next one (2562; gemm_stream_kernel): forced or recorded by the tuner (see below why it is
+//     not a default);
 //   * wide tiles on the columns that fill whole rounds and narrow tiles on the rest (2563;
 //     launch_column_split) where the problem has that shape;
 //   * the eight-wave 256x256 kernel for large problems the ring kernel cannot take whose
@@ -505,7 +501,15 @@ static int pick_tile(hipStream_t s, const GemmArgs& g, int64_t batch) {
     if (force == 2560) {
         if (gemm256_eligible(g, batch, TA, TB, dt)) return chose(2560, launch_gemm256(s, g, batch, TA, TB, dt));
     }
-    if (force == 2563 || (force == 0 && g.K >= 512 && tune_int("MHIP_GEMM_SPLIT", 1) != 2)) {    // 2 = off
+    // the other members of the generated tile family: ring depth 6 or 4 on the narrow tile, 4 on the wide one
+    if (force == 2564 || force == 2565) {
+        if (gemm256_eligible(g, batch, TA, TB, dt, 128))
+            return chose(force, launch_gemm256(s, g, batch, TA, TB, dt, 128, force == 2564 ? 6 : 4));
+    }
+    if (force == 2566) {
+        if (gemm256_eligible(g, batch, TA, TB, dt)) return chose(2566, launch_gemm256(s, g, batch, TA, TB, dt, 256, 4));
+    }
+    if (force == 2563 || (force == 0 && g.K >= 512)) {
         const int st = launch_column_split<T, TA, TB>(s, g, batch, dt, force == 2563);
         if (st >= 0) return chose(2563, st);
     }
@@ -513,18 +517,11 @@ static int pick_tile(hipStream_t s, const GemmArgs& g, int64_t batch) {
         constexpr int cus = 256;                       // compute units of the device this is written for
         const int64_t narrow = tiles_m * ((g.N + 127) / 128) * batch, stages = g.K / 32;
         const bool wide_ok = gemm256_eligible(g, batch, TA, TB, dt), narrow_ok = gemm256_eligible(g, batch, TA, TB, dt, 128);
-        // (The streamed form of the narrow tile, 2562, is no longer chosen here: it is 5 % ahead of
-        // wide tiles on a few shapes when the operands sit in the L2 -- [4096,8320] x K 1024 77 against
-        // 81 us, [8192,4608] x K 768 67 against 71 -- and 10 to 15 % behind on the same shapes when
-        // they come from memory, 92 against 84 and 83 against 72, which is how a GEMM inside a
-        // model finds them; [8192,3584] x K 768: 58 / 66 us streamed, 48 / 53 on wide tiles.  The tuner
-        // still times it and records it where it wins; MHIP_GEMM_STREAM=1 restores the old choice.)
-        if (!TB && (narrow + cus - 1) / cus <= 4 && tune_int("MHIP_GEMM_STREAM", 2) == 1 &&
-            gemm_stream_eligible(g, batch, TA, TB, dt)) {
-            const double stream_us = (double)((narrow + cus - 1) / cus) * (stages * 0.3875 + 3.8) + 5.0;
-            const double wide_us = (double)((big + cus - 1) / cus) * (stages * 0.6625 + 13.8);
-            if (!wide_ok || stream_us < wide_us) return chose(2562, launch_gemm_stream(s, g, TB, dt));
-        }
+        // (The streamed form of the narrow tile, 2562, is not chosen here: it is 5 % ahead of wide tiles
+        // on a few shapes when the operands sit in the L2 -- [4096,8320] x K 1024 77 against 81 us,
+        // [8192,4608] x K 768 67 against 71 -- and 10 to 15 % behind on the same shapes when they come
+        // from memory, 92 against 84 and 83 against 72, which is how a GEMM inside a model finds
+        // them.  The tuner times it and the table selects it where it wins.)
         const int64_t wide_cost = ((big + cus - 1) / cus) * (stages * 32 + 700);
         const int64_t narrow_cost = ((narrow + cus - 1) / cus) * (stages * 18 + 500);
         if (narrow_ok && (!wide_ok || narrow_cost < wide_cost)) return chose(2561, launch_gemm256(s, g, batch, TA, TB, dt, 128));

@@ -98,16 +98,22 @@ struct MnMajor {
     }
 };
 
-template <typename T, bool TA, bool TB, int BW>
+template <typename T, bool TA, bool TB, int BW, int RING>
 __device__ inline void main_loop(f32x16 (&acc)[BW / 16], u32x4 ra, u32x4 rb, u32x2& misc,
                                  __amdgpu_buffer_rsrc_t rsa, __amdgpu_buffer_rsrc_t rsb, uint32_t pa,
                                  uint32_t pb, uint32_t ta, uint32_t tb, uint32_t m0b, uint32_t kt) {
     constexpr bool bf = std::is_same<T, bf16_t>::value;
+    // the member of the generated tile family: B width x ring depth
 #define MHIP_LOOP(cond, name)                                                                        \
     if constexpr (cond) {                                                                            \
-        if constexpr (BW == 256) gemm256_loop_##name(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt); \
-        else gemm256x128_loop_##name(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt);           \
+        if constexpr (BW == 256 && RING == 5) gemm256_loop_##name(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt); \
+        else if constexpr (BW == 256 && RING == 4) gemm256r4_loop_##name(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt); \
+        else if constexpr (BW == 128 && RING == 5) gemm256x128_loop_##name(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt); \
+        else if constexpr (BW == 128 && RING == 4) gemm256x128r4_loop_##name(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt); \
+        else gemm256x128r6_loop_##name(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt);          \
     }
+    static_assert((BW == 256 && (RING == 4 || RING == 5)) || (BW == 128 && RING >= 4 && RING <= 6),
+                  "not a member of the generated tile family");
     MHIP_LOOP(bf && !TA && !TB, nn_bf16)
     MHIP_LOOP(bf && !TA && TB, nt_bf16)
     MHIP_LOOP(bf && TA && !TB, tn_bf16)
@@ -297,7 +303,8 @@ __device__ __forceinline__ void store_tile(f32x16 (&acc)[BW / 16], char* smem, c
 // BW = 256: the 256x256 tile (each wave 128x128).  BW = 128: a 256x128 tile (each wave
 // 128x64, half the accumulators, a 24 KB stage) for problems whose 256x256 tiling would
 // leave compute units idle or a last round nearly empty.
-template <typename T, bool TA, bool TB, int BW>
+// RING: stage buffers in the LDS ring (4, 5 or 6; loads run that many stages ahead).
+template <typename T, bool TA, bool TB, int BW, int RING>
 __global__ __launch_bounds__(256) void gemm256_kernel(GemmArgs g) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     using LA = typename std::conditional<TA, MnMajor<256>, KMajor>::type;
@@ -336,8 +343,8 @@ __global__ __launch_bounds__(256) void gemm256_kernel(GemmArgs g) {
         __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(b), 0, b_bytes, 0x00020000);
 
     f32x16 acc[4 * NBF];
-    main_loop<T, TA, TB, BW>(acc, ra, rb, misc, rsa, rsb, LA::pass_stride(g.lda), LB::pass_stride(g.ldb),
-                             LA::stage_stride(g.lda), LB::stage_stride(g.ldb), m0b, (uint32_t)(g.K / 32));
+    main_loop<T, TA, TB, BW, RING>(acc, ra, rb, misc, rsa, rsb, LA::pass_stride(g.lda), LB::pass_stride(g.ldb),
+                                   LA::stage_stride(g.lda), LB::stage_stride(g.ldb), m0b, (uint32_t)(g.K / 32));
 
     // (a compile-time variant: the same branch inside the epilogue upsets the compiler)
     if (g.stream_c) store_tile<T, BW, true>(acc, smem, g, c, res, m0, n0);
@@ -470,7 +477,7 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(GemmArgs g, int total)
             if (wave == 0)
                 *reinterpret_cast<uint32_t*>(smem + kStreamBias + lane * 4) =
                     bias ? *reinterpret_cast<const uint32_t*>(bias + n0 + 2 * lane) : 0u;
-            main_loop<T, false, TB, 128>(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt);
+            main_loop<T, false, TB, 128, 5>(acc, ra, rb, misc, rsa, rsb, pa, pb, ta, tb, m0b, kt);
         } else {
             const uint32_t m0bias = __builtin_amdgcn_readfirstlane(lds0 + kStreamBias + (uint32_t)(it & 1) * 256u);
             stream_prologue<T, TB>(misc, rsa, rsb, pa, pb, ta, tb, m0b, rsbias, m0bias,
@@ -508,10 +515,14 @@ int launch_stream(hipStream_t s, GemmArgs g) {
     return check_launch("gemm_stream");
 }
 
-template <typename T, bool TA, bool TB, int BW>
+template <typename T, bool TA, bool TB, int BW, int RING>
 int launch256(hipStream_t s, GemmArgs g, int64_t batch) {
-    constexpr int kSmem = 5 * (16 + BW / 16) * 1024;   // ring of five stage buffers; the epilogue staging reuses it
-    auto kern = gemm256_kernel<T, TA, TB, BW>;
+    // the ring of stage buffers; the epilogue's staging (four waves x 128 rows of WN 16-bit values + 16
+    // bytes of padding) reuses it and is the larger of the two for a short ring of wide tiles
+    constexpr int kRing = RING * (16 + BW / 16) * 1024, kStaging = 4 * 128 * (BW + 16);
+    constexpr int kSmem = kRing > kStaging ? kRing : kStaging;
+    static_assert(kSmem <= 160 * 1024, "ring or staging exceeds the LDS of a compute unit");
+    auto kern = gemm256_kernel<T, TA, TB, BW, RING>;
     static std::once_flag once;
     static hipError_t attr_err = hipSuccess;
     std::call_once(once, [&] {
@@ -534,12 +545,23 @@ int launch256(hipStream_t s, GemmArgs g, int64_t batch) {
     return check_launch("gemm256");
 }
 
-template <typename T, int BW>
+template <typename T, int BW, int RING>
 int layout256(hipStream_t s, const GemmArgs& g, int64_t batch, int ta, int tb) {
-    if (!ta && !tb) return launch256<T, false, false, BW>(s, g, batch);
-    if (!ta && tb) return launch256<T, false, true, BW>(s, g, batch);
-    if (ta && !tb) return launch256<T, true, false, BW>(s, g, batch);
-    return launch256<T, true, true, BW>(s, g, batch);
+    if (!ta && !tb) return launch256<T, false, false, BW, RING>(s, g, batch);
+    if (!ta && tb) return launch256<T, false, true, BW, RING>(s, g, batch);
+    if (ta && !tb) return launch256<T, true, false, BW, RING>(s, g, batch);
+    return launch256<T, true, true, BW, RING>(s, g, batch);
+}
+
+template <typename T>
+int family256(hipStream_t s, const GemmArgs& g, int64_t batch, int ta, int tb, int bw, int ring) {
+    if (bw == 256) {
+        if (ring == 4) return layout256<T, 256, 4>(s, g, batch, ta, tb);
+        return layout256<T, 256, 5>(s, g, batch, ta, tb);
+    }
+    if (ring == 4) return layout256<T, 128, 4>(s, g, batch, ta, tb);
+    if (ring == 6) return layout256<T, 128, 6>(s, g, batch, ta, tb);
+    return layout256<T, 128, 5>(s, g, batch, ta, tb);
 }
 
 }  // namespace
@@ -564,14 +586,11 @@ bool gemm256_eligible(const GemmArgs& g, int64_t batch, int trans_a, int trans_b
     return (tiles >= 192 || any_tile_count) && tiles <= 0x7FFFFFFF && batch <= 65535;
 }
 
+// `bw` x `ring`: the member of the tile family (256 x {4, 5}, 128 x {4, 5, 6}; anything else runs depth 5).
 int launch_gemm256(hipStream_t s, const GemmArgs& g, int64_t batch, int trans_a, int trans_b,
-                   int dtype, int bw) {
-    if (bw == 128) {
-        if (dtype == MHIP_BF16) return layout256<bf16_t, 128>(s, g, batch, trans_a, trans_b);
-        return layout256<f16_t, 128>(s, g, batch, trans_a, trans_b);
-    }
-    if (dtype == MHIP_BF16) return layout256<bf16_t, 256>(s, g, batch, trans_a, trans_b);
-    return layout256<f16_t, 256>(s, g, batch, trans_a, trans_b);
+                   int dtype, int bw, int ring) {
+    if (dtype == MHIP_BF16) return family256<bf16_t>(s, g, batch, trans_a, trans_b, bw, ring);
+    return family256<f16_t>(s, g, batch, trans_a, trans_b, bw, ring);
 }
 
 // Streamed tiles (persistent workgroups, stores inside the next tile's loop): see gemm_stream_kernel.

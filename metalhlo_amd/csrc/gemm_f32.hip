@@ -203,12 +203,11 @@ int launch_tile(hipStream_t s, GemmArgs g, int64_t batch) {
 // them for a round and a quarter, 64x64 tiles (eight per CU) below that.  Measured (TFLOP/s,
 // 64 | 128): 4096^3 101 | 116, [8192,3072] x K 768 (1536 large tiles) 100 | 113; [3000,3000] x K 1000
 // (576) 89 | 73, [2048,2048] x K 2048 (256) 99 | 91, [8192,768] x K 3072 (384) 100 | 87, 1024^3 (64)
-// 62 | 23.  MHIP_GEMM_F32_TILE = 64 | 128 forces one.
+// 62 | 23.
 template <bool TA, bool TB>
 int launch(hipStream_t s, const GemmArgs& g, int64_t batch) {
-    const int forced = tune_int("MHIP_GEMM_F32_TILE", 0);
     const int64_t large_tiles = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128) * batch;
-    if (forced == 128 || (forced != 64 && large_tiles >= 960)) return launch_tile<TA, TB, 2>(s, g, batch);
+    if (large_tiles >= 960) return launch_tile<TA, TB, 2>(s, g, batch);
     return launch_tile<TA, TB, 1>(s, g, batch);
 }
 

@@ -47,9 +47,6 @@ Register map:
   s77 = caller's M0, s[78:79] / s[80:81] = compare results of q0 / q1,
   s[82:83] / s[84:85] = lanes of q0 / q1 whose reference maximum moved
 """
-import os
-
-EXP = set(os.environ.get("FA_LOOP_EXP", "").split(","))      # timing experiments (results are wrong)
 NQ = 2
 SBUF = (0, 192)
 PX, PY = 64, 160
@@ -228,8 +225,6 @@ def body(n, order, uid):
     s_in, s_out = (SBUF[0], SBUF[1]) if n % 2 == 0 else (SBUF[1], SBUF[0])
     pprev, pnew = (PY, PX) if n % 2 == 0 else (PX, PY)
     valu = interleave(softmax_stream(0, s_in, pnew), softmax_stream(1, s_in, pnew))
-    if "novalu" in EXP:
-        valu = []
     half = len(valu) // 2
     # the scores were written by the MFMAs just before this body: the first two MFMAs of
     # phase B (64 cycles) stand between them and the first instruction that reads them
@@ -255,8 +250,7 @@ def body(n, order, uid):
         for f in first_k:
             out += order.issue(("K", uid, f), [k_read(f, slot_k, RING)])
     # ---- end of B
-    if "norescale" not in EXP:
-        out += rescale_block(f"{uid}")
+    out += rescale_block(f"{uid}")
     out.append("s_waitcnt vmcnt(8)")
     out.append("s_barrier")
     # the eight loads of K(j+4), V(j+3): M0 (the LDS target) is written one MFMA ahead of its load
@@ -393,24 +387,9 @@ def pv_tail():
     return out
 
 
-def strip(lines):
-    if "nomfma" in EXP:
-        lines = [x for x in lines if not x.startswith("v_mfma")]
-    if "nolds" in EXP:
-        lines = [x for x in lines if not x.startswith("ds_read")]
-    if "noload" in EXP:
-        lines = [x for x in lines if not x.startswith("buffer_load")]
-    if "nobarrier" in EXP:
-        lines = [x for x in lines if x != "s_barrier"]
-    for e in EXP:
-        if e.startswith("no:"):
-            lines = [x for x in lines if not x.startswith(e[3:])]
-    return lines
-
-
 def emit(lines):
     print("    asm volatile(")
-    for ln in strip(lines):
+    for ln in lines:
         print(f'        "{ln}\\n"')
 
 

@@ -44,14 +44,19 @@ An operand is either "K" (k is the contiguous axis in memory: stage tile stored
 tile stored as it lies, [32 k][256 mn], fragments transposed on the way out with
 ds_read_b64_tr_b16).
 
+The family of tiles: B width 256 or 128 columns (rows are always 256) x ring depth 4, 5 or 6.
+A member is emitted only when it passes the validity filter (`valid`): its ring fits the
+160 KB of LDS of a compute unit, and accumulators plus fragment and address registers fit the
+512 registers of a wave.  Ring depth D changes the prefetch distance (loads of stage t+D are
+triggered by the barrier of stage t) and the unrolling (a multiple of D and of 2).  The
+descriptions above are written for depth 5.
+
 Run:  python3 gen_gemm256_loop.py > gemm256_loop.inc
 """
-import os
-
-EXP = os.environ.get("GEMM256_EXP", "")   # timing experiments only: noload, nomfma, noread, nobarrier
-
-NST = 5               # ring stages
+NST = 5               # ring stages (set per emitted function, like BW)
 UNROLL = 10           # stages per loop body: lcm(ring, pair issue, fragment set rotation)
+LDS_BYTES = 160 * 1024
+WAVE_REGISTERS = 512
 OPER = 16384          # bytes of the A tile (256 rows x 32 k); the B tile follows it in a stage buffer
 # Set per emitted function: the B tile is 256 or 128 columns wide.  The narrow form gives a
 # 256x128 workgroup tile (each wave 128x64 = 4x2 accumulators, 128 AGPRs) for problems
@@ -61,9 +66,21 @@ NBF = 4               # B fragments (32 columns each) per wave = BW / 64
 STAGE = 32768         # bytes per stage buffer = OPER + BW * 64
 
 
-def configure(bw):
-    global BW, NBF, STAGE
+def configure(bw, ring=5):
+    global BW, NBF, STAGE, NST, UNROLL
     BW, NBF, STAGE = bw, bw // 64, OPER + bw * 64
+    NST = ring
+    UNROLL = ring if ring % 2 == 0 else 2 * ring
+
+
+def valid(bw, ring):
+    """The validity filter of the tile family: LDS for the ring and for the epilogue's staging, which
+    reuses it (four waves x 128 rows x (bw + 16) bytes), and registers (accumulators in AGPRs; four fragment sets, read addresses for up to six ring
+    buffers, load offsets)."""
+    lds = max(ring * (OPER + bw * 64), 4 * 128 * (bw + 16))     # the ring, or the epilogue's staging area in its place
+    accumulators = 4 * (bw // 64) * 16
+    vgprs = 4 * (16 + 4 * (bw // 64)) + 24 + 4
+    return 2 <= ring <= 6 and lds <= LDS_BYTES and accumulators <= 256 and accumulators + vgprs <= WAVE_REGISTERS
 
 SET = {n: (32 * n, 32 * n + 16) for n in range(4)}   # fragment set -> (A base vgpr, B base vgpr)
 RA, RB = 192, 204
@@ -121,15 +138,17 @@ def trigger_group(kinds, t):
     for which in ("A", "B"):
         passes = 4 if which == "A" else NBF     # 4 KB (one 1 KB slot per wave) per pass
         if kinds[which] == "K":
-            if t % 2 == 0:
+            # stages 2m and 2m + 1 are the two halves of the same cache lines: the pair goes out
+            # together, at the barrier that frees the buffer of its second stage
+            if (t + NST - 1) % 2 == 0:
                 for p in range(passes):
-                    grp.append(load_instr(which, t + 4, p))
-                    grp.append(load_instr(which, t + 5, p, second_half=True))
+                    grp.append(load_instr(which, t + NST - 1, p))
+                    grp.append(load_instr(which, t + NST, p, second_half=True))
                 grp.append(dict(stage=None, lines=[f"v_add_u32 v{GOFF[which]}, 128, v{GOFF[which]}",
                                                    f"v_add_u32 v{GOFF2[which]}, 128, v{GOFF2[which]}"]))
         else:
             for p in range(passes):
-                grp.append(load_instr(which, t + 5, p))
+                grp.append(load_instr(which, t + NST, p))
             step = "%[ta]" if which == "A" else "%[tb]"
             grp.append(dict(stage=None, lines=[f"v_add_u32 v{GOFF[which]}, {step}, v{GOFF[which]}"]))
     return grp
@@ -208,10 +227,6 @@ def simulate(kinds):
     return pro, counts
 
 
-def drop(lines, prefix):
-    return [l for l in lines if not l.startswith(prefix)]
-
-
 def stage_iteration(mnem, kinds, t, vmcnt, extra=(), extra_mid=()):
     g, nxt = t % NST, (t + 1) % NST
     r0 = all_frag_reads(kinds, nxt, 0, (2 * t + 2) % 4)
@@ -229,14 +244,6 @@ def stage_iteration(mnem, kinds, t, vmcnt, extra=(), extra_mid=()):
     out.append("s_barrier")
     out += list(extra_mid)
     out += interleave(mfmas(mnem, (2 * t + 1) % 4), r1, this_first)
-    if "noload" in EXP:
-        out = [l for l in drop(drop(out, "buffer_load"), "s_add_u32 m0") if l != "s_nop 0"]
-    if "nomfma" in EXP:
-        out = drop(out, "v_mfma")
-    if "noread" in EXP:
-        out = drop(out, "ds_read")
-    if "nobarrier" in EXP:
-        out = drop(out, "s_barrier")
     return out
 
 
@@ -480,17 +487,28 @@ def emit(name, mnem, ka, kb):
     print("}\n")
 
 
+# The tile family: (B width, ring depth) -> stem of the emitted functions.  Every member that passes
+# `valid` is emitted and becomes a kernel variant the tuner can time (gemm.hip lists the codes).
+FAMILY = [(256, 5, "gemm256_loop"), (256, 4, "gemm256r4_loop"), (256, 6, "gemm256r6_loop"),
+          (128, 5, "gemm256x128_loop"), (128, 4, "gemm256x128r4_loop"), (128, 6, "gemm256x128r6_loop")]
+
+
 def main():
     print("// Generated by gen_gemm256_loop.py -- do not edit by hand.")
     print("// Main loops of the 256x256 and 256x128 GEMM kernels (the generator documents the schedule")
     print("// and the register map).\n")
-    for bw, stem in ((256, "gemm256_loop"), (128, "gemm256x128_loop")):
-        configure(bw)
+    for bw, ring, stem in FAMILY:
+        if not valid(bw, ring):
+            print(f"// {stem}: 256x{bw} tile with a ring of {ring} stages fails the validity filter "
+                  f"({ring * (OPER + bw * 64) // 1024} KB of LDS)\n")
+            continue
+        print(f"#define MHIP_HAVE_{stem.upper()} 1\n")
+        configure(bw, ring)
         for tname, mnem in (("bf16", "v_mfma_f32_32x32x16_bf16"), ("f16", "v_mfma_f32_32x32x16_f16")):
             for lname, ka, kb in (("nn", "K", "MN"), ("nt", "K", "K"), ("tn", "MN", "MN"), ("tt", "MN", "K")):
                 emit(f"{stem}_{lname}_{tname}", mnem, ka, kb)
     # streamed tiles: the 256x128 kernel as a persistent workgroup, for A with k contiguous
-    configure(128)
+    configure(128, 5)
     for tname, mnem in (("bf16", "v_mfma_f32_32x32x16_bf16"), ("f16", "v_mfma_f32_32x32x16_f16")):
         for lname, ka, kb in (("nn", "K", "MN"), ("nt", "K", "K")):
             emit_stream(f"gemm_stream_loop_{lname}_{tname}", mnem, ka, kb)

@@ -493,7 +493,7 @@ static void check_custom_call_types(const Op& op, const std::vector<TensorType>&
         std::vector<int64_t> want(xt.shape.begin(), xt.shape.end() - 1);
         want.push_back(down.shape[1]);
         if (op.out.shape != want) throw ParseError(where(op) + "the result shape is not [.., M, d2]");
-        if (cfg.get_bool("is_gated", false)) throw UnsupportedOp(where(op) + "gated feed-forward blocks are not supported");
+        // "is_gated" is read and ignored, as the reference's handler does (CustomCallHandlers.swift:871)
     } else if (op.target == "fused_scaled_dot_product_attention" && cfg.get_int_array("views", {}).empty()) {
         const TensorType& kt = in(1);
         const size_t r = xt.shape.size();
@@ -615,8 +615,6 @@ void compile(Executable& exe) {
                 throw UnsupportedOp(where(op) + "element type not supported");
             if (op.target == "fused_matmul_bias_activation" &&
                 !kActivation.count(parse_config(op.backend_config).get_string("activation", "none")))
-                throw UnsupportedOp(where(op) + "unknown activation");
-            if (op.target == "fused_ffn" && !kActivation.count(parse_config(op.backend_config).get_string("activation", "gelu")))
                 throw UnsupportedOp(where(op) + "unknown activation");
             check_custom_call_types(op, vt);
         } else {
@@ -819,8 +817,10 @@ static std::vector<DeviceTensor> run_ops(Executable& exe, const std::vector<Devi
                     const TensorType &up = in(1).type, &down = in(2).type;
                     const int64_t F = up.shape[1], d2 = down.shape[1];
                     DeviceTensor hidden = al.allocate(TensorType{{rows, F}, dt});
+                    // an activation name the handler does not know means no activation (CustomCallHandlers.swift:905)
+                    const std::string act_name = cfg.get_string("activation", "gelu");
                     RUN(mhip_gemm(s, in(0).data(), in(1).data(), nullptr, hidden.data(), rows, F, cols, 1, 0, 0, 0, 0, 0,
-                                  kActivation.at(cfg.get_string("activation", "gelu")), dt));
+                                  kActivation.count(act_name) ? kActivation.at(act_name) : MHIP_ACT_NONE, dt));
                     RUN(mhip_gemm(s, hidden.data(), in(2).data(), nullptr, out.data(), rows, d2, F, 1, 0, 0, 0, 0, 0, MHIP_ACT_NONE, dt));
                 } else if (op.target == "fused_layer_norm" || op.target == "fused_rms_norm") {
                     const auto axes = cfg.get_int_array("axes", {-1});
@@ -999,7 +999,7 @@ static void ensure_arena(Executable& exe, size_t bytes) {
 static bool direct_results(const Executable& exe) {
     size_t escaping = 0;
     for (auto& sl : exe.plan.slots) escaping += sl.escapes;
-    return escaping == exe.fn.returns.size() && env_flag("METALHLO_GRAPH_DIRECT_RESULTS", true);
+    return escaping == exe.fn.returns.size();
 }
 
 static bool capture_graph(Executable& exe, const std::vector<DeviceTensor>& inputs, Executable::CapturedGraph& out) {

@@ -633,9 +633,7 @@ static void launch_split(const RowLaunch& c, hipStream_t s, const T* xp, const T
         // a tensor small enough to sit in the L2s between two kernels: rows by XCD (see the kernel).
         // Not for large ones: eight separate windows of memory in flight instead of one cost the
         // [32768, 4096] benchmarks 4 to 17 % (softmax 0.80 -> 0.71 of the HBM peak, RMSNorm 0.79 -> 0.65).
-        const int xcd_mode = tune_int("MHIP_ROW_XCD", 1);          // 2 = never, 3 = whatever the size
-        const bool by_xcd = units % 8 == 0 && xcd_mode != 2 &&
-                            (xcd_mode == 3 || (int64_t)rows * cols * (int64_t)sizeof(T) <= (16 << 20));
+        const bool by_xcd = units % 8 == 0 && (int64_t)rows * cols * (int64_t)sizeof(T) <= (16 << 20);
         const int chunk = by_xcd ? -1 : 1;
         if (c.r == 2)
             hipLaunchKernelGGL((row_split_kernel<T, OP, NVS, WPR, 2>), dim3((unsigned)units), dim3(256), 0, s, xp, gp, bp, yp,
@@ -665,13 +663,6 @@ static int launch_row(hipStream_t s, const void* x, const void* g, const void* b
         RowLaunch c;
         if (forced) c = *forced;
         else if (!tuned_row_launch(OP, dtype, rows, cols, gp != nullptr, OP == kLayerNorm && bp != nullptr, &c)) c = RowLaunch();
-        if (!forced) {               // environment overrides, for experiments
-            c.kind = tune_int("MHIP_ROW_KIND", c.kind);
-            c.r = tune_int("MHIP_ROW_R", c.r);
-            c.per_cu = tune_int("MHIP_ROW_BLOCKS_PER_CU", c.per_cu);
-            const int o = tune_int("MHIP_ROW_ORDERED", 0);       // 1 = ordered, 2 = persistent
-            if (o) c.ordered = o == 1;
-        }
         // defaults (measured on [32768, 4096] bf16: ordered split launches run at the rate of a plain
         // copy; with both gamma and beta two rows per wave group keep the parameters' 16 KB per row
         // from falling out of the CU's vector cache; rows of up to 256 vectors are faster two at a
@@ -734,20 +725,17 @@ static int launch_gelu(hipStream_t s, const void* x, const void* bias, void* y, 
         // tiles of `tile_rows` rows x 256 vectors in address order (two rows measured fastest on
         // [32768, 4096]: 0.775 of the HBM peak against 0.70 for one row and 0.755 for four)
         const int64_t bpr = (nvec_row + 255) / 256;
-        int tile_rows = tune_int("MHIP_GELU_TILE_ROWS", 2);
-        tile_rows = tile_rows >= 4 ? 4 : tile_rows >= 2 ? 2 : 1;
+        constexpr int tile_rows = 2;
         const int64_t tiles = bpr * ((rows + tile_rows - 1) / tile_rows);
         if (tiles <= 0x7FFFFFFFLL) {
 #define MHIP_GELU_TILE(R)                                                                              \
     hipLaunchKernelGGL((bias_gelu_tile_kernel<T, R, EXACT>), dim3((unsigned)tiles), dim3(256), 0, s, static_cast<const T*>(x), \
                        static_cast<const T*>(bias), static_cast<T*>(y), rows, (int)nvec_row, (unsigned)bpr)
-            if (tile_rows == 1) MHIP_GELU_TILE(1);
-            else if (tile_rows == 2) MHIP_GELU_TILE(2);
-            else MHIP_GELU_TILE(4);
+            MHIP_GELU_TILE(2);
 #undef MHIP_GELU_TILE
         } else {      // more tiles than a grid holds: the grid-stride kernel
             const int64_t want = (nvec + 511) / 512;
-            const int64_t cap = (int64_t)compute_units() * tune_int("MHIP_GELU_BLOCKS_PER_CU", 64);
+            const int64_t cap = (int64_t)compute_units() * 64;
             const bool in_lds = bias && cols * sizeof(float) <= 48 * 1024;
             hipLaunchKernelGGL((bias_gelu_vec_kernel<T, EXACT>), dim3((unsigned)(want < cap ? want : cap)), dim3(256),
                                in_lds ? (size_t)cols * sizeof(float) : 0, s, static_cast<const T*>(x),

@@ -14,14 +14,17 @@
 // in a process-wide table that the entry points consult before their heuristics, and can be
 // saved to / loaded from a text file (MHIP_TUNING_DB names one to load at first use).  Entries
 // of other devices are kept and written back, never used.
+#include <dlfcn.h>
 #include <stdarg.h>
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
 
+#include <algorithm>
 #include <map>
 #include <mutex>
 #include <string>
+#include <vector>
 
 #include "gemm_common.h"
 
@@ -85,7 +88,7 @@ bool valid_choice(const char* line, const std::string& choice) {
     int a = 0, b = 0, c = 0, d = 0;
     if (!strncmp(line, "gemm ", 5)) {
         const int v = atoi(choice.c_str());
-        return v == 128 || v == 256 || v == 2560 || v == 2561 || v == 2562 || v == 2563;
+        return v == 128 || v == 256 || (v >= 2560 && v <= 2566);
     }
     if (!strncmp(line, "row ", 4))
         return sscanf(choice.c_str(), "%d %d %d %d", &a, &b, &c, &d) == 4 && (a == 1 || a == 2) && (b == 1 || b == 2) &&
@@ -118,13 +121,32 @@ int load_file(const char* path, bool quiet) {
     return st;
 }
 
-// False when there is nothing to look up (the common case: no key is built then).
+// The table that ships with the library: <directory of this shared object>/../tuning/<arch>_<CUs>.txt
+// (for the device in use), written by `python -m metalhlo_amd.tune` on such a device.
+std::string shipped_table_path() {
+    Dl_info info;
+    if (!dladdr(reinterpret_cast<const void*>(&shipped_table_path), &info) || !info.dli_fname) return "";
+    std::string dir = info.dli_fname;
+    const size_t slash = dir.rfind('/');
+    dir = slash == std::string::npos ? "." : dir.substr(0, slash);
+    std::string dev = device_key();
+    std::replace(dev.begin(), dev.end(), '/', '_');
+    return dir + "/../tuning/" + dev + ".txt";
+}
+
+// False when there is nothing to look up (no key is built then).  At first use the shipped table of
+// the device is loaded, then the file MHIP_TUNING_DB names (its entries win); MHIP_TUNING_DB=none
+// loads neither.
 bool have_entries() {
     std::lock_guard<std::mutex> lk(g_mu);
     if (!g_env_loaded) {
         g_env_loaded = true;
         const char* p = getenv("MHIP_TUNING_DB");
-        if (p && *p) load_file(p, true);
+        if (!p || strcmp(p, "none") != 0) {
+            const std::string shipped = shipped_table_path();
+            if (!shipped.empty()) load_file(shipped.c_str(), true);
+            if (p && *p) load_file(p, true);
+        }
     }
     return !g_table.empty();
 }
@@ -174,7 +196,7 @@ int tuned_gemm_variant(const GemmArgs& g, int64_t batch, int ta, int tb, int dty
     std::string c;
     if (!have_entries() || !lookup(gemm_key(g.M, g.N, g.K, batch, ta, tb, dtype), &c)) return 0;
     const int v = atoi(c.c_str());
-    return (v == 128 || v == 256 || v == 2560 || v == 2561 || v == 2562 || v == 2563) ? v : 0;
+    return (v == 128 || v == 256 || (v >= 2560 && v <= 2566)) ? v : 0;
 }
 
 bool tuned_row_launch(int op, int dtype, int64_t rows, int64_t cols, bool has_gamma, bool has_beta, RowLaunch* out) {
@@ -199,6 +221,19 @@ int tuned_attention_variant(int dtype, int64_t batch_heads, int64_t Sq, int64_t 
 
 using namespace mhip;
 
+// GEMM candidates a problem can run (the validity filter: shape, alignment, LDS and tile count rules of each kernel).
+static std::vector<int> gemm_candidates(const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype) {
+    std::vector<int> out;
+    for (int v : {128, 256, 2560, 2561, 2562, 2563, 2564, 2565, 2566}) {
+        if ((v == 2560 || v == 2566) && !gemm256_eligible(g, batch, trans_a, trans_b, dtype)) continue;
+        if ((v == 2561 || v == 2564 || v == 2565) && !gemm256_eligible(g, batch, trans_a, trans_b, dtype, 128)) continue;
+        if (v == 2562 && !gemm_stream_eligible(g, batch, trans_a, trans_b, dtype)) continue;
+        if (v == 2563 && !(gemm_split_shape(g, batch, nullptr) && gemm256_eligible(g, batch, trans_a, trans_b, dtype))) continue;
+        out.push_back(v);
+    }
+    return out;
+}
+
 extern "C" int mhip_gemm_autotune(void* stream, const void* a, const void* b, const void* bias, void* c,
                                   int64_t M, int64_t N, int64_t K, int64_t batch, int64_t stride_a,
                                   int64_t stride_b, int64_t stride_c, int trans_a, int trans_b,
@@ -215,25 +250,99 @@ extern "C" int mhip_gemm_autotune(void* stream, const void* a, const void* b, co
     g.M = (int)M; g.N = (int)N; g.K = (int)K;
     g.lda = (int)(trans_a ? M : K); g.ldb = (int)(trans_b ? K : N);
     g.sa = stride_a; g.sb = stride_b; g.sc = stride_c;
-    const int candidates[6] = {128, 256, 2560, 2561, 2562, 2563};
+    const std::vector<int> cand = gemm_candidates(g, batch, trans_a, trans_b, dtype);
+    std::vector<float> us(cand.size(), -1.f);
+    // two passes over the candidates, the better time of each counts: the first candidates of the
+    // first pass run on a device that is still raising its clocks
+    for (int pass = 0; pass < 2; pass++)
+        for (size_t i = 0; i < cand.size(); i++) {
+            g_forced_gemm = cand[i];
+            const float t_us = t.time(s, iters, [&] {
+                return mhip_gemm(stream, a, b, bias, c, M, N, K, batch, stride_a, stride_b, stride_c, trans_a, trans_b, activation, dtype);
+            });
+            g_forced_gemm = 0;
+            if (t_us < 0.f) return MHIP_ERR_LAUNCH;
+            if (us[i] < 0.f || t_us < us[i]) us[i] = t_us;
+        }
+    size_t best = 0;
+    for (size_t i = 1; i < cand.size(); i++)
+        if (us[i] < us[best]) best = i;
+    record(gemm_key(M, N, K, batch, trans_a, trans_b, dtype), std::to_string(cand[best]), us[best]);
+    if (out_variant) *out_variant = cand[best];
+    if (out_us) *out_us = us[best];
+    return MHIP_OK;
+}
+
+// The same search with every launch timed on its own as a model finds its operands: `flush` is
+// overwritten first (64 to 128 MB empty the L2s and leave most of the 256 MB memory-side cache, the
+// state of weights that were written a millisecond ago; 512 MB and more empty both), then A is
+// rewritten in place the way the kernel in front of a GEMM leaves its result, then one launch between
+// two events.  The median of `iters` such launches decides.  A GEMM in a loop of its own finds both
+// operands in the caches, which favours other tile widths and ring depths than a model does.
+extern "C" int mhip_gemm_autotune_in_model(void* stream, const void* a, const void* b, const void* bias, void* c,
+                                           int64_t M, int64_t N, int64_t K, int64_t batch, int64_t stride_a,
+                                           int64_t stride_b, int64_t stride_c, int trans_a, int trans_b,
+                                           int activation, int dtype, int iters, void* flush, int64_t flush_bytes,
+                                           int* out_variant, float* out_us) {
+    if (dtype != MHIP_BF16 && dtype != MHIP_F16)
+        return fail(MHIP_ERR_UNSUPPORTED, "mhip_gemm_autotune_in_model: only the 16-bit MFMA kernels have variants");
+    if (iters <= 0 || M <= 0 || N <= 0 || K <= 0 || batch <= 0 || !a || !b || !c || !flush || flush_bytes < (64ll << 20))
+        return fail(MHIP_ERR_INVALID_ARGUMENT, "mhip_gemm_autotune_in_model: bad argument (the flush buffer needs at least 64 MB)");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    Timer t;
+    if (!t.ok()) return fail(MHIP_ERR_LAUNCH, "mhip_gemm_autotune_in_model: cannot create events");
+    GemmArgs g{};
+    g.a = a; g.b = b; g.bias = bias; g.c = c;
+    g.M = (int)M; g.N = (int)N; g.K = (int)K;
+    g.lda = (int)(trans_a ? M : K); g.ldb = (int)(trans_b ? K : N);
+    g.sa = stride_a; g.sb = stride_b; g.sc = stride_c;
+    const int64_t a_bytes = (batch == 1 || stride_a == M * K) ? M * K * batch * 2 : M * K * 2;
     int best = 0;
     float best_us = 0.f;
-    for (int v : candidates) {
-        if (v == 2560 && !gemm256_eligible(g, batch, trans_a, trans_b, dtype)) continue;    // validity filter
-        if (v == 2561 && !gemm256_eligible(g, batch, trans_a, trans_b, dtype, 128)) continue;
-        if (v == 2562 && !gemm_stream_eligible(g, batch, trans_a, trans_b, dtype)) continue;
-        if (v == 2563 && !(gemm_split_shape(g, batch, nullptr) && gemm256_eligible(g, batch, trans_a, trans_b, dtype))) continue;
-        g_forced_gemm = v;
-        const float us = t.time(s, iters, [&] {
-            return mhip_gemm(stream, a, b, bias, c, M, N, K, batch, stride_a, stride_b, stride_c, trans_a, trans_b, activation, dtype);
-        });
-        g_forced_gemm = 0;
-        if (us < 0.f) return MHIP_ERR_LAUNCH;
-        if (!best || us < best_us) { best = v; best_us = us; }
+    std::vector<float> us(iters);
+    for (int v : gemm_candidates(g, batch, trans_a, trans_b, dtype)) {
+        for (int i = -1; i < iters; i++) {            // launch -1 is not counted
+            if (mhip_fill(stream, flush, flush_bytes / 4, (uint64_t)(i + 2), 4) != MHIP_OK) return MHIP_ERR_LAUNCH;
+            if (mhip_copy(stream, a, const_cast<void*>(a), a_bytes) != MHIP_OK) return MHIP_ERR_LAUNCH;
+            (void)hipEventRecord(t.e0, s);
+            g_forced_gemm = v;
+            const int st = mhip_gemm(stream, a, b, bias, c, M, N, K, batch, stride_a, stride_b, stride_c, trans_a, trans_b, activation, dtype);
+            g_forced_gemm = 0;
+            if (st != MHIP_OK) return st;
+            (void)hipEventRecord(t.e1, s);
+            float ms = 0.f;
+            if (hipEventSynchronize(t.e1) != hipSuccess || hipEventElapsedTime(&ms, t.e0, t.e1) != hipSuccess)
+                return fail(MHIP_ERR_LAUNCH, "autotune: timing failed: %s", hipGetErrorString(hipGetLastError()));
+            if (i >= 0) us[i] = ms * 1000.f;
+        }
+        std::sort(us.begin(), us.end());
+        const float med = us[iters / 2];
+        if (!best || med < best_us) { best = v; best_us = med; }
     }
     record(gemm_key(M, N, K, batch, trans_a, trans_b, dtype), std::to_string(best), best_us);
     if (out_variant) *out_variant = best;
     if (out_us) *out_us = best_us;
+    return MHIP_OK;
+}
+
+// A search that times something larger than one kernel (a whole forward pass, say) records its
+// result here: the GEMM problem's entry becomes `variant` (0 removes the entry).
+extern "C" int mhip_tuning_set_gemm(int64_t M, int64_t N, int64_t K, int64_t batch, int trans_a, int trans_b, int dtype,
+                                    int variant, float us) {
+    const std::string key = gemm_key(M, N, K, batch, trans_a, trans_b, dtype);
+    if (variant == 0) {
+        std::lock_guard<std::mutex> lk(g_mu);
+        g_table.erase(key);
+        g_env_loaded = true;
+        return MHIP_OK;
+    }
+    if (!valid_choice("gemm ", std::to_string(variant)))
+        return fail(MHIP_ERR_INVALID_ARGUMENT, "mhip_tuning_set_gemm: %d is no kernel variant", variant);
+    {
+        std::lock_guard<std::mutex> lk(g_mu);
+        g_env_loaded = true;
+    }
+    record(key, std::to_string(variant), us);
     return MHIP_OK;
 }
 
@@ -340,6 +449,7 @@ extern "C" int mhip_tuning_load(const char* path) {
 extern "C" void mhip_tuning_clear(void) {
     std::lock_guard<std::mutex> lk(g_mu);
     g_table.clear();
+    g_env_loaded = true;        // an explicit clear also cancels the automatic load at first use
 }
 
 extern "C" int mhip_tuning_count(void) {

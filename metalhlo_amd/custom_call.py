@@ -140,15 +140,16 @@ _ACTIVATION_ALIASES = {"gelu_approximate": "gelu", "geluApproximate": "gelu", "s
 
 def _ffn(operands, cfg):
     """act(x . up) . down, operands [x, up, down], config {activation: "gelu"}
-    (CustomCallHandlers.swift:849-910; "gelu_exact" is the erf form here)."""
+    (CustomCallHandlers.swift:849-910).  As there, "is_gated" is read and ignored and an activation
+    name the handler does not know means no activation; "gelu_exact" is the erf form here (the
+    reference computes the tanh form for it)."""
     _need(operands, 3)
     x, up, down = operands[:3]
     act = P.get_string(cfg, "activation", "gelu")
     act = _ACTIVATION_ALIASES.get(act, act)
     if act not in kernels.ACTIVATION_CODE:
-        raise CustomCallError(f"fused_ffn: unknown activation '{act}'")
-    if P.get_bool(cfg, "is_gated", False):
-        raise CustomCallError("fused_ffn: gated feed-forward blocks are not supported")
+        act = "none"
+    P.get_bool(cfg, "is_gated", False)          # reserved by the reference, ignored
     return [kernels.matmul(kernels.matmul(x, up, activation=act), down)]
 
 

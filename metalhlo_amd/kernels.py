@@ -348,6 +348,13 @@ def tuning_load(path: str) -> None:
     _lib.check(_lib.load().mhip_tuning_load(str(path).encode()))
 
 
+def shipped_tuning_table() -> str:
+    """Path of the table that ships for the current device (it may not exist); the kernel library
+    loads it by itself at first use unless the table was cleared before."""
+    import os
+    return os.path.join(os.path.dirname(os.path.abspath(__file__)), "tuning", tuning_device().replace("/", "_") + ".txt")
+
+
 def tuning_clear() -> None:
     _lib.load().mhip_tuning_clear()
 

@@ -343,7 +343,8 @@ def custom_call(target: str, operands, backend_config: str = "") -> np.ndarray:
             raise ValueError("expected 3 inputs")
         act = str(cfg.get("activation", "gelu"))                  # CustomCallHandlers.swift:870
         act = {"gelu_approximate": "gelu", "geluApproximate": "gelu", "swish": "silu"}.get(act, act)
-        return gemm(ACTIVATIONS[act](gemm(operands[0], operands[1])), operands[2])
+        # an unknown name means no activation (CustomCallHandlers.swift:905); "is_gated" is ignored (:871)
+        return gemm(ACTIVATIONS.get(act, ACTIVATIONS["none"])(gemm(operands[0], operands[1])), operands[2])
     if target == "fused_matmul_bias_activation":
         bias = operands[2] if len(operands) > 2 else None
         return matmul_bias_act(operands[0], operands[1], bias,

@@ -28,3 +28,19 @@ def oracle_c():
         import subprocess
         subprocess.check_call(["make", "-C", os.path.join(ROOT, "oracle"), "liboracle.so"])
     return ctypes.CDLL(path)
+
+
+@pytest.fixture(scope="module", autouse=True)
+def shipped_tuning_table(request):
+    """Every GPU test module starts in the product's configuration: the tuning table holds the
+    entries that ship for this device and nothing else (a test of the heuristics clears it)."""
+    if not any(item.get_closest_marker("gpu") for item in request.session.items if item.module is request.module):
+        yield
+        return
+    import os
+    from metalhlo_amd import kernels
+    kernels.tuning_clear()
+    path = kernels.shipped_tuning_table()
+    if os.path.exists(path):
+        kernels.tuning_load(path)
+    yield

@@ -171,8 +171,11 @@ def test_erf_gelu_one_pass_layer_norm_and_calls(sess):
     assert np.array_equal(t, r0 * r1) and np.array_equal(u, np.where(r1 < 0, r1, r0 * r1))
 
 
-@pytest.mark.parametrize("act", ["gelu", "gelu_exact", "relu", "silu"])
+@pytest.mark.parametrize("act", ["gelu", "gelu_exact", "relu", "silu", "mish"])
 def test_fused_ffn(sess, act):
+    """("mish": a name the reference's handler does not know, which there and here means no
+    activation, CustomCallHandlers.swift:905.  "gelu_exact" is the erf form: this build's choice, the
+    reference computes the tanh form under that name; the expectation is not pinned by the reference.)"""
     rng = np.random.default_rng(85)
     x = rng.standard_normal((4, 32, 64)).astype(np.float32)
     up = (0.2 * rng.standard_normal((64, 256))).astype(np.float32)
@@ -180,7 +183,7 @@ def test_fused_ffn(sess, act):
     exe = sess.compile(M.FFN_CUSTOM_CALL.replace("ACT", act))
     (got,) = sess.run(exe, [(x, "f32"), (up, "f32"), (down, "f32")])
     sess.lib.mhlo_executable_destroy(exe)
-    h = oracle.ACTIVATIONS[act](oracle.gemm(x.astype(np.float64).reshape(-1, 64), up.astype(np.float64)))
+    h = oracle.ACTIVATIONS.get(act, oracle.ACTIVATIONS["none"])(oracle.gemm(x.astype(np.float64).reshape(-1, 64), up.astype(np.float64)))
     close(got, oracle.gemm(h, down.astype(np.float64)).reshape(x.shape), 2e-5)
 
 

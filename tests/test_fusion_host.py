@@ -280,8 +280,10 @@ def test_calls_are_inlined(sess):
 def test_fused_ffn_custom_call(sess):
     assert ops(sess, M.FFN_CUSTOM_CALL.replace("ACT", "gelu")) == ["fused_ffn"]
     assert ops(sess, M.FFN_CUSTOM_CALL.replace("ACT", "gelu_exact")) == ["fused_ffn"]
-    with pytest.raises(capi.MHLOError):
-        ops(sess, M.FFN_CUSTOM_CALL.replace("ACT", "mish"))
+    # as in the reference's handler, an activation it does not know means none and "is_gated" is ignored
+    assert ops(sess, M.FFN_CUSTOM_CALL.replace("ACT", "mish")) == ["fused_ffn"]
+    assert ops(sess, M.FFN_CUSTOM_CALL.replace('\\"ACT\\"', '\\"gelu\\", \\"is_gated\\": true')) == ["fused_ffn"]
+    assert "is_gated" in M.FFN_CUSTOM_CALL.replace('\\"ACT\\"', '\\"gelu\\", \\"is_gated\\": true')
     with pytest.raises(capi.MHLOError):         # the down projection does not follow the up projection
         ops(sess, M.FFN_CUSTOM_CALL.replace("ACT", "gelu").replace("256x64xf32", "128x64xf32"))
 

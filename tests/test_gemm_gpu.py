@@ -197,10 +197,11 @@ BIG = [(4096, 3072, 32), (3585, 3848, 96), (4000, 3608, 160), (3600, 4104, 448),
 @pytest.mark.parametrize("layout", [(False, False), (False, True), (True, False), (True, True)],
                          ids=["nn", "nt", "tn", "tt"])
 @pytest.mark.parametrize("shape", BIG, ids=lambda s: "x".join(map(str, s)))
-@pytest.mark.parametrize("tile", ["2560", "2561"], ids=["256x256", "256x128"])
-def test_gemm_large_tiles(shape, layout, dtype, tile):
-    """The four-wave ring kernel on both of its tile widths (forced: also where the default picks
-    another kernel), ragged M and N included."""
+@pytest.mark.parametrize("tile", ["2560", "2561", "2564", "2565", "2566"],
+                         ids=["256x256", "256x128", "256x128-ring6", "256x128-ring4", "256x256-ring4"])
+def test_gemm_large_tiles(shape, layout, dtype, tile, lib):
+    """The four-wave ring kernel in every member of its generated family (tile width x ring depth;
+    forced: also where the default picks another kernel), ragged M and N included."""
     from metalhlo_amd import kernels
     M, N, K = shape
     ta, tb = layout
@@ -210,6 +211,9 @@ def test_gemm_large_tiles(shape, layout, dtype, tile):
     os.environ["MHIP_GEMM_TILE"] = tile
     try:
         c = kernels.matmul(a, b, bias, "relu", trans_a=ta, trans_b=tb)
+        # (operand rows that are not 16-byte aligned -- a transposed A with odd M -- run the scalar kernel)
+        aligned = (not ta or M % 8 == 0) and (tb or N % 8 == 0)
+        assert lib.mhip_gemm_last_variant() == (int(tile) if aligned else 0)
     finally:
         del os.environ["MHIP_GEMM_TILE"]
     assert c.shape == (M, N)
@@ -340,10 +344,12 @@ def test_gemm_split_is_the_default_from_a_third_round_on(lib, monkeypatch):
     """[8192, 768] x [768, 2304] and x [768, 3072] (more than two rounds of narrow tiles, a band of
     at most one round) take the split by default: same bits as forcing it."""
     from metalhlo_amd import kernels
+    kernels.tuning_clear()                 # the heuristic's choice, not a table entry's
     for N in (2304, 3072):
         a, b = _ab(8192, N, 768, torch.bfloat16, 67)
         monkeypatch.delenv("MHIP_GEMM_TILE", raising=False)
         c = kernels.matmul(a, b, None, "gelu")
+        assert lib.mhip_gemm_last_variant() == 2563
         monkeypatch.setenv("MHIP_GEMM_TILE", "2563")
         assert torch.equal(c, kernels.matmul(a, b, None, "gelu"))
 
@@ -457,7 +463,7 @@ def test_gemm_ring_kernel_takes_wide_and_deep_operands(lib):
         a = to_dev(rng.uniform(-1, 1, (M, K)), torch.bfloat16)
         b = to_dev(rng.uniform(-1, 1, (K, N)) * (K ** -0.5), torch.bfloat16)
         c = kernels.matmul(a, b)
-        assert lib.mhip_gemm_last_variant() in (2560, 2561, 2563), (M, N, K, lib.mhip_gemm_last_variant())
+        assert 2560 <= lib.mhip_gemm_last_variant() <= 2566, (M, N, K, lib.mhip_gemm_last_variant())
         rows = np.r_[0, 255, 256, M - 1, rng.integers(0, M, 12)]
         assert_close(c[rows], as_f64(a[rows]) @ as_f64(b), 2e-2, f"gemm {M}x{N}x{K}")
     # fp32 operands run none of the 16-bit variants

@@ -62,7 +62,8 @@ def test_gemm_autotune_picks_a_valid_variant_and_keeps_results():
         before = kernels.matmul(a, b, trans_b=tb)
         variant, us = kernels.autotune_matmul(a, b, trans_b=tb, iters=5)
         tiles = ((M + 255) // 256) * ((N + 255) // 256)
-        assert variant in ((128, 256, 2560, 2561) if tiles >= 192 else (128, 256, 2561)) and us > 0
+        ring = (2560, 2561, 2562, 2563, 2564, 2565, 2566)      # the generated family, streamed tiles, the column split
+        assert variant in ((128, 256) + ring if tiles >= 192 else (128, 256, 2561, 2564, 2565)) and us > 0
         tuned = kernels.matmul(a, b, trans_b=tb)
         # the tuned launch against the oracle on sampled rows ...
         rows = [0, 1, M // 2, M - 1]
@@ -126,3 +127,55 @@ def test_attention_autotune_matches_the_oracle(causal):
         # each variant on its own, forced through the table, against the same oracle
     assert kernels.tuning_count() == 2
     kernels.tuning_clear()
+
+
+@pytest.mark.gpu
+def test_gemm_autotune_in_model_and_the_shipped_table(lib, tmp_path):
+    """The in-model pass (caches emptied and A rewritten before every timed launch) records a valid
+    variant, and a table entry really moves the choice: for a GEMM of the GPT-2 forward pass the
+    heuristic's variant and a different variant named by a loaded table are both observed through
+    mhip_gemm_last_variant, with bit-identical results.  The table that ships with the library (when
+    there is one for this device) parses, names this device and only variants that exist."""
+    import ctypes as C
+    import os
+    import torch
+    from metalhlo_amd import kernels
+    kernels.tuning_clear()
+    torch.manual_seed(4)
+    M, N, K = 8192, 768, 768                                    # the attention output projection of GPT-2-small B8 S1024
+    a = (torch.rand(M, K, device="cuda") * 2 - 1).bfloat16()
+    b = ((torch.rand(K, N, device="cuda") * 2 - 1) * K ** -0.5).bfloat16()
+    plain = kernels.matmul(a, b)
+    default_variant = lib.mhip_gemm_last_variant()
+    assert default_variant in (128, 256, 2560, 2561, 2563)      # what the heuristic can choose
+    other = 2564 if default_variant != 2564 else 2561
+    table = tmp_path / "t.txt"
+    table.write_text(f"gemm {kernels.tuning_device()} {M} {N} {K} 1 0 0 3 = {other} @ 1.0\n")
+    kernels.tuning_load(table)
+    tuned = kernels.matmul(a, b)
+    assert lib.mhip_gemm_last_variant() == other
+    assert torch.equal(tuned, plain)
+    kernels.tuning_clear()
+    kernels.matmul(a, b)
+    assert lib.mhip_gemm_last_variant() == default_variant
+    # the in-model pass
+    flush = torch.empty(512 << 20, dtype=torch.uint8, device="cuda")
+    c = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    var, us = C.c_int(), C.c_float()
+    st = torch.cuda.current_stream().cuda_stream
+    assert lib.mhip_gemm_autotune_in_model(st, a.data_ptr(), b.data_ptr(), None, c.data_ptr(), M, N, K, 1, 0, 0, 0, 0, 0, 0, 3, 5,
+                                           flush.data_ptr(), flush.numel(), C.byref(var), C.byref(us)) == 0, lib.mhip_last_error()
+    assert var.value in (128, 256, 2561, 2564, 2565) and us.value > 0 and kernels.tuning_count() == 1
+    assert torch.equal(kernels.matmul(a, b), plain) and lib.mhip_gemm_last_variant() == var.value
+    assert torch.equal(a, a.clone())                             # (A was rewritten in place with its own values)
+    assert lib.mhip_gemm_autotune_in_model(st, a.data_ptr(), b.data_ptr(), None, c.data_ptr(), M, N, K, 1, 0, 0, 0, 0, 0, 0, 3, 5,
+                                           flush.data_ptr(), 1 << 20, C.byref(var), C.byref(us)) == 1      # flush buffer too small
+    kernels.tuning_clear()
+    shipped = kernels.shipped_tuning_table()
+    if os.path.exists(shipped):
+        kernels.tuning_load(shipped)
+        assert kernels.tuning_count() >= 5
+        text = open(shipped).read()
+        assert f"gemm {kernels.tuning_device()} 4096 4096 4096 1 0 0 3 = " in text
+        assert f"attention {kernels.tuning_device()} 3 128 4096 4096 128 1 = " in text
+        kernels.tuning_clear()
