@@ -41,17 +41,17 @@ PEAK_CLOCK_MHZ = 2400.0     # the shader clock the matrix peak is quoted at
 # HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by what the same
 # counter reads for the 'copy' workload (256 MiB in, 256 MiB out); see profiles/<workload>.txt.
 # TRAFFIC_COMMIT: the commit of this repository the counter runs were taken at (the profiles say so too).
-TRAFFIC_COMMIT = "aabac17"
+TRAFFIC_COMMIT = "59bc453"
 MEASURED_TRAFFIC = {
-    "gemm": 237446022,
-    "gemm_f32": 812745437,
-    "attention": 752630452,
-    "attention_full": 268946537,
-    "attention_f32": 1823030837,
-    "softmax": 536779900,
-    "layer_norm": 536936179,
-    "rms_norm": 536839114,
-    "bias_gelu": 536823915,
+    "gemm": 237460344,
+    "gemm_f32": 812973234,
+    "attention": 750479127,
+    "attention_full": 268940504,
+    "attention_f32": 1902930596,
+    "softmax": 536731572,
+    "layer_norm": 536898484,
+    "rms_norm": 536796223,
+    "bias_gelu": 536763241,
     "copy": 536870912,
 }
 
