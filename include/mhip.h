@@ -247,10 +247,34 @@ int mhip_iota(void* stream, void* y, int64_t outer, int64_t n, int64_t inner, in
 int mhip_argmax(void* stream, const void* x, void* out_idx, void* out_val, int64_t rows,
                 int64_t cols, int dtype, int idx_dtype);
 
+/* Rotary position embedding (FusedRoPEHandler, Compiler/CustomCallHandlers.swift:720-846):
+ * x and y are [rows, D] with rows = (leading axes) x S; the row's position is row % S.  With
+ * x = [x1 | x2] (halves of D / 2 elements): y = [x1 cos - x2 sin | x1 sin + x2 cos].
+ * freqs_are_angles = 0: freqs is [S, D], cos in the first half of a row and sin in the second
+ * (:783-808); 1: freqs is [S, D / 2] angles and cos / sin are computed (:809-812).  freqs has the
+ * element type of x.  F32 / F16 / BF16, fp32 arithmetic, one rounding. */
+int mhip_rope(void* stream, const void* x, const void* freqs, void* y, int64_t rows, int64_t S,
+              int64_t D, int freqs_are_angles, int dtype);
+
+/* A chain of elementwise operations in one launch (FusedElementwiseHandler,
+ * CustomCallHandlers.swift:927-1079): the running value starts as inputs[0]; ops[i] is either a
+ * mhip_unary_op code, applied to the running value, or MHIP_CHAIN_BINARY + a mhip_binary_op code,
+ * which combines the running value (left) with the next input (right).  The chain must consume
+ * exactly n_inputs inputs.  input_elements[k] is n, or 1 for an input used at every position.
+ * F32 / F16 / BF16; the whole chain is computed in fp32 and rounded once at the store (the
+ * reference's graph rounds after every operation). */
+#define MHIP_CHAIN_MAX_INPUTS 8
+#define MHIP_CHAIN_MAX_OPS 16
+#define MHIP_CHAIN_BINARY 100
+int mhip_elementwise_chain(void* stream, int n_inputs, const void* const* inputs,
+                           const int64_t* input_elements, int n_ops, const int* ops, void* y,
+                           int64_t n, int dtype);
+
 /* Unfused StableHLO glue for a host executor ------------------------------- */
 
 typedef enum { MHIP_UN_EXP = 0, MHIP_UN_TANH, MHIP_UN_RSQRT, MHIP_UN_SQRT, MHIP_UN_NEG,
-               MHIP_UN_LOGISTIC, MHIP_UN_ABS, MHIP_UN_LOG, MHIP_UN_ERF } mhip_unary_op;
+               MHIP_UN_LOGISTIC, MHIP_UN_ABS, MHIP_UN_LOG, MHIP_UN_ERF, MHIP_UN_SIN, MHIP_UN_COS,
+               MHIP_UN_FLOOR, MHIP_UN_CEIL } mhip_unary_op;
 typedef enum { MHIP_BIN_ADD = 0, MHIP_BIN_SUB, MHIP_BIN_MUL, MHIP_BIN_DIV, MHIP_BIN_MAX,
                MHIP_BIN_MIN, MHIP_BIN_POW } mhip_binary_op;
 typedef enum { MHIP_CMP_EQ = 0, MHIP_CMP_NE, MHIP_CMP_LT, MHIP_CMP_LE, MHIP_CMP_GT,

@@ -14,7 +14,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 ROOT = os.path.dirname(HERE)
 
-HIP_SOURCES = ["runtime.hip", "row_kernels.hip", "gemm.hip", "gemm_f32.hip", "gemm256.hip", "tuning.hip", "attention.hip", "attention_pipe.hip", "attention_f32.hip", "glue_kernels.hip", "elementwise.hip"]
+HIP_SOURCES = ["runtime.hip", "row_kernels.hip", "gemm.hip", "gemm_f32.hip", "gemm256.hip", "tuning.hip", "attention.hip", "attention_pipe.hip", "attention_f32.hip", "glue_kernels.hip", "elementwise.hip", "fused_misc.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=fast",

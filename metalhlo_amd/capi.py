@@ -153,8 +153,10 @@ class Session:
         return out
 
     def buffer(self, array: np.ndarray, element_type: str):
-        a = np.ascontiguousarray(array)
-        shape = (C.c_int64 * a.ndim)(*a.shape)
+        a = np.asarray(array)
+        if not a.flags.c_contiguous:
+            a = np.ascontiguousarray(a)
+        shape = (C.c_int64 * max(a.ndim, 1))(*a.shape)      # (a rank-0 array stays rank 0)
         buf = _vp()
         _check(self.lib.mhlo_buffer_create(self.client, a.ctypes.data_as(_vp), a.nbytes, shape, a.ndim,
                                            ELEMENT_TYPE[element_type], C.byref(buf)))

@@ -50,6 +50,10 @@ __global__ __launch_bounds__(256) void unary_kernel(const T* __restrict__ x, T* 
         case MHIP_UN_ABS: r = fabs(v); break;
         case MHIP_UN_LOG: r = log(v); break;
         case MHIP_UN_ERF: r = erf(v); break;
+        case MHIP_UN_SIN: r = sin(v); break;
+        case MHIP_UN_COS: r = cos(v); break;
+        case MHIP_UN_FLOOR: r = floor(v); break;
+        case MHIP_UN_CEIL: r = ceil(v); break;
         default: r = v; break;
     }
     Num<T>::st(y, i, r);
@@ -272,7 +276,7 @@ extern "C" int mhip_unary(void* stream, int op, const void* x, void* y, int64_t 
     if (n < 0) return fail(MHIP_ERR_INVALID_ARGUMENT, "%s: negative size", what);
     if (n == 0) return MHIP_OK;
     if (!x || !y) return fail(MHIP_ERR_INVALID_ARGUMENT, "%s: NULL pointer", what);
-    if (op < MHIP_UN_EXP || op > MHIP_UN_ERF) return fail(MHIP_ERR_INVALID_ARGUMENT, "%s: unknown op %d", what, op);
+    if (op < MHIP_UN_EXP || op > MHIP_UN_CEIL) return fail(MHIP_ERR_INVALID_ARGUMENT, "%s: unknown op %d", what, op);
     unsigned grid;
     if (ew_grid(n, &grid)) return MHIP_ERR_UNSUPPORTED;
     hipStream_t s = as_stream(stream);

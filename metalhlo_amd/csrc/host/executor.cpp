@@ -204,7 +204,7 @@ static size_t place_slots_recent(ArenaPlan& plan, bool escaping, size_t floor) {
 static const std::map<std::string, int> kUnary = {
     {"exponential", MHIP_UN_EXP}, {"tanh", MHIP_UN_TANH}, {"rsqrt", MHIP_UN_RSQRT}, {"sqrt", MHIP_UN_SQRT},
     {"negate", MHIP_UN_NEG}, {"logistic", MHIP_UN_LOGISTIC}, {"abs", MHIP_UN_ABS}, {"log", MHIP_UN_LOG},
-    {"erf", MHIP_UN_ERF}};
+    {"erf", MHIP_UN_ERF}, {"sine", MHIP_UN_SIN}, {"cosine", MHIP_UN_COS}, {"floor", MHIP_UN_FLOOR}, {"ceil", MHIP_UN_CEIL}};
 static const std::map<std::string, int> kBinary = {
     {"add", MHIP_BIN_ADD}, {"subtract", MHIP_BIN_SUB}, {"multiply", MHIP_BIN_MUL}, {"divide", MHIP_BIN_DIV},
     {"maximum", MHIP_BIN_MAX}, {"minimum", MHIP_BIN_MIN}, {"power", MHIP_BIN_POW}};
@@ -220,7 +220,32 @@ static const std::map<std::string, int> kActivation = {{"none", MHIP_ACT_NONE}, 
 // custom_call targets served by a kernel (Compiler/CustomCallHandlers.swift:75-89)
 static const char* kTargets[] = {"fused_scaled_dot_product_attention", "fused_layer_norm", "fused_rms_norm",
                                  "fused_softmax", "fused_gelu", "fused_matmul_bias_activation", "fused_ffn",
-                                 "fused_token_embedding"};
+                                 "fused_rope", "fused_elementwise", "fused_token_embedding"};
+
+// The operation list of a fused_elementwise call ("ops", or "operations": CustomCallHandlers.swift:941-943)
+// as codes for mhip_elementwise_chain, and the number of inputs the chain consumes.  The names are
+// the reference's (:969-1065): six binary operations and twelve unary ones.
+static std::vector<int> chain_ops(const Op& op, const Config& cfg, size_t* inputs_needed) {
+    static const std::map<std::string, int> binary = {{"add", MHIP_BIN_ADD}, {"subtract", MHIP_BIN_SUB}, {"multiply", MHIP_BIN_MUL},
+                                                      {"divide", MHIP_BIN_DIV}, {"maximum", MHIP_BIN_MAX}, {"minimum", MHIP_BIN_MIN}};
+    static const std::map<std::string, int> unary = {{"negate", MHIP_UN_NEG}, {"abs", MHIP_UN_ABS}, {"exponential", MHIP_UN_EXP},
+                                                     {"log", MHIP_UN_LOG}, {"sqrt", MHIP_UN_SQRT}, {"rsqrt", MHIP_UN_RSQRT},
+                                                     {"tanh", MHIP_UN_TANH}, {"logistic", MHIP_UN_LOGISTIC}, {"sine", MHIP_UN_SIN},
+                                                     {"cosine", MHIP_UN_COS}, {"floor", MHIP_UN_FLOOR}, {"ceil", MHIP_UN_CEIL}};
+    std::vector<std::string> names = cfg.get_string_array("ops");
+    if (names.empty()) names = cfg.get_string_array("operations");
+    if (names.empty()) throw ParseError("line " + std::to_string(op.line) + " (fused_elementwise): Missing 'ops' or 'operations' in the config");
+    if (names.size() > MHIP_CHAIN_MAX_OPS) throw UnsupportedOp("line " + std::to_string(op.line) + " (fused_elementwise): more than 16 operations in one chain");
+    std::vector<int> codes;
+    size_t need = 1;
+    for (auto& n : names) {
+        if (binary.count(n)) { codes.push_back(MHIP_CHAIN_BINARY + binary.at(n)); need++; }
+        else if (unary.count(n)) codes.push_back(unary.at(n));
+        else throw ParseError("line " + std::to_string(op.line) + " (fused_elementwise): Unsupported operation in fused chain: " + n);
+    }
+    if (inputs_needed) *inputs_needed = need;
+    return codes;
+}
 
 static std::string where(const Op& op) { return "line " + std::to_string(op.line) + " (stablehlo." + op.name + "): "; }
 
@@ -463,6 +488,27 @@ static void check_custom_call_types(const Op& op, const std::vector<TensorType>&
     const Config cfg = parse_config(op.backend_config);
     const TensorType& xt = in(0);
     const int64_t cols = xt.shape.empty() ? 1 : xt.shape.back();
+    if (op.target == "fused_rope") {
+        // x [.., S, D], freqs [S, D] (cos | sin) or [S, D / 2] (angles), leading axes of extent 1 allowed
+        // (CustomCallHandlers.swift:733-812); the third form there, separate cos and sin operands of
+        // another width, is not served
+        const TensorType& ft = in(1);
+        if (xt.shape.size() < 2 || cols % 2 != 0 || !(xt == op.out)) throw ParseError(where(op) + "expected x [.., S, D] with even D and a result of x's type");
+        const int64_t S = xt.shape[xt.shape.size() - 2], fd = ft.shape.empty() ? 0 : ft.shape.back();
+        if ((fd != cols && fd != cols / 2) || ft.numel() != S * fd)
+            throw UnsupportedOp(where(op) + "frequencies must be [S, D] (cos | sin) or [S, D / 2] (angles)");
+        return;
+    }
+    if (op.target == "fused_elementwise") {
+        size_t need = 0;
+        (void)chain_ops(op, cfg, &need);
+        if (need > MHIP_CHAIN_MAX_INPUTS) throw UnsupportedOp(where(op) + "more than 8 inputs in one chain");
+        if (op.operands.size() < need) throw ParseError(where(op) + "Not enough inputs for the operations of the chain");
+        for (size_t i = 0; i < need; i++)
+            if (in(i).numel() != op.out.numel() && in(i).numel() != 1)
+                throw UnsupportedOp(where(op) + "every input must have the result's shape or one element");
+        return;
+    }
     if (op.target == "fused_softmax" || op.target == "fused_gelu" || op.target == "fused_layer_norm" || op.target == "fused_rms_norm") {
         if (!(xt == op.out)) throw ParseError(where(op) + "the result type must be the input's");
         if (op.target == "fused_layer_norm" || op.target == "fused_rms_norm") {
@@ -608,7 +654,7 @@ void compile(Executable& exe) {
             if (!ok) throw UnsupportedOp(where(op) + "Unsupported custom call target: " + op.target);
             const size_t need = op.target == "fused_scaled_dot_product_attention" || op.target == "fused_layer_norm" || op.target == "fused_ffn" ||
                                         op.target == "fused_token_embedding" ? 3
-                              : op.target == "fused_rms_norm" || op.target == "fused_matmul_bias_activation" ? 2 : 1;
+                              : op.target == "fused_rms_norm" || op.target == "fused_matmul_bias_activation" || op.target == "fused_rope" ? 2 : 1;
             if (op.operands.size() < need)
                 throw ParseError(where(op) + "Invalid input count: expected " + std::to_string(need) + ", got " + std::to_string(op.operands.size()));
             if (!is_kernel_float(op.target == "fused_token_embedding" ? op.out.dtype : in(0).dtype))
@@ -797,6 +843,16 @@ static std::vector<DeviceTensor> run_ops(Executable& exe, const std::vector<Devi
                     const int64_t d = table.shape[1], p0 = cfg.get_int("first_position", 0);
                     RUN(mhip_embed_tokens(s, in(0).data(), in(1).data(), static_cast<const float*>(in(2).data()) + p0 * d, out.data(),
                                           ids.shape[0], ids.shape[1], d, table.shape[0], MHIP_F32, dt));
+                } else if (op.target == "fused_rope") {
+                    const int64_t S = xt.shape[xt.shape.size() - 2], fd = in(1).type.shape.back();
+                    RUN(mhip_rope(s, in(0).data(), in(1).data(), out.data(), rows, S, cols, fd == cols / 2 ? 1 : 0, dt));
+                } else if (op.target == "fused_elementwise") {
+                    size_t need = 0;
+                    const std::vector<int> codes = chain_ops(op, cfg, &need);
+                    std::vector<const void*> ptrs;
+                    std::vector<int64_t> counts;
+                    for (size_t i = 0; i < need; i++) { ptrs.push_back(in(i).data()); counts.push_back(in(i).type.numel()); }
+                    RUN(mhip_elementwise_chain(s, (int)need, ptrs.data(), counts.data(), (int)codes.size(), codes.data(), out.data(), cnt, dt));
                 } else if (op.target == "fused_softmax") {
                     int64_t axis = cfg.get_int("axis", -1);
                     if (axis < 0) axis += (int64_t)xt.shape.size();

@@ -102,11 +102,13 @@ struct Config {
     std::map<std::string, bool> boolean;
     std::map<std::string, std::string> str;
     std::map<std::string, std::vector<double>> arr;
+    std::map<std::string, std::vector<std::string>> sarr;
     double get_float(const std::string& k, double d) const;
     int64_t get_int(const std::string& k, int64_t d) const;
     bool get_bool(const std::string& k, bool d) const;
     std::string get_string(const std::string& k, const std::string& d) const;
     std::vector<int64_t> get_int_array(const std::string& k, const std::vector<int64_t>& d) const;
+    std::vector<std::string> get_string_array(const std::string& k) const { auto it = sarr.find(k); return it == sarr.end() ? std::vector<std::string>() : it->second; }
 };
 Config parse_config(const std::string& json);
 

@@ -819,9 +819,19 @@ Config parse_config(const std::string& j) {
         else if (j[i] == '[') {
             i++;
             std::vector<double> v;
+            std::vector<std::string> sv;
             for (;;) {
                 ws();
                 if (i < j.size() && j[i] == ']') { i++; break; }
+                if (i < j.size() && j[i] == '"') {          // an array of strings (the operation list of fused_elementwise)
+                    const size_t e3 = j.find('"', i + 1);
+                    if (e3 == std::string::npos) return empty;
+                    sv.push_back(j.substr(i + 1, e3 - i - 1));
+                    i = e3 + 1;
+                    ws();
+                    if (i < j.size() && j[i] == ',') i++;
+                    continue;
+                }
                 char* e2;
                 const double d = strtod(j.c_str() + i, &e2);
                 if (e2 == j.c_str() + i) return empty;
@@ -830,7 +840,12 @@ Config parse_config(const std::string& j) {
                 ws();
                 if (i < j.size() && j[i] == ',') i++;
             }
-            c.arr[key] = v;
+            if (!sv.empty()) {
+                if (!v.empty()) return empty;
+                c.sarr[key] = sv;
+            } else {
+                c.arr[key] = v;
+            }
         } else {
             char* e2;
             const double d = strtod(j.c_str() + i, &e2);

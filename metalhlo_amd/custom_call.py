@@ -153,6 +153,22 @@ def _ffn(operands, cfg):
     return [kernels.matmul(kernels.matmul(x, up, activation=act), down)]
 
 
+def _rope(operands, cfg):
+    """Rotary position embedding, operands [x, freqs] (CustomCallHandlers.swift:720-846)."""
+    _need(operands, 2)
+    return [kernels.rope(operands[0], operands[1])]
+
+
+def _elementwise(operands, cfg):
+    """A chain of elementwise operations, config {"ops": [...]} or {"operations": [...]}
+    (CustomCallHandlers.swift:927-1079)."""
+    ops = cfg.get("ops", cfg.get("operations"))
+    if not isinstance(ops, list) or not all(isinstance(o, str) for o in ops):
+        raise CustomCallError("Missing 'ops' or 'operations' in fused_elementwise config")
+    _need(operands, 1)
+    return [kernels.elementwise_chain(list(operands), ops)]
+
+
 def _matmul_bias_act(operands, cfg):
     _need(operands, 2)
     x, w = operands[:2]
@@ -179,6 +195,8 @@ class CustomCallRegistry:
             ("fused_gelu", _gelu),
             ("fused_matmul_bias_activation", _matmul_bias_act),
             ("fused_ffn", _ffn),
+            ("fused_rope", _rope),
+            ("fused_elementwise", _elementwise),
         ):
             self.register(name, fn)
 
@@ -203,5 +221,4 @@ shared = CustomCallRegistry()
 
 # Targets the reference registers that lie outside the attention / GEMM / row-kernel
 # path (CustomCallHandlers.swift:75-89); asking for them raises UnsupportedTarget.
-NOT_ON_PATH = ("fused_batch_norm", "fused_conv_bias_act", "fused_rope",
-               "fused_elementwise", "fused_depth_attention")
+NOT_ON_PATH = ("fused_batch_norm", "fused_conv_bias_act", "fused_depth_attention")

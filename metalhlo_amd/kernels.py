@@ -238,6 +238,57 @@ def add(a, b):
     return y
 
 
+def rope(x, freqs):
+    """Rotary position embedding: x [.., S, D]; freqs [S, D] (cos | sin halves) or [S, D / 2] (angles)."""
+    _dev(x, freqs)
+    lib = _lib.load()
+    if x.dim() < 2 or x.shape[-1] % 2 or freqs.dtype != x.dtype:
+        raise ValueError("rope needs x [.., S, D] with even D and freqs of x's element type")
+    S, D = x.shape[-2], x.shape[-1]
+    fd = freqs.shape[-1] if freqs.dim() else 0
+    if fd not in (D, D // 2) or freqs.numel() != S * fd:
+        raise ValueError("rope: freqs must be [S, D] or [S, D / 2]")
+    y = torch.empty_like(x)
+    _lib.check(lib.mhip_rope(_stream(), x.data_ptr(), freqs.data_ptr(), y.data_ptr(), x.numel() // D if D else 0, S, D,
+                             1 if fd == D // 2 else 0, _code(x)))
+    return y
+
+
+CHAIN_UNARY_CODE = {"exponential": 0, "tanh": 1, "rsqrt": 2, "sqrt": 3, "negate": 4, "logistic": 5, "abs": 6, "log": 7,
+                    "sine": 9, "cosine": 10, "floor": 11, "ceil": 12}
+CHAIN_BINARY_CODE = {"add": 100, "subtract": 101, "multiply": 102, "divide": 103, "maximum": 104, "minimum": 105}
+
+
+def elementwise_chain(inputs, ops):
+    """One launch for a chain of elementwise operations: the running value starts as inputs[0], a
+    binary operation takes the next input as its right operand, a unary one transforms the running
+    value.  Inputs have the result's shape (that of inputs[0]) or one element."""
+    import ctypes as C
+    _dev(*inputs)
+    lib = _lib.load()
+    codes = []
+    for name in ops:
+        if name in CHAIN_BINARY_CODE:
+            codes.append(CHAIN_BINARY_CODE[name])
+        elif name in CHAIN_UNARY_CODE:
+            codes.append(CHAIN_UNARY_CODE[name])
+        else:
+            raise ValueError(f"Unsupported operation in fused chain: {name}")
+    need = 1 + sum(c >= 100 for c in codes)
+    if len(inputs) < need:
+        raise ValueError("Not enough inputs for the operations of the chain")
+    inputs = list(inputs[:need])
+    if any(t.dtype != inputs[0].dtype for t in inputs):
+        raise ValueError("every input must have one element type")
+    shape = max((t.shape for t in inputs), key=lambda sh: int(torch.Size(sh).numel()))
+    y = torch.empty(shape, dtype=inputs[0].dtype, device=inputs[0].device)
+    ptrs = (C.c_void_p * need)(*[t.data_ptr() for t in inputs])
+    counts = (C.c_int64 * need)(*[t.numel() for t in inputs])
+    arr = (C.c_int32 * len(codes))(*codes)
+    _lib.check(lib.mhip_elementwise_chain(_stream(), need, ptrs, counts, len(codes), arr, y.data_ptr(), y.numel(), _code(y)))
+    return y
+
+
 def convert(x, dtype):
     _dev(x)
     lib = _lib.load()

@@ -34,6 +34,12 @@ in tests/test_oracle.py):
                       beyond these is unpinned by the reference itself.
 * gpt2_forward      — composition of the above; parity unpinned by any
                       reference-held vector (the reference publishes none).
+* rope              — equals the complex product (x1 + i x2) e^{i theta}, preserves
+                      the norm of every rotated pair, zero angle is the identity,
+                      a quarter turn gives (-x2, x1), angles add under composition.
+* elementwise_chain — each operation against the NumPy function of its name; the
+                      reference's own example add -> multiply
+                      (CustomCallHandlers.swift:950-953).
 """
 from __future__ import annotations
 
@@ -303,6 +309,59 @@ def attention_rows(q, k, v, rows, scale=None, is_causal=False) -> np.ndarray:
 
 
 # --------------------------------------------------------------------------
+# rotary position embedding and elementwise chains
+# --------------------------------------------------------------------------
+def rope(x, freqs) -> np.ndarray:
+    """Compiler/CustomCallHandlers.swift:733-846: x [.., S, D] is split into halves x1 | x2 along the
+    last axis; freqs is [S, D] with cos in the first half of a row and sin in the second (:783-808),
+    or [S, D / 2] angles (:809-812); result [x1 cos - x2 sin | x1 sin + x2 cos]."""
+    x = np.asarray(x, dtype=np.float64)
+    f = np.asarray(freqs, dtype=np.float64)
+    d = x.shape[-1]
+    h = d // 2
+    if d % 2 or x.ndim < 2:
+        raise ValueError("x must be [.., S, D] with even D")
+    f = f.reshape(-1, f.shape[-1])
+    if f.shape[0] != x.shape[-2]:
+        raise ValueError("freqs must have one row per position")
+    if f.shape[1] == d:
+        c, s = f[:, :h], f[:, h:]
+    elif f.shape[1] == h:
+        c, s = np.cos(f), np.sin(f)
+    else:
+        raise ValueError("freqs must be [S, D] or [S, D / 2]")
+    x1, x2 = x[..., :h], x[..., h:]
+    return np.concatenate([x1 * c - x2 * s, x1 * s + x2 * c], axis=-1)
+
+
+CHAIN_BINARY = {"add": np.add, "subtract": np.subtract, "multiply": np.multiply, "divide": np.divide,
+                "maximum": np.maximum, "minimum": np.minimum}
+CHAIN_UNARY = {"negate": np.negative, "abs": np.abs, "exponential": np.exp, "log": np.log, "sqrt": np.sqrt,
+               "rsqrt": lambda v: 1.0 / np.sqrt(v), "tanh": np.tanh, "logistic": lambda v: 1.0 / (1.0 + np.exp(-v)),
+               "sine": np.sin, "cosine": np.cos, "floor": np.floor, "ceil": np.ceil}
+
+
+def elementwise_chain(inputs, ops) -> np.ndarray:
+    """CustomCallHandlers.swift:927-1079: the running value starts as inputs[0]; a binary operation
+    takes the next input as its right operand, a unary one transforms the running value."""
+    if not ops:
+        raise ValueError("No operations to fuse")
+    cur = np.asarray(inputs[0], dtype=np.float64)
+    k = 1
+    for name in ops:
+        if name in CHAIN_BINARY:
+            if k >= len(inputs):
+                raise ValueError(f"Not enough inputs for {name} operation")
+            cur = CHAIN_BINARY[name](cur, np.asarray(inputs[k], dtype=np.float64))
+            k += 1
+        elif name in CHAIN_UNARY:
+            cur = CHAIN_UNARY[name](cur)
+        else:
+            raise ValueError(f"Unsupported operation in fused chain: {name}")
+    return cur
+
+
+# --------------------------------------------------------------------------
 # operator-level dispatch: custom_call target + JSON backend_config
 # --------------------------------------------------------------------------
 def custom_call(target: str, operands, backend_config: str = "") -> np.ndarray:
@@ -338,6 +397,15 @@ def custom_call(target: str, operands, backend_config: str = "") -> np.ndarray:
         # tanh form whatever `approximate` says (CustomCallHandlers.swift:694-707); "erf": true is this
         # build's mark for a decomposed erf GELU and means the exact function
         return gelu_erf(operands[0]) if cfg.get("erf") is True else gelu_tanh(operands[0])
+    if target == "fused_rope":
+        if len(operands) < 2:
+            raise ValueError("expected 2 inputs")
+        return rope(operands[0], operands[1])
+    if target == "fused_elementwise":
+        ops = cfg.get("ops", cfg.get("operations"))               # CustomCallHandlers.swift:941-943
+        if not isinstance(ops, list):
+            raise ValueError("Missing 'ops' or 'operations' in fused_elementwise config")
+        return elementwise_chain(operands, ops)
     if target == "fused_ffn":
         if len(operands) < 3:
             raise ValueError("expected 3 inputs")

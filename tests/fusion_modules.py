@@ -366,3 +366,25 @@ def embedding(B=2, S=16, d=64, vocab=50, n_pos=24, dtype="bf16", first=0, ids_ty
         last = "%h"
     L.append(f"  return {last}, %tok : {out_t}, {x3f} }}" if keep_tokens else f"  return {last} : {out_t} }}")
     return "\n".join(L)
+
+
+def rope_call(shape=(2, 3, 16, 32), freq_cols=32, dtype="f32"):
+    """custom_call @fused_rope: x [.., S, D], frequencies [S, D] (cos | sin) or [S, D / 2] (angles)."""
+    t = "x".join(map(str, shape)) + "x" + dtype
+    f = f"{shape[-2]}x{freq_cols}x{dtype}"
+    return f"""func.func @main(%x: tensor<{t}>, %f: tensor<{f}>) -> tensor<{t}> {{
+  %r = stablehlo.custom_call @fused_rope(%x, %f) {{backend_config = "{{}}"}} : (tensor<{t}>, tensor<{f}>) -> tensor<{t}>
+  return %r : tensor<{t}> }}"""
+
+
+def elementwise_call(ops, n_inputs, shape=(6, 40), dtype="f32", key="ops", scalar_inputs=()):
+    """custom_call @fused_elementwise with the operation list under `key`; inputs listed in
+    `scalar_inputs` are rank-0 tensors."""
+    t = "x".join(map(str, shape)) + "x" + dtype
+    types = [f"tensor<{dtype}>" if i in scalar_inputs else f"tensor<{t}>" for i in range(n_inputs)]
+    args = ", ".join(f"%a{i}: {ty}" for i, ty in enumerate(types))
+    names = ", ".join(f"%a{i}" for i in range(n_inputs))
+    cfg = '{\\"' + key + '\\": [' + ", ".join('\\"' + o + '\\"' for o in ops) + "]}"
+    return f"""func.func @main({args}) -> tensor<{t}> {{
+  %r = stablehlo.custom_call @fused_elementwise({names}) {{backend_config = "{cfg}"}} : ({", ".join(types)}) -> tensor<{t}>
+  return %r : tensor<{t}> }}"""

@@ -206,3 +206,90 @@ def test_token_embedding(sess, dtype, first, d):
         assert np.array_equal(a, oracle.bf16_round_bits(exp))
     else:
         assert np.array_equal(np.asarray(a, dtype=np.float32), exp.astype({"f32": np.float32, "f16": np.float16}[dtype]).astype(np.float32))
+
+
+def _to(a, dtype):
+    """numpy float -> (array, element type name) as Session.run takes it, rounded to `dtype`."""
+    if dtype == "f32":
+        return np.asarray(a, np.float32), "f32"
+    if dtype == "bf16":
+        return oracle.bf16_round_bits(np.asarray(a, np.float32)).reshape(np.shape(a)), "bf16"
+    return np.asarray(a, np.float16), "f16"
+
+
+def _from(a, dtype):
+    return oracle.bf16_bits_to_f32(a).astype(np.float64) if dtype == "bf16" else np.asarray(a, np.float64)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16", "f16"])
+@pytest.mark.parametrize("shape,table", [((2, 3, 16, 32), True), ((2, 3, 16, 32), False), ((1, 5, 9, 6), False), ((24, 128), True),
+                                         ((4, 2, 33, 64), False)],
+                         ids=["table", "angles", "odd-half", "rank2", "ragged-seq"])
+def test_fused_rope(sess, shape, table, dtype):
+    """Rotary position embedding through the C API against the oracle: cos | sin table and angle
+    forms, half widths that are no whole 16-byte vectors, every element type."""
+    rng = np.random.default_rng(91)
+    S, D = shape[-2], shape[-1]
+    x = rng.standard_normal(shape)
+    th = rng.uniform(-3, 3, (S, D // 2))
+    f = np.concatenate([np.cos(th), np.sin(th)], -1) if table else th
+    (xa, _), (fa, _) = _to(x, dtype), _to(f, dtype)
+    exe = sess.compile(M.rope_call(shape, f.shape[-1], dtype))
+    (got,) = sess.run(exe, [(xa, dtype), (fa, dtype)])
+    sess.lib.mhlo_executable_destroy(exe)
+    exp = oracle.rope(_from(xa, dtype), _from(fa, dtype))
+    close(_from(got, dtype), exp, 1e-5 if dtype == "f32" else 2e-2)
+    if dtype == "f32":       # a rotation: every pair keeps its norm
+        g = np.asarray(got, np.float64)
+        h = D // 2
+        assert np.allclose(g[..., :h] ** 2 + g[..., h:] ** 2, x[..., :h].astype(np.float32).astype(np.float64) ** 2 +
+                           x[..., h:].astype(np.float32).astype(np.float64) ** 2, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16", "f16"])
+@pytest.mark.parametrize("ops,n_in,scalars,shape", [
+    (["add", "multiply"], 3, (), (6, 40)),                       # the reference's example
+    (["tanh", "add", "negate", "abs"], 2, (), (6, 40)),
+    (["multiply", "exponential", "logistic"], 2, (1,), (6, 40)),   # a rank-0 right operand
+    (["maximum", "minimum", "subtract", "divide"], 5, (), (3, 7)),  # no whole vectors: the scalar form
+    (["abs", "sqrt", "rsqrt", "log"], 1, (), (5, 8)),
+    (["sine", "cosine", "floor", "ceil"], 1, (), (4, 16)),
+], ids=["add-mul", "unary-mix", "scalar-rhs", "five-inputs", "roots", "trig-round"])
+def test_fused_elementwise(sess, ops, n_in, scalars, shape, dtype):
+    """Elementwise chains in one launch against the oracle (fp32 chain, one rounding at the store;
+    the bf16 / f16 bar is the per-operator 2e-2)."""
+    rng = np.random.default_rng(93)
+    ins = []
+    for i in range(n_in):
+        a = rng.uniform(0.5, 2.0, () if i in scalars else shape) * (1 if ops[0] in ("abs", "sqrt") or i else rng.choice([-1, 1], shape))
+        ins.append(_to(a, dtype))
+    text = M.elementwise_call(ops, n_in, shape, dtype, scalar_inputs=scalars)
+    exe = sess.compile(text)
+    (got,) = sess.run(exe, [(a, t) for a, t in ins])
+    sess.lib.mhlo_executable_destroy(exe)
+    exp = oracle.elementwise_chain([_from(a, dtype) for a, _ in ins], ops)
+    exp = np.broadcast_to(exp, shape)
+    g = _from(got, dtype)
+    if ops[-1] in ("floor", "ceil"):      # integers: a last-bit difference in front of the rounding may move one
+        assert np.mean(g == exp) > 0.98 and np.max(np.abs(g - exp)) <= 1.0
+    else:
+        close(g, exp, 1e-5 if dtype == "f32" else 2e-2)
+
+
+def test_trig_and_rounding_operations_of_the_front_end(sess):
+    """stablehlo.sine / cosine / floor / ceil as plain operations (they came with fused_elementwise)."""
+    text = """func.func @main(%x: tensor<4x8xf32>) -> (tensor<4x8xf32>, tensor<4x8xf32>) {
+      %0 = stablehlo.sine %x : tensor<4x8xf32>
+      %1 = stablehlo.cosine %x : tensor<4x8xf32>
+      %2 = stablehlo.multiply %0, %1 : tensor<4x8xf32>
+      %3 = stablehlo.floor %x : tensor<4x8xf32>
+      %4 = stablehlo.ceil %x : tensor<4x8xf32>
+      %5 = stablehlo.subtract %4, %3 : tensor<4x8xf32>
+      return %2, %5 : tensor<4x8xf32>, tensor<4x8xf32> }"""
+    x = np.random.default_rng(95).uniform(-4, 4, (4, 8)).astype(np.float32)
+    x[0, :3] = [-1.0, 0.0, 2.0]
+    exe = sess.compile(text)
+    a, b = sess.run(exe, [(x, "f32")])
+    sess.lib.mhlo_executable_destroy(exe)
+    close(a, np.sin(x.astype(np.float64)) * np.cos(x.astype(np.float64)), 1e-5)
+    assert np.array_equal(b, np.ceil(x) - np.floor(x))

@@ -340,3 +340,38 @@ def test_token_and_position_embedding_is_one_call(sess):
         assert ops(sess, M.embedding()) == ["gather", "slice", "broadcast_in_dim", "add", "convert"]
     finally:
         del os.environ["METALHLO_DISABLED_PASSES"]
+
+
+def test_rope_and_elementwise_custom_calls_compile_and_reject(sess):
+    """fused_rope and fused_elementwise (Compiler/CustomCallHandlers.swift:720-846, 927-1079): accepted forms and
+    the handlers' own error cases, all decided at compile time."""
+    assert ops(sess, M.rope_call()) == ["fused_rope"]
+    assert ops(sess, M.rope_call(freq_cols=16)) == ["fused_rope"]
+    assert ops(sess, M.rope_call(shape=(16, 32), dtype="bf16")) == ["fused_rope"]
+    with pytest.raises(capi.MHLOError):          # an odd last axis cannot be split into halves
+        ops(sess, M.rope_call(shape=(2, 16, 33), freq_cols=33))
+    with pytest.raises(capi.MHLOError):          # frequencies of another width (the separate cos / sin form) are not served
+        ops(sess, M.rope_call(freq_cols=8))
+    with pytest.raises(capi.MHLOError) as e:     # one operand: CustomCallError.invalidInputCount(expected: 2, ...)
+        ops(sess, M.rope_call().replace("(%x, %f)", "(%x)").replace("(tensor<2x3x16x32xf32>, tensor<16x32xf32>)", "(tensor<2x3x16x32xf32>)"))
+    assert "expected 2" in str(e.value)
+    assert ops(sess, M.elementwise_call(["add", "multiply"], 3)) == ["fused_elementwise"]
+    assert ops(sess, M.elementwise_call(["tanh", "add", "negate"], 2, key="operations")) == ["fused_elementwise"]
+    assert ops(sess, M.elementwise_call(["multiply", "exponential"], 2, dtype="bf16", scalar_inputs=(1,))) == ["fused_elementwise"]
+    with pytest.raises(capi.MHLOError) as e:
+        ops(sess, M.elementwise_call(["add", "atan2"], 3))
+    assert "Unsupported operation in fused chain: atan2" in str(e.value)
+    with pytest.raises(capi.MHLOError) as e:
+        ops(sess, M.elementwise_call(["add", "multiply"], 2))
+    assert "Not enough inputs" in str(e.value)
+    with pytest.raises(capi.MHLOError) as e:
+        ops(sess, M.elementwise_call(["add"], 2).replace("ops", "steps"))
+    assert "Missing 'ops' or 'operations'" in str(e.value)
+    # sine, cosine, floor and ceil are also plain operations of the front end now
+    text = """func.func @main(%x: tensor<8xf32>) -> tensor<8xf32> {
+      %0 = stablehlo.sine %x : tensor<8xf32>
+      %1 = stablehlo.cosine %0 : tensor<8xf32>
+      %2 = stablehlo.floor %1 : tensor<8xf32>
+      %3 = stablehlo.ceil %2 : tensor<8xf32>
+      return %3 : tensor<8xf32> }"""
+    assert ops(sess, text) == ["sine", "cosine", "floor", "ceil"]

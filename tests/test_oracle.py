@@ -160,7 +160,7 @@ def test_custom_call_dispatch_contract():
     with pytest.raises(ValueError):
         oracle.custom_call("fused_layer_norm", [q, k], "")
     with pytest.raises(KeyError):
-        oracle.custom_call("fused_rope", [q], "")
+        oracle.custom_call("fused_depth_attention", [q], "")
 
 
 # ---------------------------------------------------------------- C restatement vs float64 closed forms
@@ -391,3 +391,57 @@ def test_gelu_erf_is_the_exact_gelu():
     assert np.max(np.abs(oracle.gelu_erf(x) - oracle.gelu_tanh(x))) > 1e-4
     assert np.allclose(oracle.custom_call("fused_gelu", [x], '{"approximate": false, "erf": true}'), oracle.gelu_erf(x))
     assert np.allclose(oracle.custom_call("fused_gelu", [x], '{"approximate": false}'), oracle.gelu_tanh(x))
+
+
+def test_rope_is_a_rotation():
+    """Pins oracle.rope without retyping it: the half-split rotation equals the complex product
+    (x1 + i x2) e^{i theta}; every rotated pair keeps its norm; zero angles are the identity; a
+    quarter turn gives (-x2, x1); rotating by a then by b is rotating by a + b; a table of
+    cos | sin halves gives what the angles give; a transposed sign or swapped halves fail."""
+    rng = np.random.default_rng(201)
+    B, H, S, D = 2, 3, 7, 10
+    h = D // 2
+    x = rng.standard_normal((B, H, S, D))
+    th = rng.uniform(-3, 3, (S, h))
+    got = oracle.rope(x, th)
+    z = (x[..., :h] + 1j * x[..., h:]) * np.exp(1j * th)
+    assert np.allclose(got[..., :h], z.real, atol=1e-14) and np.allclose(got[..., h:], z.imag, atol=1e-14)
+    assert np.allclose(got[..., :h] ** 2 + got[..., h:] ** 2, x[..., :h] ** 2 + x[..., h:] ** 2, atol=1e-13)
+    assert np.array_equal(oracle.rope(x, np.zeros((S, h))), x)
+    q = oracle.rope(x, np.full((S, h), np.pi / 2))
+    assert np.allclose(q[..., :h], -x[..., h:], atol=1e-15) and np.allclose(q[..., h:], x[..., :h], atol=1e-15)
+    th2 = rng.uniform(-3, 3, (S, h))
+    assert np.allclose(oracle.rope(oracle.rope(x, th), th2), oracle.rope(x, th + th2), atol=1e-13)
+    table = np.concatenate([np.cos(th), np.sin(th)], axis=-1)          # [S, D]: cos | sin
+    assert np.allclose(oracle.rope(x, table), got, atol=1e-15)
+    assert np.allclose(oracle.custom_call("fused_rope", [x, th], "{}"), got)
+    wrong_sign = np.concatenate([x[..., :h] * np.cos(th) + x[..., h:] * np.sin(th),
+                                 -x[..., :h] * np.sin(th) + x[..., h:] * np.cos(th)], axis=-1)
+    assert np.max(np.abs(wrong_sign - got)) > 0.1
+    interleaved = x.reshape(B, H, S, h, 2)                                # the pairing (2i, 2i+1) is NOT what the handler does
+    assert np.max(np.abs(np.stack([interleaved[..., 0] * np.cos(th) - interleaved[..., 1] * np.sin(th),
+                                   interleaved[..., 0] * np.sin(th) + interleaved[..., 1] * np.cos(th)], -1).reshape(x.shape) - got)) > 0.1
+    with pytest.raises(ValueError):
+        oracle.rope(x, np.zeros((S, 3)))
+
+
+def test_elementwise_chain_semantics():
+    """Pins oracle.elementwise_chain: the reference's example (add then multiply with three inputs,
+    CustomCallHandlers.swift:950-953), every operation against a closed value, unary operations
+    consuming no input, errors for a missing input or an unknown name."""
+    a, b, c = np.array([1.0, -2.0, 3.0]), np.array([0.5, 0.5, 0.5]), np.array([2.0, 4.0, -1.0])
+    assert np.array_equal(oracle.elementwise_chain([a, b, c], ["add", "multiply"]), (a + b) * c)
+    assert np.array_equal(oracle.elementwise_chain([a, b], ["subtract", "negate", "abs"]), np.abs(-(a - b)))
+    assert np.array_equal(oracle.elementwise_chain([a, b, c], ["maximum", "minimum"]), np.minimum(np.maximum(a, b), c))
+    assert np.allclose(oracle.elementwise_chain([np.array([4.0])], ["sqrt", "rsqrt", "log", "exponential"]), [1 / np.sqrt(2.0)])
+    assert np.allclose(oracle.elementwise_chain([np.array([0.0])], ["logistic", "tanh", "sine", "cosine"]), [np.cos(np.sin(np.tanh(0.5)))])
+    assert np.array_equal(oracle.elementwise_chain([np.array([1.5, -1.5]), np.array([2.0, 2.0])], ["divide", "floor"]), [0.0, -1.0])
+    assert np.array_equal(oracle.elementwise_chain([np.array([0.2, -0.2])], ["ceil"]), [1.0, -0.0])
+    assert np.array_equal(oracle.custom_call("fused_elementwise", [a, b, c], '{"ops": ["add", "multiply"]}'), (a + b) * c)
+    assert np.array_equal(oracle.custom_call("fused_elementwise", [a, b], '{"operations": ["multiply"]}'), a * b)
+    with pytest.raises(ValueError):
+        oracle.elementwise_chain([a], ["add"])
+    with pytest.raises(ValueError):
+        oracle.elementwise_chain([a, b], ["atan2"])
+    with pytest.raises(ValueError):
+        oracle.custom_call("fused_elementwise", [a, b], "{}")
