@@ -400,6 +400,7 @@ static int launch_mfma(hipStream_t s, GemmArgs g, int64_t batch) {
 // gemm256.hip: 4-wave 256x256 kernel with a hand-scheduled main loop.
 bool gemm256_eligible(const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype, int bw = 256, bool any_tile_count = false);
 int launch_gemm256(hipStream_t s, const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype, int bw = 256, int ring = 5);
+bool gemm384_activation_ok(int act);
 bool gemm_stream_eligible(const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype);
 int launch_gemm_stream(hipStream_t s, const GemmArgs& g, int trans_b, int dtype);
 // gemm_f32.hip: fp32 operands on the fp32 matrix instruction, 128x128 tiles.
@@ -461,9 +462,9 @@ static int launch_column_split(hipStream_t s, const GemmArgs& g, int64_t batch, 
     return launch_gemm256(s, w, 1, TA, TB, dt);
 }
 
-// Which kernel serves a 16-bit problem (MHIP_GEMM_TILE = 128 | 256 | 2560 ... 2566 forces one; 2564 / 2565 = the
-// 256x128 tile with a ring of six / four stages, 2566 = the 256x256 tile with four: members of the
-// generated family that only a forced choice or the tuning table selects):
+// Which kernel serves a 16-bit problem (MHIP_GEMM_TILE = 128 | 256 | 2560 ... 2567 forces one; 2564 / 2565 = the
+// 256x128 tile with a ring of six / four stages, 2566 = the 256x256 tile with four, 2567 = the 256x384
+// tile: members of the generated family that only a forced choice or the tuning table selects):
 //   * the four-wave ring kernel (gemm256.hip) on 256x256 tiles (2560) or 256x128 tiles
 //     (2561) when K >= 512 and the problem is eligible: one workgroup per CU, so its time is
 //     rounds x (stages x per-stage time + prologue and epilogue), rounds = ceil(tiles / 256 CUs);
@@ -477,6 +478,8 @@ static int launch_column_split(hipStream_t s, const GemmArgs& g, int64_t batch, 
 //     not a default);
 //   * wide tiles on the columns that fill whole rounds and narrow tiles on the rest (2563;
 //     launch_column_split) where the problem has that shape;
+//   * 256x384 tiles (2567; no activation, relu or tanh-GELU) where one round of them replaces two
+//     or three of the others;
 //   * the eight-wave 256x256 kernel for large problems the ring kernel cannot take whose
 //     rows of C are not 16-byte aligned (odd N): its eight waves hide the narrow stores;
 //   * otherwise 128x128 tiles, two workgroups per CU (short K, few tiles).
@@ -509,21 +512,41 @@ static int pick_tile(hipStream_t s, const GemmArgs& g, int64_t batch) {
     if (force == 2566) {
         if (gemm256_eligible(g, batch, TA, TB, dt)) return chose(2566, launch_gemm256(s, g, batch, TA, TB, dt, 256, 4));
     }
+    // the 256x384 tile (ring of four)
+    if (force == 2567) {
+        if (gemm256_eligible(g, batch, TA, TB, dt, 384) && gemm384_activation_ok(g.act)) return chose(2567, launch_gemm256(s, g, batch, TA, TB, dt, 384, 4));
+    }
+    constexpr int cus = 256;                           // compute units of the device this is written for
+    const int64_t narrow = tiles_m * ((g.N + 127) / 128) * batch, stages = g.K / 32;
+    const int64_t wide_cost = ((big + cus - 1) / cus) * (stages * 32 + 700);
+    const int64_t narrow_cost = ((narrow + cus - 1) / cus) * (stages * 18 + 500);
+    if (force == 0 && g.K >= 512 && gemm256_eligible(g, batch, TA, TB, dt, 384) && gemm384_activation_ok(g.act)) {
+        // The 256x384 tile where it saves a round: its stage costs 53 slots (48 MFMAs, and only
+        // one k-step of fragments read ahead), its prologue and epilogue 1050 (half as many
+        // accumulators again to convert and store) -- fitted to [8192,2304..12288] x K 768..6144:
+        // one round of it beats two of wide or three of narrow tiles ([8192,3072] x K 768 44 us
+        // against 49; inside a GPT-2 pass 50.3 against 55, and [8192,2304] 41.8 against 45.8 for
+        // the column split), while from two rounds on the wide tile's shorter epilogue wins
+        // ([8192,12288] x K 768: 170 us against 159).
+        const int64_t wider = tiles_m * ((g.N + 383) / 384) * batch;
+        const int64_t wider_cost = ((wider + cus - 1) / cus) * (stages * 53 + 1050);
+        int n_wide = 0;
+        int64_t other = wide_cost < narrow_cost ? wide_cost : narrow_cost;
+        if (gemm_split_shape(g, batch, &n_wide) && narrow > 2 * cus)
+            other = (tiles_m * (n_wide / 256) / cus) * (stages * 32 + 700) + (stages * 18 + 500);
+        if (wider_cost < other) return chose(2567, launch_gemm256(s, g, batch, TA, TB, dt, 384, 4));
+    }
     if (force == 2563 || (force == 0 && g.K >= 512)) {
         const int st = launch_column_split<T, TA, TB>(s, g, batch, dt, force == 2563);
         if (st >= 0) return chose(2563, st);
     }
     if (force == 0 && g.K >= 512) {
-        constexpr int cus = 256;                       // compute units of the device this is written for
-        const int64_t narrow = tiles_m * ((g.N + 127) / 128) * batch, stages = g.K / 32;
         const bool wide_ok = gemm256_eligible(g, batch, TA, TB, dt), narrow_ok = gemm256_eligible(g, batch, TA, TB, dt, 128);
         // (The streamed form of the narrow tile, 2562, is not chosen here: it is 5 % ahead of wide tiles
         // on a few shapes when the operands sit in the L2 -- [4096,8320] x K 1024 77 against 81 us,
         // [8192,4608] x K 768 67 against 71 -- and 10 to 15 % behind on the same shapes when they come
         // from memory, 92 against 84 and 83 against 72, which is how a GEMM inside a model finds
         // them.  The tuner times it and the table selects it where it wins.)
-        const int64_t wide_cost = ((big + cus - 1) / cus) * (stages * 32 + 700);
-        const int64_t narrow_cost = ((narrow + cus - 1) / cus) * (stages * 18 + 500);
         if (narrow_ok && (!wide_ok || narrow_cost < wide_cost)) return chose(2561, launch_gemm256(s, g, batch, TA, TB, dt, 128));
         if (wide_ok) return chose(2560, launch_gemm256(s, g, batch, TA, TB, dt));
     }

@@ -487,6 +487,216 @@ def emit(name, mnem, ka, kb):
     print("}\n")
 
 
+# ---- the 256x384 tile ----------------------------------------------------------------------------
+# The widest member: 256 rows x 384 columns per workgroup, each wave 128 x 192 = 4 x 6 accumulator
+# blocks = 384 registers, the first sixteen blocks in the AGPRs, the last eight in v[128:255].  It
+# moves 17 % fewer bytes from the L2s to LDS per FLOP than the 256x256 tile, which is what a GEMM
+# with short K whose operands come from memory is short of.  What it costs:
+#   * two fragment sets instead of four (k-step s of every stage uses set s): the fragments of a
+#     k-step are read during the k-step before it, 24 MFMAs = 768 cycles ahead;
+#   * a stage is 40 KB -- [A 16 KB][B 16 KB][B2 8 KB] -- and the ring four stages deep (160 KB);
+#     stage t+4 is asked for behind the barrier of stage t and must have landed at the barrier of
+#     stage t+3 (the reads of buffer t+1 start behind the barrier of stage t).
+# B is kept as the 256-column tile of the wide kernel followed by the 128-column tile of the narrow
+# one (B2: columns 256..383 of the workgroup's 384), each in its own layout, so that loads, LDS
+# layouts and fragment addresses are those of the two existing kernels; wave (wm, wn) owns columns
+# 128 wn .. + 127 of B (blocks j = 0..3) and 64 wn .. + 63 of B2 (j = 4, 5).
+#
+# Register map (VGPR): fragment set n: A v[40n : 40n+15], B v[40n+16 : 40n+31], B2 v[40n+32 : 40n+39];
+#   v[80:87] A read addresses, v[88:95] B, v[96:99] B2 (k-contiguous: element 2h + s; other: (blocks
+#   per wave) h + j; ring buffers 2h and 2h+1); v100 / v101 / v102 global byte offsets of this thread's
+#   chunk of A / B / B2, v103 / v104 / v105 the same + 64; v[128:255] accumulator blocks 16..23.
+# AGPR: accumulator block b = 6 i + j < 16 at a[16 b : +15].
+# SGPR: as above (s[72:74] A pass strides, s[76:78] B pass strides, s80 stage counter, s81 caller's M0).
+X_NST, X_STAGE, X_UNROLL = 4, 40960, 4
+X_REGION = {"A": 0, "B": 16384, "B2": 32768}
+X_SET = {0: {"A": 0, "B": 16, "B2": 32}, 1: {"A": 40, "B": 56, "B2": 72}}
+X_RADDR = {"A": 80, "B": 88, "B2": 96}
+X_GOFF = {"A": 100, "B": 101, "B2": 102}
+X_GOFF2 = {"A": 103, "B": 104, "B2": 105}
+X_BLOCKS = {"A": 4, "B": 4, "B2": 2}          # 32-wide fragment blocks per wave
+X_PASSES = {"A": 4, "B": 4, "B2": 2}          # 4 KB load passes per stage
+X_ROWB = {"A": 512, "B": 512, "B2": 256}      # bytes per k-row of a tile whose k axis is the slow one
+X_VACC = 128
+
+
+def x_kind(kinds, which):
+    return kinds["B" if which == "B2" else which]
+
+
+def x_frag_reads(kinds, g, s, fset):
+    per = {}
+    for which in ("A", "B", "B2"):
+        kind, base, addr = x_kind(kinds, which), X_SET[fset][which], X_RADDR[which]
+        h, lo = g >> 1, (g & 1) * X_STAGE
+        out = []
+        for j in range(X_BLOCKS[which]):
+            dst = base + 4 * j
+            if kind == "K":
+                out.append(f"ds_read_b128 {vr(dst, 4)}, v{addr + 2 * h + s} offset:{lo + j * 2048}")
+            else:
+                off = lo + s * 16 * X_ROWB[which]
+                a = addr + X_BLOCKS[which] * h + j
+                out.append(f"ds_read_b64_tr_b16 {vr(dst, 2)}, v{a} offset:{off}")
+                out.append(f"ds_read_b64_tr_b16 {vr(dst + 2, 2)}, v{a} offset:{off + 4 * X_ROWB[which]}")
+        per[which] = out
+    out = []
+    for i in range(max(len(v) for v in per.values())):
+        for which in ("A", "B", "B2"):
+            out += per[which][i:i + 1]
+    return out
+
+
+def x_load(kinds, which, stage, p, second_half=False):
+    g = stage % X_NST
+    m0 = g * X_STAGE + X_REGION[which] + p * 4096
+    sp = SP["A" if which == "A" else "B"]
+    # B2 with k as the slow axis packs four k-rows into a wave's 1 KB slot where B packs two: its
+    # passes are twice as far apart
+    mult = p * (2 if which == "B2" and x_kind(kinds, which) == "MN" else 1)
+    so = "0" if mult == 0 else f"s{sp + mult - 1}"
+    voff = (X_GOFF2 if second_half else X_GOFF)[which]
+    rs = "%[rsa]" if which == "A" else "%[rsb]"
+    return dict(stage=stage, lines=[f"s_add_u32 m0, %[m0b], {m0}", "s_nop 0",
+                                    f"buffer_load_dwordx4 v{voff}, {rs}, {so} offen lds"])
+
+
+def x_trigger_group(kinds, t):
+    """Loads triggered by the barrier of stage t (buffer t % 4 has just become free)."""
+    grp = []
+    for which in ("A", "B", "B2"):
+        if x_kind(kinds, which) == "K":
+            if (t + X_NST - 1) % 2 == 0:
+                for p in range(X_PASSES[which]):
+                    grp.append(x_load(kinds, which, t + X_NST - 1, p))
+                    grp.append(x_load(kinds, which, t + X_NST, p, second_half=True))
+                grp.append(dict(stage=None, lines=[f"v_add_u32 v{X_GOFF[which]}, 128, v{X_GOFF[which]}",
+                                                   f"v_add_u32 v{X_GOFF2[which]}, 128, v{X_GOFF2[which]}"]))
+        else:
+            for p in range(X_PASSES[which]):
+                grp.append(x_load(kinds, which, t + X_NST, p))
+            step = "%[ta]" if which == "A" else "%[tb]"
+            grp.append(dict(stage=None, lines=[f"v_add_u32 v{X_GOFF[which]}, {step}, v{X_GOFF[which]}"]))
+    return grp
+
+
+def x_acc(b):
+    return f"a[{16 * b}:{16 * b + 15}]" if b < 16 else vr(X_VACC + 16 * (b - 16), 16)
+
+
+def x_mfmas(mnem, fset):
+    out = []
+    for i in range(4):
+        for j in range(6):
+            bsrc = X_SET[fset]["B"] + 4 * j if j < 4 else X_SET[fset]["B2"] + 4 * (j - 4)
+            acc = x_acc(6 * i + j)
+            # (B, A): the accumulator tile comes out transposed (lane = row m)
+            out.append(f"{mnem} {acc}, {vr(bsrc, 4)}, {vr(X_SET[fset]['A'] + 4 * i, 4)}, {acc}")
+    return out
+
+
+def x_simulate(kinds):
+    """vmcnt of the prologue wait (stage 0 landed) and of the barrier of each body position
+    (stage t + 1 landed)."""
+    tr = Tracker()
+    for t in range(-X_NST, -1):
+        tr.issue(x_trigger_group(kinds, t))
+    first, pending = halves(x_trigger_group(kinds, -1))
+    tr.issue(first)
+    pro = tr.allowed(0)
+    counts = {}
+    for t in range(4 * X_UNROLL):
+        tr.issue(pending)
+        c = tr.allowed(t + 1)
+        counts[t % X_UNROLL] = min(counts.get(t % X_UNROLL, 63), c)
+        first, pending = halves(x_trigger_group(kinds, t))
+        tr.issue(first)
+    return pro, counts
+
+
+def x_stage(mnem, kinds, t, vmcnt):
+    g, nxt = t % X_NST, (t + 1) % X_NST
+    r0 = x_frag_reads(kinds, g, 1, 1)          # this stage's second k-step
+    r1 = x_frag_reads(kinds, nxt, 0, 0)        # the next stage's first
+    _, prev_second = halves(x_trigger_group(kinds, t - 1))
+    this_first, _ = halves(x_trigger_group(kinds, t))
+    out = ["s_waitcnt lgkmcnt(0)"]             # set 0, read during the previous k-step
+    out += interleave(x_mfmas(mnem, 0), r0, prev_second)
+    # every read of buffer t % 4 is back, the own loads of stage t + 1 have landed
+    out.append(f"s_waitcnt vmcnt({min(vmcnt, 63)}) lgkmcnt(0)")
+    out.append("s_barrier")
+    out += interleave(x_mfmas(mnem, 1), r1, this_first)
+    return out
+
+
+def x_body(mnem, kinds):
+    pro_vmcnt, vmcnts = x_simulate(kinds)
+    out = []
+    for r in range(256):
+        out.append(f"v_accvgpr_write_b32 a{r}, 0")
+    for r in range(X_VACC, 256):
+        out.append(f"v_mov_b32 v{r}, 0")
+    for which, pin in (("A", "%[pa]"), ("B", "%[pb]")):
+        for i in range(1, 4):
+            out.append(f"s_mul_i32 s{SP[which] + i - 1}, {pin}, {i}")
+    out.append(f"s_mov_b32 s{ST}, 0")
+    out.append(f"s_mov_b32 s{ST + 1}, m0")
+    # fragment read addresses of ring buffers 2 and 3 from those of buffers 0 and 1
+    for which in ("A", "B", "B2"):
+        n = 2 if x_kind(kinds, which) == "K" else X_BLOCKS[which]
+        for e in range(n):
+            out.append(f"v_add_u32 v{X_RADDR[which] + n + e}, {2 * X_STAGE}, v{X_RADDR[which] + e}")
+        out.append(f"v_add_u32 v{X_GOFF2[which]}, 64, v{X_GOFF[which]}")
+    for t in range(-X_NST, -1):
+        for ld in x_trigger_group(kinds, t):
+            out += ld["lines"]
+    first, _ = halves(x_trigger_group(kinds, -1))
+    for ld in first:
+        out += ld["lines"]
+    out.append(f"s_waitcnt vmcnt({pro_vmcnt})")           # stage 0 landed
+    out.append("s_barrier")
+    out += x_frag_reads(kinds, 0, 0, 0)
+    out.append("L_gemm384_loop_%=:")
+    for t in range(X_UNROLL):
+        out += x_stage(mnem, kinds, t, vmcnts[t])
+        out.append(f"s_add_u32 s{ST}, s{ST}, 1")
+        if t < X_UNROLL - 1:
+            out.append(f"s_cmp_ge_u32 s{ST}, %[kt]")
+            out.append("s_cbranch_scc1 L_gemm384_done_%=")
+        else:
+            out.append(f"s_cmp_lt_u32 s{ST}, %[kt]")
+            out.append("s_cbranch_scc1 L_gemm384_loop_%=")
+    out.append("L_gemm384_done_%=:")
+    out.append("s_waitcnt vmcnt(0) lgkmcnt(0)")
+    out.append("s_barrier")
+    out.append(f"s_mov_b32 m0, s{ST + 1}")
+    out += ["s_nop 15", "s_nop 15"]
+    return out
+
+
+def emit384(name, mnem, ka, kb):
+    lines = x_body(mnem, {"A": ka, "B": kb})
+    print(f"// {name}: 256x384 tile, A operand {ka}-major, B operand {kb}-major, {mnem}")
+    print(f"__device__ __forceinline__ void {name}(f32x16 (&acc)[24], u32x4& ra, u32x4& rb, u32x2& rb2, u32x4& goff,")
+    print("        __amdgpu_buffer_rsrc_t rsa, __amdgpu_buffer_rsrc_t rsb, uint32_t pa, uint32_t pb,")
+    print("        uint32_t ta, uint32_t tb, uint32_t m0b, uint32_t kt) {")
+    print("    asm volatile(")
+    for ln in lines:
+        print(f'        "{ln}\\n"')
+    outs = ", ".join(f'"={{{x_acc(b)}}}"(acc[{b}])' for b in range(24))
+    print(f"        : {outs},")
+    ra, rb, rb2 = X_RADDR["A"], X_RADDR["B"], X_RADDR["B2"]
+    print(f'          "+{{v[{X_GOFF["A"]}:{X_GOFF["A"] + 3}]}}"(goff), "+{{v[{ra}:{ra + 3}]}}"(ra), "+{{v[{rb}:{rb + 3}]}}"(rb),')
+    print(f'          "+{{v[{rb2}:{rb2 + 1}]}}"(rb2)')
+    print('        : [rsa] "s"(rsa), [rsb] "s"(rsb), [pa] "s"(pa), [pb] "s"(pb), [ta] "s"(ta), [tb] "s"(tb),')
+    print('          [m0b] "s"(m0b), [kt] "s"(kt)')
+    vclob = (list(range(80)) + list(range(ra + 4, rb)) + list(range(rb + 4, rb2)) + [rb2 + 2, rb2 + 3]
+             + [X_GOFF2["B"], X_GOFF2["B2"]])
+    clob = [f'"v{i}"' for i in vclob] + [f'"s{i}"' for i in range(SP["A"], ST + 2)] + ['"scc"', '"memory"']
+    print("        : " + ", ".join(clob) + ");")
+    print("}\n")
+
+
 # The tile family: (B width, ring depth) -> stem of the emitted functions.  Every member that passes
 # `valid` is emitted and becomes a kernel variant the tuner can time (gemm.hip lists the codes).
 FAMILY = [(256, 5, "gemm256_loop"), (256, 4, "gemm256r4_loop"), (256, 6, "gemm256r6_loop"),
@@ -507,6 +717,10 @@ def main():
         for tname, mnem in (("bf16", "v_mfma_f32_32x32x16_bf16"), ("f16", "v_mfma_f32_32x32x16_f16")):
             for lname, ka, kb in (("nn", "K", "MN"), ("nt", "K", "K"), ("tn", "MN", "MN"), ("tt", "MN", "K")):
                 emit(f"{stem}_{lname}_{tname}", mnem, ka, kb)
+    print("#define MHIP_HAVE_GEMM256X384_LOOP 1\n")
+    for tname, mnem in (("bf16", "v_mfma_f32_32x32x16_bf16"), ("f16", "v_mfma_f32_32x32x16_f16")):
+        for lname, ka, kb in (("nn", "K", "MN"), ("nt", "K", "K"), ("tn", "MN", "MN"), ("tt", "MN", "K")):
+            emit384(f"gemm256x384_loop_{lname}_{tname}", mnem, ka, kb)
     # streamed tiles: the 256x128 kernel as a persistent workgroup, for A with k contiguous
     configure(128, 5)
     for tname, mnem in (("bf16", "v_mfma_f32_32x32x16_bf16"), ("f16", "v_mfma_f32_32x32x16_f16")):

@@ -32,6 +32,7 @@ namespace mhip {
 
 bool gemm256_eligible(const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype, int bw = 256, bool any_tile_count = false);
 bool gemm_stream_eligible(const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype);
+bool gemm384_activation_ok(int act);
 bool gemm_split_shape(const GemmArgs& g, int64_t batch, int* n_wide_out);
 
 namespace {
@@ -88,7 +89,7 @@ bool valid_choice(const char* line, const std::string& choice) {
     int a = 0, b = 0, c = 0, d = 0;
     if (!strncmp(line, "gemm ", 5)) {
         const int v = atoi(choice.c_str());
-        return v == 128 || v == 256 || (v >= 2560 && v <= 2566);
+        return v == 128 || v == 256 || (v >= 2560 && v <= 2567);
     }
     if (!strncmp(line, "row ", 4))
         return sscanf(choice.c_str(), "%d %d %d %d", &a, &b, &c, &d) == 4 && (a == 1 || a == 2) && (b == 1 || b == 2) &&
@@ -196,7 +197,7 @@ int tuned_gemm_variant(const GemmArgs& g, int64_t batch, int ta, int tb, int dty
     std::string c;
     if (!have_entries() || !lookup(gemm_key(g.M, g.N, g.K, batch, ta, tb, dtype), &c)) return 0;
     const int v = atoi(c.c_str());
-    return (v == 128 || v == 256 || (v >= 2560 && v <= 2566)) ? v : 0;
+    return (v == 128 || v == 256 || (v >= 2560 && v <= 2567)) ? v : 0;
 }
 
 bool tuned_row_launch(int op, int dtype, int64_t rows, int64_t cols, bool has_gamma, bool has_beta, RowLaunch* out) {
@@ -224,9 +225,10 @@ using namespace mhip;
 // GEMM candidates a problem can run (the validity filter: shape, alignment, LDS and tile count rules of each kernel).
 static std::vector<int> gemm_candidates(const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype) {
     std::vector<int> out;
-    for (int v : {128, 256, 2560, 2561, 2562, 2563, 2564, 2565, 2566}) {
+    for (int v : {128, 256, 2560, 2561, 2562, 2563, 2564, 2565, 2566, 2567}) {
         if ((v == 2560 || v == 2566) && !gemm256_eligible(g, batch, trans_a, trans_b, dtype)) continue;
         if ((v == 2561 || v == 2564 || v == 2565) && !gemm256_eligible(g, batch, trans_a, trans_b, dtype, 128)) continue;
+        if (v == 2567 && !(gemm256_eligible(g, batch, trans_a, trans_b, dtype, 384) && gemm384_activation_ok(g.act))) continue;
         if (v == 2562 && !gemm_stream_eligible(g, batch, trans_a, trans_b, dtype)) continue;
         if (v == 2563 && !(gemm_split_shape(g, batch, nullptr) && gemm256_eligible(g, batch, trans_a, trans_b, dtype))) continue;
         out.push_back(v);
@@ -250,6 +252,7 @@ extern "C" int mhip_gemm_autotune(void* stream, const void* a, const void* b, co
     g.M = (int)M; g.N = (int)N; g.K = (int)K;
     g.lda = (int)(trans_a ? M : K); g.ldb = (int)(trans_b ? K : N);
     g.sa = stride_a; g.sb = stride_b; g.sc = stride_c;
+    g.act = activation;
     const std::vector<int> cand = gemm_candidates(g, batch, trans_a, trans_b, dtype);
     std::vector<float> us(cand.size(), -1.f);
     // two passes over the candidates, the better time of each counts: the first candidates of the
@@ -296,6 +299,7 @@ extern "C" int mhip_gemm_autotune_in_model(void* stream, const void* a, const vo
     g.M = (int)M; g.N = (int)N; g.K = (int)K;
     g.lda = (int)(trans_a ? M : K); g.ldb = (int)(trans_b ? K : N);
     g.sa = stride_a; g.sb = stride_b; g.sc = stride_c;
+    g.act = activation;
     const int64_t a_bytes = (batch == 1 || stride_a == M * K) ? M * K * batch * 2 : M * K * 2;
     int best = 0;
     float best_us = 0.f;

@@ -231,6 +231,55 @@ def test_gemm_large_tiles(shape, layout, dtype, tile, lib):
     assert torch.equal(c, c128)
 
 
+# Shapes with >= 192 tiles of 256x384 (K stages of 32: a single stage, exits at every position of the
+# unrolled ring of four, several trips; M and N ragged against the tile and, once, N odd).
+WIDEST = [(8192, 2304, 32), (7944, 2408, 96), (8192, 2696, 160), (7680, 3072, 448), (8192, 2304, 768),
+          (6152, 3080, 1056), (8192, 2309, 192)]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=lambda d: NAME[d])
+@pytest.mark.parametrize("layout", [(False, False), (False, True), (True, False), (True, True)],
+                         ids=["nn", "nt", "tn", "tt"])
+@pytest.mark.parametrize("shape", WIDEST, ids=lambda s: "x".join(map(str, s)))
+def test_gemm_256x384_tile(shape, layout, dtype, lib, monkeypatch):
+    """The widest member of the family (eight of a wave's 24 accumulator blocks live in ordinary
+    registers, B is held as a 256-column and a 128-column tile): bias, activation and residual,
+    against the oracle on sampled rows and bit for bit against the 128x128 kernel, which
+    accumulates every k-block in the same order; nothing is written behind the last row."""
+    from metalhlo_amd import kernels
+    M, N, K = shape
+    ta, tb = layout
+    aligned = (not ta or M % 8 == 0) and (tb or N % 8 == 0)
+    if not aligned:
+        pytest.skip("operand rows off 16-byte boundaries run the scalar kernel")
+    a, b = _ab(M, N, K, dtype, 41, ta, tb)
+    rng = np.random.default_rng(42)
+    bias = to_dev(rng.standard_normal(N) * 0.5, dtype)
+    r = to_dev(rng.standard_normal((M, N)), dtype)
+    monkeypatch.setenv("MHIP_GEMM_TILE", "2567")
+    guard = torch.full((M * N + 64,), 7.0, dtype=dtype, device="cuda")
+    c = kernels.matmul(a, b, bias, "gelu", trans_a=ta, trans_b=tb, out=guard[:M * N].view(M, N))
+    assert lib.mhip_gemm_last_variant() == 2567
+    cr = kernels.matmul(a, b, bias, "relu", trans_a=ta, trans_b=tb, residual=r)
+    assert lib.mhip_gemm_last_variant() == 2567
+    assert torch.all(guard[M * N:] == 7.0)
+    monkeypatch.setenv("MHIP_GEMM_TILE", "128")
+    assert torch.equal(c, kernels.matmul(a, b, bias, "gelu", trans_a=ta, trans_b=tb))
+    assert torch.equal(cr, kernels.matmul(a, b, bias, "relu", trans_a=ta, trans_b=tb, residual=r))
+    rows = np.unique(np.r_[0, 31, 32, 127, 128, 255, 256, M - 1, rng.integers(0, M, 40)])
+    A = as_f64(a).T if ta else as_f64(a)
+    B = as_f64(b).T if tb else as_f64(b)
+    exp = oracle.matmul_bias_act(A[rows], B, as_f64(bias), "gelu")
+    assert_close(c[rows], exp, TOL[dtype], f"gemm 256x384 {shape} {layout}")
+    exp = oracle.matmul_bias_act(A[rows], B, as_f64(bias), "relu")
+    exp = as_f64(to_dev(exp, dtype).cpu()) + as_f64(r)[rows]          # product rounded, then the residual added
+    assert_close(cr[rows], exp, TOL[dtype], f"gemm 256x384 + residual {shape} {layout}")
+    # an activation its epilogue does not serve goes to another kernel
+    monkeypatch.setenv("MHIP_GEMM_TILE", "2567")
+    kernels.matmul(a, b, bias, "silu", trans_a=ta, trans_b=tb)
+    assert lib.mhip_gemm_last_variant() != 2567
+
+
 @pytest.mark.parametrize("tile", ["2560", "2561"], ids=["256x256", "256x128"])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=lambda d: NAME[d])
 def test_gemm_ring_kernel_rows_of_c_at_any_alignment(tile, dtype, monkeypatch):
@@ -340,18 +389,25 @@ def test_gemm_wide_tiles_plus_a_narrow_band(shape, tb, dtype, monkeypatch):
             assert_close(c[rows], exp, TOL[dtype], f"split gemm {shape} nt={tb}")
 
 
-def test_gemm_split_is_the_default_from_a_third_round_on(lib, monkeypatch):
-    """[8192, 768] x [768, 2304] and x [768, 3072] (more than two rounds of narrow tiles, a band of
-    at most one round) take the split by default: same bits as forcing it."""
+def test_gemm_one_round_of_the_widest_tile_is_the_default_where_it_saves_a_round(lib, monkeypatch):
+    """[8192, 768] x [768, 2304] and x [768, 3072]: 192 and 256 tiles of 256x384 (one round) against
+    two rounds of wide or three of narrow tiles -- the default with an activation the widest tile's
+    epilogue serves; with another one (silu) the column split as before; [8192, 768] x [768, 12288]
+    (four rounds against six) stays on wide tiles.  Always the bits of the forced choice."""
     from metalhlo_amd import kernels
     kernels.tuning_clear()                 # the heuristic's choice, not a table entry's
     for N in (2304, 3072):
         a, b = _ab(8192, N, 768, torch.bfloat16, 67)
-        monkeypatch.delenv("MHIP_GEMM_TILE", raising=False)
-        c = kernels.matmul(a, b, None, "gelu")
-        assert lib.mhip_gemm_last_variant() == 2563
-        monkeypatch.setenv("MHIP_GEMM_TILE", "2563")
-        assert torch.equal(c, kernels.matmul(a, b, None, "gelu"))
+        for act, variant in (("gelu", 2567), ("none", 2567), ("silu", 2563)):
+            monkeypatch.delenv("MHIP_GEMM_TILE", raising=False)
+            c = kernels.matmul(a, b, None, act)
+            assert lib.mhip_gemm_last_variant() == variant, (N, act)
+            monkeypatch.setenv("MHIP_GEMM_TILE", str(variant))
+            assert torch.equal(c, kernels.matmul(a, b, None, act))
+    a, b = _ab(8192, 12288, 768, torch.bfloat16, 68)
+    monkeypatch.delenv("MHIP_GEMM_TILE", raising=False)
+    kernels.matmul(a, b)
+    assert lib.mhip_gemm_last_variant() == 2560
 
 
 def test_gemm_streaming_stores_of_a_large_result(monkeypatch):
@@ -463,7 +519,7 @@ def test_gemm_ring_kernel_takes_wide_and_deep_operands(lib):
         a = to_dev(rng.uniform(-1, 1, (M, K)), torch.bfloat16)
         b = to_dev(rng.uniform(-1, 1, (K, N)) * (K ** -0.5), torch.bfloat16)
         c = kernels.matmul(a, b)
-        assert 2560 <= lib.mhip_gemm_last_variant() <= 2566, (M, N, K, lib.mhip_gemm_last_variant())
+        assert 2560 <= lib.mhip_gemm_last_variant() <= 2567, (M, N, K, lib.mhip_gemm_last_variant())
         rows = np.r_[0, 255, 256, M - 1, rng.integers(0, M, 12)]
         assert_close(c[rows], as_f64(a[rows]) @ as_f64(b), 2e-2, f"gemm {M}x{N}x{K}")
     # fp32 operands run none of the 16-bit variants
