@@ -462,9 +462,10 @@ static int launch_column_split(hipStream_t s, const GemmArgs& g, int64_t batch, 
     return launch_gemm256(s, w, 1, TA, TB, dt);
 }
 
-// Which kernel serves a 16-bit problem (MHIP_GEMM_TILE = 128 | 256 | 2560 ... 2567 forces one; 2564 / 2565 = the
-// 256x128 tile with a ring of six / four stages, 2566 = the 256x256 tile with four, 2567 = the 256x384
-// tile: members of the generated family that only a forced choice or the tuning table selects):
+// Which kernel serves a 16-bit problem (MHIP_GEMM_TILE = 128 | 256 | 2560 ... 2568 forces one; 2564 / 2565 = the
+// 256x128 tile with a ring of six / four stages, 2566 = the 256x256 tile with four, 2568 = the 256x128
+// tile as two workgroups per compute unit: members of the generated family that only a forced choice
+// or the tuning table selects; 2567 = the 256x384 tile):
 //   * the four-wave ring kernel (gemm256.hip) on 256x256 tiles (2560) or 256x128 tiles
 //     (2561) when K >= 512 and the problem is eligible: one workgroup per CU, so its time is
 //     rounds x (stages x per-stage time + prologue and epilogue), rounds = ceil(tiles / 256 CUs);
@@ -511,6 +512,10 @@ static int pick_tile(hipStream_t s, const GemmArgs& g, int64_t batch) {
     }
     if (force == 2566) {
         if (gemm256_eligible(g, batch, TA, TB, dt)) return chose(2566, launch_gemm256(s, g, batch, TA, TB, dt, 256, 4));
+    }
+    // the 256x128 tile with two workgroups per compute unit (ring of three)
+    if (force == 2568) {
+        if (gemm256_eligible(g, batch, TA, TB, dt, 128)) return chose(2568, launch_gemm256(s, g, batch, TA, TB, dt, 128, 3));
     }
     // the 256x384 tile (ring of four)
     if (force == 2567) {

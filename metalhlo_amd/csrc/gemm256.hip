@@ -138,7 +138,7 @@ __device__ __forceinline__ float acc_value(float in_agpr) {
 
 // Epilogue of one tile: bias, activation, conversion, then through LDS (the ring, free after the
 // loop's last barrier) so that every store instruction writes whole 16-byte chunks of C rows.
-template <typename T, int BW, bool STREAM_C = false>
+template <typename T, int BW, bool STREAM_C = false, int AHEAD = (BW == 256 ? 2 : 4)>
 __device__ __forceinline__ void store_tile(f32x16 (&acc)[BW / 16], char* smem, const GemmArgs& g, T* c, const T* res,
                                   int m0, int n0) {
     constexpr int WN = BW / 2;            // columns per wave
@@ -167,9 +167,10 @@ __device__ __forceinline__ void store_tile(f32x16 (&acc)[BW / 16], char* smem, c
     const int64_t step = (int64_t)kRowsPerPass * ldc;
     // Its residual chunks are asked for now: they come from memory (the tensor was written
     // several kernels ago), and a load in front of each store would be waited for pass by pass.
-    // (The wide tile has registers for half of them; the rest is fetched block by block.)
+    // (The wide tile has registers for half of them, the kernel that runs two workgroups per compute
+    // unit for a quarter; the rest is fetched block by block.)
     constexpr int kPB = kPasses / 4;                     // passes per 32-row block
-    constexpr int kAheadBlocks = BW == 256 ? 2 : 4;
+    constexpr int kAheadBlocks = AHEAD;
     u32x4 rv[kAheadBlocks * kPB];
     if (interior && res) {
         const T* rp = res + first;
@@ -581,6 +582,100 @@ int layout384(hipStream_t s, const GemmArgs& g, int64_t batch, int ta, int tb) {
     return launch384<T, true, true>(s, g, batch);
 }
 
+// ---- the 256x128 tile, two workgroups per compute unit ------------------------------------------------
+// gemm_pair_loop_* of the generated file: the narrow tile on two fragment sets, every register
+// below v64 and a[0:127] (256 registers a wave) and a ring of three 24 KB stages (72 KB), so that
+// two workgroups share a compute unit: one's prologue, epilogue and load latency run under the
+// other's MFMAs.  Accumulators and epilogue are those of the one-workgroup kernel.
+constexpr int kPairSmem = 3 * 24 * 1024;
+
+template <typename T, bool TA, bool TB>
+__device__ __forceinline__ void main_loop_pair(f32x16 (&acc)[8], u32x4 ra, u32x2 rb, u32x2& goff,
+                                               __amdgpu_buffer_rsrc_t rsa, __amdgpu_buffer_rsrc_t rsb, uint32_t pa,
+                                               uint32_t pb, uint32_t ta, uint32_t tb, uint32_t m0b, uint32_t kt) {
+    constexpr bool bf = std::is_same<T, bf16_t>::value;
+#define MHIP_LOOP(cond, name) \
+    if constexpr (cond) gemm_pair_loop_##name(acc, ra, rb, goff, rsa, rsb, pa, pb, ta, tb, m0b, kt);
+    MHIP_LOOP(bf && !TA && !TB, nn_bf16)
+    MHIP_LOOP(bf && !TA && TB, nt_bf16)
+    MHIP_LOOP(bf && TA && !TB, tn_bf16)
+    MHIP_LOOP(bf && TA && TB, tt_bf16)
+    MHIP_LOOP(!bf && !TA && !TB, nn_f16)
+    MHIP_LOOP(!bf && !TA && TB, nt_f16)
+    MHIP_LOOP(!bf && TA && !TB, tn_f16)
+    MHIP_LOOP(!bf && TA && TB, tt_f16)
+#undef MHIP_LOOP
+}
+
+template <typename T, bool TA, bool TB>
+__global__ __launch_bounds__(256, 2) void gemm_pair_kernel(GemmArgs g) {
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    using LA = typename std::conditional<TA, MnMajor<256>, KMajor>::type;
+    using LB = typename std::conditional<TB, KMajor, MnMajor<128>>::type;
+
+    int tm, tn;
+    tile_of(blockIdx.x, gridDim.x, g.tiles_m, g.tiles_n, tm, tn);
+    const int m0 = tm * 256, n0 = tn * 128;
+    const int64_t batch = blockIdx.y;
+    const char* a = reinterpret_cast<const char*>(static_cast<const T*>(g.a) + batch * g.sa);
+    const char* b = reinterpret_cast<const char*>(static_cast<const T*>(g.b) + batch * g.sb);
+    T* c = static_cast<T*>(g.c) + batch * g.sc;
+    const T* res = g.residual ? static_cast<const T*>(g.residual) + batch * g.sc : nullptr;
+    const uint32_t a_bytes = (uint32_t)(((int64_t)((TA ? g.K : g.M) - 1) * g.lda + (TA ? g.M : g.K)) * 2);
+    const uint32_t b_bytes = (uint32_t)(((int64_t)((TB ? g.N : g.K) - 1) * g.ldb + (TB ? g.K : g.N)) * 2);
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
+    const u32x4 ra = LA::raddr(lane, wm * 128, lds0);
+    const u32x4 rbw = LB::raddr(lane, wn * 64, lds0 + kOperBytes);
+    u32x2 rb;
+    rb.x = rbw.x; rb.y = rbw.y;
+    u32x2 goff;
+    goff.x = LA::goff(lane, wave, m0, g.lda, g.M);
+    goff.y = LB::goff(lane, wave, n0, g.ldb, g.N);
+    const uint32_t m0b = __builtin_amdgcn_readfirstlane(lds0 + (uint32_t)wave * 1024u);
+    const __amdgpu_buffer_rsrc_t rsa =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(a), 0, a_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsb =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(b), 0, b_bytes, 0x00020000);
+
+    f32x16 acc[8];
+    main_loop_pair<T, TA, TB>(acc, ra, rb, goff, rsa, rsb, LA::pass_stride(g.lda), LB::pass_stride(g.ldb),
+                              LA::stage_stride(g.lda), LB::stage_stride(g.ldb), m0b, (uint32_t)(g.K / 32));
+    if (g.stream_c) store_tile<T, 128, true, 1>(acc, smem, g, c, res, m0, n0);
+    else store_tile<T, 128, false, 1>(acc, smem, g, c, res, m0, n0);
+}
+
+template <typename T, bool TA, bool TB>
+int launch_pair(hipStream_t s, GemmArgs g, int64_t batch) {
+    auto kern = gemm_pair_kernel<T, TA, TB>;
+    static_assert(kPairSmem >= 4 * 128 * (128 + 16), "the epilogue's staging area reuses the ring");
+    static std::once_flag once;
+    static hipError_t attr_err = hipSuccess;
+    std::call_once(once, [&] {
+        attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kPairSmem);
+    });
+    if (attr_err != hipSuccess)
+        return fail(MHIP_ERR_LAUNCH, "gemm_pair: cannot reserve %d bytes of LDS: %s", kPairSmem,
+                    hipGetErrorString(attr_err));
+    g.tiles_m = (g.M + 255) / 256;
+    g.tiles_n = (g.N + 127) / 128;
+    g.stream_c = (int64_t)g.M * g.N * batch * 2 > (256ll << 20) && (g.ldc ? g.ldc : g.N) % 8 == 0;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(g.tiles_m * g.tiles_n), (unsigned)batch), dim3(256),
+                       kPairSmem, s, g);
+    return check_launch("gemm_pair");
+}
+
+template <typename T>
+int layout_pair(hipStream_t s, const GemmArgs& g, int64_t batch, int ta, int tb) {
+    if (!ta && !tb) return launch_pair<T, false, false>(s, g, batch);
+    if (!ta && tb) return launch_pair<T, false, true>(s, g, batch);
+    if (ta && !tb) return launch_pair<T, true, false>(s, g, batch);
+    return launch_pair<T, true, true>(s, g, batch);
+}
+
 // ---- streamed tiles ------------------------------------------------------------------------------
 // The 256x128 kernel as a persistent workgroup: one workgroup per compute unit runs tile after tile,
 // and the stores of a tile travel inside the main loop of the NEXT one (gemm_stream_loop_* of the
@@ -826,6 +921,9 @@ int launch_gemm256(hipStream_t s, const GemmArgs& g, int64_t batch, int trans_a,
     if (bw == 384)
         return dtype == MHIP_BF16 ? layout384<bf16_t>(s, g, batch, trans_a, trans_b)
                                   : layout384<f16_t>(s, g, batch, trans_a, trans_b);
+    if (bw == 128 && ring == 3)       // two workgroups per compute unit
+        return dtype == MHIP_BF16 ? layout_pair<bf16_t>(s, g, batch, trans_a, trans_b)
+                                  : layout_pair<f16_t>(s, g, batch, trans_a, trans_b);
     if (dtype == MHIP_BF16) return family256<bf16_t>(s, g, batch, trans_a, trans_b, bw, ring);
     return family256<f16_t>(s, g, batch, trans_a, trans_b, bw, ring);
 }

@@ -508,16 +508,50 @@ def emit(name, mnem, ka, kb):
 #   chunk of A / B / B2, v103 / v104 / v105 the same + 64; v[128:255] accumulator blocks 16..23.
 # AGPR: accumulator block b = 6 i + j < 16 at a[16 b : +15].
 # SGPR: as above (s[72:74] A pass strides, s[76:78] B pass strides, s80 stage counter, s81 caller's M0).
-X_NST, X_STAGE, X_UNROLL = 4, 40960, 4
-X_REGION = {"A": 0, "B": 16384, "B2": 32768}
-X_SET = {0: {"A": 0, "B": 16, "B2": 32}, 1: {"A": 40, "B": 56, "B2": 72}}
-X_RADDR = {"A": 80, "B": 88, "B2": 96}
-X_GOFF = {"A": 100, "B": 101, "B2": 102}
-X_GOFF2 = {"A": 103, "B": 104, "B2": 105}
-X_BLOCKS = {"A": 4, "B": 4, "B2": 2}          # 32-wide fragment blocks per wave
-X_PASSES = {"A": 4, "B": 4, "B2": 2}          # 4 KB load passes per stage
-X_ROWB = {"A": 512, "B": 512, "B2": 256}      # bytes per k-row of a tile whose k axis is the slow one
-X_VACC = 128
+#
+# The same two-set schedule serves a second member, the 256x128 tile for two workgroups per compute
+# unit: all of its registers below v64 and a[0:127] (256 registers per wave), a ring of three 24 KB
+# stages (72 KB), so that two workgroups share a compute unit and one's prologue, epilogue and load
+# latency run under the other's MFMAs.  Register map: fragment set n: A v[24n : 24n+15], B
+# v[24n+16 : 24n+23]; v[48:55] A read addresses, v[56:59] B; v60 / v61 global offsets, v62 / v63 the
+# same + 64; accumulator (i, j) at a[16 (2 i + j) : +15] as in the one-workgroup kernel.
+class TwoSet:
+    """One member of the two-fragment-set family: geometry and register map."""
+
+    def __init__(self, name, nst, ops, region, sets, raddr, goff, goff2, blocks, passes, rowb, passmult,
+                 acc_regs, grid, goff_span, clobber_to):
+        self.name, self.nst, self.ops = name, nst, ops
+        self.stage = sum(passes[o] * 4096 for o in ops)
+        self.unroll = nst if nst % 2 == 0 else 2 * nst
+        self.region, self.sets, self.raddr, self.goff, self.goff2 = region, sets, raddr, goff, goff2
+        self.blocks, self.passes, self.rowb, self.passmult = blocks, passes, rowb, passmult
+        self.acc_regs = acc_regs          # block index -> register range text
+        self.grid = grid                  # (accumulator block, B operand, its block, A block) per MFMA of a k-step
+        self.goff_span = goff_span        # registers of the global-offset operand handed in by the caller
+        self.clobber_to = clobber_to      # fragment registers v0 .. clobber_to - 1
+
+
+def _x384():
+    def acc(b):
+        return f"a[{16 * b}:{16 * b + 15}]" if b < 16 else vr(128 + 16 * (b - 16), 16)
+    grid = [(6 * i + j, "B" if j < 4 else "B2", j if j < 4 else j - 4, i) for i in range(4) for j in range(6)]
+    return TwoSet("384", 4, ("A", "B", "B2"), {"A": 0, "B": 16384, "B2": 32768},
+                  {0: {"A": 0, "B": 16, "B2": 32}, 1: {"A": 40, "B": 56, "B2": 72}},
+                  {"A": 80, "B": 88, "B2": 96}, {"A": 100, "B": 101, "B2": 102}, {"A": 103, "B": 104, "B2": 105},
+                  {"A": 4, "B": 4, "B2": 2}, {"A": 4, "B": 4, "B2": 2}, {"A": 512, "B": 512, "B2": 256},
+                  {"B2": 2}, [acc(b) for b in range(24)], grid, 4, 80)
+
+
+def _xpair():
+    grid = [(2 * i + j, "B", j, i) for i in range(4) for j in range(2)]
+    return TwoSet("pair", 3, ("A", "B"), {"A": 0, "B": 16384},
+                  {0: {"A": 0, "B": 16}, 1: {"A": 24, "B": 40}},
+                  {"A": 48, "B": 56}, {"A": 60, "B": 61}, {"A": 62, "B": 63},
+                  {"A": 4, "B": 2}, {"A": 4, "B": 2}, {"A": 512, "B": 256},
+                  {}, [f"a[{16 * b}:{16 * b + 15}]" for b in range(8)], grid, 2, 48)
+
+
+X = None      # the member being emitted
 
 
 def x_kind(kinds, which):
@@ -526,72 +560,66 @@ def x_kind(kinds, which):
 
 def x_frag_reads(kinds, g, s, fset):
     per = {}
-    for which in ("A", "B", "B2"):
-        kind, base, addr = x_kind(kinds, which), X_SET[fset][which], X_RADDR[which]
-        h, lo = g >> 1, (g & 1) * X_STAGE
+    for which in X.ops:
+        kind, base, addr = x_kind(kinds, which), X.sets[fset][which], X.raddr[which]
+        h, lo = g >> 1, (g & 1) * X.stage
         out = []
-        for j in range(X_BLOCKS[which]):
+        for j in range(X.blocks[which]):
             dst = base + 4 * j
             if kind == "K":
                 out.append(f"ds_read_b128 {vr(dst, 4)}, v{addr + 2 * h + s} offset:{lo + j * 2048}")
             else:
-                off = lo + s * 16 * X_ROWB[which]
-                a = addr + X_BLOCKS[which] * h + j
+                off = lo + s * 16 * X.rowb[which]
+                a = addr + X.blocks[which] * h + j
                 out.append(f"ds_read_b64_tr_b16 {vr(dst, 2)}, v{a} offset:{off}")
-                out.append(f"ds_read_b64_tr_b16 {vr(dst + 2, 2)}, v{a} offset:{off + 4 * X_ROWB[which]}")
+                out.append(f"ds_read_b64_tr_b16 {vr(dst + 2, 2)}, v{a} offset:{off + 4 * X.rowb[which]}")
         per[which] = out
     out = []
     for i in range(max(len(v) for v in per.values())):
-        for which in ("A", "B", "B2"):
+        for which in X.ops:
             out += per[which][i:i + 1]
     return out
 
 
 def x_load(kinds, which, stage, p, second_half=False):
-    g = stage % X_NST
-    m0 = g * X_STAGE + X_REGION[which] + p * 4096
+    g = stage % X.nst
+    m0 = g * X.stage + X.region[which] + p * 4096
     sp = SP["A" if which == "A" else "B"]
-    # B2 with k as the slow axis packs four k-rows into a wave's 1 KB slot where B packs two: its
-    # passes are twice as far apart
-    mult = p * (2 if which == "B2" and x_kind(kinds, which) == "MN" else 1)
+    # (B2 with k as the slow axis packs four k-rows into a wave's 1 KB slot where B packs two: its
+    # passes are twice as far apart)
+    mult = p * (X.passmult.get(which, 1) if x_kind(kinds, which) == "MN" else 1)
     so = "0" if mult == 0 else f"s{sp + mult - 1}"
-    voff = (X_GOFF2 if second_half else X_GOFF)[which]
+    voff = (X.goff2 if second_half else X.goff)[which]
     rs = "%[rsa]" if which == "A" else "%[rsb]"
     return dict(stage=stage, lines=[f"s_add_u32 m0, %[m0b], {m0}", "s_nop 0",
                                     f"buffer_load_dwordx4 v{voff}, {rs}, {so} offen lds"])
 
 
 def x_trigger_group(kinds, t):
-    """Loads triggered by the barrier of stage t (buffer t % 4 has just become free)."""
+    """Loads triggered by the barrier of stage t (buffer t % ring has just become free)."""
     grp = []
-    for which in ("A", "B", "B2"):
+    for which in X.ops:
         if x_kind(kinds, which) == "K":
-            if (t + X_NST - 1) % 2 == 0:
-                for p in range(X_PASSES[which]):
-                    grp.append(x_load(kinds, which, t + X_NST - 1, p))
-                    grp.append(x_load(kinds, which, t + X_NST, p, second_half=True))
-                grp.append(dict(stage=None, lines=[f"v_add_u32 v{X_GOFF[which]}, 128, v{X_GOFF[which]}",
-                                                   f"v_add_u32 v{X_GOFF2[which]}, 128, v{X_GOFF2[which]}"]))
+            if (t + X.nst - 1) % 2 == 0:
+                for p in range(X.passes[which]):
+                    grp.append(x_load(kinds, which, t + X.nst - 1, p))
+                    grp.append(x_load(kinds, which, t + X.nst, p, second_half=True))
+                grp.append(dict(stage=None, lines=[f"v_add_u32 v{X.goff[which]}, 128, v{X.goff[which]}",
+                                                   f"v_add_u32 v{X.goff2[which]}, 128, v{X.goff2[which]}"]))
         else:
-            for p in range(X_PASSES[which]):
-                grp.append(x_load(kinds, which, t + X_NST, p))
+            for p in range(X.passes[which]):
+                grp.append(x_load(kinds, which, t + X.nst, p))
             step = "%[ta]" if which == "A" else "%[tb]"
-            grp.append(dict(stage=None, lines=[f"v_add_u32 v{X_GOFF[which]}, {step}, v{X_GOFF[which]}"]))
+            grp.append(dict(stage=None, lines=[f"v_add_u32 v{X.goff[which]}, {step}, v{X.goff[which]}"]))
     return grp
-
-
-def x_acc(b):
-    return f"a[{16 * b}:{16 * b + 15}]" if b < 16 else vr(X_VACC + 16 * (b - 16), 16)
 
 
 def x_mfmas(mnem, fset):
     out = []
-    for i in range(4):
-        for j in range(6):
-            bsrc = X_SET[fset]["B"] + 4 * j if j < 4 else X_SET[fset]["B2"] + 4 * (j - 4)
-            acc = x_acc(6 * i + j)
-            # (B, A): the accumulator tile comes out transposed (lane = row m)
-            out.append(f"{mnem} {acc}, {vr(bsrc, 4)}, {vr(X_SET[fset]['A'] + 4 * i, 4)}, {acc}")
+    for acc_block, bop, bj, ai in X.grid:
+        acc = X.acc_regs[acc_block]
+        # (B, A): the accumulator tile comes out transposed (lane = row m)
+        out.append(f"{mnem} {acc}, {vr(X.sets[fset][bop] + 4 * bj, 4)}, {vr(X.sets[fset]['A'] + 4 * ai, 4)}, {acc}")
     return out
 
 
@@ -599,30 +627,30 @@ def x_simulate(kinds):
     """vmcnt of the prologue wait (stage 0 landed) and of the barrier of each body position
     (stage t + 1 landed)."""
     tr = Tracker()
-    for t in range(-X_NST, -1):
+    for t in range(-X.nst, -1):
         tr.issue(x_trigger_group(kinds, t))
     first, pending = halves(x_trigger_group(kinds, -1))
     tr.issue(first)
     pro = tr.allowed(0)
     counts = {}
-    for t in range(4 * X_UNROLL):
+    for t in range(4 * X.unroll):
         tr.issue(pending)
         c = tr.allowed(t + 1)
-        counts[t % X_UNROLL] = min(counts.get(t % X_UNROLL, 63), c)
+        counts[t % X.unroll] = min(counts.get(t % X.unroll, 63), c)
         first, pending = halves(x_trigger_group(kinds, t))
         tr.issue(first)
     return pro, counts
 
 
 def x_stage(mnem, kinds, t, vmcnt):
-    g, nxt = t % X_NST, (t + 1) % X_NST
+    g, nxt = t % X.nst, (t + 1) % X.nst
     r0 = x_frag_reads(kinds, g, 1, 1)          # this stage's second k-step
     r1 = x_frag_reads(kinds, nxt, 0, 0)        # the next stage's first
     _, prev_second = halves(x_trigger_group(kinds, t - 1))
     this_first, _ = halves(x_trigger_group(kinds, t))
     out = ["s_waitcnt lgkmcnt(0)"]             # set 0, read during the previous k-step
     out += interleave(x_mfmas(mnem, 0), r0, prev_second)
-    # every read of buffer t % 4 is back, the own loads of stage t + 1 have landed
+    # every read of buffer t % ring is back, the own loads of stage t + 1 have landed
     out.append(f"s_waitcnt vmcnt({min(vmcnt, 63)}) lgkmcnt(0)")
     out.append("s_barrier")
     out += interleave(x_mfmas(mnem, 1), r1, this_first)
@@ -632,22 +660,22 @@ def x_stage(mnem, kinds, t, vmcnt):
 def x_body(mnem, kinds):
     pro_vmcnt, vmcnts = x_simulate(kinds)
     out = []
-    for r in range(256):
-        out.append(f"v_accvgpr_write_b32 a{r}, 0")
-    for r in range(X_VACC, 256):
-        out.append(f"v_mov_b32 v{r}, 0")
+    for regs in X.acc_regs:
+        m = regs[2:-1].split(":")
+        for r in range(int(m[0]), int(m[1]) + 1):
+            out.append(f"v_accvgpr_write_b32 a{r}, 0" if regs[0] == "a" else f"v_mov_b32 v{r}, 0")
     for which, pin in (("A", "%[pa]"), ("B", "%[pb]")):
         for i in range(1, 4):
             out.append(f"s_mul_i32 s{SP[which] + i - 1}, {pin}, {i}")
     out.append(f"s_mov_b32 s{ST}, 0")
     out.append(f"s_mov_b32 s{ST + 1}, m0")
-    # fragment read addresses of ring buffers 2 and 3 from those of buffers 0 and 1
-    for which in ("A", "B", "B2"):
-        n = 2 if x_kind(kinds, which) == "K" else X_BLOCKS[which]
+    # fragment read addresses of the ring's last buffer(s) from those of buffers 0 and 1
+    for which in X.ops:
+        n = 2 if x_kind(kinds, which) == "K" else X.blocks[which]
         for e in range(n):
-            out.append(f"v_add_u32 v{X_RADDR[which] + n + e}, {2 * X_STAGE}, v{X_RADDR[which] + e}")
-        out.append(f"v_add_u32 v{X_GOFF2[which]}, 64, v{X_GOFF[which]}")
-    for t in range(-X_NST, -1):
+            out.append(f"v_add_u32 v{X.raddr[which] + n + e}, {2 * X.stage}, v{X.raddr[which] + e}")
+        out.append(f"v_add_u32 v{X.goff2[which]}, 64, v{X.goff[which]}")
+    for t in range(-X.nst, -1):
         for ld in x_trigger_group(kinds, t):
             out += ld["lines"]
     first, _ = halves(x_trigger_group(kinds, -1))
@@ -656,17 +684,17 @@ def x_body(mnem, kinds):
     out.append(f"s_waitcnt vmcnt({pro_vmcnt})")           # stage 0 landed
     out.append("s_barrier")
     out += x_frag_reads(kinds, 0, 0, 0)
-    out.append("L_gemm384_loop_%=:")
-    for t in range(X_UNROLL):
+    out.append(f"L_gemm{X.name}_loop_%=:")
+    for t in range(X.unroll):
         out += x_stage(mnem, kinds, t, vmcnts[t])
         out.append(f"s_add_u32 s{ST}, s{ST}, 1")
-        if t < X_UNROLL - 1:
+        if t < X.unroll - 1:
             out.append(f"s_cmp_ge_u32 s{ST}, %[kt]")
-            out.append("s_cbranch_scc1 L_gemm384_done_%=")
+            out.append(f"s_cbranch_scc1 L_gemm{X.name}_done_%=")
         else:
             out.append(f"s_cmp_lt_u32 s{ST}, %[kt]")
-            out.append("s_cbranch_scc1 L_gemm384_loop_%=")
-    out.append("L_gemm384_done_%=:")
+            out.append(f"s_cbranch_scc1 L_gemm{X.name}_loop_%=")
+    out.append(f"L_gemm{X.name}_done_%=:")
     out.append("s_waitcnt vmcnt(0) lgkmcnt(0)")
     out.append("s_barrier")
     out.append(f"s_mov_b32 m0, s{ST + 1}")
@@ -674,24 +702,42 @@ def x_body(mnem, kinds):
     return out
 
 
-def emit384(name, mnem, ka, kb):
-    lines = x_body(mnem, {"A": ka, "B": kb})
-    print(f"// {name}: 256x384 tile, A operand {ka}-major, B operand {kb}-major, {mnem}")
-    print(f"__device__ __forceinline__ void {name}(f32x16 (&acc)[24], u32x4& ra, u32x4& rb, u32x2& rb2, u32x4& goff,")
+def emit_two_set(member, name, mnem, ka, kb):
+    global X
+    X = member
+    kinds = {"A": ka, "B": kb}
+    lines = x_body(mnem, kinds)
+    nacc = len(X.acc_regs)
+    print(f"// {name}: two fragment sets, ring of {X.nst}; A operand {ka}-major, B operand {kb}-major, {mnem}")
+    args = [f"f32x16 (&acc)[{nacc}]"]
+    for which in X.ops:
+        args.append(("u32x4& r" if X.blocks[which] == 4 else "u32x2& r") + which.lower())
+    args.append(("u32x4& " if X.goff_span == 4 else "u32x2& ") + "goff")
+    print(f"__device__ __forceinline__ void {name}({', '.join(args)},")
     print("        __amdgpu_buffer_rsrc_t rsa, __amdgpu_buffer_rsrc_t rsb, uint32_t pa, uint32_t pb,")
     print("        uint32_t ta, uint32_t tb, uint32_t m0b, uint32_t kt) {")
     print("    asm volatile(")
     for ln in lines:
         print(f'        "{ln}\\n"')
-    outs = ", ".join(f'"={{{x_acc(b)}}}"(acc[{b}])' for b in range(24))
+    outs = ", ".join(f'"={{{X.acc_regs[b]}}}"(acc[{b}])' for b in range(nacc))
     print(f"        : {outs},")
-    ra, rb, rb2 = X_RADDR["A"], X_RADDR["B"], X_RADDR["B2"]
-    print(f'          "+{{v[{X_GOFF["A"]}:{X_GOFF["A"] + 3}]}}"(goff), "+{{v[{ra}:{ra + 3}]}}"(ra), "+{{v[{rb}:{rb + 3}]}}"(rb),')
-    print(f'          "+{{v[{rb2}:{rb2 + 1}]}}"(rb2)')
+    g0 = X.goff["A"]
+    io = [f'"+{{v[{g0}:{g0 + X.goff_span - 1}]}}"(goff)']
+    declared = set(range(g0, g0 + X.goff_span))
+    for which in X.ops:
+        base, n = X.raddr[which], X.blocks[which]
+        io.append(f'"+{{v[{base}:{base + n - 1}]}}"(r{which.lower()})')
+        declared |= set(range(base, base + n))
+    print("          " + ", ".join(io))
     print('        : [rsa] "s"(rsa), [rsb] "s"(rsb), [pa] "s"(pa), [pb] "s"(pb), [ta] "s"(ta), [tb] "s"(tb),')
     print('          [m0b] "s"(m0b), [kt] "s"(kt)')
-    vclob = (list(range(80)) + list(range(ra + 4, rb)) + list(range(rb + 4, rb2)) + [rb2 + 2, rb2 + 3]
-             + [X_GOFF2["B"], X_GOFF2["B2"]])
+    # everything the block may write besides its operands: fragment sets, derived addresses, the
+    # second-half offsets
+    written = set(range(X.clobber_to))
+    for which in X.ops:
+        written |= set(range(X.raddr[which], X.raddr[which] + 2 * X.blocks[which]))
+        written.add(X.goff2[which])
+    vclob = sorted(written - declared)
     clob = [f'"v{i}"' for i in vclob] + [f'"s{i}"' for i in range(SP["A"], ST + 2)] + ['"scc"', '"memory"']
     print("        : " + ", ".join(clob) + ");")
     print("}\n")
@@ -718,9 +764,10 @@ def main():
             for lname, ka, kb in (("nn", "K", "MN"), ("nt", "K", "K"), ("tn", "MN", "MN"), ("tt", "MN", "K")):
                 emit(f"{stem}_{lname}_{tname}", mnem, ka, kb)
     print("#define MHIP_HAVE_GEMM256X384_LOOP 1\n")
-    for tname, mnem in (("bf16", "v_mfma_f32_32x32x16_bf16"), ("f16", "v_mfma_f32_32x32x16_f16")):
-        for lname, ka, kb in (("nn", "K", "MN"), ("nt", "K", "K"), ("tn", "MN", "MN"), ("tt", "MN", "K")):
-            emit384(f"gemm256x384_loop_{lname}_{tname}", mnem, ka, kb)
+    for member, stem in ((_x384(), "gemm256x384_loop"), (_xpair(), "gemm_pair_loop")):
+        for tname, mnem in (("bf16", "v_mfma_f32_32x32x16_bf16"), ("f16", "v_mfma_f32_32x32x16_f16")):
+            for lname, ka, kb in (("nn", "K", "MN"), ("nt", "K", "K"), ("tn", "MN", "MN"), ("tt", "MN", "K")):
+                emit_two_set(member, f"{stem}_{lname}_{tname}", mnem, ka, kb)
     # streamed tiles: the 256x128 kernel as a persistent workgroup, for A with k contiguous
     configure(128, 5)
     for tname, mnem in (("bf16", "v_mfma_f32_32x32x16_bf16"), ("f16", "v_mfma_f32_32x32x16_f16")):

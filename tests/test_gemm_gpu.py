@@ -197,8 +197,8 @@ BIG = [(4096, 3072, 32), (3585, 3848, 96), (4000, 3608, 160), (3600, 4104, 448),
 @pytest.mark.parametrize("layout", [(False, False), (False, True), (True, False), (True, True)],
                          ids=["nn", "nt", "tn", "tt"])
 @pytest.mark.parametrize("shape", BIG, ids=lambda s: "x".join(map(str, s)))
-@pytest.mark.parametrize("tile", ["2560", "2561", "2564", "2565", "2566"],
-                         ids=["256x256", "256x128", "256x128-ring6", "256x128-ring4", "256x256-ring4"])
+@pytest.mark.parametrize("tile", ["2560", "2561", "2564", "2565", "2566", "2568"],
+                         ids=["256x256", "256x128", "256x128-ring6", "256x128-ring4", "256x256-ring4", "256x128-two-per-cu"])
 def test_gemm_large_tiles(shape, layout, dtype, tile, lib):
     """The four-wave ring kernel in every member of its generated family (tile width x ring depth;
     forced: also where the default picks another kernel), ragged M and N included."""
@@ -519,7 +519,7 @@ def test_gemm_ring_kernel_takes_wide_and_deep_operands(lib):
         a = to_dev(rng.uniform(-1, 1, (M, K)), torch.bfloat16)
         b = to_dev(rng.uniform(-1, 1, (K, N)) * (K ** -0.5), torch.bfloat16)
         c = kernels.matmul(a, b)
-        assert 2560 <= lib.mhip_gemm_last_variant() <= 2567, (M, N, K, lib.mhip_gemm_last_variant())
+        assert 2560 <= lib.mhip_gemm_last_variant() <= 2568, (M, N, K, lib.mhip_gemm_last_variant())
         rows = np.r_[0, 255, 256, M - 1, rng.integers(0, M, 12)]
         assert_close(c[rows], as_f64(a[rows]) @ as_f64(b), 2e-2, f"gemm {M}x{N}x{K}")
     # fp32 operands run none of the 16-bit variants
