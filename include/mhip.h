@@ -256,6 +256,23 @@ int mhip_argmax(void* stream, const void* x, void* out_idx, void* out_val, int64
 int mhip_rope(void* stream, const void* x, const void* freqs, void* y, int64_t rows, int64_t S,
               int64_t D, int freqs_are_angles, int dtype);
 
+/* Batch normalisation with given statistics (FusedBatchNormHandler, Compiler/CustomCallHandlers.swift:414-452;
+ * the operands the fusion pass hands it, Compiler/PassManager.swift:1006-1080): x and y are
+ * [rows, channels] (channels = the last axis), gamma / beta / mean / variance [channels] of x's
+ * element type;  y = (x - mean) / sqrt(variance + eps) * gamma + beta.  F32 / F16 / BF16, fp32
+ * arithmetic, one rounding. */
+int mhip_batch_norm(void* stream, const void* x, const void* gamma, const void* beta, const void* mean,
+                    const void* variance, void* y, int64_t rows, int64_t channels, float eps, int dtype);
+
+/* Attention of one query row over a few key / value rows (FusedDepthAttentionHandler,
+ * Compiler/CustomCallHandlers.swift:1084-1140; the reference's own kernel for it,
+ * Metal/Kernels/DepthAttentionKernel.swift:17-20): q and out [rows, hidden], k and v
+ * [rows, depth, hidden];  out = softmax(q k^T scale) v per row.  depth 1 .. 64 (the reference's
+ * kernel reads at most 32 rows and ignores the rest; more than 64 is refused here).
+ * F32 / F16 / BF16, fp32 arithmetic, one rounding. */
+int mhip_depth_attention(void* stream, const void* q, const void* k, const void* v, void* out,
+                         int64_t rows, int64_t depth, int64_t hidden, float scale, int dtype);
+
 /* A chain of elementwise operations in one launch (FusedElementwiseHandler,
  * CustomCallHandlers.swift:927-1079): the running value starts as inputs[0]; ops[i] is either a
  * mhip_unary_op code, applied to the running value, or MHIP_CHAIN_BINARY + a mhip_binary_op code,

@@ -42,6 +42,8 @@ SIGNATURES = {
     "mhip_transpose_0213": (_i32, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32]),
     "mhip_split_qkv_heads": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32]),
     "mhip_rope": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _i32]),
+    "mhip_batch_norm": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _f32, _i32]),
+    "mhip_depth_attention": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _f32, _i32]),
     "mhip_elementwise_chain": (_i32, [_vp, _i32, C.POINTER(_vp), C.POINTER(_i64), _i32, C.POINTER(_i32), _vp, _i64, _i32]),
     "mhip_iota": (_i32, [_vp, _vp, _i64, _i64, _i64, _i32]),
     "mhip_unary": (_i32, [_vp, _i32, _vp, _vp, _i64, _i32]),

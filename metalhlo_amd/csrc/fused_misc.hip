@@ -1,5 +1,9 @@
-// Two more of the reference's fused operators, both bound by memory bandwidth:
+// Four more of the reference's fused operators, all bound by memory bandwidth:
 //
+//   batch normalisation with given statistics (CustomCallHandlers.swift:414-452, "fused_batch_norm"):
+//       y = (x - mean) / sqrt(variance + eps) * gamma + beta, the four vectors along the last axis;
+//   attention over a few stored layer outputs (CustomCallHandlers.swift:1084-1140, "fused_depth_attention"):
+//       out = softmax(q K^T scale) V for one query row against `depth` <= 64 key / value rows;
 //   rotary position embedding (Compiler/CustomCallHandlers.swift:720-846, target "fused_rope"):
 //       x = [x1 | x2] along the last axis (halves of h = D / 2 elements),
 //       y = [x1 cos - x2 sin | x1 sin + x2 cos], cos / sin of shape [S, h] spread over the leading axes;
@@ -7,8 +11,9 @@
 //       the running value starts as input 0, every binary operation consumes the next input,
 //       every unary one transforms the running value.
 //
-// Both read every operand once and write the result once, 16 bytes per lane where the layout
-// allows; the arithmetic is fp32 whatever the element type, rounded once at the store.
+// All read every operand once and write the result once (rope, chains and batch normalisation 16
+// bytes per lane where the layout allows); the arithmetic is fp32 whatever the element type,
+// rounded once at the store.
 #include <math.h>
 
 #include "common.h"
@@ -195,10 +200,137 @@ int launch_chain(hipStream_t s, const ChainArgs& a, int n_inputs, void* y, int64
     return check_launch("mhip_elementwise_chain");
 }
 
+
+// ---- batch normalisation with given statistics -------------------------------------------------
+// V elements per thread along the channel axis (1, or a 16-byte vector's worth).
+template <typename T, int V>
+__global__ __launch_bounds__(256) void batch_norm_kernel(const T* __restrict__ x, const T* __restrict__ gamma,
+                                                         const T* __restrict__ beta, const T* __restrict__ mean,
+                                                         const T* __restrict__ var, T* __restrict__ y, int64_t n, int C,
+                                                         float eps) {
+    const int64_t i0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * V;
+    if (i0 >= n) return;
+    const int c0 = (int)(i0 % C);
+    auto one = [&](float xv, int c) {
+        const float inv = 1.f / sqrtf(Elem<T>::to_f32(var[c]) + eps);
+        return (xv - Elem<T>::to_f32(mean[c])) * inv * Elem<T>::to_f32(gamma[c]) + Elem<T>::to_f32(beta[c]);
+    };
+    if constexpr (V == 1) {
+        y[i0] = Elem<T>::from_f32(one(Elem<T>::to_f32(x[i0]), c0));
+    } else {
+        const Vec16<T> v = load16(x + i0);
+        Vec16<T> o;
+#pragma unroll
+        for (int e = 0; e < V; e++) o.v[e] = Elem<T>::from_f32(one(Elem<T>::to_f32(v.v[e]), c0 + e));
+        store16(y + i0, o);
+    }
+}
+
+template <typename T>
+int launch_batch_norm(hipStream_t s, const void* x, const void* g, const void* b, const void* m, const void* v, void* y,
+                      int64_t rows, int64_t C, float eps) {
+    constexpr int E = Elem<T>::kPerVec;
+    const int64_t n = rows * C;
+    const bool vec = C % E == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0;
+    const int64_t grid = ((vec ? n / E : n) + 255) / 256;
+    if (grid > 0x7FFFFFFFLL) return fail(MHIP_ERR_UNSUPPORTED, "mhip_batch_norm: tensor too large for one launch");
+#define MHIP_BN(V) hipLaunchKernelGGL((batch_norm_kernel<T, V>), dim3((unsigned)grid), dim3(256), 0, s, static_cast<const T*>(x), \
+        static_cast<const T*>(g), static_cast<const T*>(b), static_cast<const T*>(m), static_cast<const T*>(v), static_cast<T*>(y), n, (int)C, eps)
+    if (vec) MHIP_BN(E); else MHIP_BN(1);
+#undef MHIP_BN
+    return check_launch("mhip_batch_norm");
+}
+
+// ---- attention over a few rows ------------------------------------------------------------------
+// One workgroup of 256 threads per query row.  Scores: thread t sums q[h] K[l][h] over h = t, t + 256, ..
+// for every l, the 64 lanes of a wave add up, the four waves meet in LDS; lane l < depth of wave 0
+// then holds score l, and the softmax over depth is two wave reductions.  Output: thread t sums
+// w[l] V[l][h] over l for its h.
+constexpr int kDepthMax = 64;
+
+template <typename T>
+__global__ __launch_bounds__(256) void depth_attention_kernel(const T* __restrict__ q, const T* __restrict__ k,
+                                                              const T* __restrict__ v, T* __restrict__ o, int depth, int H,
+                                                              float scale) {
+    __shared__ float part[4][kDepthMax];
+    __shared__ float w[kDepthMax];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int64_t row = blockIdx.x;
+    const T* qr = q + row * H;
+    const T* kr = k + row * (int64_t)depth * H;
+    const T* vr = v + row * (int64_t)depth * H;
+    for (int l = 0; l < depth; l++) {
+        float acc = 0.f;
+        for (int h = tid; h < H; h += 256) acc += Elem<T>::to_f32(qr[h]) * Elem<T>::to_f32(kr[(int64_t)l * H + h]);
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+        if (lane == 0) part[wave][l] = acc;
+    }
+    __syncthreads();
+    if (wave == 0) {
+        const bool live = lane < depth;
+        const float sc = live ? (part[0][lane] + part[1][lane] + part[2][lane] + part[3][lane]) * scale : -INFINITY;
+        float mx = sc;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+        const float e = live ? expf(sc - mx) : 0.f;
+        float sum = e;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+        if (live) w[lane] = e / sum;
+    }
+    __syncthreads();
+    for (int h = tid; h < H; h += 256) {
+        float acc = 0.f;
+        for (int l = 0; l < depth; l++) acc += w[l] * Elem<T>::to_f32(vr[(int64_t)l * H + h]);
+        o[row * H + h] = Elem<T>::from_f32(acc);
+    }
+}
+
+template <typename T>
+int launch_depth_attention(hipStream_t s, const void* q, const void* k, const void* v, void* o, int64_t rows, int depth, int H,
+                           float scale) {
+    hipLaunchKernelGGL((depth_attention_kernel<T>), dim3((unsigned)rows), dim3(256), 0, s, static_cast<const T*>(q),
+                       static_cast<const T*>(k), static_cast<const T*>(v), static_cast<T*>(o), depth, H, scale);
+    return check_launch("mhip_depth_attention");
+}
+
 }  // namespace
 }  // namespace mhip
 
 using namespace mhip;
+
+extern "C" int mhip_batch_norm(void* stream, const void* x, const void* gamma, const void* beta, const void* mean,
+                               const void* variance, void* y, int64_t rows, int64_t channels, float eps, int dtype) {
+    if (rows < 0 || channels < 0) return fail(MHIP_ERR_INVALID_ARGUMENT, "mhip_batch_norm: negative size");
+    if (rows == 0 || channels == 0) return MHIP_OK;
+    if (!x || !gamma || !beta || !mean || !variance || !y) return fail(MHIP_ERR_INVALID_ARGUMENT, "mhip_batch_norm: NULL pointer");
+    if (channels > 0x7FFFFFFFLL) return fail(MHIP_ERR_UNSUPPORTED, "mhip_batch_norm: too many channels");
+    hipStream_t s = as_stream(stream);
+    switch (dtype) {
+        case MHIP_F32: return launch_batch_norm<float>(s, x, gamma, beta, mean, variance, y, rows, channels, eps);
+        case MHIP_BF16: return launch_batch_norm<bf16_t>(s, x, gamma, beta, mean, variance, y, rows, channels, eps);
+        case MHIP_F16: return launch_batch_norm<f16_t>(s, x, gamma, beta, mean, variance, y, rows, channels, eps);
+        default: return fail(MHIP_ERR_UNSUPPORTED, "mhip_batch_norm: dtype %d (need f32, f16 or bf16)", dtype);
+    }
+}
+
+extern "C" int mhip_depth_attention(void* stream, const void* q, const void* k, const void* v, void* out, int64_t rows,
+                                    int64_t depth, int64_t hidden, float scale, int dtype) {
+    if (rows < 0 || depth < 0 || hidden < 0) return fail(MHIP_ERR_INVALID_ARGUMENT, "mhip_depth_attention: negative size");
+    if (rows == 0 || hidden == 0) return MHIP_OK;
+    if (!q || !k || !v || !out) return fail(MHIP_ERR_INVALID_ARGUMENT, "mhip_depth_attention: NULL pointer");
+    if (depth < 1 || depth > kDepthMax)
+        return fail(MHIP_ERR_UNSUPPORTED, "mhip_depth_attention: depth %lld (1 to %d rows are served)", (long long)depth, kDepthMax);
+    if (rows > 0x7FFFFFFFLL || hidden > 0x7FFFFFFFLL) return fail(MHIP_ERR_UNSUPPORTED, "mhip_depth_attention: tensor too large for one launch");
+    hipStream_t s = as_stream(stream);
+    switch (dtype) {
+        case MHIP_F32: return launch_depth_attention<float>(s, q, k, v, out, rows, (int)depth, (int)hidden, scale);
+        case MHIP_BF16: return launch_depth_attention<bf16_t>(s, q, k, v, out, rows, (int)depth, (int)hidden, scale);
+        case MHIP_F16: return launch_depth_attention<f16_t>(s, q, k, v, out, rows, (int)depth, (int)hidden, scale);
+        default: return fail(MHIP_ERR_UNSUPPORTED, "mhip_depth_attention: dtype %d (need f32, f16 or bf16)", dtype);
+    }
+}
 
 extern "C" int mhip_rope(void* stream, const void* x, const void* freqs, void* y, int64_t rows, int64_t S, int64_t D,
                          int freqs_are_angles, int dtype) {

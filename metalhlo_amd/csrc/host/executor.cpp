@@ -220,7 +220,8 @@ static const std::map<std::string, int> kActivation = {{"none", MHIP_ACT_NONE}, 
 // custom_call targets served by a kernel (Compiler/CustomCallHandlers.swift:75-89)
 static const char* kTargets[] = {"fused_scaled_dot_product_attention", "fused_layer_norm", "fused_rms_norm",
                                  "fused_softmax", "fused_gelu", "fused_matmul_bias_activation", "fused_ffn",
-                                 "fused_rope", "fused_elementwise", "fused_token_embedding"};
+                                 "fused_rope", "fused_elementwise", "fused_batch_norm", "fused_depth_attention",
+                                 "fused_token_embedding"};
 
 // The operation list of a fused_elementwise call ("ops", or "operations": CustomCallHandlers.swift:941-943)
 // as codes for mhip_elementwise_chain, and the number of inputs the chain consumes.  The names are
@@ -499,6 +500,25 @@ static void check_custom_call_types(const Op& op, const std::vector<TensorType>&
             throw UnsupportedOp(where(op) + "frequencies must be [S, D] (cos | sin) or [S, D / 2] (angles)");
         return;
     }
+    if (op.target == "fused_batch_norm") {
+        // x [.., C], gamma / beta / mean / variance with C elements each (CustomCallHandlers.swift:430-434)
+        if (xt.shape.empty() || !(xt == op.out)) throw ParseError(where(op) + "expected x [.., C] and a result of x's type");
+        for (size_t i = 1; i < 5; i++)
+            if (in(i).numel() != cols) throw ParseError(where(op) + "gamma, beta, mean and variance must have one element per channel");
+        return;
+    }
+    if (op.target == "fused_depth_attention") {
+        // query [.., 1, H] or [.., H], keys and values [.., depth, H] (CustomCallHandlers.swift:1101-1103)
+        const TensorType &kt = in(1), &vt2 = in(2);
+        if (kt.shape.size() < 2 || !(kt == vt2) || !(xt == op.out)) throw ParseError(where(op) + "expected keys and values [.., depth, H] and a result of the query's type");
+        std::vector<int64_t> lead(kt.shape.begin(), kt.shape.end() - 2), with_row = lead, without = lead;
+        with_row.push_back(1); with_row.push_back(kt.shape.back());
+        without.push_back(kt.shape.back());
+        if (xt.shape != with_row && xt.shape != without) throw ParseError(where(op) + "the query must be [.., 1, H] or [.., H] over the keys' leading axes");
+        const int64_t depth = kt.shape[kt.shape.size() - 2];
+        if (depth < 1 || depth > 64) throw UnsupportedOp(where(op) + "1 to 64 key / value rows are served");
+        return;
+    }
     if (op.target == "fused_elementwise") {
         size_t need = 0;
         (void)chain_ops(op, cfg, &need);
@@ -654,6 +674,7 @@ void compile(Executable& exe) {
             if (!ok) throw UnsupportedOp(where(op) + "Unsupported custom call target: " + op.target);
             const size_t need = op.target == "fused_scaled_dot_product_attention" || op.target == "fused_layer_norm" || op.target == "fused_ffn" ||
                                         op.target == "fused_token_embedding" ? 3
+                              : op.target == "fused_batch_norm" ? 5 : op.target == "fused_depth_attention" ? 3
                               : op.target == "fused_rms_norm" || op.target == "fused_matmul_bias_activation" || op.target == "fused_rope" ? 2 : 1;
             if (op.operands.size() < need)
                 throw ParseError(where(op) + "Invalid input count: expected " + std::to_string(need) + ", got " + std::to_string(op.operands.size()));
@@ -846,6 +867,13 @@ static std::vector<DeviceTensor> run_ops(Executable& exe, const std::vector<Devi
                 } else if (op.target == "fused_rope") {
                     const int64_t S = xt.shape[xt.shape.size() - 2], fd = in(1).type.shape.back();
                     RUN(mhip_rope(s, in(0).data(), in(1).data(), out.data(), rows, S, cols, fd == cols / 2 ? 1 : 0, dt));
+                } else if (op.target == "fused_batch_norm") {
+                    RUN(mhip_batch_norm(s, in(0).data(), in(1).data(), in(2).data(), in(3).data(), in(4).data(), out.data(), rows, cols,
+                                        (float)cfg.get_float("eps", 1e-5), dt));
+                } else if (op.target == "fused_depth_attention") {
+                    const TensorType& kt = in(1).type;
+                    RUN(mhip_depth_attention(s, in(0).data(), in(1).data(), in(2).data(), out.data(), rows, kt.shape[kt.shape.size() - 2],
+                                             cols, (float)cfg.get_float("scale", 1.0), dt));
                 } else if (op.target == "fused_elementwise") {
                     size_t need = 0;
                     const std::vector<int> codes = chain_ops(op, cfg, &need);

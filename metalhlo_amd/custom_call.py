@@ -169,6 +169,22 @@ def _elementwise(operands, cfg):
     return [kernels.elementwise_chain(list(operands), ops)]
 
 
+def _batch_norm(operands, cfg):
+    """Normalisation with given statistics, operands [x, gamma, beta, mean, variance], config {eps}
+    (CustomCallHandlers.swift:414-452)."""
+    _need(operands, 5)
+    x, gamma, beta, mean, var = operands[:5]
+    return [kernels.batch_norm(x, gamma, beta, mean, var, eps=P.get_float(cfg, "eps", 1e-5))]
+
+
+def _depth_attention(operands, cfg):
+    """Attention of one query row over a few stored rows, operands [query, keys, values], config
+    {scale} (CustomCallHandlers.swift:1084-1140)."""
+    _need(operands, 3)
+    q, k, v = operands[:3]
+    return [kernels.depth_attention(q, k, v, scale=P.get_float(cfg, "scale", 1.0))]
+
+
 def _matmul_bias_act(operands, cfg):
     _need(operands, 2)
     x, w = operands[:2]
@@ -197,6 +213,8 @@ class CustomCallRegistry:
             ("fused_ffn", _ffn),
             ("fused_rope", _rope),
             ("fused_elementwise", _elementwise),
+            ("fused_batch_norm", _batch_norm),
+            ("fused_depth_attention", _depth_attention),
         ):
             self.register(name, fn)
 
@@ -221,4 +239,4 @@ shared = CustomCallRegistry()
 
 # Targets the reference registers that lie outside the attention / GEMM / row-kernel
 # path (CustomCallHandlers.swift:75-89); asking for them raises UnsupportedTarget.
-NOT_ON_PATH = ("fused_batch_norm", "fused_conv_bias_act", "fused_depth_attention")
+NOT_ON_PATH = ("fused_conv_bias_act",)

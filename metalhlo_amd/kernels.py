@@ -254,6 +254,38 @@ def rope(x, freqs):
     return y
 
 
+def batch_norm(x, gamma, beta, mean, variance, eps=1e-5):
+    """y = (x - mean) / sqrt(variance + eps) * gamma + beta, the four vectors along x's last axis."""
+    _dev(x, gamma, beta, mean, variance)
+    lib = _lib.load()
+    C_ = x.shape[-1] if x.dim() else 1
+    for t in (gamma, beta, mean, variance):
+        if t.numel() != C_ or t.dtype != x.dtype:
+            raise ValueError("batch_norm: gamma, beta, mean and variance must be [channels] of x's element type")
+    y = torch.empty_like(x)
+    _lib.check(lib.mhip_batch_norm(_stream(), x.data_ptr(), gamma.data_ptr(), beta.data_ptr(), mean.data_ptr(), variance.data_ptr(),
+                                   y.data_ptr(), x.numel() // C_ if C_ else 0, C_, float(eps), _code(x)))
+    return y
+
+
+def depth_attention(q, k, v, scale=1.0):
+    """softmax(q k^T scale) v for one query row per leading index: q [.., 1, H] or [.., H], k and v
+    [.., depth, H] with depth <= 64; the result has q's shape."""
+    _dev(q, k, v)
+    lib = _lib.load()
+    if k.dim() < 2 or k.shape != v.shape or not (q.dtype == k.dtype == v.dtype):
+        raise ValueError("depth_attention: k and v must be [.., depth, H] of q's element type")
+    depth, H = k.shape[-2], k.shape[-1]
+    lead = tuple(k.shape[:-2])
+    if tuple(q.shape) not in (lead + (1, H), lead + (H,)):
+        raise ValueError("depth_attention: q must be [.., 1, H] or [.., H] over k's leading axes")
+    out = torch.empty_like(q)
+    rows = q.numel() // H if H else 0
+    _lib.check(lib.mhip_depth_attention(_stream(), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), rows, depth, H,
+                                        float(scale), _code(q)))
+    return out
+
+
 CHAIN_UNARY_CODE = {"exponential": 0, "tanh": 1, "rsqrt": 2, "sqrt": 3, "negate": 4, "logistic": 5, "abs": 6, "log": 7,
                     "sine": 9, "cosine": 10, "floor": 11, "ceil": 12}
 CHAIN_BINARY_CODE = {"add": 100, "subtract": 101, "multiply": 102, "divide": 103, "maximum": 104, "minimum": 105}

@@ -37,6 +37,13 @@ in tests/test_oracle.py):
 * rope              — equals the complex product (x1 + i x2) e^{i theta}, preserves
                       the norm of every rotated pair, zero angle is the identity,
                       a quarter turn gives (-x2, x1), angles add under composition.
+* batch_norm        — a hand-computed 2 x 2 case; with the batch's own statistics it equals
+                      layer_norm of the transposed matrix (every channel normalised over the
+                      rows) and gives columns of mean beta and variance gamma^2 var / (var + eps).
+* depth_attention   — the reference's own cases (DepthAttentionTests.swift:46-137: equal keys
+                      give the mean of the value rows, one dominant key selects its value
+                      row), equals `attention` with one head and one query row, one stored
+                      row returns that row, a vector added to every key changes nothing.
 * elementwise_chain — each operation against the NumPy function of its name; the
                       reference's own example add -> multiply
                       (CustomCallHandlers.swift:950-953).
@@ -334,6 +341,31 @@ def rope(x, freqs) -> np.ndarray:
     return np.concatenate([x1 * c - x2 * s, x1 * s + x2 * c], axis=-1)
 
 
+def batch_norm(x, gamma, beta, mean, variance, eps: float = 1e-5) -> np.ndarray:
+    """Compiler/CustomCallHandlers.swift:414-452 (`graph.normalize`): (x - mean) / sqrt(variance + eps) *
+    gamma + beta with the four channel vectors spread along the last axis of x (the operands of the
+    fusion pass, Compiler/PassManager.swift:1006-1080)."""
+    x = np.asarray(x, dtype=np.float64)
+    g, b, m, v = (np.asarray(t, dtype=np.float64).reshape(-1) for t in (gamma, beta, mean, variance))
+    if not all(t.size == x.shape[-1] for t in (g, b, m, v)):
+        raise ValueError("gamma, beta, mean and variance must have one element per channel")
+    return (x - m) / np.sqrt(v + eps) * g + b
+
+
+def depth_attention(q, k, v, scale: float = 1.0) -> np.ndarray:
+    """Compiler/CustomCallHandlers.swift:1084-1140: softmax(q k^T scale, last axis) v for q [.., 1, H] or
+    [.., H] and k, v [.., depth, H]; the result has q's shape."""
+    q = np.asarray(q, dtype=np.float64)
+    k = np.asarray(k, dtype=np.float64)
+    v = np.asarray(v, dtype=np.float64)
+    q3 = q.reshape(k.shape[:-2] + (1, k.shape[-1]))
+    s = np.matmul(q3, np.swapaxes(k, -1, -2)) * scale
+    s = s - s.max(axis=-1, keepdims=True)
+    w = np.exp(s)
+    w = w / w.sum(axis=-1, keepdims=True)
+    return np.matmul(w, v).reshape(q.shape)
+
+
 CHAIN_BINARY = {"add": np.add, "subtract": np.subtract, "multiply": np.multiply, "divide": np.divide,
                 "maximum": np.maximum, "minimum": np.minimum}
 CHAIN_UNARY = {"negate": np.negative, "abs": np.abs, "exponential": np.exp, "log": np.log, "sqrt": np.sqrt,
@@ -401,6 +433,14 @@ def custom_call(target: str, operands, backend_config: str = "") -> np.ndarray:
         if len(operands) < 2:
             raise ValueError("expected 2 inputs")
         return rope(operands[0], operands[1])
+    if target == "fused_batch_norm":
+        if len(operands) < 5:
+            raise ValueError("expected 5 inputs")
+        return batch_norm(*operands[:5], eps=float(cfg.get("eps", 1e-5)))            # CustomCallHandlers.swift:438
+    if target == "fused_depth_attention":
+        if len(operands) < 3:
+            raise ValueError("expected 3 inputs")
+        return depth_attention(*operands[:3], scale=float(cfg.get("scale", 1.0)))    # :1105
     if target == "fused_elementwise":
         ops = cfg.get("ops", cfg.get("operations"))               # CustomCallHandlers.swift:941-943
         if not isinstance(ops, list):

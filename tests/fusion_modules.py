@@ -388,3 +388,24 @@ def elementwise_call(ops, n_inputs, shape=(6, 40), dtype="f32", key="ops", scala
     return f"""func.func @main({args}) -> tensor<{t}> {{
   %r = stablehlo.custom_call @fused_elementwise({names}) {{backend_config = "{cfg}"}} : ({", ".join(types)}) -> tensor<{t}>
   return %r : tensor<{t}> }}"""
+
+
+def batch_norm_call(shape=(2, 5, 5, 16), dtype="f32", eps=1e-5, n_operands=5):
+    """custom_call @fused_batch_norm: x [.., C], gamma, beta, mean, variance [C]."""
+    t = "x".join(map(str, shape)) + "x" + dtype
+    c = f"{shape[-1]}x{dtype}"
+    names = ["%x", "%g", "%b", "%m", "%v"][:n_operands]
+    types = [f"tensor<{t}>"] + [f"tensor<{c}>"] * (n_operands - 1)
+    return f"""func.func @main(%x: tensor<{t}>, %g: tensor<{c}>, %b: tensor<{c}>, %m: tensor<{c}>, %v: tensor<{c}>) -> tensor<{t}> {{
+  %r = stablehlo.custom_call @fused_batch_norm({", ".join(names)}) {{backend_config = "{{\\"eps\\": {eps}}}"}} : ({", ".join(types)}) -> tensor<{t}>
+  return %r : tensor<{t}> }}"""
+
+
+def depth_attention_call(lead=(4,), depth=8, hidden=32, dtype="f32", scale=None, query_row=True):
+    """custom_call @fused_depth_attention: query [.., 1, H] (or [.., H]), keys and values [.., depth, H]."""
+    q = "x".join(map(str, lead + ((1, hidden) if query_row else (hidden,)))) + "x" + dtype
+    kv = "x".join(map(str, lead + (depth, hidden))) + "x" + dtype
+    cfg = "{}" if scale is None else '{\\"scale\\": ' + repr(float(scale)) + "}"
+    return f"""func.func @main(%q: tensor<{q}>, %k: tensor<{kv}>, %v: tensor<{kv}>) -> tensor<{q}> {{
+  %r = stablehlo.custom_call @fused_depth_attention(%q, %k, %v) {{backend_config = "{cfg}"}} : (tensor<{q}>, tensor<{kv}>, tensor<{kv}>) -> tensor<{q}>
+  return %r : tensor<{q}> }}"""

@@ -104,9 +104,9 @@ def test_error_codes(lib, client):
     unsup = ADD.replace("stablehlo.add", "stablehlo.atan2")
     assert lib.mhlo_compile(client, unsup.encode(), C.byref(exe)) == 4
     cc = """func.func @main(%a: tensor<4xf32>) -> tensor<4xf32> {
-      %0 = stablehlo.custom_call @fused_batch_norm(%a) {backend_config = "{}"} : (tensor<4xf32>) -> tensor<4xf32>
+      %0 = stablehlo.custom_call @fused_conv_bias_act(%a) {backend_config = "{}"} : (tensor<4xf32>) -> tensor<4xf32>
       return %0 : tensor<4xf32> }"""
-    assert lib.mhlo_compile(client, cc.encode(), C.byref(exe)) == 4 and b"fused_batch_norm" in lib.mhlo_get_last_error()
+    assert lib.mhlo_compile(client, cc.encode(), C.byref(exe)) == 4 and b"fused_conv_bias_act" in lib.mhlo_get_last_error()
     few = """func.func @main(%a: tensor<4x8xf32>) -> tensor<4x8xf32> {
       %0 = stablehlo.custom_call @fused_layer_norm(%a) {backend_config = "{}"} : (tensor<4x8xf32>) -> tensor<4x8xf32>
       return %0 : tensor<4x8xf32> }"""

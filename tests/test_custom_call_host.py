@@ -9,7 +9,8 @@ from metalhlo_amd.custom_call import BackendConfigParser as P
 def test_registry_contents():
     reg = cc.shared
     for t in ["fused_scaled_dot_product_attention", "fused_layer_norm", "fused_rms_norm",
-              "fused_matmul_bias_activation", "fused_softmax", "fused_gelu"]:
+              "fused_matmul_bias_activation", "fused_softmax", "fused_gelu", "fused_ffn", "fused_rope",
+              "fused_elementwise", "fused_batch_norm", "fused_depth_attention"]:
         assert reg.has_handler(t)
     assert not reg.has_handler("unknown_target")
     for t in cc.NOT_ON_PATH:

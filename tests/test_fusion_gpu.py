@@ -293,3 +293,62 @@ def test_trig_and_rounding_operations_of_the_front_end(sess):
     sess.lib.mhlo_executable_destroy(exe)
     close(a, np.sin(x.astype(np.float64)) * np.cos(x.astype(np.float64)), 1e-5)
     assert np.array_equal(b, np.ceil(x) - np.floor(x))
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16", "f16"])
+@pytest.mark.parametrize("shape", [(2, 5, 5, 16), (64, 30), (3, 7, 129), (4096, 64)], ids=["nhwc", "rank2-odd", "no-vectors", "large"])
+def test_fused_batch_norm(sess, shape, dtype):
+    """Normalisation with given statistics through the C API against the oracle; with the batch's own
+    statistics every channel of the fp32 result has mean beta."""
+    rng = np.random.default_rng(95)
+    C_ = shape[-1]
+    x = rng.standard_normal(shape) * 2 + 0.5
+    g, b = rng.uniform(0.5, 1.5, C_), rng.standard_normal(C_)
+    flat = x.reshape(-1, C_)
+    mu, var = flat.mean(axis=0), flat.var(axis=0)
+    arrs = [_to(a, dtype)[0] for a in (x, g, b, mu, var)]
+    exe = sess.compile(M.batch_norm_call(shape, dtype, eps=0.001))
+    (got,) = sess.run(exe, [(a, dtype) for a in arrs])
+    sess.lib.mhlo_executable_destroy(exe)
+    exp = oracle.batch_norm(*[_from(a, dtype) for a in arrs], eps=0.001)
+    close(_from(got, dtype), exp, 1e-5 if dtype == "f32" else 2e-2)
+    if dtype == "f32":
+        assert np.allclose(np.asarray(got, np.float64).reshape(-1, C_).mean(axis=0), b, atol=1e-4)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16", "f16"])
+@pytest.mark.parametrize("lead,depth,hidden,row", [((4,), 8, 32, True), ((2, 3), 32, 768, True), ((5,), 1, 40, True),
+                                                   ((3,), 64, 257, False), ((1,), 4, 16, True)],
+                         ids=["small", "attnres-768", "one-row", "depth64-odd-hidden", "batch1"])
+def test_fused_depth_attention(sess, lead, depth, hidden, row, dtype):
+    """Attention of one query row over a few stored rows through the C API against the oracle."""
+    rng = np.random.default_rng(96)
+    q = rng.standard_normal(lead + ((1, hidden) if row else (hidden,)))
+    k, v = rng.standard_normal(lead + (depth, hidden)), rng.standard_normal(lead + (depth, hidden))
+    scale = hidden ** -0.5
+    arrs = [_to(a, dtype)[0] for a in (q, k, v)]
+    exe = sess.compile(M.depth_attention_call(lead, depth, hidden, dtype, scale, row))
+    (got,) = sess.run(exe, [(a, dtype) for a in arrs])
+    sess.lib.mhlo_executable_destroy(exe)
+    exp = oracle.depth_attention(*[_from(a, dtype) for a in arrs], scale=scale)
+    close(_from(got, dtype), exp, 1e-5 if dtype == "f32" else 2e-2)
+
+
+def test_fused_depth_attention_reference_cases(sess):
+    """The reference's own cases (Tests/MetalHLOCoreTests/DepthAttentionTests.swift:46-137) at its tolerances:
+    equal keys give the mean of the value rows (1e-3), one dominant key selects its value row (0.1)."""
+    rng = np.random.default_rng(97)
+    q = rng.uniform(-1, 1, (1, 1, 8)).astype(np.float32)
+    k = np.ones((1, 4, 8), np.float32)
+    v = np.arange(32, dtype=np.float32).reshape(1, 4, 8)
+    exe = sess.compile(M.depth_attention_call((1,), 4, 8, "f32", 8 ** -0.5))
+    (got,) = sess.run(exe, [(q, "f32"), (k, "f32"), (v, "f32")])
+    sess.lib.mhlo_executable_destroy(exe)
+    assert np.all(np.abs(np.asarray(got).reshape(8) - v.mean(axis=1).reshape(8)) < 1e-3)
+    q = np.zeros((1, 1, 16), np.float32); q[0, 0, 0] = 10.0
+    k = np.zeros((1, 4, 16), np.float32); k[0, 2, 0] = 10.0
+    v = np.zeros((1, 4, 16), np.float32); v[0, 2] = np.arange(1, 17)
+    exe = sess.compile(M.depth_attention_call((1,), 4, 16, "f32", 1.0))
+    (got,) = sess.run(exe, [(q, "f32"), (k, "f32"), (v, "f32")])
+    sess.lib.mhlo_executable_destroy(exe)
+    assert np.all(np.abs(np.asarray(got).reshape(16) - np.arange(1, 17)) < 0.1)

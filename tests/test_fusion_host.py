@@ -375,3 +375,26 @@ def test_rope_and_elementwise_custom_calls_compile_and_reject(sess):
       %3 = stablehlo.ceil %2 : tensor<8xf32>
       return %3 : tensor<8xf32> }"""
     assert ops(sess, text) == ["sine", "cosine", "floor", "ceil"]
+
+
+def test_batch_norm_and_depth_attention_custom_calls_compile_and_reject(sess):
+    """fused_batch_norm and fused_depth_attention (Compiler/CustomCallHandlers.swift:414-452, 1084-1140): accepted
+    forms and the handlers' own operand-count errors, decided at compile time."""
+    assert ops(sess, M.batch_norm_call()) == ["fused_batch_norm"]
+    assert ops(sess, M.batch_norm_call(shape=(64, 30), dtype="bf16", eps=0.001)) == ["fused_batch_norm"]
+    with pytest.raises(capi.MHLOError) as e:     # CustomCallError.invalidInputCount(expected: 5, ...)
+        ops(sess, M.batch_norm_call(n_operands=4))
+    assert "expected 5" in str(e.value)
+    with pytest.raises(capi.MHLOError):          # a statistics vector of another length
+        ops(sess, M.batch_norm_call().replace("%m: tensor<16xf32>", "%m: tensor<8xf32>").replace(
+            "tensor<16xf32>, tensor<16xf32>) ->", "tensor<8xf32>, tensor<16xf32>) ->"))
+    assert ops(sess, M.depth_attention_call()) == ["fused_depth_attention"]
+    assert ops(sess, M.depth_attention_call(lead=(2, 3), depth=32, hidden=768, dtype="bf16", scale=0.036)) == ["fused_depth_attention"]
+    assert ops(sess, M.depth_attention_call(query_row=False)) == ["fused_depth_attention"]
+    with pytest.raises(capi.MHLOError) as e:     # more stored rows than the kernel holds scores for
+        ops(sess, M.depth_attention_call(depth=65))
+    assert "64" in str(e.value)
+    with pytest.raises(capi.MHLOError) as e:
+        ops(sess, M.depth_attention_call().replace("(%q, %k, %v)", "(%q, %k)").replace(
+            "(tensor<4x1x32xf32>, tensor<4x8x32xf32>, tensor<4x8x32xf32>)", "(tensor<4x1x32xf32>, tensor<4x8x32xf32>)"))
+    assert "expected 3" in str(e.value)

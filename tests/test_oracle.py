@@ -160,7 +160,7 @@ def test_custom_call_dispatch_contract():
     with pytest.raises(ValueError):
         oracle.custom_call("fused_layer_norm", [q, k], "")
     with pytest.raises(KeyError):
-        oracle.custom_call("fused_depth_attention", [q], "")
+        oracle.custom_call("fused_conv_bias_act", [q], "")
 
 
 # ---------------------------------------------------------------- C restatement vs float64 closed forms
@@ -445,3 +445,56 @@ def test_elementwise_chain_semantics():
         oracle.elementwise_chain([a, b], ["atan2"])
     with pytest.raises(ValueError):
         oracle.custom_call("fused_elementwise", [a, b], "{}")
+
+
+def test_batch_norm_pins():
+    """Closed cases for normalisation with given statistics (CustomCallHandlers.swift:414-452)."""
+    x = np.array([[1.0, 10.0], [3.0, 30.0]])
+    got = oracle.batch_norm(x, [2.0, 0.5], [0.5, -1.0], [2.0, 20.0], [1.0, 100.0], eps=0.0)
+    assert np.allclose(got, [[-1.5, -1.5], [2.5, -0.5]], atol=1e-14)
+    rng = np.random.default_rng(81)
+    x = rng.standard_normal((37, 5)) * 3 + 1
+    mu, var = x.mean(axis=0), x.var(axis=0)
+    eps = 0.1                                          # large, so that a dropped or misplaced eps shows
+    plain = oracle.batch_norm(x, np.ones(5), np.zeros(5), mu, var, eps=eps)
+    assert np.allclose(plain, oracle.layer_norm(x.T, np.ones(37), np.zeros(37), eps=eps).T, atol=1e-13)
+    g, b = rng.standard_normal(5), rng.standard_normal(5)
+    y = oracle.batch_norm(x, g, b, mu, var, eps=eps)
+    assert np.allclose(y.mean(axis=0), b, atol=1e-13)
+    assert np.allclose(y.var(axis=0), g * g * var / (var + eps), atol=1e-13)
+    # the channel axis is the last one of a tensor of any rank
+    x4 = rng.standard_normal((2, 3, 4, 5))
+    assert np.allclose(oracle.batch_norm(x4, g, b, mu, var, eps=eps).reshape(-1, 5),
+                       oracle.batch_norm(x4.reshape(-1, 5), g, b, mu, var, eps=eps))
+    assert np.allclose(oracle.custom_call("fused_batch_norm", [x, g, b, mu, var], '{"eps": 0.1}'), y)
+    with pytest.raises(ValueError):
+        oracle.custom_call("fused_batch_norm", [x, g, b, mu], "{}")
+
+
+def test_depth_attention_pins():
+    """The reference's own cases (Tests/MetalHLOCoreTests/DepthAttentionTests.swift:46-137) and what the
+    mathematics fixes."""
+    rng = np.random.default_rng(82)
+    # equal keys: uniform weights, the mean of the value rows (:46-95)
+    q = rng.uniform(-1, 1, (1, 8))
+    k = np.ones((1, 4, 8))
+    v = np.arange(32, dtype=np.float64).reshape(1, 4, 8)
+    assert np.allclose(oracle.depth_attention(q, k, v, scale=8 ** -0.5), v.mean(axis=1), atol=1e-13)
+    # one dominant key selects its value row (:97-137: query 10 e0, key row 2 = 10 e0, scale 1)
+    q = np.zeros((1, 16)); q[0, 0] = 10.0
+    k = np.zeros((1, 4, 16)); k[0, 2, 0] = 10.0
+    v = np.zeros((1, 4, 16)); v[0, 2] = np.arange(1, 17)
+    assert np.allclose(oracle.depth_attention(q, k, v, scale=1.0), v[:, 2], atol=1e-12)
+    # one head, one query row of the attention operator
+    B, L, H = 3, 7, 12
+    q, k, v = rng.standard_normal((B, 1, H)), rng.standard_normal((B, L, H)), rng.standard_normal((B, L, H))
+    ref = oracle.attention(q[:, None], k[:, None], v[:, None], scale=0.3)[:, 0]
+    got = oracle.depth_attention(q, k, v, scale=0.3)
+    assert got.shape == (B, 1, H) and np.allclose(got, ref, atol=1e-13)
+    # the query without its row axis gives the same numbers in its own shape
+    assert np.allclose(oracle.depth_attention(q[:, 0], k, v, scale=0.3), ref[:, 0], atol=1e-13)
+    # one stored row: that row, whatever the query; a vector added to every key changes nothing
+    assert np.allclose(oracle.depth_attention(q, k[:, :1], v[:, :1], scale=5.0), v[:, :1])
+    assert np.allclose(oracle.depth_attention(q, k + rng.standard_normal((B, 1, H)), v, scale=0.3), got, atol=1e-12)
+    assert np.allclose(oracle.custom_call("fused_depth_attention", [q, k, v], '{"scale": 0.3}'), got)
+    assert not np.allclose(oracle.custom_call("fused_depth_attention", [q, k, v], "{}"), got)      # default scale 1.0 (:1105)
