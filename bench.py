@@ -41,17 +41,17 @@ PEAK_CLOCK_MHZ = 2400.0     # the shader clock the matrix peak is quoted at
 # HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by what the same
 # counter reads for the 'copy' workload (256 MiB in, 256 MiB out); see profiles/<workload>.txt.
 # TRAFFIC_COMMIT: the commit of this repository the counter runs were taken at (the profiles say so too).
-TRAFFIC_COMMIT = "59bc453"
+TRAFFIC_COMMIT = "077862c"
 MEASURED_TRAFFIC = {
-    "gemm": 237460344,
-    "gemm_f32": 812973234,
-    "attention": 750479127,
-    "attention_full": 268940504,
-    "attention_f32": 1902930596,
-    "softmax": 536731572,
-    "layer_norm": 536898484,
-    "rms_norm": 536796223,
-    "bias_gelu": 536763241,
+    "gemm": 237451617,
+    "gemm_f32": 813140220,
+    "attention": 738688261,
+    "attention_full": 268939394,
+    "attention_f32": 1883326768,
+    "softmax": 536727449,
+    "layer_norm": 536894804,
+    "rms_norm": 536791829,
+    "bias_gelu": 536753799,
     "copy": 536870912,
 }
 
