@@ -14,7 +14,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 ROOT = os.path.dirname(HERE)
 
-HIP_SOURCES = ["runtime.hip", "row_kernels.hip", "gemm.hip", "gemm_f32.hip", "gemm256.hip", "tuning.hip", "attention.hip", "attention_pipe.hip", "attention_f32.hip", "glue_kernels.hip", "elementwise.hip", "fused_misc.hip"]
+HIP_SOURCES = ["runtime.hip", "row_kernels.hip", "gemm.hip", "gemm_f32.hip", "gemm256.hip", "gemm_twoset.hip", "tuning.hip", "attention.hip", "attention_pipe.hip", "attention_f32.hip", "glue_kernels.hip", "elementwise.hip", "fused_misc.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=fast",
@@ -48,9 +48,11 @@ def _exports(lib: str) -> str:
 
 
 def generate_sources(verbose: bool = True) -> None:
-    """Regenerates the hand-scheduled loops included by gemm256.hip and attention_pipe.hip."""
-    for script, target in (("gen_gemm256_loop.py", "gemm256_loop.inc"), ("gen_fa_loop.py", "fa_loop.inc")):
-        r = subprocess.run([sys.executable, os.path.join(CSRC, script)], capture_output=True, text=True)
+    """Regenerates the hand-scheduled loops included by gemm256.hip, gemm_twoset.hip and attention_pipe.hip."""
+    for script, args, target in (("gen_gemm256_loop.py", [], "gemm256_loop.inc"),
+                                 ("gen_gemm256_loop.py", ["two_set"], "gemm_twoset_loop.inc"),
+                                 ("gen_fa_loop.py", [], "fa_loop.inc")):
+        r = subprocess.run([sys.executable, os.path.join(CSRC, script), *args], capture_output=True, text=True)
         if r.returncode != 0:
             sys.stderr.write(r.stderr)
             raise RuntimeError("build step failed: " + script)

@@ -52,6 +52,7 @@ triggered by the barrier of stage t) and the unrolling (a multiple of D and of 2
 descriptions above are written for depth 5.
 
 Run:  python3 gen_gemm256_loop.py > gemm256_loop.inc
+      python3 gen_gemm256_loop.py two_set > gemm_twoset_loop.inc      (the members on two fragment sets, below)
 """
 NST = 5               # ring stages (set per emitted function, like BW)
 UNROLL = 10           # stages per loop body: lcm(ring, pair issue, fragment set rotation)
@@ -750,7 +751,19 @@ FAMILY = [(256, 5, "gemm256_loop"), (256, 4, "gemm256r4_loop"), (256, 6, "gemm25
 
 
 def main():
+    """No argument: the four-set family and the streamed loops (gemm256_loop.inc).  `two_set`: the
+    members on two fragment sets (gemm_twoset_loop.inc)."""
+    import sys
     print("// Generated by gen_gemm256_loop.py -- do not edit by hand.")
+    if sys.argv[1:] == ["two_set"]:
+        print("// Main loops of the 256x384 GEMM kernel and of the 256x128 kernel for two workgroups per compute unit")
+        print("// (the generator documents the schedule and the register maps).\n")
+        print("#define MHIP_HAVE_GEMM256X384_LOOP 1\n")
+        for member, stem in ((_x384(), "gemm256x384_loop"), (_xpair(), "gemm_pair_loop")):
+            for tname, mnem in (("bf16", "v_mfma_f32_32x32x16_bf16"), ("f16", "v_mfma_f32_32x32x16_f16")):
+                for lname, ka, kb in (("nn", "K", "MN"), ("nt", "K", "K"), ("tn", "MN", "MN"), ("tt", "MN", "K")):
+                    emit_two_set(member, f"{stem}_{lname}_{tname}", mnem, ka, kb)
+        return
     print("// Main loops of the 256x256 and 256x128 GEMM kernels (the generator documents the schedule")
     print("// and the register map).\n")
     for bw, ring, stem in FAMILY:
@@ -763,11 +776,6 @@ def main():
         for tname, mnem in (("bf16", "v_mfma_f32_32x32x16_bf16"), ("f16", "v_mfma_f32_32x32x16_f16")):
             for lname, ka, kb in (("nn", "K", "MN"), ("nt", "K", "K"), ("tn", "MN", "MN"), ("tt", "MN", "K")):
                 emit(f"{stem}_{lname}_{tname}", mnem, ka, kb)
-    print("#define MHIP_HAVE_GEMM256X384_LOOP 1\n")
-    for member, stem in ((_x384(), "gemm256x384_loop"), (_xpair(), "gemm_pair_loop")):
-        for tname, mnem in (("bf16", "v_mfma_f32_32x32x16_bf16"), ("f16", "v_mfma_f32_32x32x16_f16")):
-            for lname, ka, kb in (("nn", "K", "MN"), ("nt", "K", "K"), ("tn", "MN", "MN"), ("tt", "MN", "K")):
-                emit_two_set(member, f"{stem}_{lname}_{tname}", mnem, ka, kb)
     # streamed tiles: the 256x128 kernel as a persistent workgroup, for A with k contiguous
     configure(128, 5)
     for tname, mnem in (("bf16", "v_mfma_f32_32x32x16_bf16"), ("f16", "v_mfma_f32_32x32x16_f16")):

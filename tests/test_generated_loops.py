@@ -1,4 +1,4 @@
-"""Host-side check of the generated inline-assembly loops (gemm256_loop.inc, fa_loop.inc): every register an
+"""Host-side check of the generated inline-assembly loops (gemm256_loop.inc, gemm_twoset_loop.inc, fa_loop.inc): every register an
 assembly block writes must be declared to the compiler as an output, an in/out operand or a
 clobber.  A persistent kernel calls these blocks several times and keeps values live across them,
 so one undeclared write lets the compiler reuse a register the block has changed (seen once: a
@@ -8,7 +8,7 @@ import re
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(os.path.dirname(HERE), "metalhlo_amd", "csrc")
-INCS = [os.path.join(CSRC, "gemm256_loop.inc"), os.path.join(CSRC, "fa_loop.inc")]
+INCS = [os.path.join(CSRC, "gemm256_loop.inc"), os.path.join(CSRC, "gemm_twoset_loop.inc"), os.path.join(CSRC, "fa_loop.inc")]
 
 NO_DEST = ("s_waitcnt", "s_barrier", "s_nop", "s_cbranch", "s_cmp", "s_branch", "buffer_load", "global_store",
            "ds_write")
