@@ -231,6 +231,26 @@ def test_gemm_large_tiles(shape, layout, dtype, tile, lib):
     assert torch.equal(c, c128)
 
 
+@pytest.mark.parametrize("tile", ["2560", "2561", "2567", "2568"], ids=["256x256", "256x128", "256x384", "256x128-two-per-cu"])
+def test_gemm_ring_kernels_batched(tile, lib, monkeypatch):
+    """The ring kernels on a strided batch (one grid row per matrix): every batch element against the
+    oracle on sampled rows and bit for bit against the 128x128 kernel."""
+    from metalhlo_amd import kernels
+    M, N, K, B = 2048, 2312, 224, 4            # 8 x 7 x 4 = 224 tiles of 256x384, ragged in N
+    a, b = _ab(M, N, K, torch.bfloat16, 51, batch=(B,))
+    rng = np.random.default_rng(52)
+    bias = to_dev(rng.standard_normal(N) * 0.5, torch.bfloat16)
+    monkeypatch.setenv("MHIP_GEMM_TILE", tile)
+    c = kernels.matmul(a, b, bias, "relu")
+    assert lib.mhip_gemm_last_variant() == int(tile)
+    monkeypatch.setenv("MHIP_GEMM_TILE", "128")
+    assert torch.equal(c, kernels.matmul(a, b, bias, "relu"))
+    rows = np.r_[0, 255, 256, M - 1, rng.integers(0, M, 12)]
+    for i in range(B):
+        exp = oracle.matmul_bias_act(as_f64(a[i])[rows], as_f64(b[i]), as_f64(bias), "relu")
+        assert_close(c[i][rows], exp, 2e-2, f"batched {tile} element {i}")
+
+
 # Shapes with >= 192 tiles of 256x384 (K stages of 32: a single stage, exits at every position of the
 # unrolled ring of four, several trips; M and N ragged against the tile and, once, N odd).
 WIDEST = [(8192, 2304, 32), (7944, 2408, 96), (8192, 2696, 160), (7680, 3072, 448), (8192, 2304, 768),
