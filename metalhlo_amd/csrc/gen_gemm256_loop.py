@@ -164,7 +164,9 @@ def mfmas(mnem, fset):
     a, b = SET[fset]
     out = []
     for i in range(4):
-        for j in range(NBF):
+        # back and forth over the B fragments: consecutive MFMAs then always share one operand
+        # (B when the row block changes), which leaves fewer operand lines toggling
+        for j in (range(NBF) if i % 2 == 0 else reversed(range(NBF))):
             acc = 16 * (NBF * i + j)
             # (B, A): the accumulator tile comes out transposed (lane = row m)
             out.append(f"{mnem} a[{acc}:{acc + 15}], {vr(b + 4 * j, 4)}, {vr(a + 4 * i, 4)}, a[{acc}:{acc + 15}]")
@@ -535,7 +537,9 @@ class TwoSet:
 def _x384():
     def acc(b):
         return f"a[{16 * b}:{16 * b + 15}]" if b < 16 else vr(128 + 16 * (b - 16), 16)
-    grid = [(6 * i + j, "B" if j < 4 else "B2", j if j < 4 else j - 4, i) for i in range(4) for j in range(6)]
+    # (back and forth over the B fragments, as in `mfmas`)
+    grid = [(6 * i + j, "B" if j < 4 else "B2", j if j < 4 else j - 4, i)
+            for i in range(4) for j in (range(6) if i % 2 == 0 else reversed(range(6)))]
     return TwoSet("384", 4, ("A", "B", "B2"), {"A": 0, "B": 16384, "B2": 32768},
                   {0: {"A": 0, "B": 16, "B2": 32}, 1: {"A": 40, "B": 56, "B2": 72}},
                   {"A": 80, "B": 88, "B2": 96}, {"A": 100, "B": 101, "B2": 102}, {"A": 103, "B": 104, "B2": 105},
@@ -544,7 +548,7 @@ def _x384():
 
 
 def _xpair():
-    grid = [(2 * i + j, "B", j, i) for i in range(4) for j in range(2)]
+    grid = [(2 * i + j, "B", j, i) for i in range(4) for j in (range(2) if i % 2 == 0 else reversed(range(2)))]
     return TwoSet("pair", 3, ("A", "B"), {"A": 0, "B": 16384},
                   {0: {"A": 0, "B": 16}, 1: {"A": 24, "B": 40}},
                   {"A": 48, "B": 56}, {"A": 60, "B": 61}, {"A": 62, "B": 63},
