@@ -462,7 +462,7 @@ static int launch_column_split(hipStream_t s, const GemmArgs& g, int64_t batch, 
     return launch_gemm256(s, w, 1, TA, TB, dt);
 }
 
-// Which kernel serves a 16-bit problem (MHIP_GEMM_TILE = 128 | 256 | 2560 ... 2568 forces one; 2564 / 2565 = the
+// Which kernel serves a 16-bit problem (MHIP_GEMM_TILE = 128 | 256 | 2560 ... 2569 forces one; 2564 / 2565 = the
 // 256x128 tile with a ring of six / four stages, 2566 = the 256x256 tile with four, 2568 = the 256x128
 // tile as two workgroups per compute unit: members of the generated family that only a forced choice
 // or the tuning table selects; 2567 = the 256x384 tile):
@@ -481,6 +481,7 @@ static int launch_column_split(hipStream_t s, const GemmArgs& g, int64_t batch, 
 //     launch_column_split) where the problem has that shape;
 //   * 256x384 tiles (2567; no activation, relu or tanh-GELU) where one round of them replaces two
 //     or three of the others;
+//   * 128x192 tiles (2569) where 256-row tiles would leave compute units idle (few columns);
 //   * the eight-wave 256x256 kernel for large problems the ring kernel cannot take whose
 //     rows of C are not 16-byte aligned (odd N): its eight waves hide the narrow stores;
 //   * otherwise 128x128 tiles, two workgroups per CU (short K, few tiles).
@@ -513,6 +514,10 @@ static int pick_tile(hipStream_t s, const GemmArgs& g, int64_t batch) {
     if (force == 2566) {
         if (gemm256_eligible(g, batch, TA, TB, dt)) return chose(2566, launch_gemm256(s, g, batch, TA, TB, dt, 256, 4));
     }
+    // the 128x192 tile (ring of six)
+    if (force == 2569) {
+        if (gemm256_eligible(g, batch, TA, TB, dt, 192)) return chose(2569, launch_gemm256(s, g, batch, TA, TB, dt, 192, 6));
+    }
     // the 256x128 tile with two workgroups per compute unit (ring of three)
     if (force == 2568) {
         if (gemm256_eligible(g, batch, TA, TB, dt, 128)) return chose(2568, launch_gemm256(s, g, batch, TA, TB, dt, 128, 3));
@@ -525,7 +530,29 @@ static int pick_tile(hipStream_t s, const GemmArgs& g, int64_t batch) {
     const int64_t narrow = tiles_m * ((g.N + 127) / 128) * batch, stages = g.K / 32;
     const int64_t wide_cost = ((big + cus - 1) / cus) * (stages * 32 + 700);
     const int64_t narrow_cost = ((narrow + cus - 1) / cus) * (stages * 18 + 500);
-    if (force == 0 && g.K >= 512 && gemm256_eligible(g, batch, TA, TB, dt, 384) && gemm384_activation_ok(g.act)) {
+    // (wide tiles on the columns that make whole rounds + one round of a narrow band, where the default takes that form)
+    int n_split = 0;
+    const bool split_ok = gemm_split_shape(g, batch, &n_split) && narrow > 2 * cus;
+    const int64_t split_cost = split_ok ? (tiles_m * (n_split / 256) / cus) * (stages * 32 + 700) + (stages * 18 + 500) : ((int64_t)1 << 62);
+    const bool wider_ok = gemm256_eligible(g, batch, TA, TB, dt, 384) && gemm384_activation_ok(g.act);
+    const int64_t wider_cost = ((tiles_m * ((g.N + 383) / 384) * batch + cus - 1) / cus) * (stages * 53 + 1050);
+    if (force == 0 && g.K >= 512 && gemm256_eligible(g, batch, TA, TB, dt, 192)) {
+        // The 128x192 tile where 256-row tiles leave compute units idle: its stage moves 20 KB
+        // from the L2s against the narrow tile's 24 and costs 14 slots, the ends 500 -- fitted to
+        // [8192,3072] x [3072,768] (256 tiles of it against 192 narrow ones: 46.4 us against 53.5
+        // in a loop of its own, 40.6 against 48.2 with the caches emptied before each launch) and
+        // K 768 (24.5 against 25.7); inside a GPT-2 pass the two GEMMs with 768 columns take
+        // 72 us less in all (3.313 -> 3.241 ms on one box).
+        const int64_t small = ((g.M + 127) / 128) * ((g.N + 191) / 192) * batch;
+        const int64_t small_cost = ((small + cus - 1) / cus) * (stages * 14 + 500);
+        int64_t other = (int64_t)1 << 62;
+        if (gemm256_eligible(g, batch, TA, TB, dt) && wide_cost < other) other = wide_cost;
+        if (gemm256_eligible(g, batch, TA, TB, dt, 128) && narrow_cost < other) other = narrow_cost;
+        if (wider_ok && wider_cost < other) other = wider_cost;
+        if (split_cost < other) other = split_cost;
+        if (small_cost < other) return chose(2569, launch_gemm256(s, g, batch, TA, TB, dt, 192, 6));
+    }
+    if (force == 0 && g.K >= 512 && wider_ok) {
         // The 256x384 tile where it saves a round: its stage costs 53 slots (48 MFMAs, and only
         // one k-step of fragments read ahead), its prologue and epilogue 1050 (half as many
         // accumulators again to convert and store) -- fitted to [8192,2304..12288] x K 768..6144:
@@ -533,12 +560,8 @@ static int pick_tile(hipStream_t s, const GemmArgs& g, int64_t batch) {
         // against 49; inside a GPT-2 pass 50.3 against 55, and [8192,2304] 41.8 against 45.8 for
         // the column split), while from two rounds on the wide tile's shorter epilogue wins
         // ([8192,12288] x K 768: 170 us against 159).
-        const int64_t wider = tiles_m * ((g.N + 383) / 384) * batch;
-        const int64_t wider_cost = ((wider + cus - 1) / cus) * (stages * 53 + 1050);
-        int n_wide = 0;
         int64_t other = wide_cost < narrow_cost ? wide_cost : narrow_cost;
-        if (gemm_split_shape(g, batch, &n_wide) && narrow > 2 * cus)
-            other = (tiles_m * (n_wide / 256) / cus) * (stages * 32 + 700) + (stages * 18 + 500);
+        if (split_ok) other = split_cost;
         if (wider_cost < other) return chose(2567, launch_gemm256(s, g, batch, TA, TB, dt, 384, 4));
     }
     if (force == 2563 || (force == 0 && g.K >= 512)) {

@@ -25,6 +25,7 @@ namespace mhip {
 // gemm_twoset.hip: the 256x384 tile and the 256x128 tile for two workgroups per compute unit
 int launch_gemm384(hipStream_t s, const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype);
 int launch_gemm_pair(hipStream_t s, const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype);
+int launch_gemm192(hipStream_t s, const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype);
 
 namespace {
 
@@ -337,7 +338,8 @@ bool gemm256_eligible(const GemmArgs& g, int64_t batch, int trans_a, int trans_b
     const int64_t a_bytes = ((int64_t)((trans_a ? g.K : g.M) - 1) * g.lda + (trans_a ? g.M : g.K)) * 2;
     const int64_t b_bytes = ((int64_t)((trans_b ? g.N : g.K) - 1) * g.ldb + (trans_b ? g.K : g.N)) * 2;
     if (a_bytes >= 0x70000000LL || b_bytes >= 0x70000000LL) return false;
-    const int64_t tiles = (int64_t)((g.M + 255) / 256) * ((g.N + bw - 1) / bw) * batch;
+    const int tile_rows = bw == 192 ? 128 : 256;
+    const int64_t tiles = (int64_t)((g.M + tile_rows - 1) / tile_rows) * ((g.N + bw - 1) / bw) * batch;
     return (tiles >= 192 || any_tile_count) && tiles <= 0x7FFFFFFF && batch <= 65535;
 }
 
@@ -346,6 +348,7 @@ bool gemm256_eligible(const GemmArgs& g, int64_t batch, int trans_a, int trans_b
 int launch_gemm256(hipStream_t s, const GemmArgs& g, int64_t batch, int trans_a, int trans_b,
                    int dtype, int bw, int ring) {
     if (bw == 384) return launch_gemm384(s, g, batch, trans_a, trans_b, dtype);
+    if (bw == 192) return launch_gemm192(s, g, batch, trans_a, trans_b, dtype);                     // 128-row tiles
     if (bw == 128 && ring == 3) return launch_gemm_pair(s, g, batch, trans_a, trans_b, dtype);      // two workgroups per compute unit
     if (dtype == MHIP_BF16) return family256<bf16_t>(s, g, batch, trans_a, trans_b, bw, ring);
     return family256<f16_t>(s, g, batch, trans_a, trans_b, bw, ring);

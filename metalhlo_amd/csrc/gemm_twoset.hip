@@ -334,6 +334,202 @@ int layout_pair(hipStream_t s, const GemmArgs& g, int64_t batch, int ta, int tb)
     return launch_pair<T, true, true>(s, g, batch);
 }
 
+// ---- the 128x192 tile --------------------------------------------------------------------------------
+// gemm128x192_loop_* of the generated file: a tile for problems with so few columns that 256-row
+// tiles leave compute units idle ([8192, 768] has 192 tiles of 256x128 and 256 of 128x192; the sum of
+// rows and columns, which is what a stage moves from the L2s, is the smallest for that area).  Each
+// wave 64 x 96 = 2 x 3 accumulator blocks; A is 128 rows; B's 192 columns lie in the 256-column layout
+// of the wide kernel (loads of the last quarter carry an out-of-range offset and move nothing); a
+// stage is 24 KB, the ring six deep.
+constexpr int k192Stage = 24 * 1024;
+constexpr int k192Smem = 6 * k192Stage;
+constexpr uint32_t k192BOffset = 8 * 1024;   // B tile behind the 8 KB A tile of a stage
+
+template <typename T, bool TA, bool TB>
+__device__ __forceinline__ void main_loop192(f32x16 (&acc)[6], u32x2 ra, u32x4 rb, u32x2& goff,
+                                             __amdgpu_buffer_rsrc_t rsa, __amdgpu_buffer_rsrc_t rsb, uint32_t pa,
+                                             uint32_t pb, uint32_t ta, uint32_t tb, uint32_t m0b, uint32_t kt) {
+    constexpr bool bf = std::is_same<T, bf16_t>::value;
+#define MHIP_LOOP(cond, name) \
+    if constexpr (cond) gemm128x192_loop_##name(acc, ra, rb, goff, rsa, rsb, pa, pb, ta, tb, m0b, kt);
+    MHIP_LOOP(bf && !TA && !TB, nn_bf16)
+    MHIP_LOOP(bf && !TA && TB, nt_bf16)
+    MHIP_LOOP(bf && TA && !TB, tn_bf16)
+    MHIP_LOOP(bf && TA && TB, tt_bf16)
+    MHIP_LOOP(!bf && !TA && !TB, nn_f16)
+    MHIP_LOOP(!bf && !TA && TB, nt_f16)
+    MHIP_LOOP(!bf && TA && !TB, tn_f16)
+    MHIP_LOOP(!bf && TA && TB, tt_f16)
+#undef MHIP_LOOP
+}
+
+// Epilogue: a wave's 64 x 96 sub-tile through LDS one 32-row block at a time (32 rows of 192 + 16
+// bytes per wave); a block goes out as six instructions of 64 lanes x 16 bytes: lane slot
+// (u % 3) * 64 + lane = row 16 (u / 3) + slot / 12 of the block, chunk slot % 12.
+template <typename T>
+__device__ __forceinline__ void store_tile192(f32x16 (&acc)[6], char* smem, const GemmArgs& g, T* c, const T* res,
+                                              int m0, int n0) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int lrow = lane & 31, lhalf = lane >> 5;
+    const T* bias = static_cast<const T*>(g.bias);
+    constexpr int kRowPad = 96 * 2 + 16;
+    char* stage = smem + wave * (32 * kRowPad);
+    const int ldc = g.ldc ? g.ldc : g.N;
+    const int nw = n0 + wn * 96;                         // the wave's first column
+    const bool full_cols = __builtin_amdgcn_readfirstlane(n0 + 192 <= g.N);
+    const bool interior = __builtin_amdgcn_readfirstlane(full_cols && m0 + wm * 64 + 64 <= g.M && ldc % 8 == 0);
+    Pack4<T> bq[12];
+    static_for<12>([&](auto jq_tag) {
+        constexpr int jq = decltype(jq_tag)::value;
+        bq[jq] = __builtin_bit_cast(Pack4<T>, u32x2{0u, 0u});
+    });
+    if (bias) {
+        if (full_cols) {
+            static_for<12>([&](auto jq_tag) {
+                constexpr int jq = decltype(jq_tag)::value;
+                bq[jq] = __builtin_bit_cast(Pack4<T>, *reinterpret_cast<const u32x2*>(bias + nw + 8 * jq + 4 * lhalf));
+            });
+        } else {
+            static_for<12>([&](auto jq_tag) {
+                constexpr int jq = decltype(jq_tag)::value;
+                const int n = nw + 8 * jq + 4 * lhalf;
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    if (n + e < g.N) bq[jq].v[e] = bias[n + e];
+            });
+        }
+    }
+    dispatch_act(g.act, [&](auto act_tag) __attribute__((always_inline)) {
+    constexpr int ACT = decltype(act_tag)::value;
+    static_for<2>([&](auto i_tag) __attribute__((always_inline)) {
+        constexpr int i = decltype(i_tag)::value;
+        static_for<12>([&](auto jq_tag) __attribute__((always_inline)) {
+            constexpr int j = decltype(jq_tag)::value >> 2, q = decltype(jq_tag)::value & 3;
+            Pack4<T> o;
+            static_for<4>([&](auto e_tag) {
+                constexpr int e = decltype(e_tag)::value;
+                float v = acc_value(acc[3 * i + j][4 * q + e]) + Elem<T>::to_f32(bq[j * 4 + q].v[e]);
+                v = apply_act_c<ACT>(v);
+                o.v[e] = Elem<T>::from_f32(v);
+            });
+            *reinterpret_cast<u32x2*>(stage + lrow * kRowPad + (j * 32 + 8 * q + 4 * lhalf) * 2) =
+                __builtin_bit_cast(u32x2, o);
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // a wave re-reads only its own rows
+        if (interior) {
+            u32x4 w[6], r[6];
+            int64_t off[6];
+#pragma unroll
+            for (int u = 0; u < 6; u++) {
+                const int slot = (u % 3) * 64 + lane;
+                const int rl = 16 * (u / 3) + slot / 12, ch = slot % 12;
+                off[u] = (int64_t)(m0 + wm * 64 + i * 32 + rl) * ldc + nw + 8 * ch;
+                if (res) r[u] = *reinterpret_cast<const u32x4*>(res + off[u]);
+                w[u] = *reinterpret_cast<const u32x4*>(stage + rl * kRowPad + ch * 16);
+            }
+#pragma unroll
+            for (int u = 0; u < 6; u++) {
+                if (res) w[u] = add_chunk<T>(w[u], r[u]);
+                *reinterpret_cast<u32x4*>(c + off[u]) = w[u];
+            }
+        } else {
+#pragma unroll 1
+            for (int u = 0; u < 6; u++) {
+                const int slot = (u % 3) * 64 + lane;
+                const int rl = 16 * (u / 3) + slot / 12, ch = slot % 12;
+                const int m = m0 + wm * 64 + i * 32 + rl;
+                const int n = nw + 8 * ch;
+                T* cp = c + (int64_t)m * ldc + n;
+                const T* rp = res + (int64_t)m * ldc + n;
+                if (m < g.M && n + 8 <= g.N) {
+                    u32x4 w = *reinterpret_cast<const u32x4*>(stage + rl * kRowPad + ch * 16);
+                    if (res) w = add_chunk<T>(w, *reinterpret_cast<const u32x4_unaligned*>(rp));
+                    *reinterpret_cast<u32x4_unaligned*>(cp) = w;
+                } else if (m < g.M && n < g.N) {                 // the last, partial chunk of a row
+                    const T* sv = reinterpret_cast<const T*>(stage + rl * kRowPad + ch * 16);
+                    for (int e = 0; e < g.N - n; e++) {
+                        T val = sv[e];
+                        if (res) val = Elem<T>::from_f32(Elem<T>::to_f32(val) + Elem<T>::to_f32(rp[e]));
+                        cp[e] = val;
+                    }
+                }
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the next block overwrites the rows just read
+        __builtin_amdgcn_sched_barrier(0);
+    });
+    });
+}
+
+template <typename T, bool TA, bool TB>
+__global__ __launch_bounds__(256) void gemm192_kernel(GemmArgs g) {
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    using LA = typename std::conditional<TA, MnMajor<128>, KMajor>::type;
+    using LB = typename std::conditional<TB, KMajor, MnMajor<256>>::type;
+
+    int tm, tn;
+    tile_of(blockIdx.x, gridDim.x, g.tiles_m, g.tiles_n, tm, tn);
+    const int m0 = tm * 128, n0 = tn * 192;
+    const int64_t batch = blockIdx.y;
+    const char* a = reinterpret_cast<const char*>(static_cast<const T*>(g.a) + batch * g.sa);
+    const char* b = reinterpret_cast<const char*>(static_cast<const T*>(g.b) + batch * g.sb);
+    T* c = static_cast<T*>(g.c) + batch * g.sc;
+    const T* res = g.residual ? static_cast<const T*>(g.residual) + batch * g.sc : nullptr;
+    const uint32_t a_bytes = (uint32_t)(((int64_t)((TA ? g.K : g.M) - 1) * g.lda + (TA ? g.M : g.K)) * 2);
+    const uint32_t b_bytes = (uint32_t)(((int64_t)((TB ? g.N : g.K) - 1) * g.ldb + (TB ? g.K : g.N)) * 2);
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
+    const u32x4 raw = LA::raddr(lane, wm * 64, lds0);
+    u32x2 ra;
+    ra.x = raw.x; ra.y = raw.y;
+    const u32x4 rb = LB::raddr(lane, wn * 96, lds0 + k192BOffset);
+    u32x2 goff;
+    goff.x = LA::goff(lane, wave, m0, g.lda, g.M);
+    // (columns past the tile's 192 are not asked for: the layout is 256 wide)
+    goff.y = LB::goff(lane, wave, n0, g.ldb, min(g.N, n0 + 192));
+    const uint32_t m0b = __builtin_amdgcn_readfirstlane(lds0 + (uint32_t)wave * 1024u);
+    const __amdgpu_buffer_rsrc_t rsa =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(a), 0, a_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsb =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(b), 0, b_bytes, 0x00020000);
+
+    f32x16 acc[6];
+    main_loop192<T, TA, TB>(acc, ra, rb, goff, rsa, rsb, LA::pass_stride(g.lda), LB::pass_stride(g.ldb),
+                            LA::stage_stride(g.lda), LB::stage_stride(g.ldb), m0b, (uint32_t)(g.K / 32));
+    store_tile192<T>(acc, smem, g, c, res, m0, n0);
+}
+
+template <typename T, bool TA, bool TB>
+int launch192(hipStream_t s, GemmArgs g, int64_t batch) {
+    auto kern = gemm192_kernel<T, TA, TB>;
+    static std::once_flag once;
+    static hipError_t attr_err = hipSuccess;
+    std::call_once(once, [&] {
+        attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, k192Smem);
+    });
+    if (attr_err != hipSuccess)
+        return fail(MHIP_ERR_LAUNCH, "gemm192: cannot reserve %d bytes of LDS: %s", k192Smem,
+                    hipGetErrorString(attr_err));
+    g.tiles_m = (g.M + 127) / 128;
+    g.tiles_n = (g.N + 191) / 192;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(g.tiles_m * g.tiles_n), (unsigned)batch), dim3(256),
+                       k192Smem, s, g);
+    return check_launch("gemm192");
+}
+
+template <typename T>
+int layout192(hipStream_t s, const GemmArgs& g, int64_t batch, int ta, int tb) {
+    if (!ta && !tb) return launch192<T, false, false>(s, g, batch);
+    if (!ta && tb) return launch192<T, false, true>(s, g, batch);
+    if (ta && !tb) return launch192<T, true, false>(s, g, batch);
+    return launch192<T, true, true>(s, g, batch);
+}
+
 }  // namespace
 
 // The activations the 256x384 kernel's epilogue serves.
@@ -341,6 +537,10 @@ bool gemm384_activation_ok(int act) { return act == MHIP_ACT_NONE || act == MHIP
 
 int launch_gemm384(hipStream_t s, const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype) {
     return dtype == MHIP_BF16 ? layout384<bf16_t>(s, g, batch, trans_a, trans_b) : layout384<f16_t>(s, g, batch, trans_a, trans_b);
+}
+
+int launch_gemm192(hipStream_t s, const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype) {
+    return dtype == MHIP_BF16 ? layout192<bf16_t>(s, g, batch, trans_a, trans_b) : layout192<f16_t>(s, g, batch, trans_a, trans_b);
 }
 
 int launch_gemm_pair(hipStream_t s, const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype) {

@@ -522,9 +522,11 @@ class TwoSet:
     """One member of the two-fragment-set family: geometry and register map."""
 
     def __init__(self, name, nst, ops, region, sets, raddr, goff, goff2, blocks, passes, rowb, passmult,
-                 acc_regs, grid, goff_span, clobber_to):
+                 acc_regs, grid, goff_span, clobber_to, stage=None, a_blocks=4):
         self.name, self.nst, self.ops = name, nst, ops
-        self.stage = sum(passes[o] * 4096 for o in ops)
+        # (`passes` of an operand: a number, or one per layout {"K": .., "MN": ..})
+        self.stage = stage if stage else sum(passes[o] * 4096 for o in ops)
+        self.a_blocks = a_blocks          # 32-row blocks of A per wave
         self.unroll = nst if nst % 2 == 0 else 2 * nst
         self.region, self.sets, self.raddr, self.goff, self.goff2 = region, sets, raddr, goff, goff2
         self.blocks, self.passes, self.rowb, self.passmult = blocks, passes, rowb, passmult
@@ -556,7 +558,26 @@ def _xpair():
                   {}, [f"a[{16 * b}:{16 * b + 15}]" for b in range(8)], grid, 2, 48)
 
 
+def _x192():
+    """128 x 192 tile: each wave 64 x 96 = 2 x 3 accumulator blocks in a[0:95]; A is 128 rows, B 192
+    columns held in the 256-column layout of the wide kernel (its last quarter is never asked
+    for); a stage is 24 KB, the ring six deep.  Register map: fragment set n: A v[20n : 20n+7], B
+    v[20n+8 : 20n+19]; v[40:45] A read addresses, v[48:56] B; v60 / v61 global offsets, v62 / v63
+    the same + 64."""
+    grid = [(3 * i + j, "B", j, i) for i in range(2) for j in (range(3) if i % 2 == 0 else reversed(range(3)))]
+    return TwoSet("x192", 6, ("A", "B"), {"A": 0, "B": 8192},
+                  {0: {"A": 0, "B": 8}, 1: {"A": 20, "B": 28}},
+                  {"A": 40, "B": 48}, {"A": 60, "B": 61}, {"A": 62, "B": 63},
+                  {"A": 2, "B": 3}, {"A": 2, "B": {"K": 3, "MN": 4}}, {"A": 256, "B": 512},
+                  {}, [f"a[{16 * b}:{16 * b + 15}]" for b in range(6)], grid, 2, 40, stage=24576, a_blocks=2)
+
+
 X = None      # the member being emitted
+
+
+def x_passes(kinds, which):
+    p = X.passes[which]
+    return p[x_kind(kinds, which)] if isinstance(p, dict) else p
 
 
 def x_kind(kinds, which):
@@ -606,13 +627,13 @@ def x_trigger_group(kinds, t):
     for which in X.ops:
         if x_kind(kinds, which) == "K":
             if (t + X.nst - 1) % 2 == 0:
-                for p in range(X.passes[which]):
+                for p in range(x_passes(kinds, which)):
                     grp.append(x_load(kinds, which, t + X.nst - 1, p))
                     grp.append(x_load(kinds, which, t + X.nst, p, second_half=True))
                 grp.append(dict(stage=None, lines=[f"v_add_u32 v{X.goff[which]}, 128, v{X.goff[which]}",
                                                    f"v_add_u32 v{X.goff2[which]}, 128, v{X.goff2[which]}"]))
         else:
-            for p in range(X.passes[which]):
+            for p in range(x_passes(kinds, which)):
                 grp.append(x_load(kinds, which, t + X.nst, p))
             step = "%[ta]" if which == "A" else "%[tb]"
             grp.append(dict(stage=None, lines=[f"v_add_u32 v{X.goff[which]}, {step}, v{X.goff[which]}"]))
@@ -677,8 +698,9 @@ def x_body(mnem, kinds):
     # fragment read addresses of the ring's last buffer(s) from those of buffers 0 and 1
     for which in X.ops:
         n = 2 if x_kind(kinds, which) == "K" else X.blocks[which]
-        for e in range(n):
-            out.append(f"v_add_u32 v{X.raddr[which] + n + e}, {2 * X.stage}, v{X.raddr[which] + e}")
+        for h in range(1, (X.nst + 1) // 2):
+            for e in range(n):
+                out.append(f"v_add_u32 v{X.raddr[which] + n * h + e}, {h * 2 * X.stage}, v{X.raddr[which] + e}")
         out.append(f"v_add_u32 v{X.goff2[which]}, 64, v{X.goff[which]}")
     for t in range(-X.nst, -1):
         for ld in x_trigger_group(kinds, t):
@@ -716,7 +738,7 @@ def emit_two_set(member, name, mnem, ka, kb):
     print(f"// {name}: two fragment sets, ring of {X.nst}; A operand {ka}-major, B operand {kb}-major, {mnem}")
     args = [f"f32x16 (&acc)[{nacc}]"]
     for which in X.ops:
-        args.append(("u32x4& r" if X.blocks[which] == 4 else "u32x2& r") + which.lower())
+        args.append(("u32x4& r" if X.blocks[which] > 2 else "u32x2& r") + which.lower())
     args.append(("u32x4& " if X.goff_span == 4 else "u32x2& ") + "goff")
     print(f"__device__ __forceinline__ void {name}({', '.join(args)},")
     print("        __amdgpu_buffer_rsrc_t rsa, __amdgpu_buffer_rsrc_t rsb, uint32_t pa, uint32_t pb,")
@@ -730,7 +752,7 @@ def emit_two_set(member, name, mnem, ka, kb):
     io = [f'"+{{v[{g0}:{g0 + X.goff_span - 1}]}}"(goff)']
     declared = set(range(g0, g0 + X.goff_span))
     for which in X.ops:
-        base, n = X.raddr[which], X.blocks[which]
+        base, n = X.raddr[which], (4 if X.blocks[which] > 2 else 2)
         io.append(f'"+{{v[{base}:{base + n - 1}]}}"(r{which.lower()})')
         declared |= set(range(base, base + n))
     print("          " + ", ".join(io))
@@ -740,7 +762,7 @@ def emit_two_set(member, name, mnem, ka, kb):
     # second-half offsets
     written = set(range(X.clobber_to))
     for which in X.ops:
-        written |= set(range(X.raddr[which], X.raddr[which] + 2 * X.blocks[which]))
+        written |= set(range(X.raddr[which], X.raddr[which] + ((X.nst + 1) // 2) * max(2, X.blocks[which])))
         written.add(X.goff2[which])
     vclob = sorted(written - declared)
     clob = [f'"v{i}"' for i in vclob] + [f'"s{i}"' for i in range(SP["A"], ST + 2)] + ['"scc"', '"memory"']
@@ -763,7 +785,7 @@ def main():
         print("// Main loops of the 256x384 GEMM kernel and of the 256x128 kernel for two workgroups per compute unit")
         print("// (the generator documents the schedule and the register maps).\n")
         print("#define MHIP_HAVE_GEMM256X384_LOOP 1\n")
-        for member, stem in ((_x384(), "gemm256x384_loop"), (_xpair(), "gemm_pair_loop")):
+        for member, stem in ((_x384(), "gemm256x384_loop"), (_xpair(), "gemm_pair_loop"), (_x192(), "gemm128x192_loop")):
             for tname, mnem in (("bf16", "v_mfma_f32_32x32x16_bf16"), ("f16", "v_mfma_f32_32x32x16_f16")):
                 for lname, ka, kb in (("nn", "K", "MN"), ("nt", "K", "K"), ("tn", "MN", "MN"), ("tt", "MN", "K")):
                     emit_two_set(member, f"{stem}_{lname}_{tname}", mnem, ka, kb)

@@ -32,7 +32,7 @@ MODEL_GEMMS = [
 ]
 # the logits GEMM as the program from text writes it (N = 50257): timed on its own, caches emptied
 TEXT_LOGITS = (8192, 50257, 768, 1)
-GEMM_VARIANTS = [128, 256, 2560, 2561, 2562, 2563, 2564, 2565, 2566, 2567, 2568]
+GEMM_VARIANTS = [128, 256, 2560, 2561, 2562, 2563, 2564, 2565, 2566, 2567, 2568, 2569]
 ATTENTION = [(4, 32, 4096, 128, 1), (4, 32, 2048, 128, 0)]            # B, H, S, D, causal
 # operator (0 softmax, 1 LayerNorm, 2 RMSNorm), rows, cols.  Only the benchmark shapes: a row kernel between two
 # GEMMs of a model is not timed in a loop of its own -- there the launch form decides which XCD's L2 holds
@@ -106,7 +106,7 @@ def main():
             check(lib.mhip_tuning_set_gemm(M, N, K, 1, 0, tb, 3, v, 0.0), "set")
             t = _forward_us(model, ids, torch)
             print(f"  {name} [{M},{K}] x [{K},{N}] as variant {v}: forward {t:.1f} us", flush=True)
-            if t < best_t * 0.998:              # a candidate must beat the incumbent by more than the noise
+            if t < best_t * 0.995:              # a candidate must beat the incumbent by more than the noise (+-0.3 % from run to run)
                 best_v, best_t = v, t
         check(lib.mhip_tuning_set_gemm(M, N, K, 1, 0, tb, 3, best_v, best_t), "set")
         print(f"{name}: " + (f"variant {best_v}, forward {best_t:.1f} us" if best_v else "the heuristic's choice stays"), flush=True)

@@ -231,7 +231,50 @@ def test_gemm_large_tiles(shape, layout, dtype, tile, lib):
     assert torch.equal(c, c128)
 
 
-@pytest.mark.parametrize("tile", ["2560", "2561", "2567", "2568"], ids=["256x256", "256x128", "256x384", "256x128-two-per-cu"])
+# Shapes with >= 192 tiles of 128x192 (single stage, exits at every position of the unrolled ring of six,
+# several trips; M and N ragged against the tile and, once, N odd).
+SMALL_ROWS = [(8192, 768, 32), (4104, 1160, 96), (8192, 776, 160), (6152, 960, 224), (8192, 768, 768), (4096, 1544, 1056),
+              (8192, 773, 192), (8192, 768, 3072)]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=lambda d: NAME[d])
+@pytest.mark.parametrize("layout", [(False, False), (False, True), (True, False), (True, True)],
+                         ids=["nn", "nt", "tn", "tt"])
+@pytest.mark.parametrize("shape", SMALL_ROWS, ids=lambda s: "x".join(map(str, s)))
+def test_gemm_128x192_tile(shape, layout, dtype, lib, monkeypatch):
+    """The 128-row member of the family (B's 192 columns in a 256-column layout whose last quarter is
+    never loaded): bias, activation and residual, against the oracle on sampled rows and bit for bit
+    against the 128x128 kernel; nothing is written behind the last row."""
+    from metalhlo_amd import kernels
+    M, N, K = shape
+    ta, tb = layout
+    if not ((not ta or M % 8 == 0) and (tb or N % 8 == 0)):
+        pytest.skip("operand rows off 16-byte boundaries run the scalar kernel")
+    a, b = _ab(M, N, K, dtype, 43, ta, tb)
+    rng = np.random.default_rng(44)
+    bias = to_dev(rng.standard_normal(N) * 0.5, dtype)
+    r = to_dev(rng.standard_normal((M, N)), dtype)
+    monkeypatch.setenv("MHIP_GEMM_TILE", "2569")
+    guard = torch.full((M * N + 64,), 7.0, dtype=dtype, device="cuda")
+    c = kernels.matmul(a, b, bias, "silu", trans_a=ta, trans_b=tb, out=guard[:M * N].view(M, N))
+    assert lib.mhip_gemm_last_variant() == 2569
+    cr = kernels.matmul(a, b, bias, "none", trans_a=ta, trans_b=tb, residual=r)
+    assert lib.mhip_gemm_last_variant() == 2569
+    assert torch.all(guard[M * N:] == 7.0)
+    monkeypatch.setenv("MHIP_GEMM_TILE", "128")
+    assert torch.equal(c, kernels.matmul(a, b, bias, "silu", trans_a=ta, trans_b=tb))
+    assert torch.equal(cr, kernels.matmul(a, b, bias, "none", trans_a=ta, trans_b=tb, residual=r))
+    rows = np.unique(np.r_[0, 31, 32, 63, 64, 127, 128, M - 1, rng.integers(0, M, 40)])
+    A = as_f64(a).T if ta else as_f64(a)
+    B = as_f64(b).T if tb else as_f64(b)
+    exp = oracle.matmul_bias_act(A[rows], B, as_f64(bias), "silu")
+    assert_close(c[rows], exp, TOL[dtype], f"gemm 128x192 {shape} {layout}")
+    exp = oracle.matmul_bias_act(A[rows], B, as_f64(bias), "none")
+    exp = as_f64(to_dev(exp, dtype).cpu()) + as_f64(r)[rows]          # product rounded, then the residual added
+    assert_close(cr[rows], exp, TOL[dtype], f"gemm 128x192 + residual {shape} {layout}")
+
+
+@pytest.mark.parametrize("tile", ["2560", "2561", "2567", "2568", "2569"], ids=["256x256", "256x128", "256x384", "256x128-two-per-cu", "128x192"])
 def test_gemm_ring_kernels_batched(tile, lib, monkeypatch):
     """The ring kernels on a strided batch (one grid row per matrix): every batch element against the
     oracle on sampled rows and bit for bit against the 128x128 kernel."""
@@ -428,6 +471,14 @@ def test_gemm_one_round_of_the_widest_tile_is_the_default_where_it_saves_a_round
     monkeypatch.delenv("MHIP_GEMM_TILE", raising=False)
     kernels.matmul(a, b)
     assert lib.mhip_gemm_last_variant() == 2560
+    # 768 columns: 192 tiles of 256x128 would leave a quarter of the device idle, 256 of 128x192 do not
+    for K in (768, 3072):
+        a, b = _ab(8192, 768, K, torch.bfloat16, 69)
+        monkeypatch.delenv("MHIP_GEMM_TILE", raising=False)
+        c = kernels.matmul(a, b)
+        assert lib.mhip_gemm_last_variant() == 2569, K
+        monkeypatch.setenv("MHIP_GEMM_TILE", "2561")
+        assert torch.equal(c, kernels.matmul(a, b))
 
 
 def test_gemm_streaming_stores_of_a_large_result(monkeypatch):
@@ -539,7 +590,7 @@ def test_gemm_ring_kernel_takes_wide_and_deep_operands(lib):
         a = to_dev(rng.uniform(-1, 1, (M, K)), torch.bfloat16)
         b = to_dev(rng.uniform(-1, 1, (K, N)) * (K ** -0.5), torch.bfloat16)
         c = kernels.matmul(a, b)
-        assert 2560 <= lib.mhip_gemm_last_variant() <= 2568, (M, N, K, lib.mhip_gemm_last_variant())
+        assert 2560 <= lib.mhip_gemm_last_variant() <= 2569, (M, N, K, lib.mhip_gemm_last_variant())
         rows = np.r_[0, 255, 256, M - 1, rng.integers(0, M, 12)]
         assert_close(c[rows], as_f64(a[rows]) @ as_f64(b), 2e-2, f"gemm {M}x{N}x{K}")
     # fp32 operands run none of the 16-bit variants

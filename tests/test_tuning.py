@@ -62,8 +62,8 @@ def test_gemm_autotune_picks_a_valid_variant_and_keeps_results():
         before = kernels.matmul(a, b, trans_b=tb)
         variant, us = kernels.autotune_matmul(a, b, trans_b=tb, iters=5)
         tiles = ((M + 255) // 256) * ((N + 255) // 256)
-        ring = (2560, 2561, 2562, 2563, 2564, 2565, 2566, 2567, 2568)      # the generated family, streamed tiles, the column split
-        assert variant in ((128, 256) + ring if tiles >= 192 else (128, 256, 2561, 2564, 2565, 2568)) and us > 0
+        ring = (2560, 2561, 2562, 2563, 2564, 2565, 2566, 2567, 2568, 2569)      # the generated family, streamed tiles, the column split
+        assert variant in ((128, 256) + ring if tiles >= 192 else (128, 256, 2561, 2564, 2565, 2568, 2569)) and us > 0
         tuned = kernels.matmul(a, b, trans_b=tb)
         # the tuned launch against the oracle on sampled rows ...
         rows = [0, 1, M // 2, M - 1]
@@ -147,7 +147,7 @@ def test_gemm_autotune_in_model_and_the_shipped_table(lib, tmp_path):
     b = ((torch.rand(K, N, device="cuda") * 2 - 1) * K ** -0.5).bfloat16()
     plain = kernels.matmul(a, b)
     default_variant = lib.mhip_gemm_last_variant()
-    assert default_variant in (128, 256, 2560, 2561, 2563, 2567)      # what the heuristic can choose
+    assert default_variant in (128, 256, 2560, 2561, 2563, 2567, 2569)      # what the heuristic can choose
     other = 2564 if default_variant != 2564 else 2561
     table = tmp_path / "t.txt"
     table.write_text(f"gemm {kernels.tuning_device()} {M} {N} {K} 1 0 0 3 = {other} @ 1.0\n")
@@ -165,7 +165,7 @@ def test_gemm_autotune_in_model_and_the_shipped_table(lib, tmp_path):
     st = torch.cuda.current_stream().cuda_stream
     assert lib.mhip_gemm_autotune_in_model(st, a.data_ptr(), b.data_ptr(), None, c.data_ptr(), M, N, K, 1, 0, 0, 0, 0, 0, 0, 3, 5,
                                            flush.data_ptr(), flush.numel(), C.byref(var), C.byref(us)) == 0, lib.mhip_last_error()
-    assert var.value in (128, 256, 2561, 2564, 2565, 2568) and us.value > 0 and kernels.tuning_count() == 1
+    assert var.value in (128, 256, 2561, 2564, 2565, 2568, 2569) and us.value > 0 and kernels.tuning_count() == 1
     assert torch.equal(kernels.matmul(a, b), plain) and lib.mhip_gemm_last_variant() == var.value
     assert torch.equal(a, a.clone())                             # (A was rewritten in place with its own values)
     assert lib.mhip_gemm_autotune_in_model(st, a.data_ptr(), b.data_ptr(), None, c.data_ptr(), M, N, K, 1, 0, 0, 0, 0, 0, 0, 3, 5,
