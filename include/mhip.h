@@ -351,7 +351,8 @@ int mhip_fill(void* stream, void* y, int64_t n, uint64_t pattern, int elem_size)
  * with four, 2567 = 256x384 with four (a third of its accumulators in ordinary registers; no
  * activation, relu or tanh-GELU), 2568 = 256x128 with three, in 256 registers a wave, two workgroups
  * per compute unit, 2569 = 128x192 with six (for problems with so few columns that 256-row tiles
- * leave compute units idle);
+ * leave compute units idle), 2570 = 256x288 with four (four waves one above the other; the same
+ * activations as 2567);
  * microseconds per launch. */
 int mhip_gemm_autotune(void* stream, const void* a, const void* b, const void* bias, void* c,
                        int64_t M, int64_t N, int64_t K, int64_t batch, int64_t stride_a,

@@ -462,7 +462,7 @@ static int launch_column_split(hipStream_t s, const GemmArgs& g, int64_t batch, 
     return launch_gemm256(s, w, 1, TA, TB, dt);
 }
 
-// Which kernel serves a 16-bit problem (MHIP_GEMM_TILE = 128 | 256 | 2560 ... 2569 forces one; 2564 / 2565 = the
+// Which kernel serves a 16-bit problem (MHIP_GEMM_TILE = 128 | 256 | 2560 ... 2570 forces one; 2570 = the 256x288 tile; 2564 / 2565 = the
 // 256x128 tile with a ring of six / four stages, 2566 = the 256x256 tile with four, 2568 = the 256x128
 // tile as two workgroups per compute unit: members of the generated family that only a forced choice
 // or the tuning table selects; 2567 = the 256x384 tile):
@@ -513,6 +513,10 @@ static int pick_tile(hipStream_t s, const GemmArgs& g, int64_t batch) {
     }
     if (force == 2566) {
         if (gemm256_eligible(g, batch, TA, TB, dt)) return chose(2566, launch_gemm256(s, g, batch, TA, TB, dt, 256, 4));
+    }
+    // the 256x288 tile (ring of four)
+    if (force == 2570) {
+        if (gemm256_eligible(g, batch, TA, TB, dt, 288) && gemm384_activation_ok(g.act)) return chose(2570, launch_gemm256(s, g, batch, TA, TB, dt, 288, 4));
     }
     // the 128x192 tile (ring of six)
     if (force == 2569) {

@@ -26,6 +26,7 @@ namespace mhip {
 int launch_gemm384(hipStream_t s, const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype);
 int launch_gemm_pair(hipStream_t s, const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype);
 int launch_gemm192(hipStream_t s, const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype);
+int launch_gemm288(hipStream_t s, const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype);
 
 namespace {
 
@@ -349,6 +350,7 @@ int launch_gemm256(hipStream_t s, const GemmArgs& g, int64_t batch, int trans_a,
                    int dtype, int bw, int ring) {
     if (bw == 384) return launch_gemm384(s, g, batch, trans_a, trans_b, dtype);
     if (bw == 192) return launch_gemm192(s, g, batch, trans_a, trans_b, dtype);                     // 128-row tiles
+    if (bw == 288) return launch_gemm288(s, g, batch, trans_a, trans_b, dtype);
     if (bw == 128 && ring == 3) return launch_gemm_pair(s, g, batch, trans_a, trans_b, dtype);      // two workgroups per compute unit
     if (dtype == MHIP_BF16) return family256<bf16_t>(s, g, batch, trans_a, trans_b, bw, ring);
     return family256<f16_t>(s, g, batch, trans_a, trans_b, bw, ring);

@@ -530,13 +530,229 @@ int layout192(hipStream_t s, const GemmArgs& g, int64_t batch, int ta, int tb) {
     return launch192<T, true, true>(s, g, batch);
 }
 
+// ---- the 256x288 tile --------------------------------------------------------------------------------
+// gemm256x288_loop_* of the generated file: for problems whose 256x384 tiling leaves a quarter of the
+// compute units idle ([8192, 2304]: 192 tiles of 256x384, 256 of 256x288).  Four waves one above the
+// other, each 64 x 288 = 2 x 9 accumulator blocks (sixteen in the accumulation registers, two in
+// v[128:159]); every wave reads all of B, which lies as in the 256x384 kernel -- the 256-column tile,
+// then the 128-column tile, of which only the first 32 columns are ever loaded.
+template <typename T, bool TA, bool TB>
+__device__ __forceinline__ void main_loop288(f32x16 (&acc)[18], u32x2 ra, u32x4 rb, u32x2 rb2, u32x4& goff,
+                                             __amdgpu_buffer_rsrc_t rsa, __amdgpu_buffer_rsrc_t rsb, uint32_t pa,
+                                             uint32_t pb, uint32_t ta, uint32_t tb, uint32_t m0b, uint32_t kt) {
+    constexpr bool bf = std::is_same<T, bf16_t>::value;
+#define MHIP_LOOP(cond, name) \
+    if constexpr (cond) gemm256x288_loop_##name(acc, ra, rb, rb2, goff, rsa, rsb, pa, pb, ta, tb, m0b, kt);
+    MHIP_LOOP(bf && !TA && !TB, nn_bf16)
+    MHIP_LOOP(bf && !TA && TB, nt_bf16)
+    MHIP_LOOP(bf && TA && !TB, tn_bf16)
+    MHIP_LOOP(bf && TA && TB, tt_bf16)
+    MHIP_LOOP(!bf && !TA && !TB, nn_f16)
+    MHIP_LOOP(!bf && !TA && TB, nt_f16)
+    MHIP_LOOP(!bf && TA && !TB, tn_f16)
+    MHIP_LOOP(!bf && TA && TB, tt_f16)
+#undef MHIP_LOOP
+}
+
+// Epilogue: a wave's 64 x 288 sub-tile through LDS one 32-row block at a time (32 rows of 576 + 16
+// bytes per wave); a block goes out as eighteen instructions of 64 lanes x 16 bytes: lane slot
+// (u % 9) * 64 + lane = row 16 (u / 9) + slot / 36 of the block, chunk slot % 36.  The activation
+// is a uniform branch around each group of four values, as in store_tile384 and for its reason.
+template <typename T>
+__device__ __forceinline__ void store_tile288(f32x16 (&acc)[18], char* smem, const GemmArgs& g, T* c, const T* res,
+                                              int m0, int n0) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int lrow = lane & 31, lhalf = lane >> 5;
+    const T* bias = static_cast<const T*>(g.bias);
+    constexpr int kRowPad = 288 * 2 + 16;
+    char* stage = smem + wave * (32 * kRowPad);
+    const int ldc = g.ldc ? g.ldc : g.N;
+    const bool full_cols = __builtin_amdgcn_readfirstlane(n0 + 288 <= g.N);
+    const bool interior = __builtin_amdgcn_readfirstlane(full_cols && m0 + wave * 64 + 64 <= g.M && ldc % 8 == 0);
+    const bool stream = __builtin_amdgcn_readfirstlane(g.stream_c != 0);
+    Pack4<T> bq[36];
+    static_for<36>([&](auto jq_tag) {
+        constexpr int jq = decltype(jq_tag)::value;
+        bq[jq] = __builtin_bit_cast(Pack4<T>, u32x2{0u, 0u});
+    });
+    if (bias) {
+        if (full_cols) {
+            static_for<36>([&](auto jq_tag) {
+                constexpr int jq = decltype(jq_tag)::value;
+                bq[jq] = __builtin_bit_cast(Pack4<T>, *reinterpret_cast<const u32x2*>(bias + n0 + 8 * jq + 4 * lhalf));
+            });
+        } else {
+            static_for<36>([&](auto jq_tag) {
+                constexpr int jq = decltype(jq_tag)::value;
+                const int n = n0 + 8 * jq + 4 * lhalf;
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    if (n + e < g.N) bq[jq].v[e] = bias[n + e];
+            });
+        }
+    }
+    const int act = __builtin_amdgcn_readfirstlane(g.act);
+    static_for<2>([&](auto i_tag) {
+        constexpr int i = decltype(i_tag)::value;
+        static_for<36>([&](auto jq_tag) {
+            constexpr int j = decltype(jq_tag)::value >> 2, q = decltype(jq_tag)::value & 3;
+            constexpr int b = 9 * i + j;
+            Pack4<T> o;
+            float v4[4];
+            static_for<4>([&](auto e_tag) {
+                constexpr int e = decltype(e_tag)::value;
+                if constexpr (b < 16) v4[e] = acc_value(acc[b][4 * q + e]);
+                else v4[e] = acc[b][4 * q + e];
+                v4[e] += Elem<T>::to_f32(bq[j * 4 + q].v[e]);
+            });
+            if (act == MHIP_ACT_GELU) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) v4[e] = apply_act_c<MHIP_ACT_GELU>(v4[e]);
+            } else if (act == MHIP_ACT_RELU) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) v4[e] = apply_act_c<MHIP_ACT_RELU>(v4[e]);
+            }
+#pragma unroll
+            for (int e = 0; e < 4; e++) o.v[e] = Elem<T>::from_f32(v4[e]);
+            *reinterpret_cast<u32x2*>(stage + lrow * kRowPad + (j * 32 + 8 * q + 4 * lhalf) * 2) =
+                __builtin_bit_cast(u32x2, o);
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // a wave re-reads only its own rows
+        if (interior) {
+#pragma unroll
+            for (int h = 0; h < 3; h++) {
+                u32x4 w[6], r[6];
+                int64_t off[6];
+#pragma unroll
+                for (int u = 0; u < 6; u++) {
+                    const int U = 6 * h + u;
+                    const int slot = (U % 9) * 64 + lane;
+                    const int rl = 16 * (U / 9) + slot / 36, ch = slot % 36;
+                    off[u] = (int64_t)(m0 + wave * 64 + i * 32 + rl) * ldc + n0 + 8 * ch;
+                    if (res) r[u] = *reinterpret_cast<const u32x4*>(res + off[u]);
+                    w[u] = *reinterpret_cast<const u32x4*>(stage + rl * kRowPad + ch * 16);
+                }
+#pragma unroll
+                for (int u = 0; u < 6; u++) {
+                    if (res) w[u] = add_chunk<T>(w[u], r[u]);
+                    if (stream) __builtin_nontemporal_store(w[u], reinterpret_cast<u32x4*>(c + off[u]));
+                    else *reinterpret_cast<u32x4*>(c + off[u]) = w[u];
+                }
+            }
+        } else {
+#pragma unroll 1
+            for (int u = 0; u < 18; u++) {
+                const int slot = (u % 9) * 64 + lane;
+                const int rl = 16 * (u / 9) + slot / 36, ch = slot % 36;
+                const int m = m0 + wave * 64 + i * 32 + rl;
+                const int n = n0 + 8 * ch;
+                T* cp = c + (int64_t)m * ldc + n;
+                const T* rp = res + (int64_t)m * ldc + n;
+                if (m < g.M && n + 8 <= g.N) {
+                    u32x4 w = *reinterpret_cast<const u32x4*>(stage + rl * kRowPad + ch * 16);
+                    if (res) w = add_chunk<T>(w, *reinterpret_cast<const u32x4_unaligned*>(rp));
+                    *reinterpret_cast<u32x4_unaligned*>(cp) = w;
+                } else if (m < g.M && n < g.N) {                 // the last, partial chunk of a row
+                    const T* sv = reinterpret_cast<const T*>(stage + rl * kRowPad + ch * 16);
+                    for (int e = 0; e < g.N - n; e++) {
+                        T val = sv[e];
+                        if (res) val = Elem<T>::from_f32(Elem<T>::to_f32(val) + Elem<T>::to_f32(rp[e]));
+                        cp[e] = val;
+                    }
+                }
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the next block overwrites the rows just read
+        __builtin_amdgcn_sched_barrier(0);
+    });
+}
+
+template <typename T, bool TA, bool TB>
+__global__ __launch_bounds__(256) void gemm288_kernel(GemmArgs g) {
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    using LA = typename std::conditional<TA, MnMajor<256>, KMajor>::type;
+    using LB = typename std::conditional<TB, KMajor, MnMajor<256>>::type;
+    using LB2 = typename std::conditional<TB, KMajor, MnMajor<128>>::type;
+
+    int tm, tn;
+    tile_of(blockIdx.x, gridDim.x, g.tiles_m, g.tiles_n, tm, tn);
+    const int m0 = tm * 256, n0 = tn * 288;
+    const int64_t batch = blockIdx.y;
+    const char* a = reinterpret_cast<const char*>(static_cast<const T*>(g.a) + batch * g.sa);
+    const char* b = reinterpret_cast<const char*>(static_cast<const T*>(g.b) + batch * g.sb);
+    T* c = static_cast<T*>(g.c) + batch * g.sc;
+    const T* res = g.residual ? static_cast<const T*>(g.residual) + batch * g.sc : nullptr;
+    const uint32_t a_bytes = (uint32_t)(((int64_t)((TA ? g.K : g.M) - 1) * g.lda + (TA ? g.M : g.K)) * 2);
+    const uint32_t b_bytes = (uint32_t)(((int64_t)((TB ? g.N : g.K) - 1) * g.ldb + (TB ? g.K : g.N)) * 2);
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
+    const u32x4 raw = LA::raddr(lane, wave * 64, lds0);
+    u32x2 ra;
+    ra.x = raw.x; ra.y = raw.y;
+    const u32x4 rb = LB::raddr(lane, 0, lds0 + kOperBytes);
+    const u32x4 rb2w = LB2::raddr(lane, 0, lds0 + 2 * kOperBytes);
+    u32x2 rb2;
+    rb2.x = rb2w.x; rb2.y = rb2w.y;
+    const int n_end = min(g.N, n0 + 288);                    // nothing past the tile's 288 columns is asked for
+    u32x4 goff;
+    goff.x = LA::goff(lane, wave, m0, g.lda, g.M);
+    goff.y = LB::goff(lane, wave, n0, g.ldb, n_end);
+    goff.z = LB2::goff(lane, wave, n0 + 256, g.ldb, n_end);
+    if (TB && n0 + 256 + 16 * wave + (lane >> 2) >= n_end) goff.z = kOob;     // (a k-contiguous tile is bounded by rows)
+    goff.w = 0;
+    const uint32_t m0b = __builtin_amdgcn_readfirstlane(lds0 + (uint32_t)wave * 1024u);
+    const __amdgpu_buffer_rsrc_t rsa =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(a), 0, a_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsb =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(b), 0, b_bytes, 0x00020000);
+
+    f32x16 acc[18];
+    main_loop288<T, TA, TB>(acc, ra, rb, rb2, goff, rsa, rsb, LA::pass_stride(g.lda), LB::pass_stride(g.ldb),
+                            LA::stage_stride(g.lda), LB::stage_stride(g.ldb), m0b, (uint32_t)(g.K / 32));
+    store_tile288<T>(acc, smem, g, c, res, m0, n0);
+}
+
+template <typename T, bool TA, bool TB>
+int launch288(hipStream_t s, GemmArgs g, int64_t batch) {
+    auto kern = gemm288_kernel<T, TA, TB>;
+    static std::once_flag once;
+    static hipError_t attr_err = hipSuccess;
+    std::call_once(once, [&] {
+        attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, k384Smem);
+    });
+    if (attr_err != hipSuccess)
+        return fail(MHIP_ERR_LAUNCH, "gemm288: cannot reserve %d bytes of LDS: %s", k384Smem,
+                    hipGetErrorString(attr_err));
+    g.tiles_m = (g.M + 255) / 256;
+    g.tiles_n = (g.N + 287) / 288;
+    g.stream_c = (int64_t)g.M * g.N * batch * 2 > (256ll << 20) && (g.ldc ? g.ldc : g.N) % 8 == 0;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(g.tiles_m * g.tiles_n), (unsigned)batch), dim3(256),
+                       k384Smem, s, g);
+    return check_launch("gemm288");
+}
+
+template <typename T>
+int layout288(hipStream_t s, const GemmArgs& g, int64_t batch, int ta, int tb) {
+    if (!ta && !tb) return launch288<T, false, false>(s, g, batch);
+    if (!ta && tb) return launch288<T, false, true>(s, g, batch);
+    if (ta && !tb) return launch288<T, true, false>(s, g, batch);
+    return launch288<T, true, true>(s, g, batch);
+}
+
 }  // namespace
 
-// The activations the 256x384 kernel's epilogue serves.
+// The activations the epilogues of the 256x384 and the 256x288 kernel serve.
 bool gemm384_activation_ok(int act) { return act == MHIP_ACT_NONE || act == MHIP_ACT_RELU || act == MHIP_ACT_GELU; }
 
 int launch_gemm384(hipStream_t s, const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype) {
     return dtype == MHIP_BF16 ? layout384<bf16_t>(s, g, batch, trans_a, trans_b) : layout384<f16_t>(s, g, batch, trans_a, trans_b);
+}
+
+int launch_gemm288(hipStream_t s, const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype) {
+    return dtype == MHIP_BF16 ? layout288<bf16_t>(s, g, batch, trans_a, trans_b) : layout288<f16_t>(s, g, batch, trans_a, trans_b);
 }
 
 int launch_gemm192(hipStream_t s, const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype) {

@@ -522,11 +522,15 @@ class TwoSet:
     """One member of the two-fragment-set family: geometry and register map."""
 
     def __init__(self, name, nst, ops, region, sets, raddr, goff, goff2, blocks, passes, rowb, passmult,
-                 acc_regs, grid, goff_span, clobber_to, stage=None, a_blocks=4):
+                 acc_regs, grid, goff_span, clobber_to, stage=None, a_blocks=4, mn_fold=None):
         self.name, self.nst, self.ops = name, nst, ops
         # (`passes` of an operand: a number, or one per layout {"K": .., "MN": ..})
         self.stage = stage if stage else sum(passes[o] * 4096 for o in ops)
         self.a_blocks = a_blocks          # 32-row blocks of A per wave
+        # An operand in the 256-column layout of which a wave reads more than four blocks: block j
+        # uses the address register of block j % 4 and an offset of 256 bytes per four blocks (the
+        # swizzle of that layout only touches the two low bits of the block index).
+        self.mn_fold = mn_fold or {}
         self.unroll = nst if nst % 2 == 0 else 2 * nst
         self.region, self.sets, self.raddr, self.goff, self.goff2 = region, sets, raddr, goff, goff2
         self.blocks, self.passes, self.rowb, self.passmult = blocks, passes, rowb, passmult
@@ -572,7 +576,32 @@ def _x192():
                   {}, [f"a[{16 * b}:{16 * b + 15}]" for b in range(6)], grid, 2, 40, stage=24576, a_blocks=2)
 
 
+def _x288():
+    """256 x 288 tile: four waves one above the other, each 64 x 288 = 2 x 9 accumulator blocks, the
+    first sixteen in a[0:255] and the last two in v[128:159].  Every wave reads all of B: its 256-column
+    tile (eight blocks) and the first block of the 128-column tile behind it (columns 256..287; the
+    rest of that tile is never loaded).  Register map: fragment set n: A v[44n : 44n+7], B
+    v[44n+8 : 44n+39], B2 v[44n+40 : 44n+43]; v[88:91] A read addresses, v[92:99] B, v[100:103] B2;
+    v104 / v105 / v106 global offsets, v107 / v108 / v109 the same + 64."""
+    def acc(b):
+        return f"a[{16 * b}:{16 * b + 15}]" if b < 16 else vr(128 + 16 * (b - 16), 16)
+    grid = [(9 * i + j, "B" if j < 8 else "B2", j if j < 8 else 0, i)
+            for i in range(2) for j in (range(9) if i % 2 == 0 else reversed(range(9)))]
+    return TwoSet("x288", 4, ("A", "B", "B2"), {"A": 0, "B": 16384, "B2": 32768},
+                  {0: {"A": 0, "B": 8, "B2": 40}, 1: {"A": 44, "B": 52, "B2": 84}},
+                  {"A": 88, "B": 92, "B2": 100}, {"A": 104, "B": 105, "B2": 106}, {"A": 107, "B": 108, "B2": 109},
+                  {"A": 2, "B": 8, "B2": 1}, {"A": 4, "B": 4, "B2": {"K": 1, "MN": 2}}, {"A": 512, "B": 512, "B2": 256},
+                  {"B2": 2}, [acc(b) for b in range(18)], grid, 4, 88, stage=40960, a_blocks=2, mn_fold={"B": 4})
+
+
 X = None      # the member being emitted
+
+
+def x_addr_regs(kinds, which):
+    """Fragment address registers of an operand per pair of ring buffers."""
+    if x_kind(kinds, which) == "K":
+        return 2
+    return min(X.blocks[which], X.mn_fold.get(which, X.blocks[which]))
 
 
 def x_passes(kinds, which):
@@ -595,8 +624,9 @@ def x_frag_reads(kinds, g, s, fset):
             if kind == "K":
                 out.append(f"ds_read_b128 {vr(dst, 4)}, v{addr + 2 * h + s} offset:{lo + j * 2048}")
             else:
-                off = lo + s * 16 * X.rowb[which]
-                a = addr + X.blocks[which] * h + j
+                fold = X.mn_fold.get(which, X.blocks[which])
+                off = lo + s * 16 * X.rowb[which] + (j // fold) * 256
+                a = addr + min(X.blocks[which], fold) * h + j % fold
                 out.append(f"ds_read_b64_tr_b16 {vr(dst, 2)}, v{a} offset:{off}")
                 out.append(f"ds_read_b64_tr_b16 {vr(dst + 2, 2)}, v{a} offset:{off + 4 * X.rowb[which]}")
         per[which] = out
@@ -697,7 +727,7 @@ def x_body(mnem, kinds):
     out.append(f"s_mov_b32 s{ST + 1}, m0")
     # fragment read addresses of the ring's last buffer(s) from those of buffers 0 and 1
     for which in X.ops:
-        n = 2 if x_kind(kinds, which) == "K" else X.blocks[which]
+        n = x_addr_regs(kinds, which)
         for h in range(1, (X.nst + 1) // 2):
             for e in range(n):
                 out.append(f"v_add_u32 v{X.raddr[which] + n * h + e}, {h * 2 * X.stage}, v{X.raddr[which] + e}")
@@ -762,7 +792,7 @@ def emit_two_set(member, name, mnem, ka, kb):
     # second-half offsets
     written = set(range(X.clobber_to))
     for which in X.ops:
-        written |= set(range(X.raddr[which], X.raddr[which] + ((X.nst + 1) // 2) * max(2, X.blocks[which])))
+        written |= set(range(X.raddr[which], X.raddr[which] + ((X.nst + 1) // 2) * max(2, x_addr_regs({"A": "MN", "B": "MN"}, which))))
         written.add(X.goff2[which])
     vclob = sorted(written - declared)
     clob = [f'"v{i}"' for i in vclob] + [f'"s{i}"' for i in range(SP["A"], ST + 2)] + ['"scc"', '"memory"']
@@ -785,7 +815,8 @@ def main():
         print("// Main loops of the 256x384 GEMM kernel and of the 256x128 kernel for two workgroups per compute unit")
         print("// (the generator documents the schedule and the register maps).\n")
         print("#define MHIP_HAVE_GEMM256X384_LOOP 1\n")
-        for member, stem in ((_x384(), "gemm256x384_loop"), (_xpair(), "gemm_pair_loop"), (_x192(), "gemm128x192_loop")):
+        for member, stem in ((_x384(), "gemm256x384_loop"), (_xpair(), "gemm_pair_loop"), (_x192(), "gemm128x192_loop"),
+                             (_x288(), "gemm256x288_loop")):
             for tname, mnem in (("bf16", "v_mfma_f32_32x32x16_bf16"), ("f16", "v_mfma_f32_32x32x16_f16")):
                 for lname, ka, kb in (("nn", "K", "MN"), ("nt", "K", "K"), ("tn", "MN", "MN"), ("tt", "MN", "K")):
                     emit_two_set(member, f"{stem}_{lname}_{tname}", mnem, ka, kb)

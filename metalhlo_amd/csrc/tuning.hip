@@ -89,7 +89,7 @@ bool valid_choice(const char* line, const std::string& choice) {
     int a = 0, b = 0, c = 0, d = 0;
     if (!strncmp(line, "gemm ", 5)) {
         const int v = atoi(choice.c_str());
-        return v == 128 || v == 256 || (v >= 2560 && v <= 2569);
+        return v == 128 || v == 256 || (v >= 2560 && v <= 2570);
     }
     if (!strncmp(line, "row ", 4))
         return sscanf(choice.c_str(), "%d %d %d %d", &a, &b, &c, &d) == 4 && (a == 1 || a == 2) && (b == 1 || b == 2) &&
@@ -197,7 +197,7 @@ int tuned_gemm_variant(const GemmArgs& g, int64_t batch, int ta, int tb, int dty
     std::string c;
     if (!have_entries() || !lookup(gemm_key(g.M, g.N, g.K, batch, ta, tb, dtype), &c)) return 0;
     const int v = atoi(c.c_str());
-    return (v == 128 || v == 256 || (v >= 2560 && v <= 2569)) ? v : 0;
+    return (v == 128 || v == 256 || (v >= 2560 && v <= 2570)) ? v : 0;
 }
 
 bool tuned_row_launch(int op, int dtype, int64_t rows, int64_t cols, bool has_gamma, bool has_beta, RowLaunch* out) {
@@ -225,9 +225,10 @@ using namespace mhip;
 // GEMM candidates a problem can run (the validity filter: shape, alignment, LDS and tile count rules of each kernel).
 static std::vector<int> gemm_candidates(const GemmArgs& g, int64_t batch, int trans_a, int trans_b, int dtype) {
     std::vector<int> out;
-    for (int v : {128, 256, 2560, 2561, 2562, 2563, 2564, 2565, 2566, 2567, 2568, 2569}) {
+    for (int v : {128, 256, 2560, 2561, 2562, 2563, 2564, 2565, 2566, 2567, 2568, 2569, 2570}) {
         if ((v == 2560 || v == 2566) && !gemm256_eligible(g, batch, trans_a, trans_b, dtype)) continue;
         if ((v == 2561 || v == 2564 || v == 2565 || v == 2568) && !gemm256_eligible(g, batch, trans_a, trans_b, dtype, 128)) continue;
+        if (v == 2570 && !(gemm256_eligible(g, batch, trans_a, trans_b, dtype, 288) && gemm384_activation_ok(g.act))) continue;
         if (v == 2569 && !gemm256_eligible(g, batch, trans_a, trans_b, dtype, 192)) continue;
         if (v == 2567 && !(gemm256_eligible(g, batch, trans_a, trans_b, dtype, 384) && gemm384_activation_ok(g.act))) continue;
         if (v == 2562 && !gemm_stream_eligible(g, batch, trans_a, trans_b, dtype)) continue;

@@ -32,7 +32,7 @@ MODEL_GEMMS = [
 ]
 # the logits GEMM as the program from text writes it (N = 50257): timed on its own, caches emptied
 TEXT_LOGITS = (8192, 50257, 768, 1)
-GEMM_VARIANTS = [128, 256, 2560, 2561, 2562, 2563, 2564, 2565, 2566, 2567, 2568, 2569]
+GEMM_VARIANTS = [128, 256, 2560, 2561, 2562, 2563, 2564, 2565, 2566, 2567, 2568, 2569, 2570]
 ATTENTION = [(4, 32, 4096, 128, 1), (4, 32, 2048, 128, 0)]            # B, H, S, D, causal
 # operator (0 softmax, 1 LayerNorm, 2 RMSNorm), rows, cols.  Only the benchmark shapes: a row kernel between two
 # GEMMs of a model is not timed in a loop of its own -- there the launch form decides which XCD's L2 holds

@@ -231,6 +231,49 @@ def test_gemm_large_tiles(shape, layout, dtype, tile, lib):
     assert torch.equal(c, c128)
 
 
+# Shapes with >= 192 tiles of 256x288 (as above for the ring of four).
+NINE_BLOCKS = [(8192, 2304, 32), (7944, 2312, 96), (8192, 1736, 160), (6152, 2304, 448), (8192, 2304, 768),
+               (8192, 2024, 1056), (8192, 2309, 192)]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=lambda d: NAME[d])
+@pytest.mark.parametrize("layout", [(False, False), (False, True), (True, False), (True, True)],
+                         ids=["nn", "nt", "tn", "tt"])
+@pytest.mark.parametrize("shape", NINE_BLOCKS, ids=lambda s: "x".join(map(str, s)))
+def test_gemm_256x288_tile(shape, layout, dtype, lib, monkeypatch):
+    """The member whose four waves lie one above the other and all read the whole B tile (two of a
+    wave's eighteen accumulator blocks in ordinary registers): bias, activation and residual, against
+    the oracle on sampled rows and bit for bit against the 128x128 kernel; nothing is written behind
+    the last row."""
+    from metalhlo_amd import kernels
+    M, N, K = shape
+    ta, tb = layout
+    if not ((not ta or M % 8 == 0) and (tb or N % 8 == 0)):
+        pytest.skip("operand rows off 16-byte boundaries run the scalar kernel")
+    a, b = _ab(M, N, K, dtype, 45, ta, tb)
+    rng = np.random.default_rng(46)
+    bias = to_dev(rng.standard_normal(N) * 0.5, dtype)
+    r = to_dev(rng.standard_normal((M, N)), dtype)
+    monkeypatch.setenv("MHIP_GEMM_TILE", "2570")
+    guard = torch.full((M * N + 64,), 7.0, dtype=dtype, device="cuda")
+    c = kernels.matmul(a, b, bias, "gelu", trans_a=ta, trans_b=tb, out=guard[:M * N].view(M, N))
+    assert lib.mhip_gemm_last_variant() == 2570
+    cr = kernels.matmul(a, b, bias, "none", trans_a=ta, trans_b=tb, residual=r)
+    assert lib.mhip_gemm_last_variant() == 2570
+    assert torch.all(guard[M * N:] == 7.0)
+    monkeypatch.setenv("MHIP_GEMM_TILE", "128")
+    assert torch.equal(c, kernels.matmul(a, b, bias, "gelu", trans_a=ta, trans_b=tb))
+    assert torch.equal(cr, kernels.matmul(a, b, bias, "none", trans_a=ta, trans_b=tb, residual=r))
+    rows = np.unique(np.r_[0, 31, 32, 63, 64, 255, 256, M - 1, rng.integers(0, M, 40)])
+    A = as_f64(a).T if ta else as_f64(a)
+    B = as_f64(b).T if tb else as_f64(b)
+    exp = oracle.matmul_bias_act(A[rows], B, as_f64(bias), "gelu")
+    assert_close(c[rows], exp, TOL[dtype], f"gemm 256x288 {shape} {layout}")
+    exp = oracle.matmul_bias_act(A[rows], B, as_f64(bias), "none")
+    exp = as_f64(to_dev(exp, dtype).cpu()) + as_f64(r)[rows]          # product rounded, then the residual added
+    assert_close(cr[rows], exp, TOL[dtype], f"gemm 256x288 + residual {shape} {layout}")
+
+
 # Shapes with >= 192 tiles of 128x192 (single stage, exits at every position of the unrolled ring of six,
 # several trips; M and N ragged against the tile and, once, N odd).
 SMALL_ROWS = [(8192, 768, 32), (4104, 1160, 96), (8192, 776, 160), (6152, 960, 224), (8192, 768, 768), (4096, 1544, 1056),
@@ -274,7 +317,8 @@ def test_gemm_128x192_tile(shape, layout, dtype, lib, monkeypatch):
     assert_close(cr[rows], exp, TOL[dtype], f"gemm 128x192 + residual {shape} {layout}")
 
 
-@pytest.mark.parametrize("tile", ["2560", "2561", "2567", "2568", "2569"], ids=["256x256", "256x128", "256x384", "256x128-two-per-cu", "128x192"])
+@pytest.mark.parametrize("tile", ["2560", "2561", "2567", "2568", "2569", "2570"],
+                         ids=["256x256", "256x128", "256x384", "256x128-two-per-cu", "128x192", "256x288"])
 def test_gemm_ring_kernels_batched(tile, lib, monkeypatch):
     """The ring kernels on a strided batch (one grid row per matrix): every batch element against the
     oracle on sampled rows and bit for bit against the 128x128 kernel."""
@@ -590,7 +634,7 @@ def test_gemm_ring_kernel_takes_wide_and_deep_operands(lib):
         a = to_dev(rng.uniform(-1, 1, (M, K)), torch.bfloat16)
         b = to_dev(rng.uniform(-1, 1, (K, N)) * (K ** -0.5), torch.bfloat16)
         c = kernels.matmul(a, b)
-        assert 2560 <= lib.mhip_gemm_last_variant() <= 2569, (M, N, K, lib.mhip_gemm_last_variant())
+        assert 2560 <= lib.mhip_gemm_last_variant() <= 2570, (M, N, K, lib.mhip_gemm_last_variant())
         rows = np.r_[0, 255, 256, M - 1, rng.integers(0, M, 12)]
         assert_close(c[rows], as_f64(a[rows]) @ as_f64(b), 2e-2, f"gemm {M}x{N}x{K}")
     # fp32 operands run none of the 16-bit variants

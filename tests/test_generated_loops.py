@@ -56,7 +56,7 @@ def test_every_written_register_is_declared():
             written |= regs
         assert written, name
         assert not (written - declared), f"{name} writes undeclared registers {sorted(written - declared)}"
-    for stem in ("gemm_stream_loop_", "gemm256_loop_", "gemm256x128_loop_", "gemm256x384_loop_", "gemm_pair_loop_", "gemm128x192_loop_", "fa_pipe_loop_"):
+    for stem in ("gemm_stream_loop_", "gemm256_loop_", "gemm256x128_loop_", "gemm256x384_loop_", "gemm_pair_loop_", "gemm128x192_loop_", "gemm256x288_loop_", "fa_pipe_loop_"):
         assert any(n.startswith(stem) for n in names), stem
 
 

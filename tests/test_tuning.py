@@ -62,7 +62,7 @@ def test_gemm_autotune_picks_a_valid_variant_and_keeps_results():
         before = kernels.matmul(a, b, trans_b=tb)
         variant, us = kernels.autotune_matmul(a, b, trans_b=tb, iters=5)
         tiles = ((M + 255) // 256) * ((N + 255) // 256)
-        ring = (2560, 2561, 2562, 2563, 2564, 2565, 2566, 2567, 2568, 2569)      # the generated family, streamed tiles, the column split
+        ring = (2560, 2561, 2562, 2563, 2564, 2565, 2566, 2567, 2568, 2569, 2570)      # the generated family, streamed tiles, the column split
         assert variant in ((128, 256) + ring if tiles >= 192 else (128, 256, 2561, 2564, 2565, 2568, 2569)) and us > 0
         tuned = kernels.matmul(a, b, trans_b=tb)
         # the tuned launch against the oracle on sampled rows ...
