@@ -41,17 +41,17 @@ PEAK_CLOCK_MHZ = 2400.0     # the shader clock the matrix peak is quoted at
 # HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by what the same
 # counter reads for the 'copy' workload (256 MiB in, 256 MiB out); see profiles/<workload>.txt.
 # TRAFFIC_COMMIT: the commit of this repository the counter runs were taken at (the profiles say so too).
-TRAFFIC_COMMIT = "1a0c8b4"
+TRAFFIC_COMMIT = "78f698b"
 MEASURED_TRAFFIC = {
-    "gemm": 237457913,
-    "gemm_f32": 813052194,
-    "attention": 750939674,
-    "attention_full": 268935613,
-    "attention_f32": 1879698027,
-    "softmax": 536712540,
-    "layer_norm": 536879315,
-    "rms_norm": 536776598,
-    "bias_gelu": 536737125,
+    "gemm": 237458425,
+    "gemm_f32": 812880561,
+    "attention": 753138116,
+    "attention_full": 268936609,
+    "attention_f32": 1879189489,
+    "softmax": 536739646,
+    "layer_norm": 536883062,
+    "rms_norm": 536780726,
+    "bias_gelu": 536741693,
     "copy": 536870912,
 }
 
