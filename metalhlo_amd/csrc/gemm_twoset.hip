@@ -1,7 +1,8 @@
 // The members of the ring-kernel family that run on two fragment sets (gen_gemm256_loop.py, second part ->
-// gemm_twoset_loop.inc): the 256x384 tile, whose accumulators do not fit the accumulation registers, and
-// the 256x128 tile in 256 registers a wave for two workgroups per compute unit.  Operand layouts and the
-// epilogue of the narrow tile are those of gemm256.hip (gemm_ring.h).
+// gemm_twoset_loop.inc): the 256x384 and the 256x288 tile, whose accumulators do not fit the accumulation
+// registers, the 128x192 tile for problems with few columns, and the 256x128 tile in 256 registers a wave
+// for two workgroups per compute unit.  Operand layouts and the epilogue of the narrow tile are those of
+// gemm256.hip (gemm_ring.h).
 #include "gemm_ring.h"
 
 namespace mhip {

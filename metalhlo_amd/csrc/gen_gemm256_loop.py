@@ -518,6 +518,8 @@ def emit(name, mnem, ka, kb):
 # latency run under the other's MFMAs.  Register map: fragment set n: A v[24n : 24n+15], B
 # v[24n+16 : 24n+23]; v[48:55] A read addresses, v[56:59] B; v60 / v61 global offsets, v62 / v63 the
 # same + 64; accumulator (i, j) at a[16 (2 i + j) : +15] as in the one-workgroup kernel.
+# Two more members, described where they are defined: the 128x192 tile (`_x192`) and the 256x288
+# tile (`_x288`).
 class TwoSet:
     """One member of the two-fragment-set family: geometry and register map."""
 
